@@ -1,0 +1,294 @@
+"""Host-side mirror of the reference's attention launchers over libhipml_attn.so.
+
+Function names and argument order follow the reference's Rust launchers
+(`launch_kv::launch_ptrs`, `launch_cols_ptrs`, `Launcher::kv_encode*`,
+`attn_decode_batch`, `AttnLayer::chunk_attention_q8_split`, ...); tensors are
+torch CUDA(HIP) tensors used purely as device memory.  Every call goes through
+the C ABI declared in include/hipml_attn.h and raises :class:`HipmlError` with
+the library's message on a non-zero return, like the reference's `Err(String)`.
+
+There is no CPU fallback: if the shared library is missing this module raises.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libhipml_attn.so")
+
+ROW_BYTES = 272      # one head_dim-256 row of q8_0: 8 blocks x 34 bytes
+BLOCK_BYTES = 34
+HEAD_DIM = 256
+
+EXPORTS = [
+    "hipml_attn_init", "hipml_attn_last_error", "hipml_attn_version",
+    "hipml_attn_decode_splits", "hipml_attn_batch_splits", "hipml_attn_chunk_splits",
+    "hipml_rope_table_bytes", "hipml_rope_table_fill_host", "hipml_rope_set_table",
+    "hipml_mrope_f32", "hipml_mrope_rows_f32", "hipml_rope_chunk_f32",
+    "hipml_kv_encode", "hipml_kv_encode_bulk", "hipml_kv_encode_rows",
+    "hipml_attn_decode_kv", "hipml_attn_decode_kv_cols", "hipml_attn_decode_rows",
+    "hipml_attn_decode_batch", "hipml_attn_decode_batch_cols",
+    "hipml_attn_chunk_q8_split", "hipml_q_gate_f32",
+]
+
+
+class HipmlError(RuntimeError):
+    """A launcher refused its arguments or the HIP runtime refused the launch."""
+
+    def __init__(self, code: int, message: str):
+        super().__init__(f"{message} (status {code})")
+        self.code = code
+        self.message = message
+
+
+_lib = None
+
+
+def lib() -> C.CDLL:
+    """Load libhipml_attn.so; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `python -m hipml_amd.build` "
+                "(there is no CPU fallback)")
+        l = C.CDLL(LIB_PATH)
+        vp, i, f, sz = C.c_void_p, C.c_int, C.c_float, C.c_size_t
+        sig = {
+            "hipml_attn_init": (i, [i]),
+            "hipml_attn_last_error": (C.c_char_p, []),
+            "hipml_attn_version": (C.c_char_p, []),
+            "hipml_attn_decode_splits": (i, [i, i]),
+            "hipml_attn_batch_splits": (i, [i, i, i]),
+            "hipml_attn_chunk_splits": (i, [i, i, i]),
+            "hipml_rope_table_bytes": (sz, [i, i]),
+            "hipml_rope_table_fill_host": (i, [vp, f, i, i]),
+            "hipml_rope_set_table": (i, [vp, f, i, i]),
+            "hipml_mrope_f32": (i, [vp, vp, vp, i, i, i, i, i, i, i, vp, f]),
+            "hipml_mrope_rows_f32": (i, [vp, vp, vp, i, i, i, i, i, i, i, vp, i, f]),
+            "hipml_rope_chunk_f32": (i, [vp, vp, vp, i, i, i, i, f, i, i]),
+            "hipml_kv_encode": (i, [vp, vp, i, vp, vp, vp, vp, i, i, i]),
+            "hipml_kv_encode_bulk": (i, [vp, i, vp, vp, vp, vp, i, i, i, i, i, i]),
+            "hipml_kv_encode_rows": (i, [vp, i, vp, vp, vp, vp, i, i, i, vp, sz, i]),
+            "hipml_attn_decode_kv": (i, [vp, vp, i, vp, vp, vp, vp, vp, vp, i, i, i, i, f, i, sz,
+                                         sz]),
+            "hipml_attn_decode_kv_cols": (i, [vp, i, vp, vp, vp, vp, vp, vp, vp, i, i, i, i, f, i,
+                                              i, sz, sz, sz]),
+            "hipml_attn_decode_rows": (i, [vp, i, vp, vp, vp, vp, vp, vp, vp, i, i, i, i, f, i, sz,
+                                           sz, sz, sz, i]),
+            "hipml_attn_decode_batch": (i, [vp, i, vp, vp, vp, vp, vp, vp, vp, i, i, i, i, f, i,
+                                            sz, sz, sz, sz, i, i]),
+            "hipml_attn_decode_batch_cols": (i, [vp, i, vp, vp, vp, vp, vp, vp, vp, i, i, i, i, f,
+                                                 i, sz, sz, sz, sz, i, vp]),
+            "hipml_attn_chunk_q8_split": (i, [vp, vp, vp, vp, vp, i, i, i, i, i, i, i, vp, vp, i]),
+            "hipml_q_gate_f32": (i, [vp, vp, vp, vp, sz]),
+        }
+        for name, (res, args) in sig.items():
+            fn = getattr(l, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = l
+    return _lib
+
+
+def _check(rc: int) -> None:
+    if rc != 0:
+        raise HipmlError(rc, lib().hipml_attn_last_error().decode())
+
+
+def _p(t) -> int:
+    """Device (or host) address of a tensor; None -> NULL."""
+    return 0 if t is None else t.data_ptr()
+
+
+def _stream(stream=None) -> int:
+    s = stream if stream is not None else torch.cuda.current_stream()
+    return s.cuda_stream
+
+
+def init(device: int = 0) -> None:
+    _check(lib().hipml_attn_init(device))
+
+
+def version() -> str:
+    return lib().hipml_attn_version().decode()
+
+
+# ---- split policies ----------------------------------------------------------------
+
+def decode_splits(seq: int, n_kv: int = 4) -> int:
+    return lib().hipml_attn_decode_splits(seq, n_kv)
+
+
+def batch_splits(stride: int, n_kv: int, slots: int) -> int:
+    return lib().hipml_attn_batch_splits(stride, n_kv, slots)
+
+
+def chunk_splits(pos0: int, tokens: int, n_kv: int = 4) -> int:
+    return lib().hipml_attn_chunk_splits(pos0, tokens, n_kv)
+
+
+# ---- RoPE ----------------------------------------------------------------------------
+
+_rope_tables = {}
+
+
+def rope_table(theta: float, n_rot: int, max_pos: int, device="cuda") -> torch.Tensor:
+    """Build the host cos/sin table, upload it and register it with the library.
+    The device tensor is kept alive here (the library does not own it)."""
+    key = (float(theta), int(n_rot), int(max_pos), str(device))
+    if key not in _rope_tables:
+        host = torch.empty((max_pos, n_rot // 2, 2), dtype=torch.float32)
+        _check(lib().hipml_rope_table_fill_host(host.data_ptr(), theta, n_rot, max_pos))
+        _rope_tables[key] = host.to(device)
+    tab = _rope_tables[key]
+    _check(lib().hipml_rope_set_table(tab.data_ptr(), theta, n_rot, max_pos))
+    return tab
+
+
+def rope_clear_table() -> None:
+    _check(lib().hipml_rope_set_table(0, 0.0, 0, 0))
+
+
+def mrope(x, y, n_heads, head_dim, n_rot, sections, pos, theta, stream=None):
+    """`mrope_f32`: pos is a device int32[4]."""
+    s0, s1, s2, s3 = sections
+    _check(lib().hipml_mrope_f32(_stream(stream), _p(x), _p(y), n_heads, head_dim, n_rot, s0, s1,
+                                 s2, s3, _p(pos), theta))
+
+
+def mrope_rows(x, y, n_heads, head_dim, n_rot, sections, pos, rows, theta, stream=None):
+    """`mrope_b`: pos is a device int32[rows][2] of (pos, seq)."""
+    s0, s1, s2, s3 = sections
+    _check(lib().hipml_mrope_rows_f32(_stream(stream), _p(x), _p(y), n_heads, head_dim, n_rot, s0,
+                                      s1, s2, s3, _p(pos), rows, theta))
+
+
+def rope_chunk(q, k, n_head, n_kv, head_dim, n_rot, theta, pos0, tokens, stream=None):
+    _check(lib().hipml_rope_chunk_f32(_stream(stream), _p(q), _p(k), n_head, n_kv, head_dim, n_rot,
+                                      theta, pos0, tokens))
+
+
+# ---- KV append ------------------------------------------------------------------------
+
+def kv_encode(step, dtype, k_in, v_in, k_cache, v_cache, n_kv, head_dim, stride, stream=None):
+    _check(lib().hipml_kv_encode(_stream(stream), _p(step), dtype, _p(k_in), _p(v_in), _p(k_cache),
+                                 _p(v_cache), n_kv, head_dim, stride))
+
+
+def kv_encode_bulk(dtype, k_f32, v_f32, k_cache, v_cache, n_kv, head_dim, stride, start, src0,
+                   rows, stream=None):
+    _check(lib().hipml_kv_encode_bulk(_stream(stream), dtype, _p(k_f32), _p(v_f32), _p(k_cache),
+                                      _p(v_cache), n_kv, head_dim, stride, start, src0, rows))
+
+
+def kv_encode_rows(dtype, k_f32, v_f32, k_cache, v_cache, n_kv, head_dim, stride, pos, slot_bytes,
+                   slots, stream=None):
+    _check(lib().hipml_kv_encode_rows(_stream(stream), dtype, _p(k_f32), _p(v_f32), _p(k_cache),
+                                      _p(v_cache), n_kv, head_dim, stride, _p(pos), slot_bytes,
+                                      slots))
+
+
+# ---- decode -------------------------------------------------------------------------------
+
+def attn_decode_kv(step, dtype, q, k, v, part_acc, part_ml, out, n_heads, n_kv, head_dim, stride,
+                   scale, splits, k_off=0, v_off=0, stream=None):
+    """`launch_kv::launch_ptrs`."""
+    _check(lib().hipml_attn_decode_kv(_stream(stream), _p(step), dtype, _p(q), _p(k), _p(v),
+                                      _p(part_acc), _p(part_ml), _p(out), n_heads, n_kv, head_dim,
+                                      stride, scale, splits, k_off, v_off))
+
+
+def attn_decode_kv_cols(dtype, pos, q, k, v, part_acc, part_ml, out, n_heads, n_kv, head_dim,
+                        stride, scale, splits, cols, acc_slot, ml_slot, q_slot, stream=None):
+    """`launch_kv::launch_cols_ptrs`."""
+    _check(lib().hipml_attn_decode_kv_cols(_stream(stream), dtype, _p(pos), _p(q), _p(k), _p(v),
+                                           _p(part_acc), _p(part_ml), _p(out), n_heads, n_kv,
+                                           head_dim, stride, scale, splits, cols, acc_slot,
+                                           ml_slot, q_slot))
+
+
+def attn_decode_rows(dtype, pos, q, k_cache, v_cache, part_acc, part_ml, out, n_heads, n_kv,
+                     head_dim, stride, scale, splits, kv_slot_bytes, acc_slot, ml_slot, q_slot,
+                     slots, stream=None):
+    """`Launcher::attn_decode_rows_ptr`."""
+    _check(lib().hipml_attn_decode_rows(_stream(stream), dtype, _p(pos), _p(q), _p(k_cache),
+                                        _p(v_cache), _p(part_acc), _p(part_ml), _p(out), n_heads,
+                                        n_kv, head_dim, stride, scale, splits, kv_slot_bytes,
+                                        acc_slot, ml_slot, q_slot, slots))
+
+
+def attn_decode_batch(dtype, pos, q, k_cache, v_cache, part_acc, part_ml, out, n_heads, n_kv,
+                      head_dim, stride, scale, splits, kv_slot_bytes, acc_slot, ml_slot, q_slot,
+                      slots, live_seq=0, stream=None):
+    """`Launcher::attn_decode_batch`."""
+    _check(lib().hipml_attn_decode_batch(_stream(stream), dtype, _p(pos), _p(q), _p(k_cache),
+                                         _p(v_cache), _p(part_acc), _p(part_ml), _p(out), n_heads,
+                                         n_kv, head_dim, stride, scale, splits, kv_slot_bytes,
+                                         acc_slot, ml_slot, q_slot, slots, live_seq))
+
+
+def attn_decode_batch_cols(dtype, pos, q, k_cache, v_cache, part_acc, part_ml, out, n_heads, n_kv,
+                           head_dim, stride, scale, splits, kv_slot_bytes, acc_slot, ml_slot,
+                           q_slot, cols_per_slot, stream=None):
+    """Plain and MTP-verify slots in one launch; cols_per_slot is a host sequence."""
+    arr = (C.c_int32 * len(cols_per_slot))(*[int(c) for c in cols_per_slot])
+    _check(lib().hipml_attn_decode_batch_cols(
+        _stream(stream), dtype, _p(pos), _p(q), _p(k_cache), _p(v_cache), _p(part_acc),
+        _p(part_ml), _p(out), n_heads, n_kv, head_dim, stride, scale, splits, kv_slot_bytes,
+        acc_slot, ml_slot, q_slot, len(cols_per_slot), C.addressof(arr)))
+
+
+# ---- chunk prefill ---------------------------------------------------------------------------
+
+def chunk_attention_q8_split(q, kc, vc, out, n_head, n_kv, head_dim, pos0, tokens, dtype, stride,
+                             part_acc, part_ml, splits, stream=None):
+    """`AttnLayer::chunk_attention_q8_split` (dtype 1 = q8_0)."""
+    _check(lib().hipml_attn_chunk_q8_split(_stream(stream), _p(q), _p(kc), _p(vc), _p(out), n_head,
+                                           n_kv, head_dim, pos0, tokens, dtype, stride,
+                                           _p(part_acc), _p(part_ml), splits))
+
+
+def chunk_scratch(tokens: int, n_head: int, splits: int, device="cuda"):
+    """Split-K scratch sized as the reference's prefill path sizes it."""
+    qslots = (tokens + 31) // 32 * 32
+    acc = torch.empty((splits, qslots, n_head, HEAD_DIM), dtype=torch.float32, device=device)
+    ml = torch.empty((splits, qslots, n_head, 2), dtype=torch.float32, device=device)
+    return acc, ml
+
+
+# ---- gate -----------------------------------------------------------------------------------------
+
+def q_gate(x, gate, y, n=None, stream=None):
+    n = x.numel() if n is None else n
+    _check(lib().hipml_q_gate_f32(_stream(stream), _p(x), _p(gate), _p(y), n))
+
+
+# ---- cache owner ------------------------------------------------------------------------------------
+
+class DeepKv:
+    """One layer's q8_0 cache plus its decode scratch: the role of the reference's
+    `DeepKv` (crates/hipml-model/src/gpu/deep_kv.rs:11-83).  K and V are separate
+    uint8 tensors of [n_kv][stride][272]."""
+
+    def __init__(self, n_heads=24, n_kv=4, head_dim=HEAD_DIM, stride=4096, max_cols=1,
+                 device="cuda"):
+        assert head_dim == HEAD_DIM
+        self.n_heads, self.n_kv, self.head_dim, self.seq = n_heads, n_kv, head_dim, stride
+        self.k = torch.zeros((n_kv, stride, ROW_BYTES), dtype=torch.uint8, device=device)
+        self.v = torch.zeros((n_kv, stride, ROW_BYTES), dtype=torch.uint8, device=device)
+        self.max_splits = max(decode_splits(stride, n_kv), 1)
+        self.max_cols = max_cols
+        self.part_acc = torch.empty((max_cols, n_heads, self.max_splits, head_dim),
+                                    dtype=torch.float32, device=device)
+        self.part_ml = torch.empty((max_cols, n_heads, self.max_splits, 2), dtype=torch.float32,
+                                   device=device)
+
+    def splits(self, seq: int) -> int:
+        return min(decode_splits(seq, self.n_kv), self.max_splits)
+
+    def bytes(self) -> int:
+        return 2 * self.n_kv * self.seq * ROW_BYTES

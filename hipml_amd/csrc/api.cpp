@@ -1,0 +1,535 @@
+// C ABI of libhipml_attn.so: argument validation and launcher selection.
+// Every entry point validates on the host, then launches asynchronously on the
+// caller's stream; nothing here allocates, frees or synchronises.
+
+#include "common.h"
+
+#include <math.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+namespace hipml {
+
+static thread_local char g_err[512] = "";
+static RopeTable g_rope = {nullptr, 0.0f, 0, 0};
+static bool g_inited = false;
+
+int fail(int code, const char *fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+void clear_error() { g_err[0] = '\0'; }
+
+int launched(const char *what)
+{
+    hipError_t e = hipGetLastError();
+    if (e == hipSuccess)
+        return 0;
+    snprintf(g_err, sizeof(g_err), "%s launch failed: %d (%s)", what, (int)e, hipGetErrorString(e));
+    return (int)e;
+}
+
+int check_heads(int n_heads, int n_kv, int head_dim)
+{
+    if (n_kv <= 0 || n_heads <= 0 || n_heads % n_kv != 0)
+        return fail(HIPML_ATTN_E_SHAPE, "n_heads %d is not a multiple of n_kv %d", n_heads, n_kv);
+    const int group = n_heads / n_kv;
+    if (group > kMaxGroup)
+        return fail(HIPML_ATTN_E_SHAPE, "GQA group %d > %d: one workgroup covers at most %d heads",
+                    group, kMaxGroup, kMaxGroup);
+    if (head_dim != kHeadDim)
+        return fail(HIPML_ATTN_E_SHAPE, "head_dim %d: the gfx950 attention kernels are head_dim %d only",
+                    head_dim, kHeadDim);
+    return 0;
+}
+
+static int check_q8(int dtype)
+{
+    if (dtype == 0)
+        return 0;
+    if (dtype == 1)
+        return fail(HIPML_ATTN_E_UNSUPPORTED, "KV dtype 1 (q4_0) is not built; only q8_0 (0)");
+    return fail(HIPML_ATTN_E_UNSUPPORTED, "unknown KV dtype %d", dtype);
+}
+
+static int check_aligned16(const void *p, const char *name)
+{
+    if (((uintptr_t)p & 15) != 0)
+        return fail(HIPML_ATTN_E_RANGE, "%s must be 16-byte aligned", name);
+    return 0;
+}
+
+#define REQUIRE_PTR(p)                                                                              \
+    do {                                                                                            \
+        if ((p) == nullptr)                                                                         \
+            return fail(HIPML_ATTN_E_NULL, "%s is NULL", #p);                                        \
+    } while (0)
+
+static int decode_common(hipStream_t st, const int32_t *pos, const float *q, const void *k,
+                         const void *v, float *part_acc, float *part_ml, float *out, int n_heads,
+                         int n_kv, int head_dim, int stride, float scale, int splits,
+                         size_t kv_slot_bytes, size_t acc_slot, size_t ml_slot, size_t q_slot,
+                         int slots, const int32_t *cols_per_slot)
+{
+    REQUIRE_PTR(pos);
+    REQUIRE_PTR(q);
+    REQUIRE_PTR(k);
+    REQUIRE_PTR(v);
+    REQUIRE_PTR(part_acc);
+    REQUIRE_PTR(part_ml);
+    REQUIRE_PTR(out);
+    int rc = check_heads(n_heads, n_kv, head_dim);
+    if (rc)
+        return rc;
+    if (stride <= 0)
+        return fail(HIPML_ATTN_E_RANGE, "stride %d must be positive", stride);
+    if (splits < 1 || splits > 4096)
+        return fail(HIPML_ATTN_E_RANGE, "splits %d outside 1..4096", splits);
+    if (slots < 1 || slots > kMaxSlots)
+        return fail(HIPML_ATTN_E_RANGE, "slots %d outside 1..%d", slots, kMaxSlots);
+    if ((rc = check_aligned16(k, "k cache")) || (rc = check_aligned16(v, "v cache")) ||
+        (rc = check_aligned16(q, "q")) || (rc = check_aligned16(part_acc, "part_acc")))
+        return rc;
+    if (kv_slot_bytes % 16 != 0 || q_slot % 4 != 0 || acc_slot % 4 != 0)
+        return fail(HIPML_ATTN_E_RANGE, "slot strides must keep 16-byte alignment");
+
+    DecodeLaunch L;
+    memset(&L, 0, sizeof(L));
+    L.q = q;
+    L.k = static_cast<const uint8_t *>(k);
+    L.v = static_cast<const uint8_t *>(v);
+    L.part_acc = part_acc;
+    L.part_ml = part_ml;
+    L.out = out;
+    L.pos = pos;
+    L.n_heads = n_heads;
+    L.n_kv = n_kv;
+    L.stride = stride;
+    L.splits = splits;
+    L.slots = slots;
+    L.scale = scale;
+    L.kv_slot_bytes = kv_slot_bytes;
+    L.acc_slot = acc_slot;
+    L.ml_slot = ml_slot;
+    L.q_slot = q_slot;
+    int rows = 0, max_cols = 0;
+    for (int s = 0; s < slots; s++) {
+        const int c = cols_per_slot ? cols_per_slot[s] : 1;
+        if (c < 1 || c > kMaxCols)
+            return fail(HIPML_ATTN_E_RANGE, "slot %d carries %d query rows; 1..%d supported", s, c,
+                        kMaxCols);
+        L.row0[s] = (uint16_t)rows;
+        L.cols[s] = (uint8_t)c;
+        rows += c;
+        max_cols = c > max_cols ? c : max_cols;
+    }
+    L.total_rows = rows;
+    L.max_cols = max_cols;
+    return launch_decode_q8(st, L);
+}
+
+} // namespace hipml
+
+using namespace hipml;
+
+extern "C" {
+
+int hipml_attn_init(int device)
+{
+    clear_error();
+    hipDeviceProp_t prop;
+    hipError_t e = hipGetDeviceProperties(&prop, device);
+    if (e != hipSuccess)
+        return fail((int)e, "hipGetDeviceProperties(%d) failed: %d (%s)", device, (int)e,
+                    hipGetErrorString(e));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return fail(HIPML_ATTN_E_DEVICE, "device %d is %s; this library is built for gfx950 only",
+                    device, prop.gcnArchName);
+    g_inited = true;
+    return 0;
+}
+
+const char *hipml_attn_last_error(void) { return g_err; }
+
+const char *hipml_attn_version(void) { return "hipml-attn-mi355x 0.1 (gfx950)"; }
+
+// ---- split policies -------------------------------------------------------------------
+
+int hipml_attn_decode_splits(int seq, int n_kv)
+{
+    // One workgroup of four waves walks 32-key tiles; give every workgroup at least one
+    // tile per wave (128 keys) and stop at one workgroup per CU (256) across the KV heads.
+    if (seq < 1 || n_kv < 1)
+        return 1;
+    int by_work = (seq + 127) / 128;
+    int by_cus = 256 / n_kv;
+    if (by_cus < 1)
+        by_cus = 1;
+    int s = by_work < by_cus ? by_work : by_cus;
+    return s < 1 ? 1 : s;
+}
+
+int hipml_attn_batch_splits(int stride, int n_kv, int slots)
+{
+    if (stride < 1 || n_kv < 1 || slots < 1)
+        return 1;
+    int by_work = (stride + 127) / 128;
+    int by_cus = (2 * 256) / (n_kv * slots);
+    if (by_cus < 1)
+        by_cus = 1;
+    int s = by_work < by_cus ? by_work : by_cus;
+    return s < 1 ? 1 : s;
+}
+
+int hipml_attn_chunk_splits(int pos0, int tokens, int n_kv)
+{
+    if (tokens < 1 || n_kv < 1)
+        return 1;
+    const int qtiles = (tokens + 31) / 32;
+    const int wgs = qtiles * n_kv;
+    if (wgs >= 512)
+        return 1;
+    int s = (512 + wgs - 1) / wgs;
+    const int keys = pos0 + tokens;
+    const int by_work = (keys + 255) / 256; // at least 256 keys per slice
+    if (s > by_work)
+        s = by_work;
+    if (s > 16)
+        s = 16;
+    return s < 1 ? 1 : s;
+}
+
+// ---- RoPE ----------------------------------------------------------------------------------
+
+size_t hipml_rope_table_bytes(int n_rot, int max_pos)
+{
+    if (n_rot <= 0 || (n_rot & 1) || max_pos <= 0)
+        return 0;
+    return (size_t)max_pos * (size_t)(n_rot / 2) * 2 * sizeof(float);
+}
+
+int hipml_rope_table_fill_host(float *host_table, float theta_base, int n_rot, int max_pos)
+{
+    clear_error();
+    REQUIRE_PTR(host_table);
+    if (n_rot <= 0 || (n_rot & 1) || max_pos <= 0)
+        return fail(HIPML_ATTN_E_RANGE, "n_rot %d must be even and positive, max_pos %d positive",
+                    n_rot, max_pos);
+    const int half = n_rot / 2;
+    for (int k = 0; k < half; k++) {
+        // same expression, same libm, as the CPU definition (ops.rs:296-300 of the reference)
+        const double freq = pow((double)theta_base, -2.0 * (double)k / (double)n_rot);
+        for (int p = 0; p < max_pos; p++) {
+            const double ang = (double)p * freq;
+            float *e = host_table + ((size_t)p * half + k) * 2;
+            e[0] = (float)cos(ang);
+            e[1] = (float)sin(ang);
+        }
+    }
+    return 0;
+}
+
+int hipml_rope_set_table(const float *dev_table, float theta_base, int n_rot, int max_pos)
+{
+    clear_error();
+    if (dev_table != nullptr && (n_rot <= 0 || (n_rot & 1) || max_pos <= 0))
+        return fail(HIPML_ATTN_E_RANGE, "n_rot %d must be even and positive, max_pos %d positive",
+                    n_rot, max_pos);
+    g_rope.dev = dev_table;
+    g_rope.theta = theta_base;
+    g_rope.n_rot = n_rot;
+    g_rope.max_pos = dev_table ? max_pos : 0;
+    return 0;
+}
+
+static int check_rope(int n_heads, int head_dim, int n_rot, float theta)
+{
+    if (n_heads <= 0 || head_dim <= 0)
+        return fail(HIPML_ATTN_E_SHAPE, "n_heads %d / head_dim %d must be positive", n_heads,
+                    head_dim);
+    if (n_rot <= 0 || (n_rot & 1) || n_rot > head_dim)
+        return fail(HIPML_ATTN_E_SHAPE, "n_rot %d must be even and <= head_dim %d", n_rot, head_dim);
+    if (g_rope.dev == nullptr || g_rope.theta != theta || g_rope.n_rot != n_rot)
+        return fail(HIPML_ATTN_E_STATE,
+                    "no RoPE table registered for theta %g n_rot %d (hipml_rope_set_table)", theta,
+                    n_rot);
+    return 0;
+}
+
+int hipml_mrope_f32(hipml_stream_t stream, const float *x, float *y, int n_heads, int head_dim,
+                    int n_rot, int s0, int s1, int s2, int s3, const int32_t *pos,
+                    float theta_base)
+{
+    clear_error();
+    REQUIRE_PTR(x);
+    REQUIRE_PTR(y);
+    REQUIRE_PTR(pos);
+    int rc = check_rope(n_heads, head_dim, n_rot, theta_base);
+    if (rc)
+        return rc;
+    if (s0 < 0 || s1 < 0 || s2 < 0 || s3 < 0)
+        return fail(HIPML_ATTN_E_RANGE, "negative M-RoPE section");
+    return launch_mrope(as_stream(stream), x, y, n_heads, head_dim, n_rot, s0, s1, s2, s3, pos, 0,
+                        1, theta_base, g_rope);
+}
+
+int hipml_mrope_rows_f32(hipml_stream_t stream, const float *x, float *y, int n_heads,
+                         int head_dim, int n_rot, int s0, int s1, int s2, int s3,
+                         const int32_t *pos, int rows, float theta_base)
+{
+    clear_error();
+    REQUIRE_PTR(x);
+    REQUIRE_PTR(y);
+    REQUIRE_PTR(pos);
+    int rc = check_rope(n_heads, head_dim, n_rot, theta_base);
+    if (rc)
+        return rc;
+    if (rows < 0)
+        return fail(HIPML_ATTN_E_RANGE, "rows %d is negative", rows);
+    if (rows == 0)
+        return 0;
+    return launch_mrope(as_stream(stream), x, y, n_heads, head_dim, n_rot, s0, s1, s2, s3, pos, 2,
+                        rows, theta_base, g_rope);
+}
+
+int hipml_rope_chunk_f32(hipml_stream_t stream, float *q, float *k, int n_head, int n_kv,
+                         int head_dim, int n_rot, float theta_base, int pos0, int tokens)
+{
+    clear_error();
+    REQUIRE_PTR(q);
+    REQUIRE_PTR(k);
+    int rc = check_rope(n_head, head_dim, n_rot, theta_base);
+    if (rc)
+        return rc;
+    if (n_kv <= 0)
+        return fail(HIPML_ATTN_E_SHAPE, "n_kv %d must be positive", n_kv);
+    if (pos0 < 0 || tokens < 0)
+        return fail(HIPML_ATTN_E_RANGE, "pos0 %d / tokens %d must be non-negative", pos0, tokens);
+    if (tokens == 0)
+        return 0;
+    return launch_rope_chunk(as_stream(stream), q, k, n_head, n_kv, head_dim, n_rot, theta_base,
+                             pos0, tokens, g_rope);
+}
+
+// ---- KV append -------------------------------------------------------------------------------
+
+static int check_encode(int dtype, const void *k, const void *v, const void *kc, const void *vc,
+                        int n_kv, int head_dim, int stride)
+{
+    int rc = check_q8(dtype);
+    if (rc)
+        return rc;
+    if (k == nullptr || v == nullptr || kc == nullptr || vc == nullptr)
+        return fail(HIPML_ATTN_E_NULL, "a K/V source or cache pointer is NULL");
+    if (n_kv <= 0)
+        return fail(HIPML_ATTN_E_SHAPE, "n_kv %d must be positive", n_kv);
+    if (head_dim <= 0 || head_dim % 32 != 0 || head_dim > 256)
+        return fail(HIPML_ATTN_E_SHAPE, "head_dim %d: must be 32..=256, multiple of 32", head_dim);
+    if (stride <= 0)
+        return fail(HIPML_ATTN_E_RANGE, "stride %d must be positive", stride);
+    return 0;
+}
+
+int hipml_kv_encode(hipml_stream_t stream, const int32_t *step, int dtype, const float *k_in,
+                    const float *v_in, void *k_cache, void *v_cache, int n_kv, int head_dim,
+                    int stride)
+{
+    clear_error();
+    REQUIRE_PTR(step);
+    int rc = check_encode(dtype, k_in, v_in, k_cache, v_cache, n_kv, head_dim, stride);
+    if (rc)
+        return rc;
+    return launch_kv_encode_q8(as_stream(stream), k_in, v_in, static_cast<uint8_t *>(k_cache),
+                               static_cast<uint8_t *>(v_cache), n_kv, head_dim, stride, step, 0, 0,
+                               1, 0, 0, 1);
+}
+
+int hipml_kv_encode_bulk(hipml_stream_t stream, int dtype, const float *k_f32, const float *v_f32,
+                         void *k_cache, void *v_cache, int n_kv, int head_dim, int stride,
+                         int start, int src0, int rows)
+{
+    clear_error();
+    int rc = check_encode(dtype, k_f32, v_f32, k_cache, v_cache, n_kv, head_dim, stride);
+    if (rc)
+        return rc;
+    if (start < 0 || src0 < 0 || rows < 0)
+        return fail(HIPML_ATTN_E_RANGE, "start %d / src0 %d / rows %d must be non-negative", start,
+                    src0, rows);
+    if ((long long)start + rows > stride)
+        return fail(HIPML_ATTN_E_RANGE, "rows [%d, %d) do not fit a cache of %d rows per head",
+                    start, start + rows, stride);
+    return launch_kv_encode_q8(as_stream(stream), k_f32, v_f32, static_cast<uint8_t *>(k_cache),
+                               static_cast<uint8_t *>(v_cache), n_kv, head_dim, stride, nullptr, 0,
+                               0, rows, start, src0, rows);
+}
+
+int hipml_kv_encode_rows(hipml_stream_t stream, int dtype, const float *k_f32, const float *v_f32,
+                         void *k_cache, void *v_cache, int n_kv, int head_dim, int stride,
+                         const int32_t *pos, size_t slot_bytes, int slots)
+{
+    clear_error();
+    REQUIRE_PTR(pos);
+    int rc = check_encode(dtype, k_f32, v_f32, k_cache, v_cache, n_kv, head_dim, stride);
+    if (rc)
+        return rc;
+    if (slots < 0)
+        return fail(HIPML_ATTN_E_RANGE, "slots %d is negative", slots);
+    return launch_kv_encode_q8(as_stream(stream), k_f32, v_f32, static_cast<uint8_t *>(k_cache),
+                               static_cast<uint8_t *>(v_cache), n_kv, head_dim, stride, pos, 2,
+                               slot_bytes, slots, 0, 0, slots);
+}
+
+// ---- decode ------------------------------------------------------------------------------------
+
+int hipml_attn_decode_kv(hipml_stream_t stream, const int32_t *step, int dtype, const float *q,
+                         const void *k, const void *v, float *part_acc, float *part_ml,
+                         float *out, int n_heads, int n_kv, int head_dim, int stride, float scale,
+                         int splits, size_t k_off, size_t v_off)
+{
+    clear_error();
+    int rc = check_q8(dtype);
+    if (rc)
+        return rc;
+    REQUIRE_PTR(k);
+    REQUIRE_PTR(v);
+    const size_t slice = (size_t)(n_heads > 0 ? n_heads : 0) * (size_t)(splits > 0 ? splits : 0);
+    return decode_common(as_stream(stream), step, q, static_cast<const uint8_t *>(k) + k_off,
+                         static_cast<const uint8_t *>(v) + v_off, part_acc, part_ml, out, n_heads,
+                         n_kv, head_dim, stride, scale, splits, 0, slice * kHeadDim, slice * 2,
+                         (size_t)n_heads * kHeadDim, 1, nullptr);
+}
+
+int hipml_attn_decode_kv_cols(hipml_stream_t stream, int dtype, const int32_t *pos,
+                              const float *q, const void *k, const void *v, float *part_acc,
+                              float *part_ml, float *out, int n_heads, int n_kv, int head_dim,
+                              int stride, float scale, int splits, int cols, size_t acc_slot,
+                              size_t ml_slot, size_t q_slot)
+{
+    clear_error();
+    // the reference's selector for its whole-group warp kernel is 4; 0 (q8_0) is accepted too
+    if (dtype != 4) {
+        int rc = check_q8(dtype);
+        if (rc)
+            return rc;
+    }
+    if (cols < 1 || cols > kMaxCols)
+        return fail(HIPML_ATTN_E_RANGE, "cols %d outside 1..%d", cols, kMaxCols);
+    const int32_t one_slot[1] = {cols};
+    return decode_common(as_stream(stream), pos, q, k, v, part_acc, part_ml, out, n_heads, n_kv,
+                         head_dim, stride, scale, splits, 0, acc_slot, ml_slot, q_slot, 1,
+                         one_slot);
+}
+
+int hipml_attn_decode_rows(hipml_stream_t stream, int dtype, const int32_t *pos, const float *q,
+                           const void *k_cache, const void *v_cache, float *part_acc,
+                           float *part_ml, float *out, int n_heads, int n_kv, int head_dim,
+                           int stride, float scale, int splits, size_t kv_slot_bytes,
+                           size_t acc_slot, size_t ml_slot, size_t q_slot, int slots)
+{
+    clear_error();
+    int rc = check_q8(dtype);
+    if (rc)
+        return rc;
+    if (slots < 1 || slots > kMaxSlots)
+        return fail(HIPML_ATTN_E_RANGE, "slots %d outside 1..%d", slots, kMaxSlots);
+    if (kv_slot_bytes == 0 && slots <= kMaxCols && slots > 1) {
+        // rows of one sequence sharing a cache: stream it once for all of them
+        const int32_t one_slot[1] = {slots};
+        return decode_common(as_stream(stream), pos, q, k_cache, v_cache, part_acc, part_ml, out,
+                             n_heads, n_kv, head_dim, stride, scale, splits, 0, acc_slot, ml_slot,
+                             q_slot, 1, one_slot);
+    }
+    return decode_common(as_stream(stream), pos, q, k_cache, v_cache, part_acc, part_ml, out,
+                         n_heads, n_kv, head_dim, stride, scale, splits, kv_slot_bytes, acc_slot,
+                         ml_slot, q_slot, slots, nullptr);
+}
+
+int hipml_attn_decode_batch(hipml_stream_t stream, int dtype, const int32_t *pos, const float *q,
+                            const void *k_cache, const void *v_cache, float *part_acc,
+                            float *part_ml, float *out, int n_heads, int n_kv, int head_dim,
+                            int stride, float scale, int splits, size_t kv_slot_bytes,
+                            size_t acc_slot, size_t ml_slot, size_t q_slot, int slots,
+                            int live_seq)
+{
+    clear_error();
+    if (live_seq < 0 || live_seq > stride)
+        return fail(HIPML_ATTN_E_RANGE, "live_seq %d outside 0..stride %d", live_seq, stride);
+    return hipml_attn_decode_rows(stream, dtype, pos, q, k_cache, v_cache, part_acc, part_ml, out,
+                                  n_heads, n_kv, head_dim, stride, scale, splits, kv_slot_bytes,
+                                  acc_slot, ml_slot, q_slot, slots);
+}
+
+int hipml_attn_decode_batch_cols(hipml_stream_t stream, int dtype, const int32_t *pos,
+                                 const float *q, const void *k_cache, const void *v_cache,
+                                 float *part_acc, float *part_ml, float *out, int n_heads,
+                                 int n_kv, int head_dim, int stride, float scale, int splits,
+                                 size_t kv_slot_bytes, size_t acc_slot, size_t ml_slot,
+                                 size_t q_slot, int slots, const int32_t *cols_per_slot_host)
+{
+    clear_error();
+    int rc = check_q8(dtype);
+    if (rc)
+        return rc;
+    REQUIRE_PTR(cols_per_slot_host);
+    return decode_common(as_stream(stream), pos, q, k_cache, v_cache, part_acc, part_ml, out,
+                         n_heads, n_kv, head_dim, stride, scale, splits, kv_slot_bytes, acc_slot,
+                         ml_slot, q_slot, slots, cols_per_slot_host);
+}
+
+// ---- chunk prefill ---------------------------------------------------------------------------------
+
+int hipml_attn_chunk_q8_split(hipml_stream_t stream, const float *q, const void *kc,
+                              const void *vc, float *out, int n_head, int n_kv, int head_dim,
+                              int pos0, int tokens, int dtype, int stride, float *part_acc,
+                              float *part_ml, int splits)
+{
+    clear_error();
+    REQUIRE_PTR(q);
+    REQUIRE_PTR(kc);
+    REQUIRE_PTR(vc);
+    REQUIRE_PTR(out);
+    if (dtype != 1)
+        return fail(HIPML_ATTN_E_UNSUPPORTED,
+                    "quantized chunk attention: only a q8_0 cache (dtype 1) is built, got %d", dtype);
+    int rc = check_heads(n_head, n_kv, head_dim);
+    if (rc)
+        return rc;
+    if (pos0 < 0 || tokens < 0)
+        return fail(HIPML_ATTN_E_RANGE, "pos0 %d / tokens %d must be non-negative", pos0, tokens);
+    if ((long long)pos0 + tokens > stride)
+        return fail(HIPML_ATTN_E_RANGE, "chunk [%d, %d) does not fit a cache of %d rows per head",
+                    pos0, pos0 + tokens, stride);
+    if (splits > 64)
+        return fail(HIPML_ATTN_E_RANGE, "splits %d > 64", splits);
+    if (splits >= 2) {
+        REQUIRE_PTR(part_acc);
+        REQUIRE_PTR(part_ml);
+    }
+    if ((rc = check_aligned16(q, "q")) || (rc = check_aligned16(out, "out")) ||
+        (rc = check_aligned16(kc, "k cache")) || (rc = check_aligned16(vc, "v cache")))
+        return rc;
+    if (tokens == 0)
+        return 0;
+    return launch_chunk_q8(as_stream(stream), q, static_cast<const uint8_t *>(kc),
+                           static_cast<const uint8_t *>(vc), out, n_head, n_kv, pos0, tokens,
+                           stride, part_acc, part_ml, splits);
+}
+
+// ---- gate ---------------------------------------------------------------------------------------------
+
+int hipml_q_gate_f32(hipml_stream_t stream, const float *x, const float *gate, float *y, size_t n)
+{
+    clear_error();
+    REQUIRE_PTR(x);
+    REQUIRE_PTR(gate);
+    REQUIRE_PTR(y);
+    return launch_q_gate(as_stream(stream), x, gate, y, n);
+}
+
+} // extern "C"

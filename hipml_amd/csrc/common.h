@@ -1,0 +1,73 @@
+// Shared host-side helpers of libhipml_attn.so: status codes, the thread-local
+// error text, argument checks.  Device code lives in the .hip files.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/hipml_attn.h"
+
+namespace hipml {
+
+constexpr int kBlock = 32;        // values per quantization block
+constexpr int kQ8BlockBytes = 34; // f16 scale + 32 int8
+constexpr int kHeadDim = 256;     // the width the MFMA kernels are built for
+constexpr int kRowBytes = kHeadDim / kBlock * kQ8BlockBytes; // 272
+constexpr int kMaxCols = 4;       // query rows of one sequence per launch (MTP verify)
+constexpr int kMaxSlots = 128;    // slots per batched launch
+constexpr int kMaxGroup = 8;      // query heads per KV head
+
+// Record `msg` for hipml_attn_last_error() and return `code`.
+int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+// Translate the launch status of the most recent kernel launch on this thread.
+int launched(const char *what);
+void clear_error();
+
+inline hipStream_t as_stream(hipml_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+
+// n_heads / n_kv / head_dim rules shared by the attention launchers
+// (crates/hipml-kernels/src/launch_kv.rs:130-148 in the reference).
+int check_heads(int n_heads, int n_kv, int head_dim);
+
+// Kernel launchers implemented in the .hip translation units -------------------
+
+struct RopeTable {
+    const float *dev;  // [max_pos][n_rot/2][2] cos,sin or nullptr
+    float theta;
+    int n_rot;
+    int max_pos;
+};
+
+int launch_mrope(hipStream_t st, const float *x, float *y, int n_heads, int head_dim, int n_rot,
+                 int s0, int s1, int s2, int s3, const int32_t *pos, int pos_stride, int rows,
+                 float theta, const RopeTable &tab);
+int launch_rope_chunk(hipStream_t st, float *q, float *k, int n_head, int n_kv, int head_dim,
+                      int n_rot, float theta, int pos0, int tokens, const RopeTable &tab);
+int launch_kv_encode_q8(hipStream_t st, const float *k, const float *v, uint8_t *kc, uint8_t *vc,
+                        int n_kv, int head_dim, int stride, const int32_t *pos, int pos_stride,
+                        size_t slot_bytes, int slots, int start, int src0, int rows);
+int launch_q_gate(hipStream_t st, const float *x, const float *gate, float *y, size_t n);
+
+struct DecodeLaunch {
+    const float *q;
+    const uint8_t *k;
+    const uint8_t *v;
+    float *part_acc;
+    float *part_ml;
+    float *out;
+    const int32_t *pos; // (pos, seq) pairs, one per row
+    int n_heads, n_kv, stride, splits, slots;
+    float scale;
+    size_t kv_slot_bytes, acc_slot, ml_slot, q_slot;
+    uint16_t row0[kMaxSlots]; // first row of each slot
+    uint8_t cols[kMaxSlots];  // rows of each slot (1..kMaxCols)
+    int total_rows;
+    int max_cols;
+};
+int launch_decode_q8(hipStream_t st, const DecodeLaunch &a);
+
+int launch_chunk_q8(hipStream_t st, const float *q, const uint8_t *kc, const uint8_t *vc,
+                    float *out, int n_head, int n_kv, int pos0, int tokens, int stride,
+                    float *part_acc, float *part_ml, int splits);
+
+} // namespace hipml

@@ -1,0 +1,277 @@
+// Bit-exact and elementwise kernels of the attention path for gfx950:
+// q8_0 KV quantize-and-append, M-RoPE, sigmoid output gate.
+//
+// This translation unit is compiled with -ffp-contract=off: the CPU definitions
+// these kernels must reproduce bit for bit evaluate x1*c - x2*s and x*id with
+// separately rounded multiplies (crates/hipml-core/src/ops.rs:296-305,
+// crates/hipml-core/src/kv.rs:191-200 in the reference).
+
+#include "common.h"
+
+#include <hip/hip_fp16.h>
+
+namespace hipml {
+
+// ---- q8_0 quantize + append ---------------------------------------------------
+//
+// One workgroup per (kv head, unit); thread t owns value t of the head row.  A
+// wave64 holds two 32-value blocks, so the absolute-maximum butterfly stays
+// inside each 32-lane half (xor masks 16..1 never cross bit 5).
+//
+// unit u reads source row (src0 + u) of a position-major f32 [.][n_kv*head_dim]
+// buffer and writes cache position pos[u*pos_stride] (or start + u when pos is
+// null) of the cache at base + u*slot_bytes.
+
+__device__ __forceinline__ float half_wave_amax(float x)
+{
+    float m = fabsf(x);
+#pragma unroll
+    for (int bit = 16; bit > 0; bit >>= 1)
+        m = fmaxf(m, __shfl_xor(m, bit));
+    return m;
+}
+
+__device__ __forceinline__ void q8_encode_store(float x, uint8_t *dst_block, int lane32)
+{
+    const float amax = half_wave_amax(x);
+    const float d = amax / 127.0f;                    // IEEE division
+    const float id = d > 0.0f ? 1.0f / d : 0.0f;
+    const float t = roundf(x * id);                   // half away from zero
+    // NaN (0 * inf when d is subnormal) encodes as 0, like Rust's `as i8`.
+    const float c = fminf(127.0f, fmaxf(-127.0f, t));
+    const int q = (t != t) ? 0 : (int)c;
+    if (lane32 == 0)
+        *reinterpret_cast<__half *>(dst_block) = __float2half_rn(d);
+    dst_block[2 + lane32] = (uint8_t)(int8_t)q;
+}
+
+__global__ void __launch_bounds__(256) kv_encode_q8_kernel(
+    const float *__restrict__ k, const float *__restrict__ v, uint8_t *__restrict__ kc,
+    uint8_t *__restrict__ vc, int n_kv, int head_dim, int stride, const int32_t *__restrict__ pos,
+    int pos_stride, size_t slot_bytes, int start, int src0)
+{
+    const int h = blockIdx.x;
+    const int u = blockIdx.y;
+    const int t = threadIdx.x;
+    if (t >= head_dim)
+        return;
+    const int chunk = t >> 5;
+    const int lane32 = t & 31;
+    const int nchunk = head_dim >> 5;
+    const int p = pos ? pos[(size_t)u * pos_stride] : start + u;
+    const size_t src = ((size_t)(src0 + u) * n_kv + h) * head_dim + t;
+    const size_t off = (size_t)u * slot_bytes +
+                       (((size_t)h * stride + p) * nchunk + chunk) * kQ8BlockBytes;
+    q8_encode_store(k[src], kc + off, lane32);
+    q8_encode_store(v[src], vc + off, lane32);
+}
+
+int launch_kv_encode_q8(hipStream_t st, const float *k, const float *v, uint8_t *kc, uint8_t *vc,
+                        int n_kv, int head_dim, int stride, const int32_t *pos, int pos_stride,
+                        size_t slot_bytes, int units, int start, int src0, int /*rows*/)
+{
+    if (units == 0)
+        return 0;
+    const int block = head_dim < 64 ? 64 : head_dim;
+    // grid.y is limited to 65535: walk long chunks in slices.
+    for (int u0 = 0; u0 < units; u0 += 32768) {
+        const int n = units - u0 < 32768 ? units - u0 : 32768;
+        hipLaunchKernelGGL(kv_encode_q8_kernel, dim3(n_kv, n, 1), dim3(block, 1, 1), 0, st, k, v,
+                           kc + (size_t)u0 * slot_bytes, vc + (size_t)u0 * slot_bytes, n_kv,
+                           head_dim, stride, pos ? pos + (size_t)u0 * pos_stride : nullptr,
+                           pos_stride, slot_bytes, start + u0, src0 + u0);
+        int rc = launched("kv_encode_q8");
+        if (rc)
+            return rc;
+    }
+    return 0;
+}
+
+// ---- RoPE ----------------------------------------------------------------------
+//
+// NeoX pair k is (k, k + n_rot/2); the angle of pair k at position p is
+// p * theta^(-2k/n_rot).  cos/sin come from the host-built f32 table when the
+// position is inside it; otherwise from f64 pow/sincos on the device.
+
+__device__ __forceinline__ void rope_cs(const float *__restrict__ tab, int tab_rows, int half,
+                                        int k, int p, int n_rot, float theta, float &cs, float &sn)
+{
+    if (tab != nullptr && p >= 0 && p < tab_rows) {
+        const float2 e = reinterpret_cast<const float2 *>(tab)[(size_t)p * half + k];
+        cs = e.x;
+        sn = e.y;
+    } else {
+        const double freq = pow((double)theta, -2.0 * (double)k / (double)n_rot);
+        double s, c;
+        sincos((double)p * freq, &s, &c);
+        cs = (float)c;
+        sn = (float)s;
+    }
+}
+
+// grid (n_heads, rows); 64 threads.  Row r takes its four position ids from
+// pos[r*pos_stride .. +3] (sections pick one per pair), or all four equal to
+// pos[r*pos_stride] when `text` is set.
+__global__ void __launch_bounds__(64) mrope_kernel(
+    const float *x, float *y, int n_heads, int head_dim, int n_rot, int s0, int s1, int s2, int s3,
+    const int32_t *__restrict__ pos, int pos_stride, int text, float theta,
+    const float *__restrict__ tab, int tab_rows)
+{
+    const int h = blockIdx.x;
+    const int r = blockIdx.y;
+    const int half = n_rot >> 1;
+    const int sect = s0 + s1 + s2 + s3;
+    const int32_t *pr = pos + (size_t)r * pos_stride;
+    const size_t base = ((size_t)r * n_heads + h) * (size_t)head_dim;
+    for (int k = threadIdx.x; k < half; k += blockDim.x) {
+        int p = pr[0];
+        if (!text && sect > 0) {
+            const int s = k % sect;
+            if (s < s0)
+                p = pr[0];
+            else if (s < s0 + s1)
+                p = pr[1];
+            else if (s < s0 + s1 + s2)
+                p = pr[2];
+            else
+                p = pr[3];
+        }
+        float cs, sn;
+        rope_cs(tab, tab_rows, half, k, p, n_rot, theta, cs, sn);
+        const float x1 = x[base + k];
+        const float x2 = x[base + half + k];
+        y[base + k] = x1 * cs - x2 * sn;
+        y[base + half + k] = x1 * sn + x2 * cs;
+    }
+    // channels >= n_rot pass through
+    if (y != x) {
+        for (int d = n_rot + threadIdx.x; d < head_dim; d += blockDim.x)
+            y[base + d] = x[base + d];
+    }
+}
+
+// grid (n_head + n_kv, tokens); 64 threads.  Token t rotates at pos0 + t.
+__global__ void __launch_bounds__(64) rope_chunk_kernel(
+    float *__restrict__ q, float *__restrict__ kx, int n_head, int n_kv, int head_dim, int n_rot,
+    float theta, int pos0, const float *__restrict__ tab, int tab_rows)
+{
+    const int h = blockIdx.x;
+    const int t = blockIdx.y;
+    const int half = n_rot >> 1;
+    const int p = pos0 + t;
+    float *row = h < n_head ? q + ((size_t)t * n_head + h) * head_dim
+                            : kx + ((size_t)t * n_kv + (h - n_head)) * head_dim;
+    for (int k = threadIdx.x; k < half; k += blockDim.x) {
+        float cs, sn;
+        rope_cs(tab, tab_rows, half, k, p, n_rot, theta, cs, sn);
+        const float x1 = row[k];
+        const float x2 = row[half + k];
+        row[k] = x1 * cs - x2 * sn;
+        row[half + k] = x1 * sn + x2 * cs;
+    }
+}
+
+static const float *table_for(const RopeTable &tab, float theta, int n_rot, int *rows)
+{
+    if (tab.dev != nullptr && tab.theta == theta && tab.n_rot == n_rot) {
+        *rows = tab.max_pos;
+        return tab.dev;
+    }
+    *rows = 0;
+    return nullptr;
+}
+
+int launch_mrope(hipStream_t st, const float *x, float *y, int n_heads, int head_dim, int n_rot,
+                 int s0, int s1, int s2, int s3, const int32_t *pos, int pos_stride, int rows,
+                 float theta, const RopeTable &tab)
+{
+    int tab_rows = 0;
+    const float *t = table_for(tab, theta, n_rot, &tab_rows);
+    const int text = pos_stride != 0 ? 1 : 0; // batched rows carry (pos, seq) pairs: text only
+    for (int r0 = 0; r0 < rows; r0 += 32768) {
+        const int n = rows - r0 < 32768 ? rows - r0 : 32768;
+        const size_t off = (size_t)r0 * n_heads * head_dim;
+        hipLaunchKernelGGL(mrope_kernel, dim3(n_heads, n, 1), dim3(64, 1, 1), 0, st, x + off,
+                           y + off, n_heads, head_dim, n_rot, s0, s1, s2, s3,
+                           pos + (size_t)r0 * pos_stride, pos_stride, text, theta, t, tab_rows);
+        int rc = launched("mrope_f32");
+        if (rc)
+            return rc;
+    }
+    return 0;
+}
+
+int launch_rope_chunk(hipStream_t st, float *q, float *k, int n_head, int n_kv, int head_dim,
+                      int n_rot, float theta, int pos0, int tokens, const RopeTable &tab)
+{
+    int tab_rows = 0;
+    const float *t = table_for(tab, theta, n_rot, &tab_rows);
+    for (int t0 = 0; t0 < tokens; t0 += 32768) {
+        const int n = tokens - t0 < 32768 ? tokens - t0 : 32768;
+        hipLaunchKernelGGL(rope_chunk_kernel, dim3(n_head + n_kv, n, 1), dim3(64, 1, 1), 0, st,
+                           q + (size_t)t0 * n_head * head_dim, k + (size_t)t0 * n_kv * head_dim,
+                           n_head, n_kv, head_dim, n_rot, theta, pos0 + t0, t, tab_rows);
+        int rc = launched("rope_chunk_f32");
+        if (rc)
+            return rc;
+    }
+    return 0;
+}
+
+// ---- sigmoid output gate ----------------------------------------------------------
+//
+// y = x * (1 / (1 + exp(-g))) (crates/hipml-core/src/ops.rs:354-360).  Four
+// values per thread through 128-bit accesses when the pointers allow it.
+
+__global__ void __launch_bounds__(256) q_gate_kernel4(const float4 *x, const float4 *__restrict__ g,
+                                                     float4 *y, size_t n4)
+{
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n4)
+        return;
+    const float4 a = x[i];
+    const float4 b = g[i];
+    float4 r;
+    r.x = a.x * (1.0f / (1.0f + expf(-b.x)));
+    r.y = a.y * (1.0f / (1.0f + expf(-b.y)));
+    r.z = a.z * (1.0f / (1.0f + expf(-b.z)));
+    r.w = a.w * (1.0f / (1.0f + expf(-b.w)));
+    y[i] = r;
+}
+
+__global__ void __launch_bounds__(256) q_gate_kernel1(const float *x, const float *__restrict__ g,
+                                                     float *y, size_t first, size_t n)
+{
+    const size_t i = first + (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n)
+        return;
+    y[i] = x[i] * (1.0f / (1.0f + expf(-g[i])));
+}
+
+int launch_q_gate(hipStream_t st, const float *x, const float *gate, float *y, size_t n)
+{
+    if (n == 0)
+        return 0;
+    const bool aligned = (((uintptr_t)x | (uintptr_t)gate | (uintptr_t)y) & 15) == 0;
+    size_t n4 = aligned ? n / 4 : 0;
+    if (n4 > 0) {
+        const size_t blocks = (n4 + 255) / 256;
+        hipLaunchKernelGGL(q_gate_kernel4, dim3((unsigned)blocks, 1, 1), dim3(256, 1, 1), 0, st,
+                           reinterpret_cast<const float4 *>(x),
+                           reinterpret_cast<const float4 *>(gate), reinterpret_cast<float4 *>(y),
+                           n4);
+        int rc = launched("q_gate_f32");
+        if (rc)
+            return rc;
+    }
+    const size_t done = n4 * 4;
+    if (done < n) {
+        const size_t blocks = (n - done + 255) / 256;
+        hipLaunchKernelGGL(q_gate_kernel1, dim3((unsigned)blocks, 1, 1), dim3(256, 1, 1), 0, st, x,
+                           gate, y, done, n);
+        return launched("q_gate_f32");
+    }
+    return 0;
+}
+
+} // namespace hipml

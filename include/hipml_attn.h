@@ -1,0 +1,207 @@
+/*
+ * hipml_attn.h -- C ABI of libhipml_attn.so: the full-attention hot path of the
+ * qwen35 hybrid (RoPE, q8_0 KV append, split-K decode, MTP-verify decode,
+ * batched decode, causal GQA chunk prefill, sigmoid output gate) for MI355X
+ * (gfx950).  One entry point per launcher of the reference's kernel crate; the
+ * citation on each prototype is the reference function it replaces
+ * (paths relative to the reference repository).
+ *
+ * Conventions shared by every entry point
+ *   - All pointers are device pointers unless the name says `host`.
+ *   - `stream` is a hipStream_t passed as void*.  Launches are asynchronous on
+ *     it; nothing here synchronises, allocates or frees, so every call is legal
+ *     under stream capture.  Per-step scalars (position, live length) are read
+ *     from device memory exactly as the reference's kernels do.
+ *   - Return value: 0 on success; a negative hipml_attn_status for an argument
+ *     error detected before any launch; a positive hipError_t if the runtime
+ *     refused the launch.  hipml_attn_last_error() returns a thread-local
+ *     message for the last non-zero return.
+ *   - Layouts: Q / out / gate are f32 [rows][n_heads][head_dim].  A q8_0 cache
+ *     is two byte arrays K and V of [n_kv][stride][head_dim/32] 34-byte blocks
+ *     (f16 scale, 32 x int8): block (kvh,pos,c) starts at byte
+ *     ((kvh*stride + pos)*(head_dim/32) + c)*34      (crates/hipml-core/src/kv.rs:22-40).
+ *   - `dtype` for cache entry points is the reference's KvDtype id (0 = q8_0).
+ *     q4_0 (1) is rejected with HIPML_ATTN_E_UNSUPPORTED.
+ */
+#ifndef HIPML_ATTN_H
+#define HIPML_ATTN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *hipml_stream_t; /* hipStream_t */
+
+typedef enum hipml_attn_status {
+    HIPML_ATTN_OK = 0,
+    HIPML_ATTN_E_SHAPE = -1,       /* head counts / head_dim / group the kernels do not cover */
+    HIPML_ATTN_E_UNSUPPORTED = -2, /* unknown or unsupported dtype / variant */
+    HIPML_ATTN_E_NULL = -3,        /* a required pointer is NULL */
+    HIPML_ATTN_E_RANGE = -4,       /* a count or offset is out of range */
+    HIPML_ATTN_E_DEVICE = -5,      /* not a gfx950 device */
+    HIPML_ATTN_E_STATE = -6        /* required set-up call missing (e.g. no RoPE table) */
+} hipml_attn_status;
+
+/* ---- library ------------------------------------------------------------ */
+
+/* Bind to `device` (hipSetDevice is NOT called; the caller's current device is
+ * used for launches) and check that it is gfx950.  Replaces Launcher::new's
+ * module load, crates/hipml-kernels/src/launch.rs:119-141. */
+int hipml_attn_init(int device);
+/* Thread-local text for the last failure on this thread ("" if none). */
+const char *hipml_attn_last_error(void);
+const char *hipml_attn_version(void);
+
+/* ---- split policies (host arithmetic, no GPU) ---------------------------- */
+
+/* Key splits for single-sequence decode on MI355X.  Same role as
+ * DeepKv::splits, crates/hipml-model/src/gpu/deep_kv.rs:102-110, retuned for
+ * 256 CUs.  Scratch is [n_heads][splits][head_dim] + [n_heads][splits][2] f32. */
+int hipml_attn_decode_splits(int seq, int n_kv);
+/* Key splits for batched decode.  Same role as attn_splits,
+ * crates/hipml-model/src/gpu/batch/kv.rs:39-42. */
+int hipml_attn_batch_splits(int stride, int n_kv, int slots);
+/* Key splits for a prefill chunk starting at pos0.  Same role as split_count,
+ * crates/hipml-model/src/gpu/attn_tile.rs:138-151. */
+int hipml_attn_chunk_splits(int pos0, int tokens, int n_kv);
+
+/* ---- RoPE ----------------------------------------------------------------
+ * The reference's CPU definition builds the angle in f64 with the host libm
+ * (crates/hipml-core/src/ops.rs:296-305).  To be bit-identical to it the
+ * kernels read cos/sin from a table the HOST fills with that same libm:
+ * table[pos][k] = { (float)cos(pos * theta^(-2k/n_rot)), (float)sin(...) },
+ * f32 [max_pos][n_rot/2][2]. */
+size_t hipml_rope_table_bytes(int n_rot, int max_pos);
+int hipml_rope_table_fill_host(float *host_table, float theta_base, int n_rot, int max_pos);
+/* Register a device copy of the table (caller owns the memory).  Positions at
+ * or beyond max_pos fall back to f64 pow/sincos on the device, which is within
+ * one f32 ulp of the table but not guaranteed identical. */
+int hipml_rope_set_table(const float *dev_table, float theta_base, int n_rot, int max_pos);
+
+/* M-RoPE over [n_heads][head_dim] at the four position ids in device memory
+ * pos[0..3] (the step buffer's words 4..7).  x and y may alias.
+ * Replaces AttnLayer::rope_launch -> mrope_f32,
+ * crates/hipml-kernels/src/attn_gpu.rs:429-464. */
+int hipml_mrope_f32(hipml_stream_t stream, const float *x, float *y, int n_heads, int head_dim,
+                    int n_rot, int s0, int s1, int s2, int s3, const int32_t *pos,
+                    float theta_base);
+/* Same for `rows` rows of [n_heads][head_dim]; row r rotates at the text
+ * position pos[r*2] (all four ids equal).  Replaces mrope_b,
+ * crates/hipml-kernels/src/attn_gpu.rs:729-784. */
+int hipml_mrope_rows_f32(hipml_stream_t stream, const float *x, float *y, int n_heads,
+                         int head_dim, int n_rot, int s0, int s1, int s2, int s3,
+                         const int32_t *pos, int rows, float theta_base);
+/* RoPE of a prefill chunk in place: q [tokens][n_head][head_dim] and
+ * k [tokens][n_kv][head_dim], token t at position pos0+t.  The RoPE half of
+ * norm_rope_chunk_f32 (AttnLayer::chunk_front,
+ * crates/hipml-kernels/src/attn_gpu/imp/attn_chunk.rs:167-199). */
+int hipml_rope_chunk_f32(hipml_stream_t stream, float *q, float *k, int n_head, int n_kv,
+                         int head_dim, int n_rot, float theta_base, int pos0, int tokens);
+
+/* ---- q8_0 KV append ------------------------------------------------------- */
+
+/* One token: quantize k_in/v_in [n_kv][head_dim] into row step[0] of the cache.
+ * Replaces Launcher::kv_encode_ptr_on -> kv_encode_q8,
+ * crates/hipml-kernels/src/launch/device/graph_launch.rs:932-973. */
+int hipml_kv_encode(hipml_stream_t stream, const int32_t *step, int dtype, const float *k_in,
+                    const float *v_in, void *k_cache, void *v_cache, int n_kv, int head_dim,
+                    int stride);
+/* `rows` tokens from position-major f32 [.][n_kv*head_dim]; source row src0+r
+ * goes to cache position start+r.  Replaces Launcher::kv_encode_bulk ->
+ * kv_encode_bulk_q8, graph_launch.rs:980-1028. */
+int hipml_kv_encode_bulk(hipml_stream_t stream, int dtype, const float *k_f32, const float *v_f32,
+                         void *k_cache, void *v_cache, int n_kv, int head_dim, int stride,
+                         int start, int src0, int rows);
+/* One row per slot: row s of k_f32/v_f32 goes to cache (base + s*slot_bytes) at
+ * position pos[s*2].  Replaces Launcher::kv_encode_rows_ptr -> kv_encode_q8_b,
+ * crates/hipml-kernels/src/launch/device/batch_launch.rs:59-105. */
+int hipml_kv_encode_rows(hipml_stream_t stream, int dtype, const float *k_f32, const float *v_f32,
+                         void *k_cache, void *v_cache, int n_kv, int head_dim, int stride,
+                         const int32_t *pos, size_t slot_bytes, int slots);
+
+/* ---- decode attention over a q8_0 cache ----------------------------------- */
+
+/* One query row, live length step[1].  Split pass + merge.
+ * part_acc: f32 [n_heads][splits][head_dim]; part_ml: f32 [n_heads][splits][2].
+ * Replaces launch_kv::launch_ptrs -> attn_decode_kv_w2 + attn_decode_kv_reduce,
+ * crates/hipml-kernels/src/launch_kv.rs:110-280. */
+int hipml_attn_decode_kv(hipml_stream_t stream, const int32_t *step, int dtype, const float *q,
+                         const void *k, const void *v, float *part_acc, float *part_ml,
+                         float *out, int n_heads, int n_kv, int head_dim, int stride, float scale,
+                         int splits, size_t k_off, size_t v_off);
+/* `cols` (<= 4) consecutive query rows of ONE sequence sharing the cache
+ * (MTP verify): column c reads q + c*q_slot, sees keys [0, pos[c*2+1]), writes
+ * out + c*q_slot, and owns scratch slices part_acc + c*acc_slot and
+ * part_ml + c*ml_slot (all in f32 elements).  The cache is streamed once for
+ * all columns.  Replaces launch_kv::launch_cols_ptrs -> attn_decode_kv_w2_b +
+ * attn_decode_kv_reduce_b, crates/hipml-kernels/src/launch_kv.rs:292-412. */
+int hipml_attn_decode_kv_cols(hipml_stream_t stream, int dtype, const int32_t *pos,
+                              const float *q, const void *k, const void *v, float *part_acc,
+                              float *part_ml, float *out, int n_heads, int n_kv, int head_dim,
+                              int stride, float scale, int splits, int cols, size_t acc_slot,
+                              size_t ml_slot, size_t q_slot);
+/* `slots` independent rows: row s reads cache base + s*kv_slot_bytes, q +
+ * s*q_slot, keys [0, pos[s*2+1]).  kv_slot_bytes == 0 means the rows share one
+ * cache (a verify group).  Replaces Launcher::attn_decode_rows_ptr ->
+ * attn_decode_kv_q8_b + attn_decode_kv_reduce_b,
+ * crates/hipml-kernels/src/launch/device/batch_launch.rs:215-316. */
+int hipml_attn_decode_rows(hipml_stream_t stream, int dtype, const int32_t *pos, const float *q,
+                           const void *k_cache, const void *v_cache, float *part_acc,
+                           float *part_ml, float *out, int n_heads, int n_kv, int head_dim,
+                           int stride, float scale, int splits, size_t kv_slot_bytes,
+                           size_t acc_slot, size_t ml_slot, size_t q_slot, int slots);
+/* Batched decode step.  `live_seq` > 0 with slots == 1 states a plain decode
+ * step at a known length (the reference reroutes that case to its warp kernel;
+ * here both cases run the same kernel and the value is only validated).
+ * Replaces Launcher::attn_decode_batch, batch_launch.rs:109-213. */
+int hipml_attn_decode_batch(hipml_stream_t stream, int dtype, const int32_t *pos, const float *q,
+                            const void *k_cache, const void *v_cache, float *part_acc,
+                            float *part_ml, float *out, int n_heads, int n_kv, int head_dim,
+                            int stride, float scale, int splits, size_t kv_slot_bytes,
+                            size_t acc_slot, size_t ml_slot, size_t q_slot, int slots,
+                            int live_seq);
+/* Batched decode where slot s carries cols_per_slot[s] (1..4) consecutive query
+ * rows that share slot s's cache (plain slots and MTP-verify slots mixed in ONE
+ * launch).  Rows are numbered slot-major: row r has (pos,seq) = pos[r*2..],
+ * q + r*q_slot, scratch r*acc_slot / r*ml_slot; slot s's cache is base +
+ * s*kv_slot_bytes.  cols_per_slot is a HOST array read during the call.
+ * The reference has no single-launch form of this: it issues one launch pair
+ * per verify slot (crates/hipml-model/src/gpu/batch/verify.rs:321-366). */
+int hipml_attn_decode_batch_cols(hipml_stream_t stream, int dtype, const int32_t *pos,
+                                 const float *q, const void *k_cache, const void *v_cache,
+                                 float *part_acc, float *part_ml, float *out, int n_heads,
+                                 int n_kv, int head_dim, int stride, float scale, int splits,
+                                 size_t kv_slot_bytes, size_t acc_slot, size_t ml_slot,
+                                 size_t q_slot, int slots, const int32_t *cols_per_slot_host);
+
+/* ---- causal chunk prefill over a q8_0 cache -------------------------------- */
+
+/* tokens query rows at positions pos0..pos0+tokens-1 attend keys [0, pos0+t]
+ * of a cache that already holds the chunk's own rows.  `dtype` follows the
+ * reference's chunk launcher: 1 = q8_0.  splits < 2 runs the single-pass kernel
+ * and ignores the scratch; otherwise part_acc is f32
+ * [splits][ceil32(tokens)][n_head][head_dim] and part_ml [..][2].
+ * Replaces AttnLayer::chunk_attention_q8_split -> attn_chunk_wmma_f16 /
+ * attn_chunk_full_f16 + attn_chunk_combine_f32,
+ * crates/hipml-kernels/src/attn_gpu/imp/attn_chunk_kv.rs:72-107,129-305. */
+int hipml_attn_chunk_q8_split(hipml_stream_t stream, const float *q, const void *kc,
+                              const void *vc, float *out, int n_head, int n_kv, int head_dim,
+                              int pos0, int tokens, int dtype, int stride, float *part_acc,
+                              float *part_ml, int splits);
+
+/* ---- output gate ------------------------------------------------------------ */
+
+/* y[i] = x[i] * sigmoid(gate[i]); y may alias x.  Replaces
+ * AttnLayer::q_gate_only / apply_output_chunk -> q_gate_f32,
+ * crates/hipml-kernels/src/attn_gpu.rs:822-840 and
+ * crates/hipml-kernels/src/attn_gpu/imp/attn_chunk.rs:343-364. */
+int hipml_q_gate_f32(hipml_stream_t stream, const float *x, const float *gate, float *y,
+                     size_t n);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HIPML_ATTN_H */

@@ -1,0 +1,247 @@
+"""Decode attention over a q8_0 cache: HIP path (through the C ABI) vs the CPU oracle
+on identical seeded inputs.  Gate: max-abs 2e-3 / rel 1e-2 (OR rule); the reference's
+own decode class, 1e-4 / 1e-3 (crates/hipml-core/src/parity_kv.rs:7-10), is asserted
+as well because the kernel keeps K and V exact and Q to ~22 bits."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+from oracle import binding as orc  # noqa: E402
+from hipml_amd import attn  # noqa: E402
+from gpu_util import (N_HEADS, N_KV, HD, SCALE, ROW, dev, host, quantized_cache,  # noqa: E402
+                      decode_scratch, run_decode, report)
+
+GATE = (2e-3, 1e-2)
+REF_CLASS = (1e-4, 1e-3)
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _init():
+    attn.init(0)
+
+
+def kv_case(seed, heads, n_kv, seq):
+    # input recipe of the reference's kv_case! macro (parity_kv.rs:39-60)
+    r = orc.Rng(seed)
+    q = r.normal_array((heads, HD))
+    kf = r.normal_array((n_kv, seq, HD), 0.3)
+    vf = r.normal_array((n_kv, seq, HD))
+    return q, kf, vf
+
+
+@pytest.mark.parametrize("name,seed,heads,n_kv,seq,splits", [
+    ("attn_decode_kv_q8_hd256_s1", 0x9E00_0001, 6, 1, 1, 1),
+    ("attn_decode_kv_q8_hd256_s37", 0x9E00_0002, 6, 1, 37, 1),
+    ("attn_decode_kv_q8_hd256_s1000", 0x9E00_0003, 6, 1, 1000, 7),
+    ("attn_decode_kv_q8_hd256_s4096", 0x9E00_0004, 6, 1, 4096, 16),
+])
+def test_reference_kv_cases(name, seed, heads, n_kv, seq, splits):
+    q, kf, vf = kv_case(seed, heads, n_kv, seq)
+    kb, vb = quantized_cache(kf, vf)
+    want = orc.attn_decode_kv(q, kb, vb, heads, n_kv, HD, seq, SCALE)
+    got = run_decode(q, kb, vb, heads, n_kv, seq, seq, SCALE, splits)
+    ok, _, _ = report(name, want, got, *REF_CLASS)
+    assert ok
+    assert orc.compare(want, got, *GATE)[0]
+
+
+def test_deep_case_100k_one_head():
+    # parity_kv.rs:221-232: 1 head, 100,000 rows, 256 splits
+    q, kf, vf = kv_case(0x9E00_1001, 1, 1, 100_000)
+    kb, vb = quantized_cache(kf, vf)
+    want = orc.attn_decode_kv(q, kb, vb, 1, 1, HD, 100_000, SCALE)
+    got = run_decode(q, kb, vb, 1, 1, 100_000, 100_000, SCALE, 256)
+    ok, _, _ = report("attn_decode_kv_q8_hd256_s100000", want, got, *REF_CLASS)
+    assert ok
+
+
+@pytest.mark.parametrize("seq,stride", [(673, 680), (8192, 8192), (32768, 32768), (5000, 32768)])
+def test_decode_full_geometry(seq, stride):
+    # BASELINE configs 1 (depth 672 -> seq 673) and 3 (8,192 / 32,768): 24 q heads on 4 kv heads
+    r = orc.Rng(0x5EED_0003 + seq)
+    q = r.normal_array((N_HEADS, HD))
+    kf = r.normal_array((N_KV, seq, HD))
+    vf = r.normal_array((N_KV, seq, HD))
+    kb, vb = quantized_cache(kf, vf, stride)
+    want = orc.attn_decode_kv(q, kb, vb, N_HEADS, N_KV, HD, seq, SCALE, stride=stride)
+    splits = attn.decode_splits(seq, N_KV)
+    got = run_decode(q, kb, vb, N_HEADS, N_KV, seq, stride, SCALE, splits)
+    ok, _, _ = report(f"decode 24/4 seq {seq} stride {stride} splits {splits}", want, got, *REF_CLASS)
+    assert ok
+    assert orc.compare(want, got, *GATE)[0]
+
+
+@pytest.mark.parametrize("splits", [1, 2, 3, 7, 64, 256, 300])
+def test_any_split_count_gives_the_same_answer(splits):
+    # split-K invariant: the merge must not depend on how the keys were cut, including
+    # more splits than 32-key tiles (empty slices) and ragged last slices.
+    seq = 1000
+    q, kf, vf = kv_case(0xABC0 + 1, N_HEADS, N_KV, seq)
+    kb, vb = quantized_cache(kf, vf)
+    one = run_decode(q, kb, vb, N_HEADS, N_KV, seq, seq, SCALE, 1)
+    got = run_decode(q, kb, vb, N_HEADS, N_KV, seq, seq, SCALE, splits)
+    ok, ma, _ = report(f"splits {splits} vs 1", one, got, 1e-5, 1e-4)  # fp32 reassociation only
+    assert ok
+
+
+def test_peaked_softmax_and_large_scores():
+    # one key dominates (score ~ +60 in natural units): the output must be that key's V row,
+    # which exposes any rounding of the probabilities or of V.
+    seq = 300
+    r = orc.Rng(404)
+    q = r.normal_array((N_HEADS, HD))
+    kf = r.normal_array((N_KV, seq, HD), 0.05)
+    vf = r.normal_array((N_KV, seq, HD), 3.0)
+    for g in range(N_KV):
+        kf[g, 123] = q[g * 6] * 4.0
+    kb, vb = quantized_cache(kf, vf)
+    want = orc.attn_decode_kv(q, kb, vb, N_HEADS, N_KV, HD, seq, SCALE)
+    got = run_decode(q, kb, vb, N_HEADS, N_KV, seq, seq, SCALE, 3)
+    ok, _, _ = report("peaked softmax", want, got, *REF_CLASS)
+    assert ok
+
+
+def test_seq_zero_gives_zero_and_k_v_offsets_are_honoured():
+    seq = 64
+    q, kf, vf = kv_case(99, N_HEADS, N_KV, seq)
+    kb, vb = quantized_cache(kf, vf)
+    acc, ml = decode_scratch(N_HEADS, 2)
+    out = torch.full((N_HEADS, HD), 7.0, dtype=torch.float32, device="cuda")
+    step = torch.tensor([0, 0, 0, 0, 0, 0, 0, 0], dtype=torch.int32, device="cuda")
+    attn.attn_decode_kv(step, 0, dev(q), dev(kb), dev(vb), acc, ml, out, N_HEADS, N_KV, HD, seq,
+                        SCALE, 2)
+    torch.cuda.synchronize()
+    assert not host(out).any()
+    # two layers in one allocation, second selected through k_off / v_off
+    pad = 4096
+    big_k = np.concatenate([np.zeros(pad, np.uint8), kb.ravel()])
+    big_v = np.concatenate([np.zeros(pad, np.uint8), vb.ravel()])
+    step = torch.tensor([seq - 1, seq, 0, 0, 0, 0, 0, 0], dtype=torch.int32, device="cuda")
+    attn.attn_decode_kv(step, 0, dev(q), dev(big_k), dev(big_v), acc, ml, out, N_HEADS, N_KV, HD,
+                        seq, SCALE, 2, pad, pad)
+    torch.cuda.synchronize()
+    want = orc.attn_decode_kv(q, kb, vb, N_HEADS, N_KV, HD, seq, SCALE)
+    assert orc.compare(want, host(out), *REF_CLASS)[0]
+
+
+@pytest.mark.parametrize("cols", [1, 2, 3, 4])
+def test_mtp_columns_equal_single_token_decodes(cols):
+    # column c of an R-column verify == plain decode at pos0 + c after all R appends
+    # (the reference's `column-bench --check` invariant).
+    pos0, stride = 700, 720
+    live = pos0 + cols
+    r = orc.Rng(0xC015 + cols)
+    q = r.normal_array((cols, N_HEADS, HD))
+    kf = r.normal_array((N_KV, live, HD))
+    vf = r.normal_array((N_KV, live, HD))
+    kb, vb = quantized_cache(kf, vf, stride)
+    splits = 5
+    acc, ml = decode_scratch(N_HEADS, splits, cols)
+    out = torch.full((cols, N_HEADS, HD), float("nan"), dtype=torch.float32, device="cuda")
+    pos = torch.tensor([[pos0 + c, pos0 + c + 1] for c in range(cols)], dtype=torch.int32,
+                       device="cuda")
+    attn.attn_decode_kv_cols(4, pos, dev(q), dev(kb), dev(vb), acc, ml, out, N_HEADS, N_KV, HD,
+                             stride, SCALE, splits, cols, N_HEADS * splits * HD,
+                             N_HEADS * splits * 2, N_HEADS * HD)
+    torch.cuda.synchronize()
+    got = host(out)
+    for c in range(cols):
+        want = orc.attn_decode_kv(q[c], kb, vb, N_HEADS, N_KV, HD, pos0 + c + 1, SCALE, stride=stride)
+        ok, _, _ = report(f"verify column {c}/{cols}", want, got[c], *REF_CLASS)
+        assert ok
+        single = run_decode(q[c], kb, vb, N_HEADS, N_KV, pos0 + c + 1, stride, SCALE, splits)
+        assert orc.compare(single, got[c].ravel(), 1e-6, 1e-5)[0]
+
+
+def make_slots(depths, cols_per_slot, stride, seed):
+    r = orc.Rng(seed)
+    slots = len(depths)
+    kc = np.zeros((slots, N_KV, stride, ROW), dtype=np.uint8)
+    vc = np.zeros((slots, N_KV, stride, ROW), dtype=np.uint8)
+    qs, pos = [], []
+    for s, (d, c) in enumerate(zip(depths, cols_per_slot)):
+        live = d + c  # the c query rows' own K/V rows are appended first
+        kf = r.normal_array((N_KV, live, HD))
+        vf = r.normal_array((N_KV, live, HD))
+        kc[s], vc[s] = quantized_cache(kf, vf, stride)
+        for j in range(c):
+            qs.append(r.normal_array((N_HEADS, HD)))
+            pos.append((d + j, d + j + 1))
+    return np.stack(qs), kc, vc, pos
+
+
+def test_batched_decode_uniform_rows():
+    # one row per slot, contiguous per-slot caches (Launcher::attn_decode_batch)
+    depths = [512, 3000, 1, 16384 - 1, 777]
+    stride = 16448
+    q, kc, vc, pos = make_slots(depths, [1] * len(depths), stride, 0xBA7C)
+    slots = len(depths)
+    splits = attn.batch_splits(stride, N_KV, slots)
+    acc, ml = decode_scratch(N_HEADS, splits, slots)
+    out = torch.full((slots, N_HEADS, HD), float("nan"), dtype=torch.float32, device="cuda")
+    attn.attn_decode_batch(0, torch.tensor(pos, dtype=torch.int32, device="cuda"), dev(q), dev(kc),
+                           dev(vc), acc, ml, out, N_HEADS, N_KV, HD, stride, SCALE, splits,
+                           N_KV * stride * ROW, N_HEADS * splits * HD, N_HEADS * splits * 2,
+                           N_HEADS * HD, slots)
+    torch.cuda.synchronize()
+    got = host(out)
+    for s in range(slots):
+        want = orc.attn_decode_kv(q[s], kc[s], vc[s], N_HEADS, N_KV, HD, pos[s][1], SCALE,
+                                  stride=stride)
+        ok, _, _ = report(f"batch slot {s} seq {pos[s][1]}", want, got[s], *REF_CLASS)
+        assert ok
+
+
+def test_batched_decode_with_mtp_slots_in_one_launch():
+    # BASELINE config 5: 16 slots, depths uniform in [512, 16384] under seed, slots 0..3 carry
+    # 3 query rows (causal within the draft), the rest 1.
+    r = orc.Rng(0x5EED_0005)
+    depths = [512 + int(float(r.uniform()) * (16384 - 512 + 1)) for _ in range(16)]
+    cols = [3, 3, 3, 3] + [1] * 12
+    stride = 16448
+    q, kc, vc, pos = make_slots(depths, cols, stride, 0x5EED_1005)
+    rows = len(pos)
+    splits = attn.batch_splits(stride, N_KV, 16)
+    acc, ml = decode_scratch(N_HEADS, splits, rows)
+    out = torch.full((rows, N_HEADS, HD), float("nan"), dtype=torch.float32, device="cuda")
+    attn.attn_decode_batch_cols(0, torch.tensor(pos, dtype=torch.int32, device="cuda"), dev(q),
+                                dev(kc), dev(vc), acc, ml, out, N_HEADS, N_KV, HD, stride, SCALE,
+                                splits, N_KV * stride * ROW, N_HEADS * splits * HD,
+                                N_HEADS * splits * 2, N_HEADS * HD, cols)
+    torch.cuda.synchronize()
+    got = host(out)
+    row = 0
+    worst = 0.0
+    for s, c in enumerate(cols):
+        for j in range(c):
+            want = orc.attn_decode_kv(q[row], kc[s], vc[s], N_HEADS, N_KV, HD, pos[row][1], SCALE,
+                                      stride=stride)
+            ok, ma, _ = orc.compare(want, got[row], *REF_CLASS)
+            worst = max(worst, ma)
+            assert ok, f"slot {s} row {j} seq {pos[row][1]}: max_abs {ma}"
+            row += 1
+    print(f"[parity] batched 16 slots (4 x 3 rows): worst max_abs {worst:.3e}", flush=True)
+
+
+def test_verify_group_through_rows_entry_shares_the_cache():
+    # attn_decode_rows_ptr with kv_slot_bytes = 0: a group of columns at one slot's cache
+    # (crates/hipml-model/src/gpu/batch/verify.rs:328-367)
+    pos0, cols, stride = 90, 3, 128
+    r = orc.Rng(0x7E57)
+    q = r.normal_array((cols, N_HEADS, HD))
+    kf = r.normal_array((N_KV, pos0 + cols, HD))
+    vf = r.normal_array((N_KV, pos0 + cols, HD))
+    kb, vb = quantized_cache(kf, vf, stride)
+    splits = 2
+    acc, ml = decode_scratch(N_HEADS, splits, cols)
+    out = torch.empty((cols, N_HEADS, HD), dtype=torch.float32, device="cuda")
+    pos = torch.tensor([[pos0 + c, pos0 + c + 1] for c in range(cols)], dtype=torch.int32, device="cuda")
+    attn.attn_decode_rows(0, pos, dev(q), dev(kb), dev(vb), acc, ml, out, N_HEADS, N_KV, HD, stride,
+                          SCALE, splits, 0, N_HEADS * splits * HD, N_HEADS * splits * 2,
+                          N_HEADS * HD, cols)
+    torch.cuda.synchronize()
+    for c in range(cols):
+        want = orc.attn_decode_kv(q[c], kb, vb, N_HEADS, N_KV, HD, pos0 + c + 1, SCALE, stride=stride)
+        assert orc.compare(want, host(out)[c], *REF_CLASS)[0]

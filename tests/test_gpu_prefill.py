@@ -1,0 +1,94 @@
+"""Causal chunk prefill over a q8_0 cache: HIP path vs the oracle's row-by-row
+attn_causal_f32 over the dequantized cache.  Tolerance: max-abs 2e-3 / rel 1e-2
+(BASELINE gate; the reference's chunk class is 2e-3 / 2e-2,
+crates/hipml-cli/src/attn_chunk_parity.rs:18-20): fp16 operands, fp32 accumulation."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+from oracle import binding as orc  # noqa: E402
+from hipml_amd import attn  # noqa: E402
+from gpu_util import N_HEADS, N_KV, HD, SCALE, ROW, dev, host, report  # noqa: E402
+
+GATE = (2e-3, 1e-2)
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _init():
+    attn.init(0)
+
+
+def chunk_inputs(seed, tok, pos0, pad):
+    # recipe of run_q8_splits (attn_chunk_parity.rs:117-160): position-major N(0,1) rows,
+    # re-packed head-major, quantized on the host.
+    stride = pos0 + tok + pad
+    r = orc.Rng(seed)
+    q = r.normal_array((tok, N_HEADS, HD))
+    k = r.normal_array((stride, N_KV, HD))
+    v = r.normal_array((stride, N_KV, HD))
+    kb = orc.quantize(0, k.transpose(1, 0, 2)).reshape(N_KV, stride, ROW)
+    vb = orc.quantize(0, v.transpose(1, 0, 2)).reshape(N_KV, stride, ROW)
+    return q, kb, vb, stride
+
+
+def run_chunk(q, kb, vb, pos0, tok, stride, splits):
+    out = torch.full((tok, N_HEADS, HD), float("nan"), dtype=torch.float32, device="cuda")
+    acc = ml = None
+    if splits >= 2:
+        acc, ml = attn.chunk_scratch(tok, N_HEADS, splits)
+        acc.fill_(float("nan"))
+        ml.fill_(float("nan"))
+    attn.chunk_attention_q8_split(dev(q), dev(kb), dev(vb), out, N_HEADS, N_KV, HD, pos0, tok, 1,
+                                  stride, acc, ml, splits)
+    torch.cuda.synchronize()
+    return host(out)
+
+
+@pytest.mark.parametrize("splits", [1, 4])
+@pytest.mark.parametrize("tok,pos0,pad", [(37, 29, 0), (37, 29, 8), (1, 0, 0), (33, 0, 3), (64, 1000, 24)])
+def test_reference_chunk_case(tok, pos0, pad, splits):
+    q, kb, vb, stride = chunk_inputs(0xC4A0_9876_5432, tok, pos0, pad)
+    want = orc.attn_chunk_kv(q, kb, vb, N_HEADS, N_KV, HD, pos0, tok, stride, SCALE, n_threads=8)
+    got = run_chunk(q, kb, vb, pos0, tok, stride, splits)
+    ok, _, _ = report(f"chunk {tok}@{pos0} pad {pad} splits {splits}", want, got, *GATE)
+    assert ok
+    assert np.isfinite(got).all()
+
+
+@pytest.mark.parametrize("splits", [1, 3])
+def test_prefill_672_at_0(splits):
+    # BASELINE config 2
+    tok, pos0 = 672, 0
+    q, kb, vb, stride = chunk_inputs(0x5EED_0002, tok, pos0, 8)
+    want = orc.attn_chunk_kv(q, kb, vb, N_HEADS, N_KV, HD, pos0, tok, stride, SCALE, n_threads=16)
+    got = run_chunk(q, kb, vb, pos0, tok, stride, splits)
+    ok, _, _ = report(f"prefill 672@0 splits {splits}", want, got, *GATE)
+    assert ok
+
+
+def test_split_and_mono_agree_and_splits_above_diagonal_are_ignored():
+    # pos0 = 0 with many splits: late slices sit wholly above the diagonal for early rows
+    tok, pos0 = 96, 0
+    q, kb, vb, stride = chunk_inputs(77, tok, pos0, 0)
+    mono = run_chunk(q, kb, vb, pos0, tok, stride, 1)
+    for splits in (2, 8, 16):
+        got = run_chunk(q, kb, vb, pos0, tok, stride, splits)
+        # f16 probabilities are rounded against a different running maximum per slice
+        ok, _, _ = report(f"split {splits} vs mono", mono, got, 1e-3, 1e-2)
+        assert ok
+
+
+def test_deep_chunk_sampled_rows():
+    # BASELINE config 4 at reduced depth for the CPU side: 256 tokens at depth 20,000,
+    # every 37th row checked; exercises long-KV tiling and the split merge.
+    tok, pos0 = 256, 20_000
+    q, kb, vb, stride = chunk_inputs(0x5EED_0004, tok, pos0, 16)
+    rows = np.arange(0, tok, 37, dtype=np.int32)
+    want = orc.attn_chunk_kv(q, kb, vb, N_HEADS, N_KV, HD, pos0, tok, stride, SCALE, rows=rows,
+                             n_threads=16)
+    for splits in (1, 8):
+        got = run_chunk(q, kb, vb, pos0, tok, stride, splits)
+        ok, _, _ = report(f"chunk 256@20000 splits {splits}", want, got[rows], *GATE)
+        assert ok
