@@ -1,0 +1,386 @@
+#!/usr/bin/env python3
+"""Benchmark of the full-attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--main-only] [--no-cpu]
+
+Headline workload (one "step"): one layer's attention core over a 672-token
+prompt at depth 0 -- RoPE of Q and K, q8_0 quantize-and-append of K/V, causal
+GQA attention over the q8_0 cache (24 query heads, 4 KV heads, head_dim 256),
+sigmoid output gate -- with every input already resident in HBM.  Steps rotate
+over 16 distinct layer caches.  value = tokens/s of that step.
+
+The same JSON line carries, under "also", the other workloads of the path
+(decode at 8,192 / 32,768, the 2,048-token chunk at depth 100,000, batched
+decode with MTP-verify slots), each with its own roofline object.
+
+roofline.achieved = algorithmic FLOP (prefill) or K+V cache bytes (decode) per
+attention launch / the attention launch's mean duration measured with HIP
+events on the launch stream.  cpu_baseline = the CPU oracle (a scalar restatement
+of the reference's CPU path) timed on this host on the stated sample.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+H, KV, HD, NROT, THETA = 24, 4, 256, 64, 1e7
+ROW = 272
+SCALE = 1.0 / 16.0
+HBM_PEAK_GBS = 8000.0      # MI355X HBM3E, published
+MFMA_F16_PEAK_TF = 2500.0  # MI355X dense fp16 MFMA, published
+LAYERS = 16                # distinct layer caches a pass rotates over
+
+
+def prefill_flop(pos0: int, tokens: int) -> float:
+    """Causal-useful FLOP of one layer: n_head * sum_t (pos0+t+1) * 4 * head_dim."""
+    pairs = tokens * pos0 + tokens * (tokens + 1) // 2
+    return float(H * pairs * 4 * HD)
+
+
+def decode_bytes(seq_total: int) -> float:
+    """K+V cache bytes one layer's decode must read: 2 * n_kv * rows * 272."""
+    return float(2 * KV * seq_total * ROW)
+
+
+class Timer:
+    """HIP events on torch's current stream (the stream every launch below uses)."""
+
+    def __init__(self, torch):
+        self.torch = torch
+        self.a = torch.cuda.Event(enable_timing=True)
+        self.b = torch.cuda.Event(enable_timing=True)
+
+    def __enter__(self):
+        self.a.record()
+        return self
+
+    def __exit__(self, *exc):
+        self.b.record()
+        self.b.synchronize()
+        self.ms = self.a.elapsed_time(self.b)
+
+
+def fill_cache_normal(torch, attn, k_cache, v_cache, stride, rows, gen):
+    """Quantize N(0,1) rows into a [KV][stride][272] cache pair with the library's own
+    append kernel, in slabs so the f32 source stays small."""
+    slab = 8192
+    for s0 in range(0, rows, slab):
+        n = min(slab, rows - s0)
+        kf = torch.randn((n, KV, HD), device="cuda", dtype=torch.float32, generator=gen)
+        vf = torch.randn((n, KV, HD), device="cuda", dtype=torch.float32, generator=gen)
+        attn.kv_encode_bulk(0, kf, vf, k_cache, v_cache, KV, HD, stride, s0, 0, n)
+    torch.cuda.synchronize()
+
+
+# ---------------------------------------------------------------------------------------
+# prefill: rope + append + attention + gate
+# ---------------------------------------------------------------------------------------
+
+def bench_prefill(torch, attn, tokens, pos0, steps, warmup, layers, prefix_fill=True):
+    stride = (pos0 + tokens + 63) // 64 * 64
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(0x5EED0002 + pos0)
+    caches = []
+    for _ in range(layers):
+        k = torch.zeros((KV, stride, ROW), dtype=torch.uint8, device="cuda")
+        v = torch.zeros((KV, stride, ROW), dtype=torch.uint8, device="cuda")
+        if pos0 > 0 and prefix_fill:
+            fill_cache_normal(torch, attn, k, v, stride, pos0, gen)
+        caches.append((k, v))
+    q = torch.randn((tokens, H, HD), device="cuda", generator=gen)
+    kx = torch.randn((tokens, KV, HD), device="cuda", generator=gen)
+    vx = torch.randn((tokens, KV, HD), device="cuda", generator=gen)
+    gate = torch.randn((tokens, H, HD), device="cuda", generator=gen)
+    out = torch.empty((tokens, H, HD), device="cuda")
+    splits = attn.chunk_splits(pos0, tokens, KV)
+    acc = ml = None
+    if splits >= 2:
+        acc, ml = attn.chunk_scratch(tokens, H, splits)
+    attn.rope_table(THETA, NROT, max(pos0 + tokens, 1024))
+
+    def attention(i):
+        k, v = caches[i % layers]
+        attn.chunk_attention_q8_split(q, k, v, out, H, KV, HD, pos0, tokens, 1, stride, acc, ml,
+                                      splits)
+
+    def step(i):
+        k, v = caches[i % layers]
+        attn.rope_chunk(q, kx, H, KV, HD, NROT, THETA, pos0, tokens)
+        attn.kv_encode_bulk(0, kx, vx, k, v, KV, HD, stride, pos0, 0, tokens)
+        attention(i)
+        attn.q_gate(out, gate, out)
+
+    for i in range(warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        step(i)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+
+    # the attention launch alone, HIP events on the launch stream
+    for i in range(min(warmup, 3)):
+        attention(i)
+    with Timer(torch) as t:
+        for i in range(steps):
+            attention(i)
+    attn_ms = t.ms / steps
+    flop = prefill_flop(pos0, tokens)
+    tf = flop / (attn_ms * 1e-3) / 1e12
+    return {
+        "workload": f"prefill {tokens}@{pos0}: rope + q8_0 append + causal GQA attention + gate, "
+                    f"1 layer, {H}q/{KV}kv heads, head_dim {HD}",
+        "tokens": tokens, "pos0": pos0, "splits": splits, "layers_rotated": layers,
+        "ms_per_step": wall_ms,
+        "tok_per_s": tokens / (wall_ms * 1e-3),
+        "attn_ms": attn_ms,
+        "attn_tok_per_s": tokens / (attn_ms * 1e-3),
+        "roofline": {"bound": "mfma", "achieved": tf, "peak": MFMA_F16_PEAK_TF, "unit": "TFLOP/s",
+                     "frac": tf / MFMA_F16_PEAK_TF, "traffic": None,
+                     "kernel": "chunk_q8_kernel" + (" + chunk_combine_kernel" if splits >= 2 else ""),
+                     "flop_per_launch": flop, "launch_ms": attn_ms},
+    }
+
+
+# ---------------------------------------------------------------------------------------
+# decode
+# ---------------------------------------------------------------------------------------
+
+def bench_decode(torch, attn, seq, steps, warmup, layers):
+    stride = seq
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(0x5EED0003 + seq)
+    caches = []
+    for _ in range(layers):
+        k = torch.empty((KV, stride, ROW), dtype=torch.uint8, device="cuda")
+        v = torch.empty((KV, stride, ROW), dtype=torch.uint8, device="cuda")
+        fill_cache_normal(torch, attn, k, v, stride, seq, gen)
+        caches.append((k, v))
+    q = torch.randn((H, HD), device="cuda", generator=gen)
+    out = torch.empty((H, HD), device="cuda")
+    splits = attn.decode_splits(seq, KV)
+    acc = torch.empty((H, splits, HD), device="cuda")
+    ml = torch.empty((H, splits, 2), device="cuda")
+    stepbuf = torch.tensor([seq - 1, seq, 0, 0, seq - 1, seq - 1, seq - 1, seq - 1],
+                           dtype=torch.int32, device="cuda")
+
+    def one_pass():
+        for k, v in caches:
+            attn.attn_decode_kv(stepbuf, 0, q, k, v, acc, ml, out, H, KV, HD, stride, SCALE, splits)
+
+    for _ in range(warmup):
+        one_pass()
+    with Timer(torch) as t:
+        for _ in range(steps):
+            one_pass()
+    us = t.ms * 1e3 / (steps * layers)
+    nbytes = decode_bytes(seq)
+    gbs = nbytes / (us * 1e-6) / 1e9
+    return {
+        "workload": f"decode 1 query @ depth {seq}, q8_0 cache, split-K {splits} + merge",
+        "seq": seq, "splits": splits, "layers_rotated": layers,
+        "us_per_layer": us,
+        "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": gbs / HBM_PEAK_GBS, "traffic": None,
+                     "kernel": "decode_q8_kernel + decode_reduce_kernel",
+                     "bytes_per_launch": nbytes, "launch_us": us},
+    }
+
+
+def batch_case(orc_rng_uniform, slots=16, verify=4, lo=512, hi=16384):
+    depths = [lo + int(orc_rng_uniform() * (hi - lo + 1)) for _ in range(slots)]
+    cols = [3 if s < verify else 1 for s in range(slots)]
+    return depths, cols
+
+
+def bench_batch(torch, attn, orc, steps, warmup, layers):
+    r = orc.Rng(0x5EED0005)
+    depths, cols = batch_case(lambda: float(r.uniform()))
+    slots = len(depths)
+    stride = 16448
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(0x5EED0005)
+    slot_bytes = KV * stride * ROW
+    caches = []
+    for _ in range(layers):
+        k = torch.zeros((slots, KV, stride, ROW), dtype=torch.uint8, device="cuda")
+        v = torch.zeros((slots, KV, stride, ROW), dtype=torch.uint8, device="cuda")
+        for s in range(slots):
+            fill_cache_normal(torch, attn, k[s], v[s], stride, depths[s] + cols[s], gen)
+        caches.append((k, v))
+    rows = sum(cols)
+    pos = []
+    for s in range(slots):
+        for c in range(cols[s]):
+            pos += [depths[s] + c, depths[s] + c + 1]
+    pos_d = torch.tensor(pos, dtype=torch.int32, device="cuda")
+    q = torch.randn((rows, H, HD), device="cuda", generator=gen)
+    out = torch.empty((rows, H, HD), device="cuda")
+    splits = attn.batch_splits(stride, KV, slots)
+    acc = torch.empty((rows, H, splits, HD), device="cuda")
+    ml = torch.empty((rows, H, splits, 2), device="cuda")
+
+    def one_pass():
+        for k, v in caches:
+            attn.attn_decode_batch_cols(0, pos_d, q, k, v, acc, ml, out, H, KV, HD, stride, SCALE,
+                                        splits, slot_bytes, H * splits * HD, H * splits * 2, H * HD,
+                                        cols)
+
+    for _ in range(warmup):
+        one_pass()
+    with Timer(torch) as t:
+        for _ in range(steps):
+            one_pass()
+    us = t.ms * 1e3 / (steps * layers)
+    live = sum(d + c for d, c in zip(depths, cols))
+    nbytes = decode_bytes(live)
+    gbs = nbytes / (us * 1e-6) / 1e9
+    return {
+        "workload": f"batched decode, {slots} slots, depths U[512,16384] (seeded), "
+                    f"slots 0..3 carry 3 query rows (MTP verify), one launch",
+        "slots": slots, "rows": rows, "live_rows": live, "splits": splits, "layers_rotated": layers,
+        "us_per_layer": us,
+        "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": gbs / HBM_PEAK_GBS, "traffic": None,
+                     "kernel": "decode_q8_kernel + decode_reduce_kernel",
+                     "bytes_per_launch": nbytes, "launch_us": us},
+    }
+
+
+# ---------------------------------------------------------------------------------------
+# CPU baseline (the oracle, timed; never part of the measured GPU path)
+# ---------------------------------------------------------------------------------------
+
+def cpu_prefill(orc, np, tokens, pos0, rows_sample=None):
+    """Scalar single-thread oracle on the headline workload; returns (tok/s, sample text)."""
+    r = orc.Rng(0x5EED0002)
+    stride = pos0 + tokens
+    q = r.normal_array((tokens, H, HD))
+    k = r.normal_array((stride, KV, HD))
+    v = r.normal_array((stride, KV, HD))
+    gate = r.normal_array((tokens, H, HD))
+    sec = (11, 11, 10, 0)
+    t0 = time.perf_counter()
+    for t in range(tokens):
+        p = pos0 + t
+        q[t] = orc.rope_multi(q[t], H, HD, NROT, sec, (p, p, p, p), THETA).reshape(H, HD)
+        k[p] = orc.rope_multi(k[p], KV, HD, NROT, sec, (p, p, p, p), THETA).reshape(KV, HD)
+    kb = orc.quantize(0, k.transpose(1, 0, 2)).reshape(KV, stride, ROW)
+    vb = orc.quantize(0, v.transpose(1, 0, 2)).reshape(KV, stride, ROW)
+    rows = None if rows_sample is None else np.asarray(rows_sample, dtype=np.int32)
+    o = orc.attn_chunk_kv(q, kb, vb, H, KV, HD, pos0, tokens, stride, SCALE, rows=rows, n_threads=1)
+    n = tokens if rows is None else len(rows)
+    orc.q_gate(o.ravel(), gate[:n].ravel())
+    dt = time.perf_counter() - t0
+    return n / dt, dt
+
+
+def cpu_decode(orc, seq):
+    r = orc.Rng(0x5EED0003 + seq)
+    q = r.normal_array((H, HD))
+    kb = orc.synthetic_blocks(0, KV * seq * 8, 11).reshape(KV, seq, ROW)
+    vb = orc.synthetic_blocks(0, KV * seq * 8, 12).reshape(KV, seq, ROW)
+    t0 = time.perf_counter()
+    orc.attn_decode_kv(q, kb, vb, H, KV, HD, seq, SCALE)
+    return (time.perf_counter() - t0) * 1e6
+
+
+# ---------------------------------------------------------------------------------------
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--main-only", action="store_true", help="skip the 'also' workloads")
+    ap.add_argument("--only", default="", help="run one workload alone (prefill672, decode8k, "
+                    "decode32k, chunk100k, batch16) for profiling; prints its object")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (the attention path needs no exchange "
+              "between GPUs); run with --gpus 1", file=sys.stderr)
+        return 2
+
+    import numpy as np
+    import torch
+    from hipml_amd import attn
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 3
+    attn.init(0)
+    K, W = args.steps, args.warmup
+
+    if args.only:
+        from oracle import binding as orc
+        fn = {
+            "prefill672": lambda: bench_prefill(torch, attn, 672, 0, K, W, LAYERS),
+            "decode8k": lambda: bench_decode(torch, attn, 8192, K, W, LAYERS),
+            "decode32k": lambda: bench_decode(torch, attn, 32768, K, W, LAYERS),
+            "chunk100k": lambda: bench_prefill(torch, attn, 2048, 100_000, K, W, 2),
+            "batch16": lambda: bench_batch(torch, attn, orc, K, W, 4),
+        }[args.only]
+        print(json.dumps(fn()))
+        return 0
+
+    main_r = bench_prefill(torch, attn, 672, 0, K, W, LAYERS)
+    line = {
+        "metric": "prefill_attn_tok_per_s",
+        "value": main_r["tok_per_s"],
+        "unit": "tok/s",
+        "n_gpus": 1, "steps": K, "warmup": W,
+        "ms_per_step": main_r["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16 operands (Q, dequantized q8_0 K/V, P), f32 accumulate/softmax",
+        "data": "synthetic",
+        "config": {"workload": main_r["workload"], "tokens": 672, "pos0": 0,
+                   "layers_rotated": LAYERS, "splits": main_r["splits"]},
+        "attn_only_tok_per_s": main_r["attn_tok_per_s"],
+        "roofline": main_r["roofline"],
+    }
+
+    if not args.main_only:
+        also = {}
+        d_steps = max(K // 4, 10)
+        also["decode_8192"] = bench_decode(torch, attn, 8192, d_steps, max(W // 4, 2), LAYERS)
+        torch.cuda.empty_cache()
+        also["decode_32768"] = bench_decode(torch, attn, 32768, d_steps, max(W // 4, 2), LAYERS)
+        torch.cuda.empty_cache()
+        also["chunk_2048_at_100000"] = bench_prefill(torch, attn, 2048, 100_000,
+                                                     max(K // 20, 3), 1, 2)
+        torch.cuda.empty_cache()
+        from oracle import binding as orc  # only for the seeded depth recipe and the CPU leg
+        also["batch16_mtp"] = bench_batch(torch, attn, orc, d_steps, max(W // 4, 2), 4)
+        torch.cuda.empty_cache()
+        line["also"] = also
+
+    if not args.no_cpu:
+        from oracle import binding as orc
+        tokps, secs = cpu_prefill(orc, np, 672, 0)
+        line["cpu_baseline"] = {
+            "value": tokps, "unit": "tok/s", "cores": 1, "kind": "port",
+            "sample": f"the whole headline workload once (672 tokens @ 0: rope + quantize + "
+                      f"causal attention over the dequantized cache + gate), {secs:.1f} s, "
+                      f"1 thread, scalar C restatement of the reference's CPU path",
+            "host_cpus": os.cpu_count(),
+        }
+        if not args.main_only:
+            line["cpu_baseline"]["decode_us_per_layer"] = {
+                "8192": cpu_decode(orc, 8192), "32768": cpu_decode(orc, 32768)}
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
