@@ -17,7 +17,8 @@ import os
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libhipml_attn.so")
+# HIPML_ATTN_LIB selects another build of the same library (e.g. an experimental variant).
+LIB_PATH = os.environ.get("HIPML_ATTN_LIB") or os.path.join(_HERE, "libhipml_attn.so")
 
 ROW_BYTES = 272      # one head_dim-256 row of q8_0: 8 blocks x 34 bytes
 BLOCK_BYTES = 34

@@ -151,6 +151,9 @@ int hipml_attn_init(int device)
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return fail(HIPML_ATTN_E_DEVICE, "device %d is %s; this library is built for gfx950 only",
                     device, prop.gcnArchName);
+    int rc = decode_init();
+    if (rc)
+        return rc;
     g_inited = true;
     return 0;
 }
@@ -164,11 +167,11 @@ const char *hipml_attn_version(void) { return "hipml-attn-mi355x 0.1 (gfx950)"; 
 int hipml_attn_decode_splits(int seq, int n_kv)
 {
     // One workgroup of four waves walks 32-key tiles; give every workgroup at least one
-    // tile per wave (128 keys) and stop at one workgroup per CU (256) across the KV heads.
+    // tile per wave (128 keys) and stop at two workgroups per CU (512) across the KV heads.
     if (seq < 1 || n_kv < 1)
         return 1;
     int by_work = (seq + 127) / 128;
-    int by_cus = 256 / n_kv;
+    int by_cus = 512 / n_kv;
     if (by_cus < 1)
         by_cus = 1;
     int s = by_work < by_cus ? by_work : by_cus;

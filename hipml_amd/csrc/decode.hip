@@ -1,12 +1,22 @@
 // Split-K decode attention over a q8_0 KV cache for gfx950 (wave64, MFMA).
 //
 // One workgroup (4 waves) owns one (kv head, key split, slot).  Each wave walks
-// its own 32-key tiles of the split with a private online softmax; the four
-// waves merge in LDS and write one unnormalised partial per (row, head, split).
-// A second kernel merges the splits.
+// its own 32-key tiles of the split with a private online softmax and no
+// workgroup barrier in the loop; the four waves merge in LDS at the end and
+// write one unnormalised partial per (row, head, split).  A second kernel
+// merges the splits.
 //
-// Orientation (all MFMAs are v_mfma_f32_16x16x32_f16):
-//   S^T[key][n]  = K[key][:] . Q^T[:][n]      A = K bytes as f16, B = Q (hi + lo f16)
+// Memory pipeline.  A tile's K (or V) rows are 32 x 272 contiguous bytes.  A
+// lane fetches "units" of 68 bytes = two whole 34-byte blocks of one key, with
+// dword-aligned 128-bit loads; a wave's load instruction covers a
+// contiguous 4,352-byte span.  Two tiles (K and V each) are kept in flight per
+// wave in registers.  On arrival a unit is realigned (the even block's payload
+// sits 2 bytes into a dword) and written to a padded, aligned LDS tile
+// [32 keys][288 B]; block scales go to a transposed f16 table [8 blocks][32 keys].
+// K and V of a tile use the same LDS tile one after the other.
+//
+// Arithmetic (all MFMAs are v_mfma_f32_16x16x32_f16):
+//   S^T[key][n]  = K[key][:] . Q^T[:][n]      A = K bytes as f16, B = Q (hi + lo f16, from LDS)
 //   O^T[d][n]   += V^T[d][key] . P'[key][n]   A = V bytes as f16 (LDS transpose read),
 //                                              B = P' = p * scale_of_block(key, d/32), hi + lo f16
 // n runs over (query row, head of the GQA group): up to 4 rows x 8 heads, in
@@ -14,32 +24,72 @@
 // is exactly the B layout the PV product needs, so probabilities never leave
 // their lane, and every per-column scalar (max, sum, rescale) lives in lane%16.
 //
-// Exactness tricks:
-//   - int8 -> f16 without arithmetic: byte b^0x80 = b+128 placed in the low byte
-//     of an f16 is the subnormal (b+128)*2^-24; MFMA multiplies subnormals
-//     exactly.  For K the +128 is cancelled by seeding the accumulator with
-//     -128*2^-24*sum(q_block); for V by one packed f16 subtract of 2^-17.
+// Exactness:
+//   - int8 -> f16 without rounding: byte b^0x80 = b+128 placed in the low byte of
+//     an f16 is the subnormal (b+128)*2^-24; one packed f16 subtract of 128*2^-24
+//     gives b*2^-24 exactly, and MFMA multiplies subnormals exactly.
 //   - one q8 block (32 values) is one MFMA contraction, so the f16 block scale
 //     multiplies an exact integer dot product in fp32 (as the CPU definition's
 //     d * q does, crates/hipml-core/src/ops.rs:486-515 of the reference).
-//   - Q is split into hi + lo f16 halves: two MFMAs, ~22 bits of Q.
+//   - Q and P' are split into hi + lo f16 halves: two MFMAs, ~22 bits each.
 
 #include "common.h"
 
 namespace hipml {
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef float float4v __attribute__((ext_vector_type(4)));
 typedef int int2v __attribute__((ext_vector_type(2)));
 typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
-typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef uint32_t uint4a4 __attribute__((ext_vector_type(4), aligned(4)));
 
-constexpr int kTileKeys = 32;         // keys per wave tile
-constexpr int kLdsRow = 288;          // 256 payload bytes + 32 pad (bank spread)
-constexpr int kWaveLds = 2 * kTileKeys * kLdsRow + 2 * kTileKeys * 16; // 19456
-constexpr int kWaves = 4;
+constexpr int kTileKeys = 32;                         // keys per wave tile
+constexpr int kLdsRow = 288;                          // 256 payload bytes + 32 pad (bank spread)
+constexpr int kTileBytes = kTileKeys * kLdsRow;       // 9216: payload tile (K, then V)
+constexpr int kScaleBytes = 8 * kTileKeys * 2;        // 512: f16 [8 blocks][32 keys]
+constexpr int kWaveLds = kTileBytes + 2 * kScaleBytes; // 10240
+#ifndef DECODE_WAVES
+#define DECODE_WAVES 4
+#endif
+constexpr int kWaves = DECODE_WAVES;   // waves per workgroup
+constexpr int kThreads = 64 * kWaves;
+constexpr int kUnitBytes = 68;                        // two q8_0 blocks
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kTwo24 = 16777216.0f;
+
+#ifndef DECODE_MIN_WAVES
+#define DECODE_MIN_WAVES 2
+#endif
+#ifndef DECODE_DEPTH
+#define DECODE_DEPTH 1
+#endif
+// Optional scheduling fence after each block of the PV loop (off: measured no faster, no leaner).
+#ifdef DECODE_FENCE
+#define SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
+#else
+#define SCHED_FENCE() do { } while (0)
+#endif
+#ifndef DECODE_PLO
+#define DECODE_PLO 0
+#endif
+#ifndef DECODE_QLO
+#define DECODE_QLO 1
+#endif
+// Opaque use-and-redefine of a register: the value must exist here, in a VGPR.
+#define PIN(x) asm volatile("" : "+v"(x))
+constexpr int kDepth = DECODE_DEPTH; // tiles in flight per wave
+
+#ifdef DBG_TIMING
+// debug builds: per-workgroup phase timestamps (100 MHz wall clock), 8 slots per workgroup
+__device__ unsigned long long g_dbg_t[8 * 4096];
+#define STAMP(i) do { if (threadIdx.x == 0 && blockIdx.y == 0 && blockIdx.x < 4096) g_dbg_t[blockIdx.x * 8 + (i)] = wall_clock64(); } while (0)
+#else
+#define STAMP(i) do { } while (0)
+#endif
+
+constexpr int decode_lds_bytes(int nt) { return nt * 16384 + kWaves * kWaveLds; }
 
 struct DecodeArgs {
     const float *q;
@@ -55,13 +105,53 @@ struct DecodeArgs {
     uint8_t cols[kMaxSlots];
 };
 
-struct __attribute__((packed, aligned(2))) Raw16 {
-    uint4v v;
+// 68 bytes of a key row starting at a block-pair boundary: [s0 | 32 x i8 | s1 | 32 x i8].
+struct Unit {
+    uint4v a, b; // dwords 0..7:  s0 and the first 30 bytes of the even block
+    uint32_t m;  // dword 8:      last 2 bytes of the even block, s1
+    uint4v c, d; // dwords 9..16: the odd block's 32 bytes (dword aligned)
 };
 
-__device__ __forceinline__ half8 bytes_to_subnormal_f16(int2v w)
+// Plain (cached) loads: the five loads of a unit and its neighbours' share 128-byte lines, and
+// a non-temporal hint makes every one of them fetch the line again (measured: 3.3 vs 5.6 TB/s).
+__device__ __forceinline__ void load_unit(Unit &u, const uint8_t *p)
 {
-    // byte u -> f16 bits 0x00uu = u * 2^-24
+    u.a = *reinterpret_cast<const uint4a4 *>(p);
+    u.b = *reinterpret_cast<const uint4a4 *>(p + 16);
+    u.m = *reinterpret_cast<const uint32_t *>(p + 32);
+    u.c = *reinterpret_cast<const uint4a4 *>(p + 36);
+    u.d = *reinterpret_cast<const uint4a4 *>(p + 52);
+}
+
+// Realign one unit and store it: payloads of blocks (2*pr, 2*pr+1) of tile row r to the padded
+// tile, their scales to the transposed table.
+__device__ __forceinline__ void store_unit(const Unit &u, uint8_t *tile, uint8_t *scales, int r,
+                                           int pr)
+{
+    uint4v e0, e1;
+    e0[0] = __builtin_amdgcn_alignbit(u.a[1], u.a[0], 16);
+    e0[1] = __builtin_amdgcn_alignbit(u.a[2], u.a[1], 16);
+    e0[2] = __builtin_amdgcn_alignbit(u.a[3], u.a[2], 16);
+    e0[3] = __builtin_amdgcn_alignbit(u.b[0], u.a[3], 16);
+    e1[0] = __builtin_amdgcn_alignbit(u.b[1], u.b[0], 16);
+    e1[1] = __builtin_amdgcn_alignbit(u.b[2], u.b[1], 16);
+    e1[2] = __builtin_amdgcn_alignbit(u.b[3], u.b[2], 16);
+    e1[3] = __builtin_amdgcn_alignbit(u.m, u.b[3], 16);
+    uint4v *dst = reinterpret_cast<uint4v *>(tile + r * kLdsRow + pr * 64);
+    dst[0] = e0;
+    dst[1] = e1;
+    dst[2] = u.c;
+    dst[3] = u.d;
+    uint16_t *sc = reinterpret_cast<uint16_t *>(scales) + (2 * pr) * kTileKeys + r;
+    sc[0] = (uint16_t)(u.a[0] & 0xffffu);
+    sc[kTileKeys] = (uint16_t)(u.m >> 16);
+}
+
+// 8 int8 b -> 8 f16 holding (b + 128) * 2^-24 exactly (byte b^0x80 in the low byte of a
+// subnormal f16).  The +128 is taken out again by a second MFMA whose A operand is the
+// constant -128 * 2^-24: sum_k (u_k - 128) x_k = sum_k u_k x_k + sum_k (-128) x_k.
+__device__ __forceinline__ half8 bytes_to_f16_biased(int2v w)
+{
     const uint32_t x0 = (uint32_t)w[0] ^ 0x80808080u;
     const uint32_t x1 = (uint32_t)w[1] ^ 0x80808080u;
     uint4v r;
@@ -72,23 +162,19 @@ __device__ __forceinline__ half8 bytes_to_subnormal_f16(int2v w)
     return __builtin_bit_cast(half8, r);
 }
 
-__device__ __forceinline__ half8 sub_bias(half8 a)
-{
-    // (b+128)*2^-24 - 128*2^-24, exact in subnormal f16 arithmetic
-    const _Float16 bias = __builtin_bit_cast(_Float16, (uint16_t)0x0080);
-    return a - bias;
-}
-
 __device__ __forceinline__ float xor_max(float x, int mask)
 {
     return fmaxf(x, __shfl_xor(x, mask));
 }
 
-template <int NT>
-__global__ void __launch_bounds__(256) decode_q8_kernel(const DecodeArgs a)
+template <int NT, int DEPTH>
+__global__ void __launch_bounds__(kThreads, DECODE_MIN_WAVES) decode_q8_kernel(const DecodeArgs a)
 {
-    __shared__ __attribute__((aligned(16))) uint8_t lds_all[kWaves * kWaveLds];
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds_all[];
+    uint8_t *Qs = lds_all;                       // [NT][hi,lo][8 blocks][64 lanes] half8
+    uint8_t *wave_base = lds_all + NT * 16384;   // per-wave tile + scale tables
 
+    STAMP(0);
     const int wave = threadIdx.x >> 6;
     const int lane = threadIdx.x & 63;
     const int lm = lane & 15; // MFMA row/col within the 16-tile
@@ -100,6 +186,28 @@ __global__ void __launch_bounds__(256) decode_q8_kernel(const DecodeArgs a)
     const int ncols = a.cols[slot];
     const int group = a.group;
     const int nvalid = ncols * group;
+
+    // ---- Q rows first: their addresses need nothing from device memory, and issued ahead of
+    // the K/V stream they are not queued behind it.  Entry (nt, c, l) of the LDS operand table
+    // = Q[col n = nt*16 + l%16][c*32 + (l/16)*8 .. +8]; a thread owns entries tid + kThreads*k.
+    constexpr int kQEntries = NT * 8 * 64 / kThreads;
+    float4v qf[kQEntries][2];
+#pragma unroll
+    for (int k = 0; k < kQEntries; k++) {
+        const int e = threadIdx.x + kThreads * k;
+        const int l = e & 63, c = (e >> 6) & 7, nt = e >> 9;
+        const int n = nt * 16 + (l & 15);
+        qf[k][0] = (float4v){0, 0, 0, 0};
+        qf[k][1] = (float4v){0, 0, 0, 0};
+        if (n < nvalid) {
+            const int col = n / group;
+            const int head = n - col * group;
+            const float *qp = a.q + (size_t)(row0 + col) * a.q_slot +
+                              (size_t)(kvh * group + head) * kHeadDim + c * 32 + (l >> 4) * 8;
+            qf[k][0] = *reinterpret_cast<const float4v *>(qp);
+            qf[k][1] = *reinterpret_cast<const float4v *>(qp + 4);
+        }
+    }
 
     // live lengths of this slot's rows
     int seqc[kMaxCols];
@@ -114,52 +222,62 @@ __global__ void __launch_bounds__(256) decode_q8_kernel(const DecodeArgs a)
     const int per = (seq_max + a.splits - 1) / a.splits;
     const int lo = split * per;
     const int hi = lo + per < seq_max ? lo + per : seq_max;
-    const int ntile = hi > lo ? (hi - lo + kTileKeys - 1) / kTileKeys : 0;
+    const int ntile_wg = hi > lo ? (hi - lo + kTileKeys - 1) / kTileKeys : 0;
+    // this wave's tiles: wave, wave + kWaves, ...
+    const int ntile = ntile_wg > wave ? (ntile_wg - wave + kWaves - 1) / kWaves : 0;
 
-    uint8_t *lds = lds_all + wave * kWaveLds;
-    uint8_t *Kp = lds;
-    uint8_t *Vp = lds + kTileKeys * kLdsRow;
-    uint8_t *sK = lds + 2 * kTileKeys * kLdsRow;
-    uint8_t *sV = sK + kTileKeys * 16;
+    uint8_t *tile_lds = wave_base + wave * kWaveLds;
+    uint8_t *sK = tile_lds + kTileBytes;
+    uint8_t *sV = sK + kScaleBytes;
 
     const uint8_t *kbase = a.k + (size_t)slot * a.kv_slot_bytes + (size_t)kvh * a.stride * kRowBytes;
     const uint8_t *vbase = a.v + (size_t)slot * a.kv_slot_bytes + (size_t)kvh * a.stride * kRowBytes;
 
-    // ---- Q operand: column n = nt*16 + lm -> (row n/group, head n%group) -------------
-    half8 qhi[NT][8], qlo[NT][8];
-    float cinit[NT][8];
+    // ---- staging registers: DEPTH tiles in flight, each 2 K units + 2 V units per lane -------
+    Unit Kst[DEPTH][2], Vst[DEPTH][2];
+    // unit j of a tile: u = lane + 64*j -> tile row u/4, block pair u%4
+    const int ur0 = lane >> 2, ur1 = 16 + (lane >> 2), upr = lane & 3;
+    auto issue = [&](Unit (&dst)[2], const uint8_t *base, int t) {
+        const int key0 = lo + (wave + kWaves * t) * kTileKeys;
+        int ka = key0 + ur0, kb = key0 + ur1;
+        ka = ka < hi ? ka : hi - 1; // never touch rows past the live range
+        kb = kb < hi ? kb : hi - 1;
+        load_unit(dst[0], base + (size_t)ka * kRowBytes + upr * kUnitBytes);
+        load_unit(dst[1], base + (size_t)kb * kRowBytes + upr * kUnitBytes);
+    };
+#pragma unroll
+    for (int st = 0; st < DEPTH; st++)
+        if (ntile > st) {
+            issue(Kst[st], kbase, st);
+            issue(Vst[st], vbase, st);
+        }
+
+    STAMP(1); // ranges known, first K/V loads issued
+    // ---- Q operands to LDS as hi + lo f16 ------------------------------------------------------
+#pragma unroll
+    for (int k = 0; k < kQEntries; k++) {
+        const int e = threadIdx.x + kThreads * k;
+        half8 h8, l8;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const float x = j < 4 ? qf[k][0][j] : qf[k][1][j - 4];
+            const _Float16 h = (_Float16)x;
+            h8[j] = h;
+            l8[j] = (_Float16)(x - (float)h);
+        }
+        const int l = e & 63, c = (e >> 6) & 7, nt = e >> 9;
+        *reinterpret_cast<half8 *>(Qs + (((nt * 2 + 0) * 8 + c) * 64 + l) * 16) = h8;
+        *reinterpret_cast<half8 *>(Qs + (((nt * 2 + 1) * 8 + c) * 64 + l) * 16) = l8;
+    }
+    __syncthreads();
+    STAMP(2); // Q staged
+
+    // per-column causal bound (MTP rows see one more key each)
     int seq_n[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; nt++) {
         const int n = nt * 16 + lm;
-        const bool valid = n < nvalid;
-        const int col = valid ? n / group : 0;
-        const int head = valid ? n - col * group : 0;
-        seq_n[nt] = valid ? seqc[col] : 0;
-        const float *qp = a.q + (size_t)(row0 + col) * a.q_slot +
-                          (size_t)(kvh * group + head) * kHeadDim + lg * 8;
-#pragma unroll
-        for (int c = 0; c < 8; c++) {
-            float4v f0 = {0, 0, 0, 0}, f1 = {0, 0, 0, 0};
-            if (valid) {
-                f0 = *reinterpret_cast<const float4v *>(qp + c * 32);
-                f1 = *reinterpret_cast<const float4v *>(qp + c * 32 + 4);
-            }
-            float sum = 0.0f;
-#pragma unroll
-            for (int j = 0; j < 8; j++) {
-                const float x = j < 4 ? f0[j] : f1[j - 4];
-                const _Float16 h = (_Float16)x;
-                const _Float16 l = (_Float16)(x - (float)h);
-                qhi[nt][c][j] = h;
-                qlo[nt][c][j] = l;
-                sum += (float)h + (float)l;
-            }
-            // the block's 32 values are spread over the four k-groups
-            sum += __shfl_xor(sum, 16);
-            sum += __shfl_xor(sum, 32);
-            cinit[nt][c] = -128.0f / kTwo24 * sum;
-        }
+        seq_n[nt] = n < nvalid ? seqc[n / group] : 0;
     }
 
     // ---- running state --------------------------------------------------------------
@@ -174,62 +292,26 @@ __global__ void __launch_bounds__(256) decode_q8_kernel(const DecodeArgs a)
             O[nt][t] = (float4v){0, 0, 0, 0};
     }
 
-    // ---- staging: lane owns blocks b = lane + 64*j of the tile (key b/8, chunk b%8) ----
-    uint4v kp0[4], kp1[4], vp0[4], vp1[4];
-    uint16_t ks[4], vs[4];
-    auto issue_loads = [&](int tile) {
-        const int key0 = lo + tile * kTileKeys;
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const int b = lane + 64 * j;
-            int key = key0 + (b >> 3);
-            key = key < hi ? key : hi - 1; // never touch rows past the live range
-            const size_t off = (size_t)key * kRowBytes + (size_t)(b & 7) * kQ8BlockBytes;
-            ks[j] = *reinterpret_cast<const uint16_t *>(kbase + off);
-            kp0[j] = reinterpret_cast<const Raw16 *>(kbase + off + 2)->v;
-            kp1[j] = reinterpret_cast<const Raw16 *>(kbase + off + 18)->v;
-            vs[j] = *reinterpret_cast<const uint16_t *>(vbase + off);
-            vp0[j] = reinterpret_cast<const Raw16 *>(vbase + off + 2)->v;
-            vp1[j] = reinterpret_cast<const Raw16 *>(vbase + off + 18)->v;
-        }
-    };
-    auto store_lds = [&]() {
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const int b = lane + 64 * j;
-            const int r = b >> 3, c = b & 7;
-            *reinterpret_cast<uint4v *>(Kp + r * kLdsRow + c * 32) = kp0[j];
-            *reinterpret_cast<uint4v *>(Kp + r * kLdsRow + c * 32 + 16) = kp1[j];
-            *reinterpret_cast<uint4v *>(Vp + r * kLdsRow + c * 32) = vp0[j];
-            *reinterpret_cast<uint4v *>(Vp + r * kLdsRow + c * 32 + 16) = vp1[j];
-            *reinterpret_cast<uint16_t *>(sK + r * 16 + c * 2) = ks[j];
-            *reinterpret_cast<uint16_t *>(sV + r * 16 + c * 2) = vs[j];
-        }
-    };
-
     // V transpose-read address: lane (2r+e) of its 16-lane group supplies key slot r
     // (slot r<4: key lg*4+r, slot r>=4: key 16+lg*4+(r-4)), bytes [8e, 8e+8) of a 16-d run.
     const int tr_r = lm >> 1;
     const int tr_key = (tr_r >> 2) * 16 + lg * 4 + (tr_r & 3);
-    const uint8_t *vtr = Vp + tr_key * kLdsRow + (lm & 1) * 8;
+    const uint8_t *vtr = tile_lds + tr_key * kLdsRow + (lm & 1) * 8;
+    const float4v zero4 = {0, 0, 0, 0};
+    const uint4v bias_bits = {0x80808080u, 0x80808080u, 0x80808080u, 0x80808080u};
+    const half8 Abias = __builtin_bit_cast(half8, bias_bits); // eight times -128 * 2^-24
 
-    int tile = wave;
-    if (tile < ntile)
-        issue_loads(tile);
-    for (; tile < ntile; tile += kWaves) {
-        store_lds();
-        if (tile + kWaves < ntile)
-            issue_loads(tile + kWaves);
-        const int key0 = lo + tile * kTileKeys;
+    auto process = [&](Unit (&Ku)[2], Unit (&Vu)[2], int t) {
+        const int key0 = lo + (wave + kWaves * t) * kTileKeys;
+        const bool more = t + DEPTH < ntile;
 
-        // ---- scores --------------------------------------------------------------------
-        half8 sk[2][4];
-#pragma unroll
-        for (int ms = 0; ms < 2; ms++)
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-                sk[ms][i] = *reinterpret_cast<const half8 *>(sK + (ms * 16 + lg * 4 + i) * 16);
+        // ---- K tile to LDS, refill the registers ------------------------------------------
+        store_unit(Ku[0], tile_lds, sK, ur0, upr);
+        store_unit(Ku[1], tile_lds, sK, ur1, upr);
+        if (more)
+            issue(Ku, kbase, t + DEPTH);
 
+        // ---- scores ------------------------------------------------------------------------
         float S[NT][2][4];
 #pragma unroll
         for (int nt = 0; nt < NT; nt++)
@@ -238,29 +320,58 @@ __global__ void __launch_bounds__(256) decode_q8_kernel(const DecodeArgs a)
 #pragma unroll
                 for (int i = 0; i < 4; i++)
                     S[nt][ms][i] = 0.0f;
-
+#ifndef DBG_NO_QK
 #pragma unroll
-        for (int ms = 0; ms < 2; ms++) {
+        for (int c = 0; c < 8; c++) {
+            half8 bh[NT], bl[NT];
 #pragma unroll
-            for (int c = 0; c < 8; c++) {
+            for (int nt = 0; nt < NT; nt++) {
+                bh[nt] = *reinterpret_cast<const half8 *>(Qs + (((nt * 2 + 0) * 8 + c) * 64 + lane) * 16);
+                bl[nt] = *reinterpret_cast<const half8 *>(Qs + (((nt * 2 + 1) * 8 + c) * 64 + lane) * 16);
+            }
+#pragma unroll
+            for (int ms = 0; ms < 2; ms++) {
                 const int2v raw = *reinterpret_cast<const int2v *>(
-                    Kp + (ms * 16 + lm) * kLdsRow + c * 32 + lg * 8);
-                const half8 A = bytes_to_subnormal_f16(raw);
+                    tile_lds + (ms * 16 + lm) * kLdsRow + c * 32 + lg * 8);
+                const half8 A = bytes_to_f16_biased(raw);
+                const half4 sk = *reinterpret_cast<const half4 *>(
+                    sK + (c * kTileKeys + ms * 16 + lg * 4) * 2);
 #pragma unroll
                 for (int nt = 0; nt < NT; nt++) {
-                    const float ci = cinit[nt][c];
-                    float4v part = {ci, ci, ci, ci};
-                    part = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, qhi[nt][c], part, 0, 0, 0);
-                    part = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, qlo[nt][c], part, 0, 0, 0);
+                    float4v part = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, bh[nt], zero4, 0, 0, 0);
+                    part = __builtin_amdgcn_mfma_f32_16x16x32_f16(Abias, bh[nt], part, 0, 0, 0);
+                    if (DECODE_QLO) {
+                        part = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, bl[nt], part, 0, 0, 0);
+                        part = __builtin_amdgcn_mfma_f32_16x16x32_f16(Abias, bl[nt], part, 0, 0, 0);
+                    }
 #pragma unroll
                     for (int i = 0; i < 4; i++)
-                        S[nt][ms][i] = fmaf((float)sk[ms][i][c], part[i], S[nt][ms][i]);
+                        S[nt][ms][i] = fmaf((float)sk[i], part[i], S[nt][ms][i]);
                 }
             }
+            // finish this block's scores here: left alone, the optimiser sinks all 8 blocks'
+            // multiply-adds below the refill branch and keeps 16 MFMA results alive
+#pragma unroll
+            for (int nt = 0; nt < NT; nt++)
+#pragma unroll
+                for (int ms = 0; ms < 2; ms++)
+#pragma unroll
+                    for (int i = 0; i < 4; i++)
+                        PIN(S[nt][ms][i]);
         }
+#endif
+
+        // ---- V tile over the K tile, refill -----------------------------------------------
+        store_unit(Vu[0], tile_lds, sV, ur0, upr);
+        store_unit(Vu[1], tile_lds, sV, ur1, upr);
+        if (more)
+            issue(Vu, vbase, t + DEPTH);
 
         // ---- online softmax (log2 units), per column n = lane%16 -----------------------
+        // The probabilities are rounded to f16 once, here; the running sum uses the rounded
+        // values, so numerator and denominator see the same weights.
         float p[NT][2][4];
+        half4 ph[NT][2];
         bool grew = false;
         float corr[NT];
 #pragma unroll
@@ -287,8 +398,14 @@ __global__ void __launch_bounds__(256) decode_q8_kernel(const DecodeArgs a)
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
                     const float e = m_new == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(S[nt][ms][i] - m_new);
-                    p[nt][ms][i] = e;
-                    ls += e;
+                    if (DECODE_PLO) {
+                        p[nt][ms][i] = e;
+                        ls += e;
+                    } else {
+                        const _Float16 eh = (_Float16)e;
+                        ph[nt][ms][i] = eh;
+                        ls += (float)eh;
+                    }
                 }
             l_run[nt] = l_run[nt] * corr[nt] + ls;
             m_run[nt] = m_new;
@@ -297,141 +414,250 @@ __global__ void __launch_bounds__(256) decode_q8_kernel(const DecodeArgs a)
 #pragma unroll
             for (int nt = 0; nt < NT; nt++)
 #pragma unroll
-                for (int t = 0; t < 16; t++)
-                    O[nt][t] *= corr[nt];
+                for (int t2 = 0; t2 < 16; t2++)
+                    O[nt][t2] *= corr[nt];
         }
 
         // ---- O^T += V^T . P' ---------------------------------------------------------------
-        half8 sv[2][4];
-#pragma unroll
-        for (int ms = 0; ms < 2; ms++)
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                // rows past `hi` are duplicates of the last live row: finite scale, p = 0
-                sv[ms][i] = *reinterpret_cast<const half8 *>(sV + (ms * 16 + lg * 4 + i) * 16);
-            }
+#ifndef DBG_NO_PV
 #pragma unroll
         for (int c = 0; c < 8; c++) {
-            // P' = p * block scale, carried as hi + lo f16 so the product keeps ~22 bits
+            // rows past `hi` are duplicates of the last live row: finite scale, p = 0
+            half4 sv[2];
+#pragma unroll
+            for (int ms = 0; ms < 2; ms++)
+                sv[ms] = *reinterpret_cast<const half4 *>(sV + (c * kTileKeys + ms * 16 + lg * 4) * 2);
+            // P' = p * block scale.  Default: one packed f16 multiply (f16-class weights);
+            // DECODE_PLO carries hi + lo f16 so the product keeps ~22 bits.
             half8 Ph[NT], Pl[NT];
 #pragma unroll
-            for (int nt = 0; nt < NT; nt++)
+            for (int nt = 0; nt < NT; nt++) {
+                if (DECODE_PLO) {
 #pragma unroll
-                for (int ms = 0; ms < 2; ms++)
+                    for (int ms = 0; ms < 2; ms++)
 #pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        const float x = p[nt][ms][i] * (float)sv[ms][i][c];
-                        const _Float16 h = (_Float16)x;
-                        Ph[nt][ms * 4 + i] = h;
-                        Pl[nt][ms * 4 + i] = (_Float16)(x - (float)h);
-                    }
+                        for (int i = 0; i < 4; i++) {
+                            const float x = p[nt][ms][i] * (float)sv[ms][i];
+                            const _Float16 h = (_Float16)x;
+                            Ph[nt][ms * 4 + i] = h;
+                            Pl[nt][ms * 4 + i] = (_Float16)(x - (float)h);
+                        }
+                } else {
+                    const half4 x0 = ph[nt][0] * sv[0];
+                    const half4 x1 = ph[nt][1] * sv[1];
+                    Ph[nt] = __builtin_shufflevector(x0, x1, 0, 1, 2, 3, 4, 5, 6, 7);
+                }
+            }
 #pragma unroll
             for (int hf = 0; hf < 2; hf++) {
                 const int2v raw = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
                     (int2v __attribute__((address_space(3))) *)(vtr + c * 32 + hf * 16));
-                const half8 A = sub_bias(bytes_to_subnormal_f16(raw));
+                const half8 A = bytes_to_f16_biased(raw);
 #pragma unroll
                 for (int nt = 0; nt < NT; nt++) {
                     float4v o = O[nt][c * 2 + hf];
                     o = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, Ph[nt], o, 0, 0, 0);
-                    o = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, Pl[nt], o, 0, 0, 0);
+                    o = __builtin_amdgcn_mfma_f32_16x16x32_f16(Abias, Ph[nt], o, 0, 0, 0);
+                    if (DECODE_PLO) {
+                        o = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, Pl[nt], o, 0, 0, 0);
+                        o = __builtin_amdgcn_mfma_f32_16x16x32_f16(Abias, Pl[nt], o, 0, 0, 0);
+                    }
                     O[nt][c * 2 + hf] = o;
                 }
             }
+            SCHED_FENCE();
         }
+#endif
+    };
+
+    for (int t = 0; t < ntile; t += DEPTH) {
+#pragma unroll
+        for (int st = 0; st < DEPTH; st++)
+            if (t + st < ntile)
+                process(Kst[st], Vst[st], t + st);
     }
 
+    STAMP(3); // wave 0 finished its tiles
     // ---- merge the four waves and write the split's partial -------------------------------
-    // O^T C layout: lane holds d = t*16 + lg*4 + i for column n = lane%16.
+    // O^T C layout: lane holds d = t*16 + lg*4 + i for column n = lane%16.  Rounds of 8 columns:
+    // each wave parks 8 columns x 256 d (8 KiB) in its own tile area.
 #pragma unroll
     for (int nt = 0; nt < NT; nt++) {
         l_run[nt] += __shfl_xor(l_run[nt], 16);
         l_run[nt] += __shfl_xor(l_run[nt], 32);
     }
-    float *wl = reinterpret_cast<float *>(lds); // per wave: [16][256] acc, then [16] m, [16] l
+    float *wl = reinterpret_cast<float *>(tile_lds); // per wave: [8][256] acc
+    float *wml = reinterpret_cast<float *>(sK);      // per wave: [8] m, [8] l
 #pragma unroll
     for (int nt = 0; nt < NT; nt++) {
-        __syncthreads(); // everyone is done with the tile buffers / previous round
 #pragma unroll
-        for (int t = 0; t < 16; t++)
+        for (int half = 0; half < 2; half++) {
+            const int nbase = nt * 16 + half * 8;
+            if (nbase >= nvalid)
+                break; // uniform over the workgroup
+            __syncthreads(); // everyone is done with the tile buffers / previous round
+            if ((lm >> 3) == half) {
+                const int n8 = lm & 7;
 #pragma unroll
-            for (int i = 0; i < 4; i++)
-                wl[lm * kHeadDim + t * 16 + lg * 4 + i] = O[nt][t][i];
-        if (lg == 0) {
-            wl[16 * kHeadDim + lm] = m_run[nt];
-            wl[16 * kHeadDim + 16 + lm] = l_run[nt];
-        }
-        __syncthreads();
-        // thread -> (column n, 16 consecutive d): 16 columns x 16 d-runs = 256 threads
-        const int n = threadIdx.x >> 4;
-        const int d0 = (threadIdx.x & 15) * 16;
-        const int ng = nt * 16 + n;
-        if (ng < nvalid) {
-            float mw[kWaves], lw[kWaves];
-            float ms = -INFINITY;
-#pragma unroll
-            for (int w = 0; w < kWaves; w++) {
-                const float *o = reinterpret_cast<const float *>(lds_all + w * kWaveLds);
-                mw[w] = o[16 * kHeadDim + n];
-                lw[w] = o[16 * kHeadDim + 16 + n];
-                ms = fmaxf(ms, mw[w]);
+                for (int t = 0; t < 16; t++)
+                    *reinterpret_cast<float4v *>(wl + n8 * kHeadDim + t * 16 + lg * 4) = O[nt][t];
+                if (lg == 0) {
+                    wml[n8] = m_run[nt];
+                    wml[8 + n8] = l_run[nt];
+                }
             }
-            float lsum = 0.0f;
-            float wgt[kWaves];
-#pragma unroll
-            for (int w = 0; w < kWaves; w++) {
-                wgt[w] = mw[w] == -INFINITY ? 0.0f : exp2f(mw[w] - ms);
-                lsum += lw[w] * wgt[w];
-            }
-            const int col = ng / group;
-            const int head = kvh * group + (ng - col * group);
-            const size_t slice = (size_t)head * a.splits + split;
-            float *pa = a.part_acc + (size_t)(row0 + col) * a.acc_slot + slice * kHeadDim + d0;
-#pragma unroll
-            for (int dd = 0; dd < 16; dd += 4) {
-                float4v acc = {0, 0, 0, 0};
+            __syncthreads();
+            // thread -> (column n8, kRun consecutive d): 8 columns x kThreads/8 d-runs
+            constexpr int kRuns = kThreads / 8, kRun = kHeadDim / kRuns;
+            const int n8 = threadIdx.x / kRuns;
+            const int d0 = (threadIdx.x % kRuns) * kRun;
+            const int ng = nbase + n8;
+            if (ng < nvalid) {
+                float mw[kWaves], lw[kWaves];
+                float ms = -INFINITY;
 #pragma unroll
                 for (int w = 0; w < kWaves; w++) {
-                    const float *o = reinterpret_cast<const float *>(lds_all + w * kWaveLds);
-                    const float4v x = *reinterpret_cast<const float4v *>(o + n * kHeadDim + d0 + dd);
-                    acc += x * (wgt[w] * kTwo24);
+                    const float *o = reinterpret_cast<const float *>(wave_base + w * kWaveLds + kTileBytes);
+                    mw[w] = o[n8];
+                    lw[w] = o[8 + n8];
+                    ms = fmaxf(ms, mw[w]);
                 }
-                *reinterpret_cast<float4v *>(pa + dd) = acc;
-            }
-            if ((threadIdx.x & 15) == 0) {
-                float *pm = a.part_ml + (size_t)(row0 + col) * a.ml_slot + slice * 2;
-                pm[0] = ms;
-                pm[1] = lsum;
+                float lsum = 0.0f;
+                float wgt[kWaves];
+#pragma unroll
+                for (int w = 0; w < kWaves; w++) {
+                    wgt[w] = mw[w] == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(mw[w] - ms);
+                    lsum += lw[w] * wgt[w];
+                    wgt[w] *= kTwo24;
+                }
+                const int col = ng / group;
+                const int head = kvh * group + (ng - col * group);
+                const size_t slice = (size_t)head * a.splits + split;
+                float *pa = a.part_acc + (size_t)(row0 + col) * a.acc_slot + slice * kHeadDim + d0;
+#pragma unroll
+                for (int dd = 0; dd < kRun; dd += 4) {
+                    float4v acc = {0, 0, 0, 0};
+#pragma unroll
+                    for (int w = 0; w < kWaves; w++) {
+                        const float *o = reinterpret_cast<const float *>(wave_base + w * kWaveLds);
+                        const float4v x = *reinterpret_cast<const float4v *>(o + n8 * kHeadDim + d0 + dd);
+                        acc += x * wgt[w];
+                    }
+                    *reinterpret_cast<float4v *>(pa + dd) = acc;
+                }
+                if (threadIdx.x % kRuns == 0) {
+                    float *pm = a.part_ml + (size_t)(row0 + col) * a.ml_slot + slice * 2;
+                    pm[0] = ms;
+                    pm[1] = lsum;
+                }
             }
         }
     }
+    STAMP(4);
 }
 
 // out[row][head][d] = sum_s acc_s[d] * 2^(m_s - m) / sum_s l_s * 2^(m_s - m); 0 when no
-// split saw a key.  grid (n_heads, rows), 256 threads = head_dim.
+// split saw a key.  grid (n_heads * 4, rows): a workgroup owns 64 d of one (row, head);
+// thread = (split group 0..15, float4 of d 0..15).
+constexpr int kReduceMaxSplits = 4096;
+
 __global__ void __launch_bounds__(256) decode_reduce_kernel(
     const float *__restrict__ part_acc, const float *__restrict__ part_ml, float *__restrict__ out,
     int splits, size_t acc_slot, size_t ml_slot, size_t q_slot)
 {
-    const int head = blockIdx.x;
+    __shared__ float w_s[kReduceMaxSplits];
+    __shared__ float red[256];
+    __shared__ float4v accs[16][16];
+    const int head = blockIdx.x >> 2;
+    const int dq = blockIdx.x & 3;
     const int row = blockIdx.y;
-    const int d = threadIdx.x;
+    const int tid = threadIdx.x;
     const float *ml = part_ml + (size_t)row * ml_slot + (size_t)head * splits * 2;
-    const float *acc = part_acc + (size_t)row * acc_slot + (size_t)head * splits * kHeadDim + d;
+
+    // weights: w_s = 2^(m_s - m) for splits that saw a key, else 0
     float m = -INFINITY;
-    for (int s = 0; s < splits; s++)
-        if (ml[s * 2 + 1] > 0.0f)
-            m = fmaxf(m, ml[s * 2]);
-    float num = 0.0f, den = 0.0f;
-    for (int s = 0; s < splits; s++) {
-        const float l = ml[s * 2 + 1];
-        if (l > 0.0f) {
-            const float w = exp2f(ml[s * 2] - m);
-            num = fmaf(acc[(size_t)s * kHeadDim], w, num);
-            den = fmaf(l, w, den);
-        }
+    for (int s = tid; s < splits; s += 256) {
+        const float2 v = *reinterpret_cast<const float2 *>(ml + s * 2);
+        w_s[s] = v.x;
+        if (v.y > 0.0f)
+            m = fmaxf(m, v.x);
     }
-    out[(size_t)row * q_slot + (size_t)head * kHeadDim + d] = den > 0.0f ? num / den : 0.0f;
+    red[tid] = m;
+    __syncthreads();
+    for (int o = 128; o > 0; o >>= 1) {
+        if (tid < o)
+            red[tid] = fmaxf(red[tid], red[tid + o]);
+        __syncthreads();
+    }
+    m = red[0];
+    __syncthreads();
+    float den = 0.0f;
+    for (int s = tid; s < splits; s += 256) {
+        const float l = ml[s * 2 + 1];
+        const float w = l > 0.0f ? __builtin_amdgcn_exp2f(w_s[s] - m) : 0.0f;
+        w_s[s] = w;
+        den = fmaf(l, w, den);
+    }
+    red[tid] = den;
+    __syncthreads();
+    for (int o = 128; o > 0; o >>= 1) {
+        if (tid < o)
+            red[tid] += red[tid + o];
+        __syncthreads();
+    }
+    den = red[0];
+
+    const int sg = tid >> 4, dl = tid & 15;
+    const float *acc = part_acc + (size_t)row * acc_slot + (size_t)head * splits * kHeadDim +
+                       dq * 64 + dl * 4;
+    float4v num = {0, 0, 0, 0};
+    // zero-weight slices may hold anything (even NaN from an untouched scratch): select, not multiply
+    auto term = [&](int s) {
+        const float w = w_s[s];
+        const float4v x = *reinterpret_cast<const float4v *>(acc + (size_t)s * kHeadDim);
+        const float4v z = {0, 0, 0, 0};
+        return w > 0.0f ? x * w : z;
+    };
+    int s = sg;
+    for (; s + 48 < splits; s += 64)
+        num += (term(s) + term(s + 16)) + (term(s + 32) + term(s + 48));
+    for (; s < splits; s += 16)
+        num += term(s);
+    accs[sg][dl] = num;
+    __syncthreads();
+    if (tid < 16) {
+        float4v t = accs[0][tid];
+#pragma unroll
+        for (int g = 1; g < 16; g++)
+            t += accs[g][tid];
+        const float inv = den > 0.0f ? 1.0f / den : 0.0f;
+        float4v r = t * inv;
+        if (!(den > 0.0f))
+            r = (float4v){0, 0, 0, 0};
+        *reinterpret_cast<float4v *>(out + (size_t)row * q_slot + (size_t)head * kHeadDim + dq * 64 +
+                                     tid * 4) = r;
+    }
+}
+
+#ifdef DBG_TIMING
+extern "C" int hipml_dbg_read_stamps(unsigned long long *host, size_t n)
+{
+    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_dbg_t), n * 8);
+}
+#endif
+
+int decode_init()
+{
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&decode_q8_kernel<1, kDepth>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       decode_lds_bytes(1));
+    if (e == hipSuccess)
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&decode_q8_kernel<2, kDepth>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, decode_lds_bytes(2));
+    if (e != hipSuccess)
+        return fail((int)e, "hipFuncSetAttribute(decode LDS) failed: %d (%s)", (int)e,
+                    hipGetErrorString(e));
+    return 0;
 }
 
 int launch_decode_q8(hipStream_t st, const DecodeLaunch &L)
@@ -458,15 +684,15 @@ int launch_decode_q8(hipStream_t st, const DecodeLaunch &L)
     }
     const dim3 grid((unsigned)(L.n_kv * L.splits), (unsigned)L.slots, 1);
     if (L.max_cols * a.group <= 16)
-        hipLaunchKernelGGL(decode_q8_kernel<1>, grid, dim3(256, 1, 1), 0, st, a);
+        hipLaunchKernelGGL((decode_q8_kernel<1, kDepth>), grid, dim3(kThreads, 1, 1), decode_lds_bytes(1), st, a);
     else
-        hipLaunchKernelGGL(decode_q8_kernel<2>, grid, dim3(256, 1, 1), 0, st, a);
+        hipLaunchKernelGGL((decode_q8_kernel<2, kDepth>), grid, dim3(kThreads, 1, 1), decode_lds_bytes(2), st, a);
     int rc = launched("attn_decode_kv_q8");
     if (rc)
         return rc;
-    hipLaunchKernelGGL(decode_reduce_kernel, dim3((unsigned)L.n_heads, (unsigned)L.total_rows, 1),
-                       dim3(256, 1, 1), 0, st, L.part_acc, L.part_ml, L.out, L.splits, L.acc_slot,
-                       L.ml_slot, L.q_slot);
+    hipLaunchKernelGGL(decode_reduce_kernel,
+                       dim3((unsigned)L.n_heads * 4, (unsigned)L.total_rows, 1), dim3(256, 1, 1), 0,
+                       st, L.part_acc, L.part_ml, L.out, L.splits, L.acc_slot, L.ml_slot, L.q_slot);
     return launched("attn_decode_kv_reduce");
 }
 

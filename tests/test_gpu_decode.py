@@ -1,7 +1,8 @@
 """Decode attention over a q8_0 cache: HIP path (through the C ABI) vs the CPU oracle
-on identical seeded inputs.  Gate: max-abs 2e-3 / rel 1e-2 (OR rule); the reference's
-own decode class, 1e-4 / 1e-3 (crates/hipml-core/src/parity_kv.rs:7-10), is asserted
-as well because the kernel keeps K and V exact and Q to ~22 bits."""
+on identical seeded inputs.  Gate: max-abs 2e-3 / rel 1e-2 (OR rule).  The kernel keeps K, V
+and the block scales exact and Q to ~22 bits, but rounds the softmax weight times the V block
+scale to f16 once (as the reference's chunk kernel rounds P), so its own class is a few 1e-4:
+KERNEL_CLASS below is asserted everywhere, a quarter of the gate."""
 import numpy as np
 import pytest
 import torch
@@ -14,7 +15,7 @@ from gpu_util import (N_HEADS, N_KV, HD, SCALE, ROW, dev, host, quantized_cache,
                       decode_scratch, run_decode, report)
 
 GATE = (2e-3, 1e-2)
-REF_CLASS = (1e-4, 1e-3)
+KERNEL_CLASS = (5e-4, 5e-3)
 
 
 @pytest.fixture(scope="module", autouse=True)
@@ -42,7 +43,7 @@ def test_reference_kv_cases(name, seed, heads, n_kv, seq, splits):
     kb, vb = quantized_cache(kf, vf)
     want = orc.attn_decode_kv(q, kb, vb, heads, n_kv, HD, seq, SCALE)
     got = run_decode(q, kb, vb, heads, n_kv, seq, seq, SCALE, splits)
-    ok, _, _ = report(name, want, got, *REF_CLASS)
+    ok, _, _ = report(name, want, got, *KERNEL_CLASS)
     assert ok
     assert orc.compare(want, got, *GATE)[0]
 
@@ -53,7 +54,7 @@ def test_deep_case_100k_one_head():
     kb, vb = quantized_cache(kf, vf)
     want = orc.attn_decode_kv(q, kb, vb, 1, 1, HD, 100_000, SCALE)
     got = run_decode(q, kb, vb, 1, 1, 100_000, 100_000, SCALE, 256)
-    ok, _, _ = report("attn_decode_kv_q8_hd256_s100000", want, got, *REF_CLASS)
+    ok, _, _ = report("attn_decode_kv_q8_hd256_s100000", want, got, *KERNEL_CLASS)
     assert ok
 
 
@@ -68,7 +69,7 @@ def test_decode_full_geometry(seq, stride):
     want = orc.attn_decode_kv(q, kb, vb, N_HEADS, N_KV, HD, seq, SCALE, stride=stride)
     splits = attn.decode_splits(seq, N_KV)
     got = run_decode(q, kb, vb, N_HEADS, N_KV, seq, stride, SCALE, splits)
-    ok, _, _ = report(f"decode 24/4 seq {seq} stride {stride} splits {splits}", want, got, *REF_CLASS)
+    ok, _, _ = report(f"decode 24/4 seq {seq} stride {stride} splits {splits}", want, got, *KERNEL_CLASS)
     assert ok
     assert orc.compare(want, got, *GATE)[0]
 
@@ -82,7 +83,7 @@ def test_any_split_count_gives_the_same_answer(splits):
     kb, vb = quantized_cache(kf, vf)
     one = run_decode(q, kb, vb, N_HEADS, N_KV, seq, seq, SCALE, 1)
     got = run_decode(q, kb, vb, N_HEADS, N_KV, seq, seq, SCALE, splits)
-    ok, ma, _ = report(f"splits {splits} vs 1", one, got, 1e-5, 1e-4)  # fp32 reassociation only
+    ok, ma, _ = report(f"splits {splits} vs 1", one, got, 2e-4, 2e-3)  # f16 weights round against a different running maximum per slice
     assert ok
 
 
@@ -99,7 +100,7 @@ def test_peaked_softmax_and_large_scores():
     kb, vb = quantized_cache(kf, vf)
     want = orc.attn_decode_kv(q, kb, vb, N_HEADS, N_KV, HD, seq, SCALE)
     got = run_decode(q, kb, vb, N_HEADS, N_KV, seq, seq, SCALE, 3)
-    ok, _, _ = report("peaked softmax", want, got, *REF_CLASS)
+    ok, _, _ = report("peaked softmax", want, got, *KERNEL_CLASS)
     assert ok
 
 
@@ -123,7 +124,7 @@ def test_seq_zero_gives_zero_and_k_v_offsets_are_honoured():
                         seq, SCALE, 2, pad, pad)
     torch.cuda.synchronize()
     want = orc.attn_decode_kv(q, kb, vb, N_HEADS, N_KV, HD, seq, SCALE)
-    assert orc.compare(want, host(out), *REF_CLASS)[0]
+    assert orc.compare(want, host(out), *KERNEL_CLASS)[0]
 
 
 @pytest.mark.parametrize("cols", [1, 2, 3, 4])
@@ -149,7 +150,7 @@ def test_mtp_columns_equal_single_token_decodes(cols):
     got = host(out)
     for c in range(cols):
         want = orc.attn_decode_kv(q[c], kb, vb, N_HEADS, N_KV, HD, pos0 + c + 1, SCALE, stride=stride)
-        ok, _, _ = report(f"verify column {c}/{cols}", want, got[c], *REF_CLASS)
+        ok, _, _ = report(f"verify column {c}/{cols}", want, got[c], *KERNEL_CLASS)
         assert ok
         single = run_decode(q[c], kb, vb, N_HEADS, N_KV, pos0 + c + 1, stride, SCALE, splits)
         assert orc.compare(single, got[c].ravel(), 1e-6, 1e-5)[0]
@@ -190,7 +191,7 @@ def test_batched_decode_uniform_rows():
     for s in range(slots):
         want = orc.attn_decode_kv(q[s], kc[s], vc[s], N_HEADS, N_KV, HD, pos[s][1], SCALE,
                                   stride=stride)
-        ok, _, _ = report(f"batch slot {s} seq {pos[s][1]}", want, got[s], *REF_CLASS)
+        ok, _, _ = report(f"batch slot {s} seq {pos[s][1]}", want, got[s], *KERNEL_CLASS)
         assert ok
 
 
@@ -218,7 +219,7 @@ def test_batched_decode_with_mtp_slots_in_one_launch():
         for j in range(c):
             want = orc.attn_decode_kv(q[row], kc[s], vc[s], N_HEADS, N_KV, HD, pos[row][1], SCALE,
                                       stride=stride)
-            ok, ma, _ = orc.compare(want, got[row], *REF_CLASS)
+            ok, ma, _ = orc.compare(want, got[row], *KERNEL_CLASS)
             worst = max(worst, ma)
             assert ok, f"slot {s} row {j} seq {pos[row][1]}: max_abs {ma}"
             row += 1
@@ -244,4 +245,4 @@ def test_verify_group_through_rows_entry_shares_the_cache():
     torch.cuda.synchronize()
     for c in range(cols):
         want = orc.attn_decode_kv(q[c], kb, vb, N_HEADS, N_KV, HD, pos0 + c + 1, SCALE, stride=stride)
-        assert orc.compare(want, host(out)[c], *REF_CLASS)[0]
+        assert orc.compare(want, host(out)[c], *KERNEL_CLASS)[0]
