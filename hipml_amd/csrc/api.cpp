@@ -152,6 +152,8 @@ int hipml_attn_init(int device)
         return fail(HIPML_ATTN_E_DEVICE, "device %d is %s; this library is built for gfx950 only",
                     device, prop.gcnArchName);
     int rc = decode_init();
+    if (rc == 0)
+        rc = prefill_init();
     if (rc)
         return rc;
     g_inited = true;
@@ -192,19 +194,32 @@ int hipml_attn_batch_splits(int stride, int n_kv, int slots)
 
 int hipml_attn_chunk_splits(int pos0, int tokens, int n_kv)
 {
+    // A prefill workgroup is 8 tasks of (32 tokens x 1 head) and owns a whole CU (two 66 KiB
+    // LDS buffers), so the launch wants a few hundred workgroups: split the keys until there
+    // are about two rounds of 256, keep at least 128 keys per slice, and prefer a slice count
+    // that makes n_kv * splits a multiple of the 8 XCDs (the kernel then keeps each slice's
+    // K/V stream inside one XCD's L2).  Heads per KV head are taken as 6, the geometry built.
     if (tokens < 1 || n_kv < 1)
         return 1;
-    const int qtiles = (tokens + 31) / 32;
-    const int wgs = qtiles * n_kv;
+    const int ntask = (tokens + 31) / 32 * 6;
+    const int wgs = n_kv * ((ntask + 7) / 8);
     if (wgs >= 512)
         return 1;
     int s = (512 + wgs - 1) / wgs;
     const int keys = pos0 + tokens;
-    const int by_work = (keys + 255) / 256; // at least 256 keys per slice
+    const int by_work = keys / 128;
     if (s > by_work)
         s = by_work;
     if (s > 16)
         s = 16;
+    int up = s;
+    while (up <= 16 && up <= by_work && (n_kv * up) % 8 != 0)
+        up++;
+    if (up <= 16 && up <= by_work)
+        s = up;
+    else
+        while (s > 1 && (n_kv * s) % 8 != 0)
+            s--;
     return s < 1 ? 1 : s;
 }
 

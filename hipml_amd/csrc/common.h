@@ -68,6 +68,8 @@ int launch_decode_q8(hipStream_t st, const DecodeLaunch &a);
 // Raise the decode kernels' dynamic LDS limit (once per process; called by hipml_attn_init).
 int decode_init();
 
+// Raise the prefill kernels' dynamic LDS limit (once per process; called by hipml_attn_init).
+int prefill_init();
 int launch_chunk_q8(hipStream_t st, const float *q, const uint8_t *kc, const uint8_t *vc,
                     float *out, int n_head, int n_kv, int pos0, int tokens, int stride,
                     float *part_acc, float *part_ml, int splits);

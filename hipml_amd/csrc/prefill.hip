@@ -1,9 +1,13 @@
 // Causal GQA chunk prefill over a q8_0 KV cache for gfx950 (wave64, MFMA).
 //
-// One workgroup = one KV head x one tile of 32 query tokens (x one key slice when
-// split).  Wave w of the workgroup owns query head kvh*group + w, so a wave's
-// MFMA column n is query token t0 + n.  All waves share the K/V tile, which is
-// dequantized once per workgroup into f16 in LDS.
+// Work unit ("task") = 32 query tokens x 1 query head.  The tasks of one KV head are
+// numbered token-tile major (task = token_tile * group + head_in_group); a workgroup of 8
+// waves takes 8 consecutive tasks (x one key slice when split), one per wave, two waves per
+// SIMD.  All 8 tasks share the K/V stream: a tile of 64 keys is fetched as 68-byte units
+// (two whole q8_0 blocks of one key per thread, dword-aligned 128-bit loads), dequantized
+// once per workgroup to f16 and written to one of two LDS buffers.  The two waves of a SIMD
+// run one slot apart, so one does VALU work (dequantization, softmax) while the other issues
+// MFMAs; LDS operand reads are pinned two MFMAs ahead with scheduling groups.
 //
 // All MFMAs are v_mfma_f32_32x32x16_f16:
 //   S^T[key 32][tok 32] += K[key][d 16] . Q^T[d 16][tok]       (16 steps over d)
@@ -27,12 +31,27 @@ typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef float float4v __attribute__((ext_vector_type(4)));
 typedef float float16v __attribute__((ext_vector_type(16)));
 typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
+typedef uint32_t uint4a4 __attribute__((ext_vector_type(4), aligned(4)));
 typedef short short4v __attribute__((ext_vector_type(4)));
 
-constexpr int kQTile = 32;   // query tokens per workgroup
-constexpr int kKTile = 32;   // keys per LDS tile
-constexpr int kRowF16 = 528; // bytes per dequantized row in LDS: 512 + 16 pad
+constexpr int kQTile = 32;    // query tokens per task
+constexpr int kTasks = 8;     // tasks (= waves) per workgroup
+constexpr int kPfThreads = 64 * kTasks;
+constexpr int kKTile = 64;    // keys per LDS tile
+// f16 rows in LDS: 512 bytes + pad.  528 keeps the K operand's 128-bit reads (lane = row) and
+// the staging writes conflict free; 544 does the same for the V transpose reads (8 rows x 64
+// bytes per instruction) at the price of 2-way conflicts on V's staging writes.
+constexpr int kKRow = 528;
+constexpr int kVRow = 544;
+constexpr int kVOff = kKTile * kKRow;                  // V tile follows the K tile
+constexpr int kBufBytes = kKTile * (kKRow + kVRow);    // 68,608
+constexpr int kQLdsSteps = 3;                          // d-steps of the Q operand parked in LDS
+constexpr int kQLdsOff = 2 * kBufBytes;                // after the two tile buffers (137,216)
+constexpr int kPfLds = kQLdsOff + kTasks * kQLdsSteps * 1024; // 161,792 of 163,840
 constexpr float kLog2e = 1.4426950408889634f;
+#ifndef PF_SKEW
+#define PF_SKEW 1
+#endif
 
 struct ChunkArgs {
     const float *q;
@@ -43,12 +62,26 @@ struct ChunkArgs {
     float *part_ml;
     int n_head, n_kv, group;
     int pos0, tokens, stride, splits, qslots;
+    int ntask;  // tasks per KV head = ceil(tokens/32) * group
+    int nblock; // task blocks per KV head = ceil(ntask/8)
     float scale_log2;
 };
 
-struct __attribute__((packed, aligned(2))) Raw16 {
-    uint4v v;
+// 68 bytes of a key row starting at a block-pair boundary: [s0 | 32 x i8 | s1 | 32 x i8].
+struct Unit {
+    uint4v a, b; // dwords 0..7
+    uint32_t m;  // dword 8
+    uint4v c, d; // dwords 9..16
 };
+
+__device__ __forceinline__ void load_unit(Unit &u, const uint8_t *p)
+{
+    u.a = *reinterpret_cast<const uint4a4 *>(p);
+    u.b = *reinterpret_cast<const uint4a4 *>(p + 16);
+    u.m = *reinterpret_cast<const uint32_t *>(p + 32);
+    u.c = *reinterpret_cast<const uint4a4 *>(p + 36);
+    u.d = *reinterpret_cast<const uint4a4 *>(p + 52);
+}
 
 // 16 int8 -> 16 f16 (value * d), d an f16 scale: the bytes become 1024 + (b+128)
 // in f16 by bit tricks, the bias is subtracted exactly, then one packed multiply
@@ -70,23 +103,120 @@ __device__ __forceinline__ void dequant16(uint4v raw, _Float16 d, uint4v &lo, ui
     hi = (uint4v){o[4], o[5], o[6], o[7]};
 }
 
-template <bool SPLIT>
-__global__ void __launch_bounds__(512) chunk_q8_kernel(const ChunkArgs a)
+// Dequantize one unit (blocks 2*pr and 2*pr+1 of one key) into 128 bytes of f16 at `dst`.
+__device__ __forceinline__ void stage_unit(const Unit &u, uint8_t *dst)
 {
-    __shared__ __attribute__((aligned(16))) uint8_t Ks[kKTile * kRowF16];
-    __shared__ __attribute__((aligned(16))) uint8_t Vs[kKTile * kRowF16];
+    uint4v e0, e1;
+    e0[0] = __builtin_amdgcn_alignbit(u.a[1], u.a[0], 16);
+    e0[1] = __builtin_amdgcn_alignbit(u.a[2], u.a[1], 16);
+    e0[2] = __builtin_amdgcn_alignbit(u.a[3], u.a[2], 16);
+    e0[3] = __builtin_amdgcn_alignbit(u.b[0], u.a[3], 16);
+    e1[0] = __builtin_amdgcn_alignbit(u.b[1], u.b[0], 16);
+    e1[1] = __builtin_amdgcn_alignbit(u.b[2], u.b[1], 16);
+    e1[2] = __builtin_amdgcn_alignbit(u.b[3], u.b[2], 16);
+    e1[3] = __builtin_amdgcn_alignbit(u.m, u.b[3], 16);
+    const _Float16 s0 = __builtin_bit_cast(_Float16, (uint16_t)(u.a[0] & 0xffffu));
+    const _Float16 s1 = __builtin_bit_cast(_Float16, (uint16_t)(u.m >> 16));
+    uint4v *d4 = reinterpret_cast<uint4v *>(dst);
+    uint4v x0, x1;
+    dequant16(e0, s0, x0, x1);
+    d4[0] = x0;
+    d4[1] = x1;
+    dequant16(e1, s0, x0, x1);
+    d4[2] = x0;
+    d4[3] = x1;
+    dequant16(u.c, s1, x0, x1);
+    d4[4] = x0;
+    d4[5] = x1;
+    dequant16(u.d, s1, x0, x1);
+    d4[6] = x0;
+    d4[7] = x1;
+}
 
-    const int wave = threadIdx.x >> 6; // query head within the group
+#ifdef PF_TIMING
+// debug builds: per-wave accumulated phase times (100 MHz ticks) for workgroup 0: [wave][6]
+__device__ unsigned long long g_pf_t[8 * 8];
+#define TSTART() unsigned long long t_prev = wall_clock64(), t_now; unsigned long long t_acc[6] = {0, 0, 0, 0, 0, 0}
+#define TMARK(i) do { t_now = wall_clock64(); t_acc[i] += t_now - t_prev; t_prev = t_now; } while (0)
+#define TDUMP() do { if (blockIdx.x == 8 && (threadIdx.x & 63) == 0) for (int i = 0; i < 6; i++) g_pf_t[(threadIdx.x >> 6) * 8 + i] = t_acc[i]; } while (0)
+#else
+#define TSTART() do { } while (0)
+#define TMARK(i) do { } while (0)
+#define TDUMP() do { } while (0)
+#endif
+
+// max(x[lane], x[lane ^ 32]) without going through LDS: swapping the upper half of one copy
+// with the lower half of another leaves {lo, lo} and {hi, hi}.  (Written as asm: the
+// compiler's builtin for this instruction returns its first result twice.)
+__device__ __forceinline__ float xor32_max(float x)
+{
+    float a = x, b = x;
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+    return fmaxf(a, b);
+}
+
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every
+// outstanding global load (vmcnt(0)), which would expose the full latency of the next tile's
+// prefetch at each phase boundary; here only LDS operations are drained.
+__device__ __forceinline__ void lds_barrier()
+{
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+template <bool SPLIT>
+__global__ void __launch_bounds__(kPfThreads, 2) chunk_q8_kernel(const ChunkArgs a)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+
+    const int wave = threadIdx.x >> 6;
     const int lane = threadIdx.x & 63;
     const int ln = lane & 31;  // MFMA column: token within the tile
     const int lh = lane >> 5;  // k half-group
-    const int kvh = blockIdx.x;
-    const int t0 = blockIdx.y * kQTile;
-    const int split = SPLIT ? blockIdx.z : 0;
-    const int head = kvh * a.group + wave;
+    // Waves w and w+4 share a SIMD.  Set 0 (waves 0..3) and set 1 (waves 4..7) run the same
+    // program half an iteration apart: while one set issues MFMAs (PV of tile t, scores of
+    // tile t+1) the other does its VALU work (softmax, dequantization of the next tile).
+    // Set 0 stages the K tiles, set 1 the V tiles.
+    const int set = wave >> 2;
 
-    // visible key range of this workgroup
-    const int last_tok = (t0 + kQTile < a.tokens ? t0 + kQTile : a.tokens) - 1;
+    // blockIdx.x -> (kv head, key slice, task block).  Consecutive workgroups go to different
+    // XCDs (8 of them, each with its own L2); the workgroups that stream the same (kv head,
+    // slice) are therefore placed 8 apart, so that slice's K/V rows pass through one L2.
+    int kvh, split, tb;
+    {
+        const int combos = a.n_kv * (SPLIT ? a.splits : 1);
+        const int bid = blockIdx.x;
+        int combo;
+        if (combos % 8 == 0) {
+            const int per = combos / 8;
+            const int xcd = bid & 7, j = bid >> 3;
+            combo = xcd + 8 * (j % per);
+            tb = j / per;
+        } else if (8 % combos == 0) {
+            const int xcd = bid & 7, j = bid >> 3;
+            const int share = 8 / combos; // XCDs per combo
+            combo = xcd % combos;
+            tb = j * share + xcd / combos;
+        } else {
+            combo = bid % combos;
+            tb = bid / combos;
+        }
+        kvh = combo % a.n_kv;
+        split = combo / a.n_kv;
+    }
+    if (tb >= a.nblock)
+        return; // uniform over the workgroup
+
+    const int task = tb * kTasks + wave;
+    const bool task_valid = task < a.ntask;
+    const int tt = (task_valid ? task : a.ntask - 1) / a.group;
+    const int hq = (task_valid ? task : a.ntask - 1) - tt * a.group;
+    const int head = kvh * a.group + hq;
+    const int t0 = tt * kQTile;
+
+    // visible key range of this workgroup: up to the last token of its last task
+    const int last_task = (tb * kTasks + kTasks - 1 < a.ntask ? tb * kTasks + kTasks - 1 : a.ntask - 1);
+    const int tt_last = last_task / a.group;
+    const int last_tok = ((tt_last + 1) * kQTile < a.tokens ? (tt_last + 1) * kQTile : a.tokens) - 1;
     const int seq_block = a.pos0 + last_tok + 1;
     int klo = 0, khi = seq_block;
     if (SPLIT) {
@@ -94,23 +224,52 @@ __global__ void __launch_bounds__(512) chunk_q8_kernel(const ChunkArgs a)
         khi = (int)((long long)seq_block * (split + 1) / a.splits);
     }
     const int tok = t0 + ln;
-    const int my_last_key = a.pos0 + tok; // inclusive causal bound of this lane's token
-    const bool tok_valid = tok < a.tokens;
+    const int my_last_key = a.pos0 + tok;               // inclusive causal bound of this lane's token
+    const int task_last_key = a.pos0 + t0 + kQTile - 1; // of the task's last token
+    const bool tok_valid = task_valid && tok < a.tokens;
+    const int ntile = khi > klo ? (khi - klo + kKTile - 1) / kKTile : 0;
+
+    // ---- staging role: thread -> one 68-byte unit of the K tile (set 0) or V tile (set 1) ----
+    const int su = threadIdx.x & 255;
+    const int srow = su >> 2, spr = su & 3;
+    const uint8_t *sbase = (set ? a.vc : a.kc) + (size_t)kvh * a.stride * kRowBytes + spr * 68;
+    const int sdst = set ? kVOff + srow * kVRow + spr * 128 : srow * kKRow + spr * 128;
+    Unit unit;
+    auto issue = [&](int t) {
+#ifdef PF_DBG_SAMETILE
+        t = t & 7; // debug: keep re-reading the first tiles (cache hits)
+#endif
+        int key = klo + t * kKTile + srow;
+        key = key < khi ? key : khi - 1;
+        load_unit(unit, sbase + (size_t)key * kRowBytes);
+    };
+    auto stage = [&](int t) { stage_unit(unit, lds + (t & 1) * kBufBytes + sdst); };
+    if (ntile > 0)
+        issue(0);
 
     // ---- Q^T operand: 16 k-steps of 8 f16 (d = ks*16 + lh*8 + j) ---------------------------
+    // Steps 0..kQLdsSteps-1 are parked in this wave's corner of LDS and re-read per use: 256
+    // registers do not hold O (128), all of Q (64), the scores, the tile prefetch and the operand
+    // pipeline at once, and what the compiler would spill instead goes to scratch memory.
     half8 qf[16];
+    uint8_t *qlds = lds + kQLdsOff + wave * kQLdsSteps * 1024 + lane * 16;
     {
-        const int tq = tok_valid ? tok : a.tokens - 1;
+        const int tq = tok < a.tokens ? tok : a.tokens - 1;
         const float *qp = a.q + ((size_t)tq * a.n_head + head) * kHeadDim + lh * 8;
 #pragma unroll
         for (int ks = 0; ks < 16; ks++) {
             const float4v f0 = *reinterpret_cast<const float4v *>(qp + ks * 16);
             const float4v f1 = *reinterpret_cast<const float4v *>(qp + ks * 16 + 4);
+            half8 h;
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                qf[ks][j] = (_Float16)f0[j];
-                qf[ks][4 + j] = (_Float16)f1[j];
+                h[j] = (_Float16)f0[j];
+                h[4 + j] = (_Float16)f1[j];
             }
+            if (ks < kQLdsSteps)
+                *reinterpret_cast<half8 *>(qlds + ks * 1024) = h;
+            else
+                qf[ks] = h;
         }
     }
 
@@ -121,132 +280,185 @@ __global__ void __launch_bounds__(512) chunk_q8_kernel(const ChunkArgs a)
         for (int i = 0; i < 16; i++)
             O[t][i] = 0.0f;
     float m_run = -INFINITY, l_run = 0.0f;
-
-    const uint8_t *kbase = a.kc + (size_t)kvh * a.stride * kRowBytes;
-    const uint8_t *vbase = a.vc + (size_t)kvh * a.stride * kRowBytes;
-
-    // staging role: thread b < 256 owns block (key b/8, chunk b%8) of the tile
-    const int sb = threadIdx.x;
-    const bool stager = sb < 256;
-    uint4v rk0, rk1, rv0, rv1;
-    uint16_t rks = 0, rvs = 0;
-    auto issue = [&](int k0) {
-        if (stager) {
-            int key = k0 + (sb >> 3);
-            key = key < khi ? key : khi - 1;
-            const size_t off = (size_t)key * kRowBytes + (size_t)(sb & 7) * kQ8BlockBytes;
-            rks = *reinterpret_cast<const uint16_t *>(kbase + off);
-            rk0 = reinterpret_cast<const Raw16 *>(kbase + off + 2)->v;
-            rk1 = reinterpret_cast<const Raw16 *>(kbase + off + 18)->v;
-            rvs = *reinterpret_cast<const uint16_t *>(vbase + off);
-            rv0 = reinterpret_cast<const Raw16 *>(vbase + off + 2)->v;
-            rv1 = reinterpret_cast<const Raw16 *>(vbase + off + 18)->v;
-        }
-    };
-    auto stage = [&]() {
-        if (stager) {
-            const int r = sb >> 3, c = sb & 7;
-            uint4v a0, a1, a2, a3;
-            dequant16(rk0, __builtin_bit_cast(_Float16, rks), a0, a1);
-            dequant16(rk1, __builtin_bit_cast(_Float16, rks), a2, a3);
-            uint4v *dk = reinterpret_cast<uint4v *>(Ks + r * kRowF16 + c * 64);
-            dk[0] = a0;
-            dk[1] = a1;
-            dk[2] = a2;
-            dk[3] = a3;
-            dequant16(rv0, __builtin_bit_cast(_Float16, rvs), a0, a1);
-            dequant16(rv1, __builtin_bit_cast(_Float16, rvs), a2, a3);
-            uint4v *dv = reinterpret_cast<uint4v *>(Vs + r * kRowF16 + c * 64);
-            dv[0] = a0;
-            dv[1] = a1;
-            dv[2] = a2;
-            dv[3] = a3;
-        }
-    };
+    float16v S;   // scores of the half that is next in line for softmax
+    half8 P[2];   // its probabilities, as the PV product's B operand
 
     // V transpose-read geometry: 16-lane group G = lane/16 covers d rows (G&1)*16.. of the
     // 32-row tile and k half-group lh = G>>1; lane L of the group supplies key (L/4), d run (L%4)*4.
     const int gl = lane & 15;
-    const int vtr_off = (gl >> 2) * kRowF16 + (((lane >> 4) & 1) * 16 + (gl & 3) * 4) * 2;
+    const int vtr_off = kVOff + (gl >> 2) * kVRow + (((lane >> 4) & 1) * 16 + (gl & 3) * 4) * 2;
 
-    if (klo < khi)
-        issue(klo);
-    for (int k0 = klo; k0 < khi; k0 += kKTile) {
-        __syncthreads(); // previous tile fully consumed
-        stage();
-        if (k0 + kKTile < khi)
-            issue(k0 + kKTile);
-        __syncthreads();
+    // a 32-key half of tile t that this task can see at all (wave-uniform)
+    auto live = [&](int t, int hk) {
+        const int k0 = klo + t * kKTile + hk * 32;
+        return task_valid && k0 <= task_last_key && k0 < khi;
+    };
 
-        // ---- S^T = K . Q^T ------------------------------------------------------------------
-        float16v S;
+    // ---- S^T = K . Q^T for half hk of tile t ------------------------------------------------------
+    // The 16 MFMAs form one accumulation chain; their A operands are read from LDS two steps
+    // ahead, and the scheduling groups below pin that interleaving (read, then MFMA) so an
+    // operand's LDS latency is covered by the two MFMAs in front of it.
+    auto scores = [&](int t, int hk) {
+        if (!live(t, hk))
+            return;
+        const uint8_t *Kh = lds + (t & 1) * kBufBytes + hk * 32 * kKRow + ln * kKRow + lh * 16;
+        float16v acc;
 #pragma unroll
         for (int i = 0; i < 16; i++)
-            S[i] = 0.0f;
+            acc[i] = 0.0f;
+        half8 A[16], B[kQLdsSteps];
 #pragma unroll
-        for (int ks = 0; ks < 16; ks++) {
-            const half8 A =
-                *reinterpret_cast<const half8 *>(Ks + ln * kRowF16 + (ks * 16 + lh * 8) * 2);
-            S = __builtin_amdgcn_mfma_f32_32x32x16_f16(A, qf[ks], S, 0, 0, 0);
+        for (int ks = 0; ks < kQLdsSteps; ks++)
+            B[ks] = *reinterpret_cast<const half8 *>(qlds + ks * 1024);
+#pragma unroll
+        for (int ks = 0; ks < 16; ks++)
+            A[ks] = *reinterpret_cast<const half8 *>(Kh + ks * 32);
+#pragma unroll
+        for (int ks = 0; ks < 16; ks++)
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[ks], ks < kQLdsSteps ? B[ks] : qf[ks], acc,
+                                                         0, 0, 0);
+        S = acc;
+        __builtin_amdgcn_sched_group_barrier(0x100, 2 + kQLdsSteps, 0); // operands of the first steps
+#pragma unroll
+        for (int ks = 0; ks < 14; ks++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // 1 MFMA
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); // 1 LDS read
         }
+        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+    };
 
-        // ---- online softmax; lane holds keys (i/4)*8 + lh*4 + i%4 of column ln ---------------
-        const bool need_mask = (k0 + kKTile - 1 > a.pos0 + t0) || (k0 + kKTile > khi);
-        float mt = -INFINITY;
+    // ---- online softmax of half hk of tile t; lane holds keys (i/4)*8 + lh*4 + i%4 ---------------
+    auto softmax = [&](int t, int hk) {
+        if (!live(t, hk))
+            return;
+        const int k0 = klo + t * kKTile + hk * 32;
+        const bool need_mask = (k0 + 31 > a.pos0 + t0) || (k0 + 32 > khi);
+        if (need_mask) {
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
-            float s = S[i] * a.scale_log2;
-            if (need_mask) {
+            for (int i = 0; i < 16; i++) {
                 const int kg = k0 + (i >> 2) * 8 + lh * 4 + (i & 3);
-                s = (kg <= my_last_key && kg < khi) ? s : -INFINITY;
+                S[i] = (kg <= my_last_key && kg < khi) ? S[i] : -INFINITY;
             }
-            S[i] = s;
-            mt = fmaxf(mt, s);
         }
-        mt = fmaxf(mt, __shfl_xor(mt, 32));
-        const float m_new = fmaxf(m_run, mt);
+        float mt = S[0];
+#pragma unroll
+        for (int i = 1; i < 16; i++)
+            mt = fmaxf(mt, S[i]);
+        mt = xor32_max(mt);
+        const float m_new = fmaxf(m_run, mt * a.scale_log2);
         const bool dead = m_new == -INFINITY;
         const float corr = dead ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_new);
+        const float mneg = dead ? 0.0f : -m_new;
         float ls = 0.0f;
-        half8 P[2];
 #pragma unroll
         for (int i = 0; i < 16; i++) {
-            const float e = dead ? 0.0f : __builtin_amdgcn_exp2f(S[i] - m_new);
-            const _Float16 eh = (_Float16)e;
-            ls += (float)eh; // the sum uses the rounded weights the PV product uses
-            P[i >> 3][i & 7] = eh;
+            const float e = __builtin_amdgcn_exp2f(fmaf(S[i], a.scale_log2, mneg));
+            ls += e;
+            P[i >> 3][i & 7] = (_Float16)e;
         }
         l_run = l_run * corr + ls;
         if (__any(m_new > m_run)) {
 #pragma unroll
-            for (int t = 0; t < 8; t++)
-                O[t] *= corr;
+            for (int dt = 0; dt < 8; dt++)
+                O[dt] *= corr;
         }
         m_run = m_new;
+    };
 
-        // ---- O^T += V^T . P^T ------------------------------------------------------------------
+    // ---- O^T += V^T . P^T for half hk of tile t ---------------------------------------------------
+    // 16 MFMAs into 8 accumulators; each A operand is two transpose reads, issued two MFMAs ahead.
+    auto pv = [&](int t, int hk) {
+        if (!live(t, hk))
+            return;
+        const uint8_t *Vh = lds + (t & 1) * kBufBytes + vtr_off + hk * 32 * kVRow;
+        half8 A[16];
 #pragma unroll
         for (int u = 0; u < 2; u++) {
 #pragma unroll
             for (int dt = 0; dt < 8; dt++) {
                 // keys of read q: (2u+q)*8 + lh*4 + {0..3}
-                const uint8_t *vp = Vs + vtr_off + dt * 64;
+                const uint8_t *vp = Vh + dt * 64;
                 const short4v r0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                    (short4v __attribute__((address_space(3))) *)(vp + ((2 * u) * 8 + lh * 4) * kRowF16));
+                    (short4v __attribute__((address_space(3))) *)(vp + ((2 * u) * 8 + lh * 4) * kVRow));
                 const short4v r1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                    (short4v __attribute__((address_space(3))) *)(vp + ((2 * u + 1) * 8 + lh * 4) * kRowF16));
-                half8 A;
+                    (short4v __attribute__((address_space(3))) *)(vp + ((2 * u + 1) * 8 + lh * 4) * kVRow));
                 const half4 h0 = __builtin_bit_cast(half4, r0);
                 const half4 h1 = __builtin_bit_cast(half4, r1);
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
-                    A[j] = h0[j];
-                    A[4 + j] = h1[j];
+                    A[u * 8 + dt][j] = h0[j];
+                    A[u * 8 + dt][4 + j] = h1[j];
                 }
-                O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A, P[u], O[dt], 0, 0, 0);
             }
         }
+#pragma unroll
+        for (int u = 0; u < 2; u++)
+#pragma unroll
+            for (int dt = 0; dt < 8; dt++)
+                O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[u * 8 + dt], P[u], O[dt], 0, 0, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 4, 0); // 2 operands up front
+#pragma unroll
+        for (int k = 0; k < 14; k++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+    };
+
+    // Tile t lives in LDS buffer t & 1.  A tile takes four slots, each closed by a barrier:
+    //   V1: dequantize this set's side of tile t+1, softmax of half 0     (VALU)
+    //   M1: PV of half 0, scores of half 1                               (MFMA)
+    //   V2: softmax of half 1                                            (VALU)
+    //   M2: PV of half 1, scores of half 0 of tile t+1                   (MFMA)
+    // Set 1 runs one slot behind set 0 (it passes one extra barrier first, set 0 one extra at
+    // the end), so in every slot one set of each SIMD issues MFMAs while the other does VALU work.
+    // Hazards: set 0 writes K(t+1) in its V1(t); the K(t-1) it replaces was last read in M1(t-1),
+    // which set 1 finished one slot before.  Set 1 writes V(t+1) in its V1(t), which is set 0's
+    // M1(t); the V(t-1) it replaces was last read in M2(t-1), finished by both sets before that.
+    if (ntile > 0) {
+        stage(0);
+        if (ntile > 1)
+            issue(1);
     }
+    lds_barrier();
+    if (PF_SKEW && set == 1)
+        lds_barrier();
+    if (ntile > 0)
+        scores(0, 0);
+    lds_barrier();
+    TSTART();
+    for (int t = 0; t < ntile; t++) {
+        if (t + 1 < ntile) {
+            stage(t + 1);
+            if (t + 2 < ntile)
+                issue(t + 2);
+        }
+        TMARK(1);
+        softmax(t, 0);
+        TMARK(0);
+        lds_barrier();
+        TMARK(2);
+        pv(t, 0);
+        TMARK(3);
+        scores(t, 1);
+        TMARK(4);
+        lds_barrier();
+        TMARK(2);
+        softmax(t, 1);
+        TMARK(0);
+        lds_barrier();
+        TMARK(5);
+        pv(t, 1);
+        TMARK(3);
+        if (t + 1 < ntile)
+            scores(t + 1, 0);
+        TMARK(4);
+        lds_barrier();
+        TMARK(5);
+    }
+    if (PF_SKEW && set == 0)
+        lds_barrier();
+    TDUMP();
 
     // ---- epilogue --------------------------------------------------------------------------
     l_run += __shfl_xor(l_run, 32);
@@ -280,31 +492,59 @@ __global__ void __launch_bounds__(512) chunk_q8_kernel(const ChunkArgs a)
     }
 }
 
-// Fold the key slices: grid (tokens, n_head), 256 threads = head_dim.
+// Fold the key slices: one workgroup per (token, 4 heads); thread = (head, float4 of d).
 __global__ void __launch_bounds__(256) chunk_combine_kernel(
     const float *__restrict__ part_acc, const float *__restrict__ part_ml, float *__restrict__ out,
     int n_head, int qslots, int splits)
 {
     const int tok = blockIdx.x;
-    const int head = blockIdx.y;
-    const int d = threadIdx.x;
+    const int head = blockIdx.y * 4 + (threadIdx.x >> 6);
+    const int d4 = (threadIdx.x & 63) * 4;
+    if (head >= n_head)
+        return;
     float m = -INFINITY;
     for (int s = 0; s < splits; s++) {
         const size_t row = ((size_t)s * qslots + tok) * n_head + head;
-        if (part_ml[row * 2 + 1] > 0.0f)
-            m = fmaxf(m, part_ml[row * 2]);
+        const float2 ml = *reinterpret_cast<const float2 *>(part_ml + row * 2);
+        if (ml.y > 0.0f)
+            m = fmaxf(m, ml.x);
     }
-    float num = 0.0f, den = 0.0f;
+    float4v num = {0, 0, 0, 0};
+    float den = 0.0f;
     for (int s = 0; s < splits; s++) {
         const size_t row = ((size_t)s * qslots + tok) * n_head + head;
-        const float l = part_ml[row * 2 + 1];
-        if (l > 0.0f) {
-            const float w = __builtin_amdgcn_exp2f(part_ml[row * 2] - m);
-            num = fmaf(part_acc[row * kHeadDim + d], w, num);
-            den = fmaf(l, w, den);
-        }
+        const float2 ml = *reinterpret_cast<const float2 *>(part_ml + row * 2);
+        const float4v x = *reinterpret_cast<const float4v *>(part_acc + row * kHeadDim + d4);
+        const float w = ml.y > 0.0f ? __builtin_amdgcn_exp2f(ml.x - m) : 0.0f;
+        const float4v z = {0, 0, 0, 0};
+        num += ml.y > 0.0f ? x * w : z;
+        den = fmaf(ml.y > 0.0f ? ml.y : 0.0f, w, den);
     }
-    out[((size_t)tok * n_head + head) * kHeadDim + d] = den > 0.0f ? num / den : 0.0f;
+    const float inv = den > 0.0f ? 1.0f / den : 0.0f;
+    float4v r = num * inv;
+    if (!(den > 0.0f))
+        r = (float4v){0, 0, 0, 0};
+    *reinterpret_cast<float4v *>(out + ((size_t)tok * n_head + head) * kHeadDim + d4) = r;
+}
+
+#ifdef PF_TIMING
+extern "C" int hipml_dbg_read_pf(unsigned long long *host, size_t n)
+{
+    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_pf_t), n * 8);
+}
+#endif
+
+int prefill_init()
+{
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&chunk_q8_kernel<false>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kPfLds);
+    if (e == hipSuccess)
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&chunk_q8_kernel<true>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, kPfLds);
+    if (e != hipSuccess)
+        return fail((int)e, "hipFuncSetAttribute(prefill LDS) failed: %d (%s)", (int)e,
+                    hipGetErrorString(e));
+    return 0;
 }
 
 int launch_chunk_q8(hipStream_t st, const float *q, const uint8_t *kc, const uint8_t *vc,
@@ -324,21 +564,31 @@ int launch_chunk_q8(hipStream_t st, const float *q, const uint8_t *kc, const uin
     a.pos0 = pos0;
     a.tokens = tokens;
     a.stride = stride;
-    a.splits = splits;
+    a.splits = splits < 2 ? 1 : splits;
     a.qslots = (tokens + 31) / 32 * 32;
+    a.ntask = (tokens + kQTile - 1) / kQTile * a.group;
+    a.nblock = (a.ntask + kTasks - 1) / kTasks;
     a.scale_log2 = kLog2e / 16.0f; // 1/sqrt(256), as the reference's chunk launcher fixes it
-    const unsigned qtiles = (unsigned)((tokens + kQTile - 1) / kQTile);
-    const dim3 block((unsigned)(a.group * 64), 1, 1);
+    const int combos = n_kv * a.splits;
+    // grid.x covers every (combo, task block); the XCD-aware decode in the kernel may leave a
+    // few trailing workgroups without work when 8 is not a multiple of `combos`.
+    unsigned grid;
+    if (combos % 8 == 0)
+        grid = (unsigned)(combos * a.nblock);
+    else if (8 % combos == 0)
+        grid = (unsigned)(8 * ((a.nblock + 8 / combos - 1) / (8 / combos)));
+    else
+        grid = (unsigned)(combos * a.nblock);
+    const dim3 block(kPfThreads, 1, 1);
     if (splits < 2) {
-        hipLaunchKernelGGL(chunk_q8_kernel<false>, dim3((unsigned)n_kv, qtiles, 1), block, 0, st, a);
+        hipLaunchKernelGGL(chunk_q8_kernel<false>, dim3(grid, 1, 1), block, kPfLds, st, a);
         return launched("attn_chunk_q8");
     }
-    hipLaunchKernelGGL(chunk_q8_kernel<true>, dim3((unsigned)n_kv, qtiles, (unsigned)splits), block,
-                       0, st, a);
+    hipLaunchKernelGGL(chunk_q8_kernel<true>, dim3(grid, 1, 1), block, kPfLds, st, a);
     int rc = launched("attn_chunk_q8_split");
     if (rc)
         return rc;
-    hipLaunchKernelGGL(chunk_combine_kernel, dim3((unsigned)tokens, (unsigned)n_head, 1),
+    hipLaunchKernelGGL(chunk_combine_kernel, dim3((unsigned)tokens, (unsigned)((n_head + 3) / 4), 1),
                        dim3(256, 1, 1), 0, st, part_acc, part_ml, out, n_head, a.qslots, splits);
     return launched("attn_chunk_combine");
 }
