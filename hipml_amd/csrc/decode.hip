@@ -162,9 +162,18 @@ __device__ __forceinline__ half8 bytes_to_f16_biased(int2v w)
     return __builtin_bit_cast(half8, r);
 }
 
-__device__ __forceinline__ float xor_max(float x, int mask)
+// max / sum over the four lanes {l, l^16, l^32, l^48} without LDS (row-swap instructions,
+// written as asm: the compiler's builtins for them return the first result twice)
+template <bool MAX>
+__device__ __forceinline__ float quad_rows(float v)
 {
-    return fmaxf(x, __shfl_xor(x, mask));
+    float a = v, b = v;
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+    v = MAX ? fmaxf(a, b) : a + b;
+    a = v;
+    b = v;
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+    return MAX ? fmaxf(a, b) : a + b;
 }
 
 template <int NT, int DEPTH>
@@ -387,8 +396,7 @@ __global__ void __launch_bounds__(kThreads, DECODE_MIN_WAVES) decode_q8_kernel(c
                     S[nt][ms][i] = s;
                     mt = fmaxf(mt, s);
                 }
-            mt = xor_max(mt, 16);
-            mt = xor_max(mt, 32);
+            mt = quad_rows<true>(mt);
             const float m_new = fmaxf(m_run[nt], mt);
             corr[nt] = m_new == -INFINITY ? 1.0f : __builtin_amdgcn_exp2f(m_run[nt] - m_new);
             grew = grew || (m_new > m_run[nt]);
@@ -483,8 +491,7 @@ __global__ void __launch_bounds__(kThreads, DECODE_MIN_WAVES) decode_q8_kernel(c
     // each wave parks 8 columns x 256 d (8 KiB) in its own tile area.
 #pragma unroll
     for (int nt = 0; nt < NT; nt++) {
-        l_run[nt] += __shfl_xor(l_run[nt], 16);
-        l_run[nt] += __shfl_xor(l_run[nt], 32);
+        l_run[nt] = quad_rows<false>(l_run[nt]);
     }
     float *wl = reinterpret_cast<float *>(tile_lds); // per wave: [8][256] acc
     float *wml = reinterpret_cast<float *>(sK);      // per wave: [8] m, [8] l
@@ -556,9 +563,34 @@ __global__ void __launch_bounds__(kThreads, DECODE_MIN_WAVES) decode_q8_kernel(c
     STAMP(4);
 }
 
+// Wave-wide reductions without LDS: DPP inside a row of 16 lanes, then the two row-swap
+// instructions (written as asm: the compiler's builtins for them return the first result twice).
+template <bool MAX>
+__device__ __forceinline__ float wave_reduce(float v)
+{
+    auto op = [](float a, float b) { return MAX ? fmaxf(a, b) : a + b; };
+#define HIPML_DPP(x, ctrl)                                                                         \
+    __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), ctrl, 0xf, \
+                                                          0xf, true))
+    v = op(v, HIPML_DPP(v, 0xB1));  // quad_perm [1,0,3,2]: lane ^ 1
+    v = op(v, HIPML_DPP(v, 0x4E));  // quad_perm [2,3,0,1]: lane ^ 2
+    v = op(v, HIPML_DPP(v, 0x141)); // row_half_mirror: the other quad of 8
+    v = op(v, HIPML_DPP(v, 0x140)); // row_mirror: the other half of 16
+#undef HIPML_DPP
+    float a = v, b = v;
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+    v = op(a, b); // rows 0|1 and 2|3 combined
+    a = v;
+    b = v;
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+    return op(a, b);
+}
+
 // out[row][head][d] = sum_s acc_s[d] * 2^(m_s - m) / sum_s l_s * 2^(m_s - m); 0 when no
 // split saw a key.  grid (n_heads * 4, rows): a workgroup owns 64 d of one (row, head);
-// thread = (split group 0..15, float4 of d 0..15).
+// thread = (split group 0..15, float4 of d 0..15).  Latency matters more than bandwidth here:
+// the first accumulator loads are issued before anything else, and the two reductions over
+// the splits cost one barrier each.
 constexpr int kReduceMaxSplits = 4096;
 
 __global__ void __launch_bounds__(256) decode_reduce_kernel(
@@ -566,59 +598,67 @@ __global__ void __launch_bounds__(256) decode_reduce_kernel(
     int splits, size_t acc_slot, size_t ml_slot, size_t q_slot)
 {
     __shared__ float w_s[kReduceMaxSplits];
-    __shared__ float red[256];
+    __shared__ float red_m[4], red_l[4];
     __shared__ float4v accs[16][16];
     const int head = blockIdx.x >> 2;
     const int dq = blockIdx.x & 3;
     const int row = blockIdx.y;
     const int tid = threadIdx.x;
+    const int sg = tid >> 4, dl = tid & 15;
     const float *ml = part_ml + (size_t)row * ml_slot + (size_t)head * splits * 2;
+    const float *acc = part_acc + (size_t)row * acc_slot + (size_t)head * splits * kHeadDim +
+                       dq * 64 + dl * 4;
+
+    // first four accumulator rows of this thread, in flight while the weights are worked out
+    float4v x0[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const int s = sg + 16 * k;
+        x0[k] = (float4v){0, 0, 0, 0};
+        if (s < splits)
+            x0[k] = *reinterpret_cast<const float4v *>(acc + (size_t)s * kHeadDim);
+    }
 
     // weights: w_s = 2^(m_s - m) for splits that saw a key, else 0
     float m = -INFINITY;
     for (int s = tid; s < splits; s += 256) {
         const float2 v = *reinterpret_cast<const float2 *>(ml + s * 2);
-        w_s[s] = v.x;
         if (v.y > 0.0f)
             m = fmaxf(m, v.x);
     }
-    red[tid] = m;
+    m = wave_reduce<true>(m);
+    if ((tid & 63) == 0)
+        red_m[tid >> 6] = m;
     __syncthreads();
-    for (int o = 128; o > 0; o >>= 1) {
-        if (tid < o)
-            red[tid] = fmaxf(red[tid], red[tid + o]);
-        __syncthreads();
-    }
-    m = red[0];
-    __syncthreads();
+    m = fmaxf(fmaxf(red_m[0], red_m[1]), fmaxf(red_m[2], red_m[3]));
     float den = 0.0f;
     for (int s = tid; s < splits; s += 256) {
-        const float l = ml[s * 2 + 1];
-        const float w = l > 0.0f ? __builtin_amdgcn_exp2f(w_s[s] - m) : 0.0f;
+        const float2 v = *reinterpret_cast<const float2 *>(ml + s * 2); // L1 hit
+        const float w = v.y > 0.0f ? __builtin_amdgcn_exp2f(v.x - m) : 0.0f;
         w_s[s] = w;
-        den = fmaf(l, w, den);
+        den = fmaf(v.y > 0.0f ? v.y : 0.0f, w, den);
     }
-    red[tid] = den;
+    den = wave_reduce<false>(den);
+    if ((tid & 63) == 0)
+        red_l[tid >> 6] = den;
     __syncthreads();
-    for (int o = 128; o > 0; o >>= 1) {
-        if (tid < o)
-            red[tid] += red[tid + o];
-        __syncthreads();
-    }
-    den = red[0];
+    den = (red_l[0] + red_l[1]) + (red_l[2] + red_l[3]);
 
-    const int sg = tid >> 4, dl = tid & 15;
-    const float *acc = part_acc + (size_t)row * acc_slot + (size_t)head * splits * kHeadDim +
-                       dq * 64 + dl * 4;
     float4v num = {0, 0, 0, 0};
+    const float4v z = {0, 0, 0, 0};
     // zero-weight slices may hold anything (even NaN from an untouched scratch): select, not multiply
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const int s = sg + 16 * k;
+        const float w = s < splits ? w_s[s] : 0.0f;
+        num += w > 0.0f ? x0[k] * w : z;
+    }
     auto term = [&](int s) {
         const float w = w_s[s];
         const float4v x = *reinterpret_cast<const float4v *>(acc + (size_t)s * kHeadDim);
-        const float4v z = {0, 0, 0, 0};
         return w > 0.0f ? x * w : z;
     };
-    int s = sg;
+    int s = sg + 64;
     for (; s + 48 < splits; s += 64)
         num += (term(s) + term(s + 16)) + (term(s + 32) + term(s + 48));
     for (; s < splits; s += 16)

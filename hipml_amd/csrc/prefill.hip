@@ -52,6 +52,11 @@ constexpr float kLog2e = 1.4426950408889634f;
 #ifndef PF_SKEW
 #define PF_SKEW 1
 #endif
+#ifdef PF_PRIO
+#define PRIO(n) __builtin_amdgcn_s_setprio(n)
+#else
+#define PRIO(n) do { } while (0)
+#endif
 
 struct ChunkArgs {
     const float *q;
@@ -429,29 +434,44 @@ __global__ void __launch_bounds__(kPfThreads, 2) chunk_q8_kernel(const ChunkArgs
     TSTART();
     for (int t = 0; t < ntile; t++) {
         if (t + 1 < ntile) {
+#ifdef PF_TIMING
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            TMARK(2); // (timing builds: the wait for the tile prefetch is booked under "barrier A")
+#endif
             stage(t + 1);
-            if (t + 2 < ntile)
-                issue(t + 2);
+#ifdef PF_TIMING
+            TMARK(1);
+#endif
         }
-        TMARK(1);
+#ifdef PF_TIMING
+        TMARK(5); // (timing builds: issuing the next prefetch is booked under "barrier B")
+#endif
         softmax(t, 0);
         TMARK(0);
         lds_barrier();
         TMARK(2);
+        PRIO(1);
         pv(t, 0);
         TMARK(3);
         scores(t, 1);
+        PRIO(0);
         TMARK(4);
         lds_barrier();
         TMARK(2);
         softmax(t, 1);
+        // the next prefetch is issued from the short slot (V2): issuing the five loads of a
+        // unit is slow enough to matter, and V1 already carries the dequantization
+        if (t + 2 < ntile)
+            issue(t + 2);
         TMARK(0);
         lds_barrier();
         TMARK(5);
+        PRIO(1);
         pv(t, 1);
         TMARK(3);
         if (t + 1 < ntile)
             scores(t + 1, 0);
+        PRIO(0);
         TMARK(4);
         lds_barrier();
         TMARK(5);
