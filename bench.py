@@ -49,6 +49,23 @@ def decode_bytes(seq_total: int) -> float:
     return float(2 * KV * seq_total * ROW)
 
 
+def measured_traffic(workload: str, kernels):
+    """HBM bytes per launch (read + written) of the named kernels, from the committed
+    counter runs in profiles/hbm_traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled
+    by a plain copy of known size); None when that file has no entry."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
+            t = json.load(f).get(workload, {})
+    except OSError:
+        return None
+    total, seen = 0.0, False
+    for name, v in t.items():
+        if any(k in name for k in kernels):
+            total += v["read_bytes"] + v["written_bytes"]
+            seen = True
+    return total if seen else None
+
+
 class Timer:
     """HIP events on torch's current stream (the stream every launch below uses)."""
 
@@ -135,6 +152,8 @@ def bench_prefill(torch, attn, tokens, pos0, steps, warmup, layers, prefix_fill=
     attn_ms = t.ms / steps
     flop = prefill_flop(pos0, tokens)
     tf = flop / (attn_ms * 1e-3) / 1e12
+    wl = {(672, 0): "prefill672", (2048, 100_000): "chunk100k"}.get((tokens, pos0), "")
+    traffic = measured_traffic(wl, ["chunk_q8_kernel", "chunk_combine_kernel"])
     return {
         "workload": f"prefill {tokens}@{pos0}: rope + q8_0 append + causal GQA attention + gate, "
                     f"1 layer, {H}q/{KV}kv heads, head_dim {HD}",
@@ -144,7 +163,7 @@ def bench_prefill(torch, attn, tokens, pos0, steps, warmup, layers, prefix_fill=
         "attn_ms": attn_ms,
         "attn_tok_per_s": tokens / (attn_ms * 1e-3),
         "roofline": {"bound": "mfma", "achieved": tf, "peak": MFMA_F16_PEAK_TF, "unit": "TFLOP/s",
-                     "frac": tf / MFMA_F16_PEAK_TF, "traffic": None,
+                     "frac": tf / MFMA_F16_PEAK_TF, "traffic": traffic,
                      "kernel": "chunk_q8_kernel" + (" + chunk_combine_kernel" if splits >= 2 else ""),
                      "flop_per_launch": flop, "launch_ms": attn_ms},
     }
@@ -184,12 +203,14 @@ def bench_decode(torch, attn, seq, steps, warmup, layers):
     us = t.ms * 1e3 / (steps * layers)
     nbytes = decode_bytes(seq)
     gbs = nbytes / (us * 1e-6) / 1e9
+    traffic = measured_traffic({8192: "decode8k", 32768: "decode32k"}.get(seq, ""),
+                               ["decode_q8_kernel", "decode_reduce_kernel"])
     return {
         "workload": f"decode 1 query @ depth {seq}, q8_0 cache, split-K {splits} + merge",
         "seq": seq, "splits": splits, "layers_rotated": layers,
         "us_per_layer": us,
         "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": gbs / HBM_PEAK_GBS, "traffic": None,
+                     "frac": gbs / HBM_PEAK_GBS, "traffic": traffic,
                      "kernel": "decode_q8_kernel + decode_reduce_kernel",
                      "bytes_per_launch": nbytes, "launch_us": us},
     }
@@ -243,16 +264,30 @@ def bench_batch(torch, attn, orc, steps, warmup, layers):
     live = sum(d + c for d, c in zip(depths, cols))
     nbytes = decode_bytes(live)
     gbs = nbytes / (us * 1e-6) / 1e9
+    traffic = measured_traffic("batch16", ["decode_q8_kernel", "decode_reduce_kernel"])
     return {
         "workload": f"batched decode, {slots} slots, depths U[512,16384] (seeded), "
                     f"slots 0..3 carry 3 query rows (MTP verify), one launch",
         "slots": slots, "rows": rows, "live_rows": live, "splits": splits, "layers_rotated": layers,
         "us_per_layer": us,
         "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": gbs / HBM_PEAK_GBS, "traffic": None,
+                     "frac": gbs / HBM_PEAK_GBS, "traffic": traffic,
                      "kernel": "decode_q8_kernel + decode_reduce_kernel",
                      "bytes_per_launch": nbytes, "launch_us": us},
     }
+
+
+def bench_copycal(torch, steps):
+    """Plain device copy of a known size: the yardstick the HBM traffic counters
+    (FETCH_SIZE / WRITE_SIZE) are scaled by."""
+    n = 64 << 20
+    a = torch.empty(n, dtype=torch.uint8, device="cuda")
+    b = torch.ones(n, dtype=torch.uint8, device="cuda")
+    with Timer(torch) as t:
+        for _ in range(steps):
+            a.copy_(b)
+    return {"workload": "device copy", "bytes_read": n, "bytes_written": n,
+            "us_per_copy": t.ms * 1e3 / steps}
 
 
 # ---------------------------------------------------------------------------------------
@@ -302,7 +337,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--main-only", action="store_true", help="skip the 'also' workloads")
     ap.add_argument("--only", default="", help="run one workload alone (prefill672, decode8k, "
-                    "decode32k, chunk100k, batch16) for profiling; prints its object")
+                    "decode32k, chunk100k, batch16, copycal) for profiling; prints its object")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -328,6 +363,7 @@ def main() -> int:
             "decode32k": lambda: bench_decode(torch, attn, 32768, K, W, LAYERS),
             "chunk100k": lambda: bench_prefill(torch, attn, 2048, 100_000, K, W, 2),
             "batch16": lambda: bench_batch(torch, attn, orc, K, W, 4),
+            "copycal": lambda: bench_copycal(torch, K),
         }[args.only]
         print(json.dumps(fn()))
         return 0
