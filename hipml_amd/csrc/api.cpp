@@ -185,7 +185,7 @@ int hipml_attn_batch_splits(int stride, int n_kv, int slots)
     if (stride < 1 || n_kv < 1 || slots < 1)
         return 1;
     int by_work = (stride + 127) / 128;
-    int by_cus = (2 * 256) / (n_kv * slots);
+    int by_cus = 1024 / (n_kv * slots);
     if (by_cus < 1)
         by_cus = 1;
     int s = by_work < by_cus ? by_work : by_cus;

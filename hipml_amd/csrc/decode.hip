@@ -177,7 +177,7 @@ __device__ __forceinline__ float quad_rows(float v)
 }
 
 template <int NT, int DEPTH>
-__global__ void __launch_bounds__(kThreads, DECODE_MIN_WAVES) decode_q8_kernel(const DecodeArgs a)
+__device__ __forceinline__ void decode_body(const DecodeArgs &a)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds_all[];
     uint8_t *Qs = lds_all;                       // [NT][hi,lo][8 blocks][64 lanes] half8
@@ -561,6 +561,18 @@ __global__ void __launch_bounds__(kThreads, DECODE_MIN_WAVES) decode_q8_kernel(c
         }
     }
     STAMP(4);
+}
+
+// NT = 1: every slot has at most 16 (row, head) columns.  NT = 2: some slot has more (MTP
+// verify, 3-4 rows x 6 heads); slots that fit one column tile still take the NT = 1 body, so a
+// mixed batch pays the wider tile only where it is needed.  LDS is sized for the launch's NT.
+template <int NT, int DEPTH>
+__global__ void __launch_bounds__(kThreads, DECODE_MIN_WAVES) decode_q8_kernel(const DecodeArgs a)
+{
+    if (NT == 1 || a.cols[blockIdx.y] * a.group <= 16)
+        decode_body<1, DEPTH>(a);
+    else
+        decode_body<NT, DEPTH>(a);
 }
 
 // Wave-wide reductions without LDS: DPP inside a row of 16 lanes, then the two row-swap
