@@ -337,7 +337,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--main-only", action="store_true", help="skip the 'also' workloads")
     ap.add_argument("--only", default="", help="run one workload alone (prefill672, decode8k, "
-                    "decode32k, chunk100k, batch16, copycal) for profiling; prints its object")
+                    "decode32k, decode128k, chunk100k, batch16, copycal) for profiling; prints its object")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -361,6 +361,7 @@ def main() -> int:
             "prefill672": lambda: bench_prefill(torch, attn, 672, 0, K, W, LAYERS),
             "decode8k": lambda: bench_decode(torch, attn, 8192, K, W, LAYERS),
             "decode32k": lambda: bench_decode(torch, attn, 32768, K, W, LAYERS),
+            "decode128k": lambda: bench_decode(torch, attn, 131072, K, W, LAYERS),
             "chunk100k": lambda: bench_prefill(torch, attn, 2048, 100_000, K, W, 2),
             "batch16": lambda: bench_batch(torch, attn, orc, K, W, 4),
             "copycal": lambda: bench_copycal(torch, K),
@@ -392,6 +393,10 @@ def main() -> int:
         also["decode_8192"] = bench_decode(torch, attn, 8192, d_steps, max(W // 4, 2), LAYERS)
         torch.cuda.empty_cache()
         also["decode_32768"] = bench_decode(torch, attn, 32768, d_steps, max(W // 4, 2), LAYERS)
+        torch.cuda.empty_cache()
+        # beyond the BASELINE depths: shows what the same kernel does once launch and ramp-up
+        # stop dominating (285 MB per layer)
+        also["decode_131072"] = bench_decode(torch, attn, 131072, max(d_steps // 4, 5), 2, LAYERS)
         torch.cuda.empty_cache()
         also["chunk_2048_at_100000"] = bench_prefill(torch, attn, 2048, 100_000,
                                                      max(K // 20, 3), 1, 2)

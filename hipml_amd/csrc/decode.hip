@@ -89,7 +89,8 @@ __device__ unsigned long long g_dbg_t[8 * 4096];
 #define STAMP(i) do { } while (0)
 #endif
 
-constexpr int decode_lds_bytes(int nt) { return nt * 16384 + kWaves * kWaveLds; }
+constexpr int kQLds = 16384 + 2048; // per column tile: Q operands (hi, lo) + bias table
+constexpr int decode_lds_bytes(int nt) { return nt * kQLds + kWaves * kWaveLds; }
 
 struct DecodeArgs {
     const float *q;
@@ -148,8 +149,10 @@ __device__ __forceinline__ void store_unit(const Unit &u, uint8_t *tile, uint8_t
 }
 
 // 8 int8 b -> 8 f16 holding (b + 128) * 2^-24 exactly (byte b^0x80 in the low byte of a
-// subnormal f16).  The +128 is taken out again by a second MFMA whose A operand is the
-// constant -128 * 2^-24: sum_k (u_k - 128) x_k = sum_k u_k x_k + sum_k (-128) x_k.
+// subnormal f16).  The +128 is taken out again on the B side: sum_k (u_k - 128) x_k =
+// sum_k u_k x_k - 128 sum_k x_k.  For the scores x = Q is fixed, so the second term is a table
+// the block's MFMA starts from; for PV it is a second MFMA whose A operand is the constant
+// -128 * 2^-24.
 __device__ __forceinline__ half8 bytes_to_f16_biased(int2v w)
 {
     const uint32_t x0 = (uint32_t)w[0] ^ 0x80808080u;
@@ -181,7 +184,8 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds_all[];
     uint8_t *Qs = lds_all;                       // [NT][hi,lo][8 blocks][64 lanes] half8
-    uint8_t *wave_base = lds_all + NT * 16384;   // per-wave tile + scale tables
+    uint8_t *CBs = lds_all + NT * 16384;         // [NT][8 blocks][16 columns] float4 (one value x4)
+    uint8_t *wave_base = lds_all + NT * kQLds;   // per-wave tile + scale tables
 
     STAMP(0);
     const int wave = threadIdx.x >> 6;
@@ -279,6 +283,24 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
         *reinterpret_cast<half8 *>(Qs + (((nt * 2 + 1) * 8 + c) * 64 + l) * 16) = l8;
     }
     __syncthreads();
+    // Bias table: the K bytes enter the MFMA as (b + 128) * 2^-24, so every score of block c
+    // carries +128 * 2^-24 * sum_k q[k][n]; its negative is the C operand the block's MFMA starts
+    // from.  One entry per (tile, block, column), replicated x4 for the accumulator layout.
+    for (int e = threadIdx.x; e < NT * 8 * 16; e += kThreads) {
+        const int n = e & 15, c = (e >> 4) & 7, nt = e >> 7;
+        float sum = 0.0f;
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            const half8 h = *reinterpret_cast<const half8 *>(Qs + (((nt * 2 + 0) * 8 + c) * 64 + g * 16 + n) * 16);
+            const half8 l = *reinterpret_cast<const half8 *>(Qs + (((nt * 2 + 1) * 8 + c) * 64 + g * 16 + n) * 16);
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+                sum += (float)h[j] + (float)l[j];
+        }
+        const float cb = -128.0f / kTwo24 * sum;
+        *reinterpret_cast<float4v *>(CBs + ((nt * 8 + c) * 16 + n) * 16) = (float4v){cb, cb, cb, cb};
+    }
+    __syncthreads();
     STAMP(2); // Q staged
 
     // per-column causal bound (MTP rows see one more key each)
@@ -306,7 +328,6 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
     const int tr_r = lm >> 1;
     const int tr_key = (tr_r >> 2) * 16 + lg * 4 + (tr_r & 3);
     const uint8_t *vtr = tile_lds + tr_key * kLdsRow + (lm & 1) * 8;
-    const float4v zero4 = {0, 0, 0, 0};
     const uint4v bias_bits = {0x80808080u, 0x80808080u, 0x80808080u, 0x80808080u};
     const half8 Abias = __builtin_bit_cast(half8, bias_bits); // eight times -128 * 2^-24
 
@@ -333,8 +354,10 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
 #pragma unroll
         for (int c = 0; c < 8; c++) {
             half8 bh[NT], bl[NT];
+            float4v cbias[NT];
 #pragma unroll
             for (int nt = 0; nt < NT; nt++) {
+                cbias[nt] = *reinterpret_cast<const float4v *>(CBs + ((nt * 8 + c) * 16 + lm) * 16);
                 bh[nt] = *reinterpret_cast<const half8 *>(Qs + (((nt * 2 + 0) * 8 + c) * 64 + lane) * 16);
                 bl[nt] = *reinterpret_cast<const half8 *>(Qs + (((nt * 2 + 1) * 8 + c) * 64 + lane) * 16);
             }
@@ -347,12 +370,9 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
                     sK + (c * kTileKeys + ms * 16 + lg * 4) * 2);
 #pragma unroll
                 for (int nt = 0; nt < NT; nt++) {
-                    float4v part = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, bh[nt], zero4, 0, 0, 0);
-                    part = __builtin_amdgcn_mfma_f32_16x16x32_f16(Abias, bh[nt], part, 0, 0, 0);
-                    if (DECODE_QLO) {
+                    float4v part = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, bh[nt], cbias[nt], 0, 0, 0);
+                    if (DECODE_QLO)
                         part = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, bl[nt], part, 0, 0, 0);
-                        part = __builtin_amdgcn_mfma_f32_16x16x32_f16(Abias, bl[nt], part, 0, 0, 0);
-                    }
 #pragma unroll
                     for (int i = 0; i < 4; i++)
                         S[nt][ms][i] = fmaf((float)sk[i], part[i], S[nt][ms][i]);
