@@ -72,20 +72,26 @@ struct ChunkArgs {
     float scale_log2;
 };
 
-// 68 bytes of a key row starting at a block-pair boundary: [s0 | 32 x i8 | s1 | 32 x i8].
-struct Unit {
-    uint4v a, b; // dwords 0..7
-    uint32_t m;  // dword 8
-    uint4v c, d; // dwords 9..16
+// Half of a 68-byte unit [s0 | 32 x i8 | s1 | 32 x i8] of a key row, as the nine dwords that cover
+// one block: dwords 0..8 for the first block (scale in the low half of dword 0), dwords 8..16 for
+// the second (scale in the high half of dword 8, payload dword-aligned behind it).
+struct Half {
+    uint4v p, q;
+    uint32_t r; // dword 8 of the unit, in both halves
 };
 
-__device__ __forceinline__ void load_unit(Unit &u, const uint8_t *p)
+__device__ __forceinline__ void load_half0(Half &h, const uint8_t *u)
 {
-    u.a = *reinterpret_cast<const uint4a4 *>(p);
-    u.b = *reinterpret_cast<const uint4a4 *>(p + 16);
-    u.m = *reinterpret_cast<const uint32_t *>(p + 32);
-    u.c = *reinterpret_cast<const uint4a4 *>(p + 36);
-    u.d = *reinterpret_cast<const uint4a4 *>(p + 52);
+    h.p = *reinterpret_cast<const uint4a4 *>(u);
+    h.q = *reinterpret_cast<const uint4a4 *>(u + 16);
+    h.r = *reinterpret_cast<const uint32_t *>(u + 32);
+}
+
+__device__ __forceinline__ void load_half1(Half &h, const uint8_t *u)
+{
+    h.r = *reinterpret_cast<const uint32_t *>(u + 32);
+    h.p = *reinterpret_cast<const uint4a4 *>(u + 36);
+    h.q = *reinterpret_cast<const uint4a4 *>(u + 52);
 }
 
 // 16 int8 -> 16 f16 (value * d), d an f16 scale: the bytes become 1024 + (b+128)
@@ -108,20 +114,20 @@ __device__ __forceinline__ void dequant16(uint4v raw, _Float16 d, uint4v &lo, ui
     hi = (uint4v){o[4], o[5], o[6], o[7]};
 }
 
-// Dequantize one unit (blocks 2*pr and 2*pr+1 of one key) into 128 bytes of f16 at `dst`.
-__device__ __forceinline__ void stage_unit(const Unit &u, uint8_t *dst)
+// Dequantize one block of a unit (block 2*pr or 2*pr+1 of one key) into its 64 bytes of the
+// unit's 128 bytes of f16 at `dst`.
+__device__ __forceinline__ void stage_block0(const Half &h, uint8_t *dst)
 {
     uint4v e0, e1;
-    e0[0] = __builtin_amdgcn_alignbit(u.a[1], u.a[0], 16);
-    e0[1] = __builtin_amdgcn_alignbit(u.a[2], u.a[1], 16);
-    e0[2] = __builtin_amdgcn_alignbit(u.a[3], u.a[2], 16);
-    e0[3] = __builtin_amdgcn_alignbit(u.b[0], u.a[3], 16);
-    e1[0] = __builtin_amdgcn_alignbit(u.b[1], u.b[0], 16);
-    e1[1] = __builtin_amdgcn_alignbit(u.b[2], u.b[1], 16);
-    e1[2] = __builtin_amdgcn_alignbit(u.b[3], u.b[2], 16);
-    e1[3] = __builtin_amdgcn_alignbit(u.m, u.b[3], 16);
-    const _Float16 s0 = __builtin_bit_cast(_Float16, (uint16_t)(u.a[0] & 0xffffu));
-    const _Float16 s1 = __builtin_bit_cast(_Float16, (uint16_t)(u.m >> 16));
+    e0[0] = __builtin_amdgcn_alignbit(h.p[1], h.p[0], 16);
+    e0[1] = __builtin_amdgcn_alignbit(h.p[2], h.p[1], 16);
+    e0[2] = __builtin_amdgcn_alignbit(h.p[3], h.p[2], 16);
+    e0[3] = __builtin_amdgcn_alignbit(h.q[0], h.p[3], 16);
+    e1[0] = __builtin_amdgcn_alignbit(h.q[1], h.q[0], 16);
+    e1[1] = __builtin_amdgcn_alignbit(h.q[2], h.q[1], 16);
+    e1[2] = __builtin_amdgcn_alignbit(h.q[3], h.q[2], 16);
+    e1[3] = __builtin_amdgcn_alignbit(h.r, h.q[3], 16);
+    const _Float16 s0 = __builtin_bit_cast(_Float16, (uint16_t)(h.p[0] & 0xffffu));
     uint4v *d4 = reinterpret_cast<uint4v *>(dst);
     uint4v x0, x1;
     dequant16(e0, s0, x0, x1);
@@ -130,20 +136,32 @@ __device__ __forceinline__ void stage_unit(const Unit &u, uint8_t *dst)
     dequant16(e1, s0, x0, x1);
     d4[2] = x0;
     d4[3] = x1;
-    dequant16(u.c, s1, x0, x1);
+}
+
+__device__ __forceinline__ void stage_block1(const Half &h, uint8_t *dst)
+{
+    const _Float16 s1 = __builtin_bit_cast(_Float16, (uint16_t)(h.r >> 16));
+    uint4v *d4 = reinterpret_cast<uint4v *>(dst);
+    uint4v x0, x1;
+    dequant16(h.p, s1, x0, x1);
     d4[4] = x0;
     d4[5] = x1;
-    dequant16(u.d, s1, x0, x1);
+    dequant16(h.q, s1, x0, x1);
     d4[6] = x0;
     d4[7] = x1;
 }
 
 #ifdef PF_TIMING
-// debug builds: per-wave accumulated phase times (100 MHz ticks) for workgroup 0: [wave][6]
-__device__ unsigned long long g_pf_t[8 * 8];
-#define TSTART() unsigned long long t_prev = wall_clock64(), t_now; unsigned long long t_acc[6] = {0, 0, 0, 0, 0, 0}
-#define TMARK(i) do { t_now = wall_clock64(); t_acc[i] += t_now - t_prev; t_prev = t_now; } while (0)
-#define TDUMP() do { if (blockIdx.x == 8 && (threadIdx.x & 63) == 0) for (int i = 0; i < 6; i++) g_pf_t[(threadIdx.x >> 6) * 8 + i] = t_acc[i]; } while (0)
+// debug builds: per-wave accumulated cycles of each slot of the tile loop, for one workgroup:
+// [wave][16] = 10 phases, total cycles, total time in 100 MHz ticks
+__device__ unsigned long long g_pf_t[8 * 16];
+#define TSTART() unsigned long long t_w0 = wall_clock64(); unsigned long long t_prev = clock64(), t_now; unsigned long long t_acc[16] = {0,0,0,0,0,0,0,0,0,0,0,0,0,0,0,0}; const unsigned long long t_c0 = t_prev
+#if PF_TIMING >= 2
+#define TMARK(i) do { t_now = clock64(); t_acc[i] += t_now - t_prev; t_prev = t_now; } while (0)
+#else
+#define TMARK(i) do { (void)t_now; (void)t_prev; } while (0)
+#endif
+#define TDUMP() do { t_acc[10] = clock64() - t_c0; t_acc[11] = wall_clock64() - t_w0; if (blockIdx.x == 8 && (threadIdx.x & 63) == 0) for (int i = 0; i < 16; i++) g_pf_t[(threadIdx.x >> 6) * 16 + i] = t_acc[i]; } while (0)
 #else
 #define TSTART() do { } while (0)
 #define TMARK(i) do { } while (0)
@@ -163,9 +181,13 @@ __device__ __forceinline__ float xor32_max(float x)
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every
 // outstanding global load (vmcnt(0)), which would expose the full latency of the next tile's
 // prefetch at each phase boundary; here only LDS operations are drained.
+// It is also a fence for the instruction scheduler: the slots of the tile loop only overlap as
+// planned if each slot's VALU work and MFMA work stay on their own side of the barrier.
 __device__ __forceinline__ void lds_barrier()
 {
+    __builtin_amdgcn_sched_barrier(0);
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
 }
 
 template <bool SPLIT>
@@ -235,22 +257,34 @@ __global__ void __launch_bounds__(kPfThreads, 2) chunk_q8_kernel(const ChunkArgs
     const int ntile = khi > klo ? (khi - klo + kKTile - 1) / kKTile : 0;
 
     // ---- staging role: thread -> one 68-byte unit of the K tile (set 0) or V tile (set 1) ----
+    // A wave of the set covers 16 rows x 4 units.  Eight consecutive lanes take 4 rows x 2 units, so
+    // that their 128-bit LDS writes (a unit's chunks are 128 bytes apart between units, rows are
+    // 528 / 544 bytes apart) fall into distinct banks; the wave still reads 16 whole contiguous rows.
     const int su = threadIdx.x & 255;
-    const int srow = su >> 2, spr = su & 3;
+    const int srow = (su >> 6) * 16 + ((su >> 1) & 7) + ((su >> 5) & 1) * 8;
+    const int spr = (su & 1) | ((su >> 3) & 2);
     const uint8_t *sbase = (set ? a.vc : a.kc) + (size_t)kvh * a.stride * kRowBytes + spr * 68;
     const int sdst = set ? kVOff + srow * kVRow + spr * 128 : srow * kKRow + spr * 128;
-    Unit unit;
-    auto issue = [&](int t) {
+    // One block of the unit is in flight at a time: block 0 of tile t+1 travels during the MFMA slot
+    // M2(t-1) and is dequantized in V1(t), block 1 travels during M1(t) and is dequantized in V2(t).
+    // (Past the last tile the loads repeat the last key: issuing unconditionally keeps the loads'
+    // registers out of a branch, where the compiler would copy them right behind the loads and wait
+    // for memory to do it.)
+    Half half;
+    auto unit_ptr = [&](int t) {
 #ifdef PF_DBG_SAMETILE
         t = t & 7; // debug: keep re-reading the first tiles (cache hits)
 #endif
         int key = klo + t * kKTile + srow;
         key = key < khi ? key : khi - 1;
-        load_unit(unit, sbase + (size_t)key * kRowBytes);
+        return sbase + (size_t)key * kRowBytes;
     };
-    auto stage = [&](int t) { stage_unit(unit, lds + (t & 1) * kBufBytes + sdst); };
+    auto issue0 = [&](int t) { load_half0(half, unit_ptr(t)); };
+    auto issue1 = [&](int t) { load_half1(half, unit_ptr(t)); };
+    auto stage0 = [&](int t) { stage_block0(half, lds + (t & 1) * kBufBytes + sdst); };
+    auto stage1 = [&](int t) { stage_block1(half, lds + (t & 1) * kBufBytes + sdst); };
     if (ntile > 0)
-        issue(0);
+        issue0(0);
 
     // ---- Q^T operand: 16 k-steps of 8 f16 (d = ks*16 + lh*8 + j) ---------------------------
     // Steps 0..kQLdsSteps-1 are parked in this wave's corner of LDS and re-read per use: 256
@@ -368,6 +402,8 @@ __global__ void __launch_bounds__(kPfThreads, 2) chunk_q8_kernel(const ChunkArgs
                 O[dt] *= corr;
         }
         m_run = m_new;
+        // computed here, in the VALU slot, not where the MFMA slot first reads them
+        asm volatile("" : "+v"(P[0]), "+v"(P[1]), "+v"(l_run), "+v"(m_run));
     };
 
     // ---- O^T += V^T . P^T for half hk of tile t ---------------------------------------------------
@@ -411,19 +447,25 @@ __global__ void __launch_bounds__(kPfThreads, 2) chunk_q8_kernel(const ChunkArgs
     };
 
     // Tile t lives in LDS buffer t & 1.  A tile takes four slots, each closed by a barrier:
-    //   V1: dequantize this set's side of tile t+1, softmax of half 0     (VALU)
-    //   M1: PV of half 0, scores of half 1                               (MFMA)
-    //   V2: softmax of half 1                                            (VALU)
-    //   M2: PV of half 1, scores of half 0 of tile t+1                   (MFMA)
+    //   V1: dequantize block 0 of this thread's unit of tile t+1, fetch its block 1, softmax of half 0
+    //   M1: PV of half 0, scores of half 1                                                   (MFMA)
+    //   V2: dequantize block 1, fetch block 0 of tile t+2, softmax of half 1
+    //   M2: PV of half 1, scores of half 0 of tile t+1                                       (MFMA)
+    // The dequantization is split so that the two VALU slots are equally long (a slot lasts as long
+    // as the longer of one set's VALU work and the other set's MFMA work), and each fetch goes out
+    // as soon as its registers are free, ahead of the softmax, so that it travels while this wave
+    // still has VALU work and through one MFMA slot.
     // Set 1 runs one slot behind set 0 (it passes one extra barrier first, set 0 one extra at
     // the end), so in every slot one set of each SIMD issues MFMAs while the other does VALU work.
-    // Hazards: set 0 writes K(t+1) in its V1(t); the K(t-1) it replaces was last read in M1(t-1),
-    // which set 1 finished one slot before.  Set 1 writes V(t+1) in its V1(t), which is set 0's
-    // M1(t); the V(t-1) it replaces was last read in M2(t-1), finished by both sets before that.
+    // Hazards: set 0 writes K(t+1) in its V1(t) and V2(t); the K(t-1) it replaces was last read in
+    // M1(t-1), which set 1 finished one slot before V1(t), and K(t+1) is first read in M2(t).  Set 1
+    // writes V(t+1) in its V1(t) and V2(t), which are set 0's M1(t) and M2(t); the V(t-1) it replaces
+    // was last read in M2(t-1), finished by both sets before that, and V(t+1) is first read in M1(t+1).
     if (ntile > 0) {
-        stage(0);
-        if (ntile > 1)
-            issue(1);
+        stage0(0);
+        issue1(0);
+        stage1(0);
+        issue0(1);
     }
     lds_barrier();
     if (PF_SKEW && set == 1)
@@ -433,48 +475,37 @@ __global__ void __launch_bounds__(kPfThreads, 2) chunk_q8_kernel(const ChunkArgs
     lds_barrier();
     TSTART();
     for (int t = 0; t < ntile; t++) {
-        if (t + 1 < ntile) {
-#ifdef PF_TIMING
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            TMARK(2); // (timing builds: the wait for the tile prefetch is booked under "barrier A")
-#endif
-            stage(t + 1);
-#ifdef PF_TIMING
-            TMARK(1);
-#endif
-        }
-#ifdef PF_TIMING
-        TMARK(5); // (timing builds: issuing the next prefetch is booked under "barrier B")
-#endif
+        if (t + 1 < ntile)
+            stage0(t + 1);
+        TMARK(12);
+        issue1(t + 1);
+        TMARK(13);
         softmax(t, 0);
         TMARK(0);
         lds_barrier();
-        TMARK(2);
-        PRIO(1);
+        TMARK(1);
         pv(t, 0);
-        TMARK(3);
-        scores(t, 1);
-        PRIO(0);
-        TMARK(4);
-        lds_barrier();
         TMARK(2);
-        softmax(t, 1);
-        // the next prefetch is issued from the short slot (V2): issuing the five loads of a
-        // unit is slow enough to matter, and V1 already carries the dequantization
-        if (t + 2 < ntile)
-            issue(t + 2);
-        TMARK(0);
-        lds_barrier();
-        TMARK(5);
-        PRIO(1);
-        pv(t, 1);
+        scores(t, 1);
         TMARK(3);
+        lds_barrier();
+        TMARK(4);
+        if (t + 1 < ntile)
+            stage1(t + 1);
+        TMARK(14);
+        issue0(t + 2);
+        TMARK(15);
+        softmax(t, 1);
+        TMARK(5);
+        lds_barrier();
+        TMARK(6);
+        pv(t, 1);
+        TMARK(7);
         if (t + 1 < ntile)
             scores(t + 1, 0);
-        PRIO(0);
-        TMARK(4);
+        TMARK(8);
         lds_barrier();
-        TMARK(5);
+        TMARK(9);
     }
     if (PF_SKEW && set == 0)
         lds_barrier();
@@ -550,7 +581,7 @@ __global__ void __launch_bounds__(256) chunk_combine_kernel(
 #ifdef PF_TIMING
 extern "C" int hipml_dbg_read_pf(unsigned long long *host, size_t n)
 {
-    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_pf_t), n * 8);
+    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_pf_t), (n < 128 ? n : 128) * 8);
 }
 #endif
 
