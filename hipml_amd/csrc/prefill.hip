@@ -69,6 +69,11 @@ struct ChunkArgs {
     int pos0, tokens, stride, splits, qslots;
     int ntask;  // tasks per KV head = ceil(tokens/32) * group
     int nblock; // task blocks per KV head = ceil(ntask/8)
+    // Key slices per task block.  A block whose last token sees few keys (the early blocks of a
+    // chunk near position 0) is cut into fewer slices than `splits`: slices(block) =
+    // min(splits, ceil(tiles(block) / slice_tiles)); a block with one slice writes its final
+    // output itself.  nslice = sum over blocks; uniform = every block has `splits` slices.
+    int slice_tiles, nslice, uniform;
     float scale_log2;
 };
 
@@ -151,6 +156,22 @@ __device__ __forceinline__ void stage_block1(const Half &h, uint8_t *dst)
     d4[7] = x1;
 }
 
+// Number of key slices of task block tb (see ChunkArgs::slice_tiles); *seq_block receives the number
+// of keys its last token sees.
+__device__ __host__ __forceinline__ int block_slices(int tb, int ntask, int group, int tokens, int pos0,
+                                                     int splits, int slice_tiles, int *seq_block)
+{
+    const int last_task = tb * kTasks + kTasks - 1 < ntask ? tb * kTasks + kTasks - 1 : ntask - 1;
+    const int tt_last = last_task / group;
+    const int last_tok = ((tt_last + 1) * kQTile < tokens ? (tt_last + 1) * kQTile : tokens) - 1;
+    const int seq = pos0 + last_tok + 1;
+    if (seq_block)
+        *seq_block = seq;
+    const int tiles = (seq + kKTile - 1) / kKTile;
+    const int n = (tiles + slice_tiles - 1) / slice_tiles;
+    return n < 1 ? 1 : (n < splits ? n : splits);
+}
+
 #ifdef PF_TIMING
 // debug builds: per-wave accumulated cycles of each slot of the tile loop, for one workgroup:
 // [wave][16] = 10 phases, total cycles, total time in 100 MHz ticks
@@ -208,8 +229,8 @@ __global__ void __launch_bounds__(kPfThreads, 2) chunk_q8_kernel(const ChunkArgs
     // blockIdx.x -> (kv head, key slice, task block).  Consecutive workgroups go to different
     // XCDs (8 of them, each with its own L2); the workgroups that stream the same (kv head,
     // slice) are therefore placed 8 apart, so that slice's K/V rows pass through one L2.
-    int kvh, split, tb;
-    {
+    int kvh, split, tb, nsp = 1;
+    if (!SPLIT || a.uniform) {
         const int combos = a.n_kv * (SPLIT ? a.splits : 1);
         const int bid = blockIdx.x;
         int combo;
@@ -229,9 +250,26 @@ __global__ void __launch_bounds__(kPfThreads, 2) chunk_q8_kernel(const ChunkArgs
         }
         kvh = combo % a.n_kv;
         split = combo / a.n_kv;
+        nsp = SPLIT ? a.splits : 1;
+        if (tb >= a.nblock)
+            return; // uniform over the workgroup
+    } else {
+        // per-block slice counts: workgroup -> (kv head, slice index), the slice index is resolved
+        // to (block, slice of the block) by walking the blocks
+        kvh = blockIdx.x % a.n_kv;
+        int sl = blockIdx.x / a.n_kv;
+        if (sl >= a.nslice)
+            return;
+        tb = 0;
+        for (;;) {
+            nsp = block_slices(tb, a.ntask, a.group, a.tokens, a.pos0, a.splits, a.slice_tiles, nullptr);
+            if (sl < nsp)
+                break;
+            sl -= nsp;
+            tb++;
+        }
+        split = sl;
     }
-    if (tb >= a.nblock)
-        return; // uniform over the workgroup
 
     const int task = tb * kTasks + wave;
     const bool task_valid = task < a.ntask;
@@ -247,8 +285,8 @@ __global__ void __launch_bounds__(kPfThreads, 2) chunk_q8_kernel(const ChunkArgs
     const int seq_block = a.pos0 + last_tok + 1;
     int klo = 0, khi = seq_block;
     if (SPLIT) {
-        klo = (int)((long long)seq_block * split / a.splits);
-        khi = (int)((long long)seq_block * (split + 1) / a.splits);
+        klo = (int)((long long)seq_block * split / nsp);
+        khi = (int)((long long)seq_block * (split + 1) / nsp);
     }
     const int tok = t0 + ln;
     const int my_last_key = a.pos0 + tok;               // inclusive causal bound of this lane's token
@@ -283,8 +321,11 @@ __global__ void __launch_bounds__(kPfThreads, 2) chunk_q8_kernel(const ChunkArgs
     auto issue1 = [&](int t) { load_half1(half, unit_ptr(t)); };
     auto stage0 = [&](int t) { stage_block0(half, lds + (t & 1) * kBufBytes + sdst); };
     auto stage1 = [&](int t) { stage_block1(half, lds + (t & 1) * kBufBytes + sdst); };
-    if (ntile > 0)
+    Half first1; // block 1 of the first tile: fetched together with block 0, ahead of the Q loads
+    if (ntile > 0) {
         issue0(0);
+        load_half1(first1, unit_ptr(0));
+    }
 
     // ---- Q^T operand: 16 k-steps of 8 f16 (d = ks*16 + lh*8 + j) ---------------------------
     // Steps 0..kQLdsSteps-1 are parked in this wave's corner of LDS and re-read per use: 256
@@ -463,8 +504,7 @@ __global__ void __launch_bounds__(kPfThreads, 2) chunk_q8_kernel(const ChunkArgs
     // was last read in M2(t-1), finished by both sets before that, and V(t+1) is first read in M1(t+1).
     if (ntile > 0) {
         stage0(0);
-        issue1(0);
-        stage1(0);
+        stage_block1(first1, lds + sdst);
         issue0(1);
     }
     lds_barrier();
@@ -515,7 +555,7 @@ __global__ void __launch_bounds__(kPfThreads, 2) chunk_q8_kernel(const ChunkArgs
     l_run += __shfl_xor(l_run, 32);
     if (!tok_valid)
         return;
-    if (SPLIT) {
+    if (SPLIT && nsp > 1) {
         const size_t row = ((size_t)split * a.qslots + tok) * a.n_head + head;
         float *pa = a.part_acc + row * kHeadDim;
 #pragma unroll
@@ -543,18 +583,27 @@ __global__ void __launch_bounds__(kPfThreads, 2) chunk_q8_kernel(const ChunkArgs
     }
 }
 
-// Fold the key slices: one workgroup per (token, 4 heads); thread = (head, float4 of d).
+// Fold the key slices: one workgroup per (token, 4 heads); thread = (head, float4 of d).  A (token,
+// head) whose task block has a single slice was written by the attention kernel itself.
 __global__ void __launch_bounds__(256) chunk_combine_kernel(
     const float *__restrict__ part_acc, const float *__restrict__ part_ml, float *__restrict__ out,
-    int n_head, int qslots, int splits)
+    int n_head, int qslots, int splits, int group, int ntask, int tokens, int pos0, int slice_tiles,
+    int uniform)
 {
     const int tok = blockIdx.x;
     const int head = blockIdx.y * 4 + (threadIdx.x >> 6);
     const int d4 = (threadIdx.x & 63) * 4;
     if (head >= n_head)
         return;
+    int nsp = splits;
+    if (!uniform) {
+        const int task = (tok / kQTile) * group + head % group;
+        nsp = block_slices(task / kTasks, ntask, group, tokens, pos0, splits, slice_tiles, nullptr);
+        if (nsp == 1)
+            return;
+    }
     float m = -INFINITY;
-    for (int s = 0; s < splits; s++) {
+    for (int s = 0; s < nsp; s++) {
         const size_t row = ((size_t)s * qslots + tok) * n_head + head;
         const float2 ml = *reinterpret_cast<const float2 *>(part_ml + row * 2);
         if (ml.y > 0.0f)
@@ -562,7 +611,7 @@ __global__ void __launch_bounds__(256) chunk_combine_kernel(
     }
     float4v num = {0, 0, 0, 0};
     float den = 0.0f;
-    for (int s = 0; s < splits; s++) {
+    for (int s = 0; s < nsp; s++) {
         const size_t row = ((size_t)s * qslots + tok) * n_head + head;
         const float2 ml = *reinterpret_cast<const float2 *>(part_ml + row * 2);
         const float4v x = *reinterpret_cast<const float4v *>(part_acc + row * kHeadDim + d4);
@@ -620,17 +669,30 @@ int launch_chunk_q8(hipStream_t st, const float *q, const uint8_t *kc, const uin
     a.ntask = (tokens + kQTile - 1) / kQTile * a.group;
     a.nblock = (a.ntask + kTasks - 1) / kTasks;
     a.scale_log2 = kLog2e / 16.0f; // 1/sqrt(256), as the reference's chunk launcher fixes it
-    const int combos = n_kv * a.splits;
-    // grid.x covers every (combo, task block); the XCD-aware decode in the kernel may leave a
-    // few trailing workgroups without work when 8 is not a multiple of `combos`.
-    unsigned grid;
-    if (combos % 8 == 0)
-        grid = (unsigned)(combos * a.nblock);
-    else if (8 % combos == 0)
-        grid = (unsigned)(8 * ((a.nblock + 8 / combos - 1) / (8 / combos)));
-    else
-        grid = (unsigned)(combos * a.nblock);
+    // slices per block: the last block (most keys) gets `splits`, a block with fewer key tiles gets
+    // proportionally fewer, so a chunk near position 0 does not write and re-read `splits` partial
+    // copies of rows that see only a few tiles
+    const int tiles_last = (pos0 + tokens + kKTile - 1) / kKTile;
+    a.slice_tiles = (tiles_last + a.splits - 1) / a.splits;
+    a.nslice = 0;
+    for (int tb = 0; tb < a.nblock; tb++)
+        a.nslice += block_slices(tb, a.ntask, a.group, tokens, pos0, a.splits, a.slice_tiles, nullptr);
+    a.uniform = a.nslice == a.nblock * a.splits;
     const dim3 block(kPfThreads, 1, 1);
+    unsigned grid;
+    if (a.splits > 1 && !a.uniform) {
+        grid = (unsigned)(n_kv * a.nslice);
+    } else {
+        // grid.x covers every (combo, task block); the XCD-aware decode in the kernel may leave a
+        // few trailing workgroups without work when 8 is not a multiple of `combos`.
+        const int combos = n_kv * a.splits;
+        if (combos % 8 == 0)
+            grid = (unsigned)(combos * a.nblock);
+        else if (8 % combos == 0)
+            grid = (unsigned)(8 * ((a.nblock + 8 / combos - 1) / (8 / combos)));
+        else
+            grid = (unsigned)(combos * a.nblock);
+    }
     if (splits < 2) {
         hipLaunchKernelGGL(chunk_q8_kernel<false>, dim3(grid, 1, 1), block, kPfLds, st, a);
         return launched("attn_chunk_q8");
@@ -640,7 +702,8 @@ int launch_chunk_q8(hipStream_t st, const float *q, const uint8_t *kc, const uin
     if (rc)
         return rc;
     hipLaunchKernelGGL(chunk_combine_kernel, dim3((unsigned)tokens, (unsigned)((n_head + 3) / 4), 1),
-                       dim3(256, 1, 1), 0, st, part_acc, part_ml, out, n_head, a.qslots, splits);
+                       dim3(256, 1, 1), 0, st, part_acc, part_ml, out, n_head, a.qslots, a.splits, a.group,
+                       a.ntask, tokens, pos0, a.slice_tiles, a.uniform);
     return launched("attn_chunk_combine");
 }
 
