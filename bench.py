@@ -128,20 +128,33 @@ def bench_prefill(torch, attn, tokens, pos0, steps, warmup, layers, prefix_fill=
                                       splits)
 
     def step(i):
+        # the gate is applied where the attention result is written (same bits as the separate
+        # gate kernel, one pass over the rows less)
+        k, v = caches[i % layers]
+        attn.rope_chunk(q, kx, H, KV, HD, NROT, THETA, pos0, tokens)
+        attn.kv_encode_bulk(0, kx, vx, k, v, KV, HD, stride, pos0, 0, tokens)
+        attn.chunk_attention_q8_split_gate(q, k, v, gate, out, H, KV, HD, pos0, tokens, 1, stride,
+                                           acc, ml, splits)
+
+    def step_unfused(i):
         k, v = caches[i % layers]
         attn.rope_chunk(q, kx, H, KV, HD, NROT, THETA, pos0, tokens)
         attn.kv_encode_bulk(0, kx, vx, k, v, KV, HD, stride, pos0, 0, tokens)
         attention(i)
         attn.q_gate(out, gate, out)
 
-    for i in range(warmup):
-        step(i)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(steps):
-        step(i)
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    def wall(fn):
+        for i in range(warmup):
+            fn(i)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(steps):
+            fn(i)
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / steps
+
+    unfused_ms = wall(step_unfused)
+    wall_ms = wall(step)
 
     # the attention launch alone, HIP events on the launch stream
     for i in range(min(warmup, 3)):
@@ -160,6 +173,7 @@ def bench_prefill(torch, attn, tokens, pos0, steps, warmup, layers, prefix_fill=
         "tokens": tokens, "pos0": pos0, "splits": splits, "layers_rotated": layers,
         "ms_per_step": wall_ms,
         "tok_per_s": tokens / (wall_ms * 1e-3),
+        "ms_per_step_separate_gate": unfused_ms,
         "attn_ms": attn_ms,
         "attn_tok_per_s": tokens / (attn_ms * 1e-3),
         "roofline": {"bound": "mfma", "achieved": tf, "peak": MFMA_F16_PEAK_TF, "unit": "TFLOP/s",

@@ -32,7 +32,7 @@ EXPORTS = [
     "hipml_kv_encode", "hipml_kv_encode_bulk", "hipml_kv_encode_rows",
     "hipml_attn_decode_kv", "hipml_attn_decode_kv_cols", "hipml_attn_decode_rows",
     "hipml_attn_decode_batch", "hipml_attn_decode_batch_cols",
-    "hipml_attn_chunk_q8_split", "hipml_q_gate_f32",
+    "hipml_attn_chunk_q8_split", "hipml_attn_chunk_q8_split_gate", "hipml_q_gate_f32",
 ]
 
 
@@ -85,6 +85,7 @@ def lib() -> C.CDLL:
             "hipml_attn_decode_batch_cols": (i, [vp, i, vp, vp, vp, vp, vp, vp, vp, i, i, i, i, f,
                                                  i, sz, sz, sz, sz, i, vp]),
             "hipml_attn_chunk_q8_split": (i, [vp, vp, vp, vp, vp, i, i, i, i, i, i, i, vp, vp, i]),
+            "hipml_attn_chunk_q8_split_gate": (i, [vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, i, vp, vp, i]),
             "hipml_q_gate_f32": (i, [vp, vp, vp, vp, sz]),
         }
         for name, (res, args) in sig.items():
@@ -251,6 +252,14 @@ def chunk_attention_q8_split(q, kc, vc, out, n_head, n_kv, head_dim, pos0, token
     _check(lib().hipml_attn_chunk_q8_split(_stream(stream), _p(q), _p(kc), _p(vc), _p(out), n_head,
                                            n_kv, head_dim, pos0, tokens, dtype, stride,
                                            _p(part_acc), _p(part_ml), splits))
+
+
+def chunk_attention_q8_split_gate(q, kc, vc, gate, out, n_head, n_kv, head_dim, pos0, tokens, dtype,
+                                  stride, part_acc, part_ml, splits, stream=None):
+    """`chunk_attention_q8_split` followed by `q_gate_only`, as one call (same bits)."""
+    _check(lib().hipml_attn_chunk_q8_split_gate(_stream(stream), _p(q), _p(kc), _p(vc), _p(gate),
+                                                _p(out), n_head, n_kv, head_dim, pos0, tokens, dtype,
+                                                stride, _p(part_acc), _p(part_ml), splits))
 
 
 def chunk_scratch(tokens: int, n_head: int, splits: int, device="cuda"):

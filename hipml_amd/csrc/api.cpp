@@ -502,16 +502,18 @@ int hipml_attn_decode_batch_cols(hipml_stream_t stream, int dtype, const int32_t
 
 // ---- chunk prefill ---------------------------------------------------------------------------------
 
-int hipml_attn_chunk_q8_split(hipml_stream_t stream, const float *q, const void *kc,
-                              const void *vc, float *out, int n_head, int n_kv, int head_dim,
-                              int pos0, int tokens, int dtype, int stride, float *part_acc,
-                              float *part_ml, int splits)
+static int chunk_q8_common(hipml_stream_t stream, const float *q, const void *kc, const void *vc,
+                           float *out, const float *gate, bool want_gate, int n_head, int n_kv,
+                           int head_dim, int pos0, int tokens, int dtype, int stride, float *part_acc,
+                           float *part_ml, int splits)
 {
     clear_error();
     REQUIRE_PTR(q);
     REQUIRE_PTR(kc);
     REQUIRE_PTR(vc);
     REQUIRE_PTR(out);
+    if (want_gate)
+        REQUIRE_PTR(gate);
     if (dtype != 1)
         return fail(HIPML_ATTN_E_UNSUPPORTED,
                     "quantized chunk attention: only a q8_0 cache (dtype 1) is built, got %d", dtype);
@@ -532,11 +534,31 @@ int hipml_attn_chunk_q8_split(hipml_stream_t stream, const float *q, const void 
     if ((rc = check_aligned16(q, "q")) || (rc = check_aligned16(out, "out")) ||
         (rc = check_aligned16(kc, "k cache")) || (rc = check_aligned16(vc, "v cache")))
         return rc;
+    if (want_gate && (rc = check_aligned16(gate, "gate")))
+        return rc;
     if (tokens == 0)
         return 0;
     return launch_chunk_q8(as_stream(stream), q, static_cast<const uint8_t *>(kc),
                            static_cast<const uint8_t *>(vc), out, n_head, n_kv, pos0, tokens,
-                           stride, part_acc, part_ml, splits);
+                           stride, part_acc, part_ml, splits, want_gate ? gate : nullptr);
+}
+
+int hipml_attn_chunk_q8_split(hipml_stream_t stream, const float *q, const void *kc,
+                              const void *vc, float *out, int n_head, int n_kv, int head_dim,
+                              int pos0, int tokens, int dtype, int stride, float *part_acc,
+                              float *part_ml, int splits)
+{
+    return chunk_q8_common(stream, q, kc, vc, out, nullptr, false, n_head, n_kv, head_dim, pos0, tokens,
+                           dtype, stride, part_acc, part_ml, splits);
+}
+
+int hipml_attn_chunk_q8_split_gate(hipml_stream_t stream, const float *q, const void *kc,
+                                   const void *vc, const float *gate, float *out, int n_head,
+                                   int n_kv, int head_dim, int pos0, int tokens, int dtype,
+                                   int stride, float *part_acc, float *part_ml, int splits)
+{
+    return chunk_q8_common(stream, q, kc, vc, out, gate, true, n_head, n_kv, head_dim, pos0, tokens,
+                           dtype, stride, part_acc, part_ml, splits);
 }
 
 // ---- gate ---------------------------------------------------------------------------------------------

@@ -72,6 +72,6 @@ int decode_init();
 int prefill_init();
 int launch_chunk_q8(hipStream_t st, const float *q, const uint8_t *kc, const uint8_t *vc,
                     float *out, int n_head, int n_kv, int pos0, int tokens, int stride,
-                    float *part_acc, float *part_ml, int splits);
+                    float *part_acc, float *part_ml, int splits, const float *gate);
 
 } // namespace hipml

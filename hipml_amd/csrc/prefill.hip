@@ -63,6 +63,7 @@ struct ChunkArgs {
     const uint8_t *kc;
     const uint8_t *vc;
     float *out;
+    const float *gate; // optional [tokens][n_head][256]: out = attention * sigmoid(gate)
     float *part_acc;
     float *part_ml;
     int n_head, n_kv, group;
@@ -154,6 +155,13 @@ __device__ __forceinline__ void stage_block1(const Half &h, uint8_t *dst)
     dequant16(h.q, s1, x0, x1);
     d4[6] = x0;
     d4[7] = x1;
+}
+
+// The output gate, written exactly as the stand-alone gate kernel writes it, so a fused call and
+// the attention followed by that kernel give the same bits.
+__device__ __forceinline__ float gated(float x, float g)
+{
+    return x * (1.0f / (1.0f + expf(-g)));
 }
 
 // Number of key slices of task block tb (see ChunkArgs::slice_tiles); *seq_block receives the number
@@ -571,7 +579,24 @@ __global__ void __launch_bounds__(kPfThreads, 2) chunk_q8_kernel(const ChunkArgs
         }
     } else {
         const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
-        float *po = a.out + ((size_t)tok * a.n_head + head) * kHeadDim;
+        const size_t orow = ((size_t)tok * a.n_head + head) * kHeadDim;
+        float *po = a.out + orow;
+        // (with key slices the merge kernel gates every row, also the ones written here: it runs at
+        // full occupancy, where the exponentials and divisions of the gate are cheap)
+        if (a.gate && !SPLIT) {
+            const float *pg = a.gate + orow;
+#pragma unroll
+            for (int dt = 0; dt < 8; dt++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const float4v gt = *reinterpret_cast<const float4v *>(pg + dt * 32 + g * 8 + lh * 4);
+                    const float4v x = {gated(O[dt][g * 4] * inv, gt[0]), gated(O[dt][g * 4 + 1] * inv, gt[1]),
+                                       gated(O[dt][g * 4 + 2] * inv, gt[2]),
+                                       gated(O[dt][g * 4 + 3] * inv, gt[3])};
+                    *reinterpret_cast<float4v *>(po + dt * 32 + g * 8 + lh * 4) = x;
+                }
+            return;
+        }
 #pragma unroll
         for (int dt = 0; dt < 8; dt++)
 #pragma unroll
@@ -586,21 +611,29 @@ __global__ void __launch_bounds__(kPfThreads, 2) chunk_q8_kernel(const ChunkArgs
 // Fold the key slices: one workgroup per (token, 4 heads); thread = (head, float4 of d).  A (token,
 // head) whose task block has a single slice was written by the attention kernel itself.
 __global__ void __launch_bounds__(256) chunk_combine_kernel(
-    const float *__restrict__ part_acc, const float *__restrict__ part_ml, float *__restrict__ out,
-    int n_head, int qslots, int splits, int group, int ntask, int tokens, int pos0, int slice_tiles,
-    int uniform)
+    const float *__restrict__ part_acc, const float *__restrict__ part_ml, float *out,
+    const float *__restrict__ gate, int n_head, int qslots, int splits, int group, int ntask, int tokens,
+    int pos0, int slice_tiles, int uniform)
 {
     const int tok = blockIdx.x;
     const int head = blockIdx.y * 4 + (threadIdx.x >> 6);
     const int d4 = (threadIdx.x & 63) * 4;
     if (head >= n_head)
         return;
+    const size_t o = ((size_t)tok * n_head + head) * kHeadDim + d4;
     int nsp = splits;
     if (!uniform) {
         const int task = (tok / kQTile) * group + head % group;
         nsp = block_slices(task / kTasks, ntask, group, tokens, pos0, splits, slice_tiles, nullptr);
-        if (nsp == 1)
+        if (nsp == 1) {
+            if (gate) {
+                const float4v x = *reinterpret_cast<const float4v *>(out + o);
+                const float4v gt = *reinterpret_cast<const float4v *>(gate + o);
+                *reinterpret_cast<float4v *>(out + o) =
+                    (float4v){gated(x[0], gt[0]), gated(x[1], gt[1]), gated(x[2], gt[2]), gated(x[3], gt[3])};
+            }
             return;
+        }
     }
     float m = -INFINITY;
     for (int s = 0; s < nsp; s++) {
@@ -624,7 +657,11 @@ __global__ void __launch_bounds__(256) chunk_combine_kernel(
     float4v r = num * inv;
     if (!(den > 0.0f))
         r = (float4v){0, 0, 0, 0};
-    *reinterpret_cast<float4v *>(out + ((size_t)tok * n_head + head) * kHeadDim + d4) = r;
+    if (gate) {
+        const float4v gt = *reinterpret_cast<const float4v *>(gate + o);
+        r = (float4v){gated(r[0], gt[0]), gated(r[1], gt[1]), gated(r[2], gt[2]), gated(r[3], gt[3])};
+    }
+    *reinterpret_cast<float4v *>(out + o) = r;
 }
 
 #ifdef PF_TIMING
@@ -649,9 +686,10 @@ int prefill_init()
 
 int launch_chunk_q8(hipStream_t st, const float *q, const uint8_t *kc, const uint8_t *vc,
                     float *out, int n_head, int n_kv, int pos0, int tokens, int stride,
-                    float *part_acc, float *part_ml, int splits)
+                    float *part_acc, float *part_ml, int splits, const float *gate)
 {
     ChunkArgs a;
+    a.gate = gate;
     a.q = q;
     a.kc = kc;
     a.vc = vc;
@@ -702,7 +740,7 @@ int launch_chunk_q8(hipStream_t st, const float *q, const uint8_t *kc, const uin
     if (rc)
         return rc;
     hipLaunchKernelGGL(chunk_combine_kernel, dim3((unsigned)tokens, (unsigned)((n_head + 3) / 4), 1),
-                       dim3(256, 1, 1), 0, st, part_acc, part_ml, out, n_head, a.qslots, a.splits, a.group,
+                       dim3(256, 1, 1), 0, st, part_acc, part_ml, out, gate, n_head, a.qslots, a.splits, a.group,
                        a.ntask, tokens, pos0, a.slice_tiles, a.uniform);
     return launched("attn_chunk_combine");
 }

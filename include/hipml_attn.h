@@ -192,6 +192,18 @@ int hipml_attn_chunk_q8_split(hipml_stream_t stream, const float *q, const void 
                               int pos0, int tokens, int dtype, int stride, float *part_acc,
                               float *part_ml, int splits);
 
+/* The same attention with the sigmoid output gate applied where the result is
+ * written (in the key-slice merge, or in the attention kernel for rows that are
+ * not sliced): out = attention * sigmoid(gate), gate f32 [tokens][n_head][head_dim].
+ * Bit-identical to hipml_attn_chunk_q8_split followed by hipml_q_gate_f32 on its
+ * output; it saves that kernel's pass over the rows.  Replaces the pair
+ * AttnLayer::chunk_attention_q8_split (attn_chunk_kv.rs:72-107) + q_gate_only
+ * (crates/hipml-kernels/src/attn_gpu.rs:822-834) of the reference's chunk path. */
+int hipml_attn_chunk_q8_split_gate(hipml_stream_t stream, const float *q, const void *kc,
+                                   const void *vc, const float *gate, float *out, int n_head,
+                                   int n_kv, int head_dim, int pos0, int tokens, int dtype,
+                                   int stride, float *part_acc, float *part_ml, int splits);
+
 /* ---- output gate ------------------------------------------------------------ */
 
 /* y[i] = x[i] * sigmoid(gate[i]); y may alias x.  Replaces

@@ -92,3 +92,28 @@ def test_deep_chunk_sampled_rows():
         got = run_chunk(q, kb, vb, pos0, tok, stride, splits)
         ok, _, _ = report(f"chunk 256@20000 splits {splits}", want, got[rows], *GATE)
         assert ok
+
+
+@pytest.mark.parametrize("tok,pos0,splits", [(37, 29, 1), (37, 29, 4), (300, 0, 5), (160, 4000, 3)])
+def test_fused_gate_equals_attention_then_gate(tok, pos0, splits):
+    # the fused call must give the bits of the two-call sequence it replaces (mono kernel, uniform
+    # key slices, per-block slice counts near position 0)
+    q, kb, vb, stride = chunk_inputs(0x6A7D + tok, tok, pos0, 11)
+    r = orc.Rng(0x6A7E + tok)
+    gate = r.normal_array((tok, N_HEADS, HD))
+    plain = run_chunk(q, kb, vb, pos0, tok, stride, splits)
+    x = dev(plain)
+    two = torch.empty_like(x)
+    attn.q_gate(x, dev(gate), two)
+    fused = torch.empty_like(x)
+    acc = ml = None
+    if splits >= 2:
+        acc, ml = attn.chunk_scratch(tok, N_HEADS, splits)
+    attn.chunk_attention_q8_split_gate(dev(q), dev(kb), dev(vb), dev(gate), fused, N_HEADS, N_KV, HD,
+                                       pos0, tok, 1, stride, acc, ml, splits)
+    torch.cuda.synchronize()
+    assert np.array_equal(host(two), host(fused)), f"fused gate differs ({tok}@{pos0} splits {splits})"
+    # and the oracle's gate of the same rows, to the gate kernel's own class (device expf vs libm)
+    want = orc.q_gate(plain.ravel(), gate.ravel())
+    ok, _, _ = report(f"fused gate {tok}@{pos0} splits {splits}", want, host(fused).ravel(), 1e-6, 1e-5)
+    assert ok
