@@ -291,6 +291,32 @@ def bench_batch(torch, attn, orc, steps, warmup, layers):
     }
 
 
+def bench_front(torch, attn, tokens, steps):
+    """Attention front end over a chunk: q|gate split + head RMS norm + RoPE (one launch)."""
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(0x5EED0006)
+    qg = torch.randn((tokens, H, 2 * HD), device="cuda", generator=gen)
+    k0 = torch.randn((tokens, KV, HD), device="cuda", generator=gen)
+    k = k0.clone()
+    qw = torch.ones(HD, device="cuda")
+    kw = torch.ones(HD, device="cuda")
+    q = torch.empty((tokens, H, HD), device="cuda")
+    gate = torch.empty((tokens, H, HD), device="cuda")
+    attn.rope_table(THETA, NROT, max(tokens, 1024))
+    for _ in range(3):
+        attn.chunk_front(qg, k, q, gate, qw, kw, H, KV, HD, NROT, THETA, 1e-6, 0, tokens)
+    with Timer(torch) as t:
+        for _ in range(steps):
+            attn.chunk_front(qg, k, q, gate, qw, kw, H, KV, HD, NROT, THETA, 1e-6, 0, tokens)
+    us = t.ms * 1e3 / steps
+    nbytes = tokens * (H * 2 * HD + 2 * H * HD + 2 * KV * HD) * 4  # qg read, q + gate written, k both
+    gbs = nbytes / (us * 1e-6) / 1e9
+    return {"workload": f"attention front end, {tokens} rows: q|gate split + head RMS norm + RoPE",
+            "us": us, "bytes": nbytes,
+            "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": gbs / HBM_PEAK_GBS, "traffic": None, "kernel": "front_kernel"}}
+
+
 def bench_copycal(torch, steps):
     """Plain device copy of a known size: the yardstick the HBM traffic counters
     (FETCH_SIZE / WRITE_SIZE) are scaled by."""
@@ -351,7 +377,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--main-only", action="store_true", help="skip the 'also' workloads")
     ap.add_argument("--only", default="", help="run one workload alone (prefill672, decode8k, "
-                    "decode32k, decode128k, chunk100k, batch16, copycal) for profiling; prints its object")
+                    "decode32k, decode128k, chunk100k, batch16, front672, copycal) for profiling; prints its object")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -379,6 +405,7 @@ def main() -> int:
             "chunk100k": lambda: bench_prefill(torch, attn, 2048, 100_000, K, W, 2),
             "batch16": lambda: bench_batch(torch, attn, orc, K, W, 4),
             "copycal": lambda: bench_copycal(torch, K),
+            "front672": lambda: bench_front(torch, attn, 672, max(K, 20)),
         }[args.only]
         print(json.dumps(fn()))
         return 0
@@ -415,6 +442,7 @@ def main() -> int:
         also["chunk_2048_at_100000"] = bench_prefill(torch, attn, 2048, 100_000,
                                                      max(K // 20, 3), 1, 2)
         torch.cuda.empty_cache()
+        also["front_672"] = bench_front(torch, attn, 672, d_steps)
         from oracle import binding as orc  # only for the seeded depth recipe and the CPU leg
         also["batch16_mtp"] = bench_batch(torch, attn, orc, d_steps, max(W // 4, 2), 4)
         torch.cuda.empty_cache()

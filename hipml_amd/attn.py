@@ -33,6 +33,7 @@ EXPORTS = [
     "hipml_attn_decode_kv", "hipml_attn_decode_kv_cols", "hipml_attn_decode_rows",
     "hipml_attn_decode_batch", "hipml_attn_decode_batch_cols",
     "hipml_attn_chunk_q8_split", "hipml_attn_chunk_q8_split_gate", "hipml_q_gate_f32",
+    "hipml_attn_front_f32", "hipml_attn_chunk_front_f32",
 ]
 
 
@@ -87,6 +88,8 @@ def lib() -> C.CDLL:
             "hipml_attn_chunk_q8_split": (i, [vp, vp, vp, vp, vp, i, i, i, i, i, i, i, vp, vp, i]),
             "hipml_attn_chunk_q8_split_gate": (i, [vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, i, vp, vp, i]),
             "hipml_q_gate_f32": (i, [vp, vp, vp, vp, sz]),
+            "hipml_attn_front_f32": (i, [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, i, i, vp, f, f]),
+            "hipml_attn_chunk_front_f32": (i, [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, f, f, i, i]),
         }
         for name, (res, args) in sig.items():
             fn = getattr(l, name)
@@ -172,6 +175,26 @@ def mrope_rows(x, y, n_heads, head_dim, n_rot, sections, pos, rows, theta, strea
 def rope_chunk(q, k, n_head, n_kv, head_dim, n_rot, theta, pos0, tokens, stream=None):
     _check(lib().hipml_rope_chunk_f32(_stream(stream), _p(q), _p(k), n_head, n_kv, head_dim, n_rot,
                                       theta, pos0, tokens))
+
+
+# ---- attention front end ---------------------------------------------------------------
+
+def attn_front(qg, q, gate, k, q_norm, k_norm, n_heads, n_kv, head_dim, n_rot, sections, pos, theta,
+               eps, stream=None):
+    """`AttnLayer::front`: q|gate split, head RMS norm of q and k, M-RoPE of both (one token);
+    `pos` is the device int32[4] of M-RoPE position ids (step buffer + 4)."""
+    s0, s1, s2, s3 = sections
+    _check(lib().hipml_attn_front_f32(_stream(stream), _p(qg), _p(q), _p(gate), _p(k), _p(q_norm),
+                                      _p(k_norm), n_heads, n_kv, head_dim, n_rot, s0, s1, s2, s3,
+                                      _p(pos), theta, eps))
+
+
+def chunk_front(qg, k, q, gate, q_norm, k_norm, n_heads, n_kv, head_dim, n_rot, theta, eps, pos0,
+                tokens, stream=None):
+    """`AttnLayer::chunk_front`: the same over `tokens` rows at text positions pos0.."""
+    _check(lib().hipml_attn_chunk_front_f32(_stream(stream), _p(qg), _p(k), _p(q), _p(gate),
+                                            _p(q_norm), _p(k_norm), n_heads, n_kv, head_dim, n_rot,
+                                            theta, eps, pos0, tokens))
 
 
 # ---- KV append ------------------------------------------------------------------------

@@ -335,6 +335,62 @@ int hipml_rope_chunk_f32(hipml_stream_t stream, float *q, float *k, int n_head, 
                              pos0, tokens, g_rope);
 }
 
+// ---- attention front end ---------------------------------------------------------------------
+
+static int check_front(const float *qg, const float *q, const float *gate, const float *k,
+                       const float *q_norm, const float *k_norm, int n_heads, int n_kv, int head_dim,
+                       int n_rot, float theta_base, float eps)
+{
+    if (qg == nullptr || q == nullptr || gate == nullptr || k == nullptr || q_norm == nullptr ||
+        k_norm == nullptr)
+        return fail(HIPML_ATTN_E_NULL, "a front-end buffer (qg, q, gate, k, q_norm, k_norm) is NULL");
+    int rc = check_rope(n_heads, head_dim, n_rot, theta_base);
+    if (rc)
+        return rc;
+    if (n_kv <= 0)
+        return fail(HIPML_ATTN_E_SHAPE, "n_kv %d must be positive", n_kv);
+    if (head_dim != kHeadDim)
+        return fail(HIPML_ATTN_E_UNSUPPORTED,
+                    "attention front end: built for head_dim %d (one square per lane slot and the "
+                    "256-wide tree of the reference), got %d", kHeadDim, head_dim);
+    if (!(eps >= 0.0f))
+        return fail(HIPML_ATTN_E_RANGE, "eps %g must be non-negative", (double)eps);
+    return 0;
+}
+
+int hipml_attn_front_f32(hipml_stream_t stream, const float *qg, float *q, float *gate, float *k,
+                         const float *q_norm, const float *k_norm, int n_heads, int n_kv,
+                         int head_dim, int n_rot, int s0, int s1, int s2, int s3,
+                         const int32_t *pos, float theta_base, float eps)
+{
+    clear_error();
+    REQUIRE_PTR(pos);
+    int rc = check_front(qg, q, gate, k, q_norm, k_norm, n_heads, n_kv, head_dim, n_rot, theta_base, eps);
+    if (rc)
+        return rc;
+    if (s0 < 0 || s1 < 0 || s2 < 0 || s3 < 0)
+        return fail(HIPML_ATTN_E_RANGE, "negative M-RoPE section");
+    return launch_front(as_stream(stream), qg, q, gate, k, q_norm, k_norm, n_heads, n_kv, n_rot, s0, s1,
+                        s2, s3, pos, 0, 1, theta_base, eps, g_rope);
+}
+
+int hipml_attn_chunk_front_f32(hipml_stream_t stream, const float *qg, float *k, float *q,
+                               float *gate, const float *q_norm, const float *k_norm, int n_heads,
+                               int n_kv, int head_dim, int n_rot, float theta_base, float eps,
+                               int pos0, int tokens)
+{
+    clear_error();
+    int rc = check_front(qg, q, gate, k, q_norm, k_norm, n_heads, n_kv, head_dim, n_rot, theta_base, eps);
+    if (rc)
+        return rc;
+    if (pos0 < 0 || tokens < 0)
+        return fail(HIPML_ATTN_E_RANGE, "pos0 %d / tokens %d must be non-negative", pos0, tokens);
+    if (tokens == 0)
+        return 0;
+    return launch_front(as_stream(stream), qg, q, gate, k, q_norm, k_norm, n_heads, n_kv, n_rot, 0, 0, 0,
+                        0, nullptr, pos0, tokens, theta_base, eps, g_rope);
+}
+
 // ---- KV append -------------------------------------------------------------------------------
 
 static int check_encode(int dtype, const void *k, const void *v, const void *kc, const void *vc,

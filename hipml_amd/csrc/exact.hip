@@ -218,6 +218,113 @@ int launch_rope_chunk(hipStream_t st, float *q, float *k, int n_head, int n_kv, 
     return 0;
 }
 
+// ---- attention front end ------------------------------------------------------------
+//
+// q|gate split, per-head RMS norm of q and k, M-RoPE of both, one wave per (row, head):
+// the reference's attn_front_f32 (crates/hipml-kernels/kernels/attn_front_f32.hip:34-135, one
+// token) and qg_split_chunk_f32 + norm_rope_chunk_f32 (attn_chunk_f32.hip:22-98, a chunk of rows).
+// The arithmetic is theirs, operation for operation, at head_dim 256: the sum of squares is
+// one square per element folded by the halving tree red[t] += red[t + off], off = 128 .. 1 (a
+// lane holds elements l, l+64, l+128, l+192, so two levels are in-lane adds and six are lane
+// exchanges; IEEE addition commutes, so every lane ends with red[0]); mean = sum / 256;
+// scale = 1 / sqrtf(mean + eps) with the correctly rounded divide and square root; the value is
+// (x * scale) * w; the rotation reads cos/sin as the other RoPE kernels here do.
+// grid: ceil((n_heads + n_kv) * rows / 4) workgroups of 4 waves.  `pos` (device int32[4]) gives
+// the four M-RoPE position ids of a single row; when it is null, row t rotates at pos0 + t.
+__global__ void __launch_bounds__(256) front_kernel(
+    const float *__restrict__ qg, float *__restrict__ q, float *__restrict__ gate, float *k,
+    const float *__restrict__ qw, const float *__restrict__ kw, int n_heads, int n_kv, int n_rot,
+    int s0, int s1, int s2, int s3, const int32_t *__restrict__ pos, int pos0, int rows, float theta,
+    float eps, const float *__restrict__ tab, int tab_rows)
+{
+    __shared__ float buf[4][kHeadDim];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int per_row = n_heads + n_kv;
+    const int idx = blockIdx.x * 4 + wave;
+    if (idx >= per_row * rows)
+        return; // no workgroup-wide barrier below: waves are independent
+    const int row = idx / per_row;
+    const int hb = idx - row * per_row;
+    const bool is_q = hb < n_heads;
+    const int h = is_q ? hb : hb - n_heads;
+    const float *src = is_q ? qg + ((size_t)row * n_heads + h) * (2 * kHeadDim)
+                            : k + ((size_t)row * n_kv + h) * kHeadDim;
+    float *dst = is_q ? q + ((size_t)row * n_heads + h) * kHeadDim
+                      : k + ((size_t)row * n_kv + h) * kHeadDim;
+    const float *w = is_q ? qw : kw;
+
+    float x[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+        x[j] = src[lane + 64 * j];
+    if (is_q) {
+        float *gd = gate + ((size_t)row * n_heads + h) * kHeadDim;
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            gd[lane + 64 * j] = src[kHeadDim + lane + 64 * j];
+    }
+    const float a0 = x[0] * x[0] + x[2] * x[2]; // off = 128
+    const float a1 = x[1] * x[1] + x[3] * x[3];
+    float sum = a0 + a1;                        // off = 64
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1)
+        sum += __shfl_xor(sum, off);
+    const float mean_sq = sum / (float)kHeadDim;
+    const float scale = 1.0f / sqrtf(mean_sq + eps);
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+        buf[wave][lane + 64 * j] = x[j] * scale * w[lane + 64 * j];
+    __builtin_amdgcn_wave_barrier();
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+
+    const int half = n_rot >> 1;
+    const int sect = s0 + s1 + s2 + s3;
+    for (int c = lane; c < half; c += 64) {
+        int p = pos ? pos[0] : pos0 + row;
+        if (pos && sect > 0) {
+            const int s = c % sect;
+            if (s < s0)
+                p = pos[0];
+            else if (s < s0 + s1)
+                p = pos[1];
+            else if (s < s0 + s1 + s2)
+                p = pos[2];
+            else
+                p = pos[3];
+        }
+        float cs, sn;
+        rope_cs(tab, tab_rows, half, c, p, n_rot, theta, cs, sn);
+        const float x1 = buf[wave][c];
+        const float x2 = buf[wave][c + half];
+        dst[c] = x1 * cs - x2 * sn;
+        dst[c + half] = x1 * sn + x2 * cs;
+    }
+    for (int d = n_rot + lane; d < kHeadDim; d += 64)
+        dst[d] = buf[wave][d];
+}
+
+int launch_front(hipStream_t st, const float *qg, float *q, float *gate, float *k, const float *qw,
+                 const float *kw, int n_heads, int n_kv, int n_rot, int s0, int s1, int s2, int s3,
+                 const int32_t *pos, int pos0, int rows, float theta, float eps, const RopeTable &tab)
+{
+    int tab_rows = 0;
+    const float *t = table_for(tab, theta, n_rot, &tab_rows);
+    const int per_row = n_heads + n_kv;
+    const int max_rows = 1 << 22; // keeps (rows * per_row) far inside int
+    for (int r0 = 0; r0 < rows; r0 += max_rows) {
+        const int n = rows - r0 < max_rows ? rows - r0 : max_rows;
+        const unsigned grid = (unsigned)(((long long)per_row * n + 3) / 4);
+        hipLaunchKernelGGL(front_kernel, dim3(grid, 1, 1), dim3(256, 1, 1), 0, st,
+                           qg + (size_t)r0 * n_heads * 2 * kHeadDim, q + (size_t)r0 * n_heads * kHeadDim,
+                           gate + (size_t)r0 * n_heads * kHeadDim, k + (size_t)r0 * n_kv * kHeadDim, qw, kw,
+                           n_heads, n_kv, n_rot, s0, s1, s2, s3, pos, pos0 + r0, n, theta, eps, t, tab_rows);
+        int rc = launched("attn_front_f32");
+        if (rc)
+            return rc;
+    }
+    return 0;
+}
+
 // ---- sigmoid output gate ----------------------------------------------------------
 //
 // y = x * (1 / (1 + exp(-g))) (crates/hipml-core/src/ops.rs:354-360).  Four

@@ -101,6 +101,33 @@ int hipml_mrope_rows_f32(hipml_stream_t stream, const float *x, float *y, int n_
 int hipml_rope_chunk_f32(hipml_stream_t stream, float *q, float *k, int n_head, int n_kv,
                          int head_dim, int n_rot, float theta_base, int pos0, int tokens);
 
+/* ---- attention front end ----------------------------------------------------- */
+
+/* One token: split the joint projection qg [n_heads][2*head_dim] into q and gate
+ * [n_heads][head_dim], RMS-normalise every q head and (in place) every k head
+ * [n_kv][head_dim] with the shared weight rows q_norm / k_norm [head_dim], then
+ * M-RoPE both with the four position ids at `pos` (device int32[4]).  Bit-identical
+ * to the reference's kernel: squares folded by its 256-wide halving tree,
+ * scale = 1/sqrtf(mean + eps), (x*scale)*w, f64 angles.  head_dim must be 256.
+ * Replaces AttnLayer::front -> attn_front_f32 (= qg_split_f32 + head_rmsnorm_f32 x2
+ * + mrope_f32 x2), crates/hipml-kernels/src/attn_gpu.rs:549-609,
+ * crates/hipml-kernels/kernels/attn_front_f32.hip:34-135. */
+int hipml_attn_front_f32(hipml_stream_t stream, const float *qg, float *q, float *gate, float *k,
+                         const float *q_norm, const float *k_norm, int n_heads, int n_kv,
+                         int head_dim, int n_rot, int s0, int s1, int s2, int s3,
+                         const int32_t *pos, float theta_base, float eps);
+
+/* The same over a chunk of `tokens` rows (qg [tokens][n_heads][2*head_dim], k
+ * [tokens][n_kv][head_dim] in place); row t rotates at text position pos0 + t.
+ * Argument order of the reference's launcher.  Replaces AttnLayer::chunk_front ->
+ * qg_split_chunk_f32 + norm_rope_chunk_f32,
+ * crates/hipml-kernels/src/attn_gpu/imp/attn_chunk.rs:129-205,
+ * crates/hipml-kernels/kernels/attn_chunk_f32.hip:22-98. */
+int hipml_attn_chunk_front_f32(hipml_stream_t stream, const float *qg, float *k, float *q,
+                               float *gate, const float *q_norm, const float *k_norm, int n_heads,
+                               int n_kv, int head_dim, int n_rot, float theta_base, float eps,
+                               int pos0, int tokens);
+
 /* ---- q8_0 KV append ------------------------------------------------------- */
 
 /* One token: quantize k_in/v_in [n_kv][head_dim] into row step[0] of the cache.

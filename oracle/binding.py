@@ -71,6 +71,10 @@ def _declare(l: C.CDLL) -> None:
         "orc_rope_neox_f32": (None, [_f32p, _f32p, sz, sz, sz, f32]),
         "orc_rope_multi_f32": (None, [_f32p, _f32p, sz, sz, sz, _szp, _szp, f32]),
         "orc_q_gate_f32": (None, [_f32p, _f32p, _f32p, sz]),
+        "orc_rmsnorm_f32": (None, [_f32p, _f32p, _f32p, sz, f32]),
+        "orc_head_rmsnorm_f32": (None, [_f32p, _f32p, _f32p, sz, sz, f32]),
+        "orc_rmsnorm_tree_f32": (None, [_f32p, _f32p, _f32p, sz, f32]),
+        "orc_qg_split_f32": (None, [_f32p, _f32p, _f32p, sz, sz]),
         "orc_kv_append_f32": (None, [_f32p, _f32p, _f32p, _f32p, sz, sz]),
         "orc_attn_causal_f32": (None, [_f32p, _f32p, _f32p, sz, sz, sz, sz, f32, _f32p]),
         "orc_attn_decode_f32": (None, [_f32p, _f32p, _f32p, sz, sz, sz, sz, f32, _f32p]),
@@ -200,6 +204,49 @@ def q_gate(q, gate) -> np.ndarray:
     out = np.empty_like(q)
     lib().orc_q_gate_f32(_pf(q), _pf(gate), _pf(out), q.size)
     return out
+
+
+def rmsnorm(x, w, eps) -> np.ndarray:
+    x, w = _f(x), _f(w)
+    y = np.empty_like(x)
+    lib().orc_rmsnorm_f32(_pf(x), _pf(w), _pf(y), x.size, eps)
+    return y
+
+
+def head_rmsnorm(x, w, n_heads, head_dim, eps, tree=False) -> np.ndarray:
+    """Per-head RMS norm; `tree` sums the squares in the order of the reference's GPU kernels."""
+    x, w = _f(x), _f(w)
+    y = np.empty_like(x)
+    if not tree:
+        lib().orc_head_rmsnorm_f32(_pf(x), _pf(w), _pf(y), n_heads, head_dim, eps)
+        return y
+    xr, yr = x.reshape(n_heads, head_dim), y.reshape(n_heads, head_dim)
+    for h in range(n_heads):
+        row = np.ascontiguousarray(xr[h])
+        out = np.empty_like(row)
+        lib().orc_rmsnorm_tree_f32(_pf(row), _pf(w), _pf(out), head_dim, eps)
+        yr[h] = out
+    return y
+
+
+def qg_split(qg, n_heads, head_dim):
+    qg = _f(qg)
+    q = np.empty(n_heads * head_dim, dtype=np.float32)
+    gate = np.empty(n_heads * head_dim, dtype=np.float32)
+    lib().orc_qg_split_f32(_pf(qg), _pf(q), _pf(gate), n_heads, head_dim)
+    return q, gate
+
+
+def attn_front(qg, k, q_norm, k_norm, n_heads, n_kv, head_dim, n_rot, sections, pos, theta, eps,
+               tree=True):
+    """q|gate split, per-head RMS norm of q and k, M-RoPE of both: the reference's decode front
+    end (attn_front_f32.hip:34-135 = qg_split + head_rmsnorm x2 + mrope x2).  Returns q, gate, k."""
+    q, gate = qg_split(qg, n_heads, head_dim)
+    q = head_rmsnorm(q, q_norm, n_heads, head_dim, eps, tree)
+    kk = head_rmsnorm(k, k_norm, n_kv, head_dim, eps, tree)
+    q = rope_multi(q, n_heads, head_dim, n_rot, sections, pos, theta)
+    kk = rope_multi(kk, n_kv, head_dim, n_rot, sections, pos, theta)
+    return q.ravel(), gate.ravel(), kk.ravel()
 
 
 def rope_neox(x, n_heads, head_dim, pos, theta) -> np.ndarray:

@@ -261,6 +261,56 @@ void orc_q_gate_f32(const float *q, const float *gate, float *y, size_t n)
         y[i] = q[i] * (1.0f / (1.0f + expf(-gate[i])));
 }
 
+/* ---- attention front end: ops.rs:178-187, 315-349 ------------------------------ */
+
+/* ops.rs:181-187: mean of squares summed in index order (Rust's f32 `sum()` is a left fold),
+ * scale = 1/sqrt(mean + eps), then the two multiplies x*scale*w left to right. */
+void orc_rmsnorm_f32(const float *x, const float *w, float *y, size_t n, float eps)
+{
+    float sum = 0.0f;
+    for (size_t i = 0; i < n; i++)
+        sum += x[i] * x[i];
+    float mean_sq = sum / (float)n;
+    float scale = 1.0f / sqrtf(mean_sq + eps);
+    for (size_t i = 0; i < n; i++)
+        y[i] = x[i] * scale * w[i];
+}
+
+/* ops.rs:337-349: every head row normalised with the shared weight row. */
+void orc_head_rmsnorm_f32(const float *x, const float *w, float *y, size_t n_heads, size_t head_dim,
+                          float eps)
+{
+    for (size_t h = 0; h < n_heads; h++)
+        orc_rmsnorm_f32(x + h * head_dim, w, y + h * head_dim, head_dim, eps);
+}
+
+/* The summation order of the reference's GPU kernels (attn_front_f32.hip:79-103,
+ * attn_chunk_f32.hip:68-81) at head_dim == block size: thread t holds x[t]^2 (its fma chain has
+ * one link), then the shared-memory tree red[t] += red[t + off] for off = n/2 .. 1.  n must be a
+ * power of two <= 256.  Everything else as orc_rmsnorm_f32. */
+void orc_rmsnorm_tree_f32(const float *x, const float *w, float *y, size_t n, float eps)
+{
+    float red[256];
+    for (size_t i = 0; i < n; i++)
+        red[i] = x[i] * x[i];
+    for (size_t off = n / 2; off > 0; off >>= 1)
+        for (size_t t = 0; t < off; t++)
+            red[t] += red[t + off];
+    float mean_sq = red[0] / (float)n;
+    float scale = 1.0f / sqrtf(mean_sq + eps);
+    for (size_t i = 0; i < n; i++)
+        y[i] = x[i] * scale * w[i];
+}
+
+/* ops.rs:315-330: joint projection [n_heads][2*head_dim] -> q [n_heads][head_dim], gate likewise. */
+void orc_qg_split_f32(const float *qg, float *q, float *gate, size_t n_heads, size_t head_dim)
+{
+    for (size_t h = 0; h < n_heads; h++) {
+        memcpy(q + h * head_dim, qg + h * 2 * head_dim, head_dim * sizeof(float));
+        memcpy(gate + h * head_dim, qg + h * 2 * head_dim + head_dim, head_dim * sizeof(float));
+    }
+}
+
 /* ---- RoPE: ops.rs:195-224, 260-309 --------------------------------------- */
 
 static void rotate_pair(const float *x, float *y, size_t lo, size_t hi, size_t p, double freq)

@@ -64,6 +64,14 @@ void orc_rope_multi_f32(const float *x, float *y, size_t n_heads, size_t head_di
                         float theta_base);
 /* ops.rs:354-360 */
 void orc_q_gate_f32(const float *q, const float *gate, float *y, size_t n);
+
+/* attention front end (ops.rs:178-187, 315-349); `_tree` sums the squares in the order of the
+ * reference's GPU kernels (one square per thread, shared-memory halving tree) */
+void orc_rmsnorm_f32(const float *x, const float *w, float *y, size_t n, float eps);
+void orc_head_rmsnorm_f32(const float *x, const float *w, float *y, size_t n_heads, size_t head_dim,
+                          float eps);
+void orc_rmsnorm_tree_f32(const float *x, const float *w, float *y, size_t n, float eps);
+void orc_qg_split_f32(const float *qg, float *q, float *gate, size_t n_heads, size_t head_dim);
 /* ops.rs:366-386 (in place on the two caches) */
 void orc_kv_append_f32(float *k_cache, float *v_cache, const float *k, const float *v,
                        size_t off, size_t width);

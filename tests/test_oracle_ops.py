@@ -284,3 +284,77 @@ def test_compare_is_abs_or_rel(orc):
     assert ok
     ok, _, _ = orc.compare([1e-9], [5e-5], 1e-4, 1e-3)  # rel fails, abs passes
     assert ok
+
+
+# ---- attention front end: rmsnorm, q|gate split -----------------------------
+
+def test_rmsnorm_unit_rms_and_elementwise_gain(orc):
+    # parity_reference.rs:64-85 (n = 513 on purpose, Rng seed 7, normal * 4)
+    n = 513
+    x = orc.Rng(7).normal_array((n,), 4.0)
+    y = orc.rmsnorm(x, np.ones(n, dtype=np.float32), 1e-6)
+    rms = math.sqrt(float(np.mean(y.astype(np.float64) ** 2)))
+    assert abs(rms - 1.0) < 1e-3
+    gain = np.array([(i % 5) + 0.5 for i in range(n)], dtype=np.float32)
+    scaled = orc.rmsnorm(x, gain, 1e-6)
+    assert np.all(np.abs(scaled - y * gain) < 1e-5)
+
+
+def test_rmsnorm_closed_forms(orc):
+    # constant row c, weight w: y = c / sqrt(c^2 + eps) * w; zero row stays zero
+    n, c, eps = 256, np.float32(3.0), np.float32(1e-6)
+    w = np.linspace(0.5, 2.0, n).astype(np.float32)
+    y = orc.rmsnorm(np.full(n, c, dtype=np.float32), w, float(eps))
+    want = (np.float64(c) / np.sqrt(np.float64(c) ** 2 + np.float64(eps))) * w.astype(np.float64)
+    assert np.allclose(y, want, rtol=3e-7, atol=0)
+    assert np.all(orc.rmsnorm(np.zeros(n, dtype=np.float32), w, 1e-6) == 0.0)
+    # float64 definition on random rows, and a sign/eps mistake would show: eps matters at tiny rows
+    x = orc.Rng(99).normal_array((n,), 1e-3)
+    y = orc.rmsnorm(x, w, 1e-6)
+    x64 = x.astype(np.float64)
+    want = x64 / np.sqrt(np.mean(x64 * x64) + 1e-6) * w
+    assert np.allclose(y, want, rtol=2e-6, atol=0)
+    assert not np.allclose(y, x64 / np.sqrt(np.mean(x64 * x64)) * w, rtol=1e-3, atol=0)
+
+
+def test_rmsnorm_tree_order_is_the_same_function(orc):
+    # the GPU summation order differs from the index-order sum only in rounding; with squares that
+    # sum exactly (small integers) the two are bit-identical, and a power-of-two case has a
+    # closed form: x = 1..256 -> sum of squares 5,625,216 exactly
+    n = 256
+    w = np.ones(n, dtype=np.float32)
+    x = np.arange(1, n + 1, dtype=np.float32)
+    a = orc.head_rmsnorm(x, w, 1, n, 0.0)
+    b = orc.head_rmsnorm(x, w, 1, n, 0.0, tree=True)
+    assert np.array_equal(a, b)
+    scale = np.float32(1.0) / np.sqrt(np.float32(5625216.0) / np.float32(256.0))
+    assert np.array_equal(a, x * scale)
+    # random rows: same value to rounding, and per-head independence
+    r = orc.Rng(5)
+    x = r.normal_array((3 * n,))
+    w = r.normal_array((n,))
+    a = orc.head_rmsnorm(x, w, 3, n, 1e-6)
+    b = orc.head_rmsnorm(x, w, 3, n, 1e-6, tree=True)
+    assert np.allclose(a, b, rtol=1e-6, atol=0)
+    assert np.array_equal(a[n:2 * n], orc.rmsnorm(x[n:2 * n], w, 1e-6))
+    # the tree pairs (t, t + 128) first: a row whose only rounding sits in that pairing tells the
+    # orders apart (1 + 2^-24 twice: index order loses both, the tree adds them together first)
+    x = np.zeros(n, dtype=np.float32)
+    x[0] = 1.0
+    x[1] = x[129] = np.float32(2.0 ** -12)      # squares 2^-24 each
+    ones = np.ones(n, dtype=np.float32)
+    seq = orc.head_rmsnorm(x, ones, 1, n, 0.0)[0]
+    tree = orc.head_rmsnorm(x, ones, 1, n, 0.0, tree=True)[0]
+    s_seq = np.float32(1.0)                       # (1 + 2^-24) rounds to 1, twice
+    s_tree = np.float32(1.0) + np.float32(2.0 ** -23)   # 2^-24 + 2^-24 joined before meeting 1
+    assert seq == np.float32(1.0) / np.sqrt(s_seq / np.float32(n))
+    assert tree == np.float32(1.0) / np.sqrt(s_tree / np.float32(n))
+
+
+def test_qg_split_layout(orc):
+    # ops.rs:315-330: head h of the joint row is [q_h | gate_h]
+    nh, hd = 3, 4
+    qg = np.arange(nh * 2 * hd, dtype=np.float32)
+    q, g = orc.qg_split(qg, nh, hd)
+    assert np.array_equal(q, [0, 1, 2, 3, 8, 9, 10, 11, 16, 17, 18, 19])
+    assert np.array_equal(g, [4, 5, 6, 7, 12, 13, 14, 15, 20, 21, 22, 23])
