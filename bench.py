@@ -84,15 +84,15 @@ class Timer:
         self.ms = self.a.elapsed_time(self.b)
 
 
-def fill_cache_normal(torch, attn, k_cache, v_cache, stride, rows, gen):
-    """Quantize N(0,1) rows into a [KV][stride][272] cache pair with the library's own
-    append kernel, in slabs so the f32 source stays small."""
+def fill_cache_normal(torch, attn, k_cache, v_cache, stride, rows, gen, dtype=0):
+    """Quantize N(0,1) rows into a [KV][stride][272] (q8_0) or [..][144] (q4_0, dtype 1) cache pair
+    with the library's own append kernel, in slabs so the f32 source stays small."""
     slab = 8192
     for s0 in range(0, rows, slab):
         n = min(slab, rows - s0)
         kf = torch.randn((n, KV, HD), device="cuda", dtype=torch.float32, generator=gen)
         vf = torch.randn((n, KV, HD), device="cuda", dtype=torch.float32, generator=gen)
-        attn.kv_encode_bulk(0, kf, vf, k_cache, v_cache, KV, HD, stride, s0, 0, n)
+        attn.kv_encode_bulk(dtype, kf, vf, k_cache, v_cache, KV, HD, stride, s0, 0, n)
     torch.cuda.synchronize()
 
 
@@ -187,15 +187,16 @@ def bench_prefill(torch, attn, tokens, pos0, steps, warmup, layers, prefix_fill=
 # decode
 # ---------------------------------------------------------------------------------------
 
-def bench_decode(torch, attn, seq, steps, warmup, layers):
+def bench_decode(torch, attn, seq, steps, warmup, layers, dtype=0):
+    row = ROW if dtype == 0 else 144
     stride = seq
     gen = torch.Generator(device="cuda")
     gen.manual_seed(0x5EED0003 + seq)
     caches = []
     for _ in range(layers):
-        k = torch.empty((KV, stride, ROW), dtype=torch.uint8, device="cuda")
-        v = torch.empty((KV, stride, ROW), dtype=torch.uint8, device="cuda")
-        fill_cache_normal(torch, attn, k, v, stride, seq, gen)
+        k = torch.empty((KV, stride, row), dtype=torch.uint8, device="cuda")
+        v = torch.empty((KV, stride, row), dtype=torch.uint8, device="cuda")
+        fill_cache_normal(torch, attn, k, v, stride, seq, gen, dtype)
         caches.append((k, v))
     q = torch.randn((H, HD), device="cuda", generator=gen)
     out = torch.empty((H, HD), device="cuda")
@@ -207,7 +208,7 @@ def bench_decode(torch, attn, seq, steps, warmup, layers):
 
     def one_pass():
         for k, v in caches:
-            attn.attn_decode_kv(stepbuf, 0, q, k, v, acc, ml, out, H, KV, HD, stride, SCALE, splits)
+            attn.attn_decode_kv(stepbuf, dtype, q, k, v, acc, ml, out, H, KV, HD, stride, SCALE, splits)
 
     for _ in range(warmup):
         one_pass()
@@ -215,12 +216,13 @@ def bench_decode(torch, attn, seq, steps, warmup, layers):
         for _ in range(steps):
             one_pass()
     us = t.ms * 1e3 / (steps * layers)
-    nbytes = decode_bytes(seq)
+    nbytes = decode_bytes(seq) * row // ROW
     gbs = nbytes / (us * 1e-6) / 1e9
-    traffic = measured_traffic({8192: "decode8k", 32768: "decode32k"}.get(seq, ""),
+    traffic = measured_traffic({8192: "decode8k", 32768: "decode32k"}.get(seq, "") if dtype == 0 else "",
                                ["decode_q8_kernel", "decode_reduce_kernel"])
     return {
-        "workload": f"decode 1 query @ depth {seq}, q8_0 cache, split-K {splits} + merge",
+        "workload": f"decode 1 query @ depth {seq}, {'q8_0' if dtype == 0 else 'q4_0'} cache, "
+                    f"split-K {splits} + merge",
         "seq": seq, "splits": splits, "layers_rotated": layers,
         "us_per_layer": us,
         "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
@@ -406,6 +408,7 @@ def main() -> int:
             "batch16": lambda: bench_batch(torch, attn, orc, K, W, 4),
             "copycal": lambda: bench_copycal(torch, K),
             "front672": lambda: bench_front(torch, attn, 672, max(K, 20)),
+            "decode32k_q4": lambda: bench_decode(torch, attn, 32768, max(K, 20), 3, LAYERS, 1),
         }[args.only]
         print(json.dumps(fn()))
         return 0
@@ -443,6 +446,7 @@ def main() -> int:
                                                      max(K // 20, 3), 1, 2)
         torch.cuda.empty_cache()
         also["front_672"] = bench_front(torch, attn, 672, d_steps)
+        also["decode_32768_q4_0"] = bench_decode(torch, attn, 32768, d_steps, max(W // 4, 2), LAYERS, 1)
         from oracle import binding as orc  # only for the seeded depth recipe and the CPU leg
         also["batch16_mtp"] = bench_batch(torch, attn, orc, d_steps, max(W // 4, 2), 4)
         torch.cuda.empty_cache()

@@ -49,13 +49,30 @@ int check_heads(int n_heads, int n_kv, int head_dim)
     return 0;
 }
 
-static int check_q8(int dtype)
+// KV dtype ids of the reference's KvDtype::id (crates/hipml-core/src/kv.rs:47-91): 0 = q8_0, 1 = q4_0.
+static int check_kv_dtype(int dtype)
 {
-    if (dtype == 0)
+    if (dtype == 0 || dtype == 1)
         return 0;
-    if (dtype == 1)
-        return fail(HIPML_ATTN_E_UNSUPPORTED, "KV dtype 1 (q4_0) is not built; only q8_0 (0)");
-    return fail(HIPML_ATTN_E_UNSUPPORTED, "unknown KV dtype %d", dtype);
+    return fail(HIPML_ATTN_E_UNSUPPORTED, "unknown KV dtype %d (0 = q8_0, 1 = q4_0)", dtype);
+}
+
+// Decode launchers: the reference's selector also names kernel variants
+// (crates/hipml-kernels/src/launch_kv.rs:146-170,329-334): 0 and 4 are its staged and warp q8_0
+// kernels, 1 and 5 the q4_0 ones.  There is one kernel per format here, so the selector only
+// picks the format; its other values (A/B variants of the reference's kernels) are refused.
+static int decode_format(int dtype, int *kv_dtype)
+{
+    if (dtype == 0 || dtype == 4) {
+        *kv_dtype = 0;
+        return 0;
+    }
+    if (dtype == 1 || dtype == 5) {
+        *kv_dtype = 1;
+        return 0;
+    }
+    return fail(HIPML_ATTN_E_UNSUPPORTED,
+                "KV dtype selector %d: 0/4 (q8_0) and 1/5 (q4_0) are built", dtype);
 }
 
 static int check_aligned16(const void *p, const char *name)
@@ -71,7 +88,7 @@ static int check_aligned16(const void *p, const char *name)
             return fail(HIPML_ATTN_E_NULL, "%s is NULL", #p);                                        \
     } while (0)
 
-static int decode_common(hipStream_t st, const int32_t *pos, const float *q, const void *k,
+static int decode_common(hipStream_t st, int dtype, const int32_t *pos, const float *q, const void *k,
                          const void *v, float *part_acc, float *part_ml, float *out, int n_heads,
                          int n_kv, int head_dim, int stride, float scale, int splits,
                          size_t kv_slot_bytes, size_t acc_slot, size_t ml_slot, size_t q_slot,
@@ -113,6 +130,7 @@ static int decode_common(hipStream_t st, const int32_t *pos, const float *q, con
     L.stride = stride;
     L.splits = splits;
     L.slots = slots;
+    L.q4 = dtype == 1 ? 1 : 0;
     L.scale = scale;
     L.kv_slot_bytes = kv_slot_bytes;
     L.acc_slot = acc_slot;
@@ -396,7 +414,7 @@ int hipml_attn_chunk_front_f32(hipml_stream_t stream, const float *qg, float *k,
 static int check_encode(int dtype, const void *k, const void *v, const void *kc, const void *vc,
                         int n_kv, int head_dim, int stride)
 {
-    int rc = check_q8(dtype);
+    int rc = check_kv_dtype(dtype);
     if (rc)
         return rc;
     if (k == nullptr || v == nullptr || kc == nullptr || vc == nullptr)
@@ -419,7 +437,7 @@ int hipml_kv_encode(hipml_stream_t stream, const int32_t *step, int dtype, const
     int rc = check_encode(dtype, k_in, v_in, k_cache, v_cache, n_kv, head_dim, stride);
     if (rc)
         return rc;
-    return launch_kv_encode_q8(as_stream(stream), k_in, v_in, static_cast<uint8_t *>(k_cache),
+    return launch_kv_encode(as_stream(stream), dtype, k_in, v_in, static_cast<uint8_t *>(k_cache),
                                static_cast<uint8_t *>(v_cache), n_kv, head_dim, stride, step, 0, 0,
                                1, 0, 0, 1);
 }
@@ -438,7 +456,7 @@ int hipml_kv_encode_bulk(hipml_stream_t stream, int dtype, const float *k_f32, c
     if ((long long)start + rows > stride)
         return fail(HIPML_ATTN_E_RANGE, "rows [%d, %d) do not fit a cache of %d rows per head",
                     start, start + rows, stride);
-    return launch_kv_encode_q8(as_stream(stream), k_f32, v_f32, static_cast<uint8_t *>(k_cache),
+    return launch_kv_encode(as_stream(stream), dtype, k_f32, v_f32, static_cast<uint8_t *>(k_cache),
                                static_cast<uint8_t *>(v_cache), n_kv, head_dim, stride, nullptr, 0,
                                0, rows, start, src0, rows);
 }
@@ -454,7 +472,7 @@ int hipml_kv_encode_rows(hipml_stream_t stream, int dtype, const float *k_f32, c
         return rc;
     if (slots < 0)
         return fail(HIPML_ATTN_E_RANGE, "slots %d is negative", slots);
-    return launch_kv_encode_q8(as_stream(stream), k_f32, v_f32, static_cast<uint8_t *>(k_cache),
+    return launch_kv_encode(as_stream(stream), dtype, k_f32, v_f32, static_cast<uint8_t *>(k_cache),
                                static_cast<uint8_t *>(v_cache), n_kv, head_dim, stride, pos, 2,
                                slot_bytes, slots, 0, 0, slots);
 }
@@ -467,13 +485,14 @@ int hipml_attn_decode_kv(hipml_stream_t stream, const int32_t *step, int dtype, 
                          int splits, size_t k_off, size_t v_off)
 {
     clear_error();
-    int rc = check_q8(dtype);
+    int fmt = 0;
+    int rc = decode_format(dtype, &fmt);
     if (rc)
         return rc;
     REQUIRE_PTR(k);
     REQUIRE_PTR(v);
     const size_t slice = (size_t)(n_heads > 0 ? n_heads : 0) * (size_t)(splits > 0 ? splits : 0);
-    return decode_common(as_stream(stream), step, q, static_cast<const uint8_t *>(k) + k_off,
+    return decode_common(as_stream(stream), fmt, step, q, static_cast<const uint8_t *>(k) + k_off,
                          static_cast<const uint8_t *>(v) + v_off, part_acc, part_ml, out, n_heads,
                          n_kv, head_dim, stride, scale, splits, 0, slice * kHeadDim, slice * 2,
                          (size_t)n_heads * kHeadDim, 1, nullptr);
@@ -486,16 +505,14 @@ int hipml_attn_decode_kv_cols(hipml_stream_t stream, int dtype, const int32_t *p
                               size_t ml_slot, size_t q_slot)
 {
     clear_error();
-    // the reference's selector for its whole-group warp kernel is 4; 0 (q8_0) is accepted too
-    if (dtype != 4) {
-        int rc = check_q8(dtype);
-        if (rc)
-            return rc;
-    }
+    int fmt = 0;
+    int rc = decode_format(dtype, &fmt);
+    if (rc)
+        return rc;
     if (cols < 1 || cols > kMaxCols)
         return fail(HIPML_ATTN_E_RANGE, "cols %d outside 1..%d", cols, kMaxCols);
     const int32_t one_slot[1] = {cols};
-    return decode_common(as_stream(stream), pos, q, k, v, part_acc, part_ml, out, n_heads, n_kv,
+    return decode_common(as_stream(stream), fmt, pos, q, k, v, part_acc, part_ml, out, n_heads, n_kv,
                          head_dim, stride, scale, splits, 0, acc_slot, ml_slot, q_slot, 1,
                          one_slot);
 }
@@ -507,7 +524,8 @@ int hipml_attn_decode_rows(hipml_stream_t stream, int dtype, const int32_t *pos,
                            size_t acc_slot, size_t ml_slot, size_t q_slot, int slots)
 {
     clear_error();
-    int rc = check_q8(dtype);
+    int fmt = 0;
+    int rc = decode_format(dtype, &fmt);
     if (rc)
         return rc;
     if (slots < 1 || slots > kMaxSlots)
@@ -515,11 +533,11 @@ int hipml_attn_decode_rows(hipml_stream_t stream, int dtype, const int32_t *pos,
     if (kv_slot_bytes == 0 && slots <= kMaxCols && slots > 1) {
         // rows of one sequence sharing a cache: stream it once for all of them
         const int32_t one_slot[1] = {slots};
-        return decode_common(as_stream(stream), pos, q, k_cache, v_cache, part_acc, part_ml, out,
+        return decode_common(as_stream(stream), fmt, pos, q, k_cache, v_cache, part_acc, part_ml, out,
                              n_heads, n_kv, head_dim, stride, scale, splits, 0, acc_slot, ml_slot,
                              q_slot, 1, one_slot);
     }
-    return decode_common(as_stream(stream), pos, q, k_cache, v_cache, part_acc, part_ml, out,
+    return decode_common(as_stream(stream), fmt, pos, q, k_cache, v_cache, part_acc, part_ml, out,
                          n_heads, n_kv, head_dim, stride, scale, splits, kv_slot_bytes, acc_slot,
                          ml_slot, q_slot, slots, nullptr);
 }
@@ -547,11 +565,12 @@ int hipml_attn_decode_batch_cols(hipml_stream_t stream, int dtype, const int32_t
                                  size_t q_slot, int slots, const int32_t *cols_per_slot_host)
 {
     clear_error();
-    int rc = check_q8(dtype);
+    int fmt = 0;
+    int rc = decode_format(dtype, &fmt);
     if (rc)
         return rc;
     REQUIRE_PTR(cols_per_slot_host);
-    return decode_common(as_stream(stream), pos, q, k_cache, v_cache, part_acc, part_ml, out,
+    return decode_common(as_stream(stream), fmt, pos, q, k_cache, v_cache, part_acc, part_ml, out,
                          n_heads, n_kv, head_dim, stride, scale, splits, kv_slot_bytes, acc_slot,
                          ml_slot, q_slot, slots, cols_per_slot_host);
 }
@@ -570,9 +589,11 @@ static int chunk_q8_common(hipml_stream_t stream, const float *q, const void *kc
     REQUIRE_PTR(out);
     if (want_gate)
         REQUIRE_PTR(gate);
-    if (dtype != 1)
+    // the reference's chunk launcher numbers the formats 1 = q8_0, 2 = q4_0
+    // (crates/hipml-kernels/src/attn_gpu/imp/attn_chunk_kv.rs:41-60)
+    if (dtype != 1 && dtype != 2)
         return fail(HIPML_ATTN_E_UNSUPPORTED,
-                    "quantized chunk attention: only a q8_0 cache (dtype 1) is built, got %d", dtype);
+                    "quantized chunk attention: dtype 1 (q8_0) or 2 (q4_0), got %d", dtype);
     int rc = check_heads(n_head, n_kv, head_dim);
     if (rc)
         return rc;
@@ -596,7 +617,7 @@ static int chunk_q8_common(hipml_stream_t stream, const float *q, const void *kc
         return 0;
     return launch_chunk_q8(as_stream(stream), q, static_cast<const uint8_t *>(kc),
                            static_cast<const uint8_t *>(vc), out, n_head, n_kv, pos0, tokens,
-                           stride, part_acc, part_ml, splits, want_gate ? gate : nullptr);
+                           stride, part_acc, part_ml, splits, want_gate ? gate : nullptr, dtype == 2 ? 1 : 0);
 }
 
 int hipml_attn_chunk_q8_split(hipml_stream_t stream, const float *q, const void *kc,

@@ -11,8 +11,10 @@ namespace hipml {
 
 constexpr int kBlock = 32;        // values per quantization block
 constexpr int kQ8BlockBytes = 34; // f16 scale + 32 int8
+constexpr int kQ4BlockBytes = 18; // f16 scale + 16 bytes of nibble pairs (j, j + 16)
 constexpr int kHeadDim = 256;     // the width the MFMA kernels are built for
 constexpr int kRowBytes = kHeadDim / kBlock * kQ8BlockBytes; // 272
+constexpr int kRowBytesQ4 = kHeadDim / kBlock * kQ4BlockBytes; // 144
 constexpr int kMaxCols = 4;       // query rows of one sequence per launch (MTP verify)
 constexpr int kMaxSlots = 128;    // slots per batched launch
 constexpr int kMaxGroup = 8;      // query heads per KV head
@@ -43,9 +45,9 @@ int launch_mrope(hipStream_t st, const float *x, float *y, int n_heads, int head
                  float theta, const RopeTable &tab);
 int launch_rope_chunk(hipStream_t st, float *q, float *k, int n_head, int n_kv, int head_dim,
                       int n_rot, float theta, int pos0, int tokens, const RopeTable &tab);
-int launch_kv_encode_q8(hipStream_t st, const float *k, const float *v, uint8_t *kc, uint8_t *vc,
-                        int n_kv, int head_dim, int stride, const int32_t *pos, int pos_stride,
-                        size_t slot_bytes, int slots, int start, int src0, int rows);
+int launch_kv_encode(hipStream_t st, int q4, const float *k, const float *v, uint8_t *kc, uint8_t *vc,
+                     int n_kv, int head_dim, int stride, const int32_t *pos, int pos_stride,
+                     size_t slot_bytes, int slots, int start, int src0, int rows);
 int launch_front(hipStream_t st, const float *qg, float *q, float *gate, float *k, const float *qw,
                  const float *kw, int n_heads, int n_kv, int n_rot, int s0, int s1, int s2, int s3,
                  const int32_t *pos, int pos0, int rows, float theta, float eps, const RopeTable &tab);
@@ -60,6 +62,7 @@ struct DecodeLaunch {
     float *out;
     const int32_t *pos; // (pos, seq) pairs, one per row
     int n_heads, n_kv, stride, splits, slots;
+    int q4; // cache format: 0 = q8_0, 1 = q4_0
     float scale;
     size_t kv_slot_bytes, acc_slot, ml_slot, q_slot;
     uint16_t row0[kMaxSlots]; // first row of each slot
@@ -75,6 +78,6 @@ int decode_init();
 int prefill_init();
 int launch_chunk_q8(hipStream_t st, const float *q, const uint8_t *kc, const uint8_t *vc,
                     float *out, int n_head, int n_kv, int pos0, int tokens, int stride,
-                    float *part_acc, float *part_ml, int splits, const float *gate);
+                    float *part_acc, float *part_ml, int splits, const float *gate, int q4);
 
 } // namespace hipml

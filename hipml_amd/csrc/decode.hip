@@ -55,7 +55,6 @@ constexpr int kWaveLds = kTileBytes + 2 * kScaleBytes; // 10240
 #endif
 constexpr int kWaves = DECODE_WAVES;   // waves per workgroup
 constexpr int kThreads = 64 * kWaves;
-constexpr int kUnitBytes = 68;                        // two q8_0 blocks
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kTwo24 = 16777216.0f;
 
@@ -148,15 +147,57 @@ __device__ __forceinline__ void store_unit(const Unit &u, uint8_t *tile, uint8_t
     sc[kTileKeys] = (uint16_t)(u.m >> 16);
 }
 
+// q4_0: a unit is two 18-byte blocks of one key, 36 bytes at a dword boundary:
+// [s0 | 16 bytes | s1 | 16 bytes]; byte j of a block holds element j in its low and element j+16
+// in its high nibble (crates/hipml-core/src/kv.rs:201-218).
+struct Unit4 {
+    uint4v a;   // dwords 0..3: s0 and the first 14 bytes of the even block
+    uint32_t m; // dword 4:     last 2 bytes of the even block, s1
+    uint4v b;   // dwords 5..8: the odd block's 16 bytes (dword aligned)
+};
+
+__device__ __forceinline__ void load_unit(Unit4 &u, const uint8_t *p)
+{
+    u.a = *reinterpret_cast<const uint4a4 *>(p);
+    u.m = *reinterpret_cast<const uint32_t *>(p + 16);
+    u.b = *reinterpret_cast<const uint4a4 *>(p + 20);
+}
+
+// Nibbles widened to one byte per element (values 0..15), element order, so the tile has the
+// q8_0 tile's shape and everything after staging is shared; the offset to remove is 8, not 128.
+__device__ __forceinline__ void store_unit(const Unit4 &u, uint8_t *tile, uint8_t *scales, int r,
+                                           int pr)
+{
+    uint4v e0;
+    e0[0] = __builtin_amdgcn_alignbit(u.a[1], u.a[0], 16);
+    e0[1] = __builtin_amdgcn_alignbit(u.a[2], u.a[1], 16);
+    e0[2] = __builtin_amdgcn_alignbit(u.a[3], u.a[2], 16);
+    e0[3] = __builtin_amdgcn_alignbit(u.m, u.a[3], 16);
+    const uint4v mask = {0x0f0f0f0fu, 0x0f0f0f0fu, 0x0f0f0f0fu, 0x0f0f0f0fu};
+    uint4v *dst = reinterpret_cast<uint4v *>(tile + r * kLdsRow + pr * 64);
+    dst[0] = e0 & mask;
+    dst[1] = (e0 >> 4) & mask;
+    dst[2] = u.b & mask;
+    dst[3] = (u.b >> 4) & mask;
+    uint16_t *sc = reinterpret_cast<uint16_t *>(scales) + (2 * pr) * kTileKeys + r;
+    sc[0] = (uint16_t)(u.a[0] & 0xffffu);
+    sc[kTileKeys] = (uint16_t)(u.m >> 16);
+}
+
+template <bool Q4> struct UnitOf { typedef Unit type; };
+template <> struct UnitOf<true> { typedef Unit4 type; };
+
 // 8 int8 b -> 8 f16 holding (b + 128) * 2^-24 exactly (byte b^0x80 in the low byte of a
 // subnormal f16).  The +128 is taken out again on the B side: sum_k (u_k - 128) x_k =
 // sum_k u_k x_k - 128 sum_k x_k.  For the scores x = Q is fixed, so the second term is a table
 // the block's MFMA starts from; for PV it is a second MFMA whose A operand is the constant
 // -128 * 2^-24.
+// (q4_0 tiles already hold unsigned bytes 0..15: no sign flip, and the offset is 8.)
+template <bool Q4>
 __device__ __forceinline__ half8 bytes_to_f16_biased(int2v w)
 {
-    const uint32_t x0 = (uint32_t)w[0] ^ 0x80808080u;
-    const uint32_t x1 = (uint32_t)w[1] ^ 0x80808080u;
+    const uint32_t x0 = Q4 ? (uint32_t)w[0] : (uint32_t)w[0] ^ 0x80808080u;
+    const uint32_t x1 = Q4 ? (uint32_t)w[1] : (uint32_t)w[1] ^ 0x80808080u;
     uint4v r;
     r[0] = __builtin_amdgcn_perm(0u, x0, 0x0c010c00u);
     r[1] = __builtin_amdgcn_perm(0u, x0, 0x0c030c02u);
@@ -179,9 +220,13 @@ __device__ __forceinline__ float quad_rows(float v)
     return MAX ? fmaxf(a, b) : a + b;
 }
 
-template <int NT, int DEPTH>
+template <int NT, int DEPTH, bool Q4>
 __device__ __forceinline__ void decode_body(const DecodeArgs &a)
 {
+    typedef typename UnitOf<Q4>::type Unit;
+    constexpr int kRowBytes = Q4 ? hipml::kRowBytesQ4 : hipml::kRowBytes;
+    constexpr int kUnitBytes = Q4 ? 36 : 68;
+    constexpr float kOffset = Q4 ? 8.0f : 128.0f; // what a staged byte carries on top of the value
     extern __shared__ __attribute__((aligned(16))) uint8_t lds_all[];
     uint8_t *Qs = lds_all;                       // [NT][hi,lo][8 blocks][64 lanes] half8
     uint8_t *CBs = lds_all + NT * 16384;         // [NT][8 blocks][16 columns] float4 (one value x4)
@@ -297,7 +342,7 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
             for (int j = 0; j < 8; j++)
                 sum += (float)h[j] + (float)l[j];
         }
-        const float cb = -128.0f / kTwo24 * sum;
+        const float cb = -kOffset / kTwo24 * sum;
         *reinterpret_cast<float4v *>(CBs + ((nt * 8 + c) * 16 + n) * 16) = (float4v){cb, cb, cb, cb};
     }
     __syncthreads();
@@ -328,8 +373,9 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
     const int tr_r = lm >> 1;
     const int tr_key = (tr_r >> 2) * 16 + lg * 4 + (tr_r & 3);
     const uint8_t *vtr = tile_lds + tr_key * kLdsRow + (lm & 1) * 8;
-    const uint4v bias_bits = {0x80808080u, 0x80808080u, 0x80808080u, 0x80808080u};
-    const half8 Abias = __builtin_bit_cast(half8, bias_bits); // eight times -128 * 2^-24
+    constexpr uint32_t kBiasBits = Q4 ? 0x80088008u : 0x80808080u;
+    const uint4v bias_bits = {kBiasBits, kBiasBits, kBiasBits, kBiasBits};
+    const half8 Abias = __builtin_bit_cast(half8, bias_bits); // eight times -offset * 2^-24
 
     auto process = [&](Unit (&Ku)[2], Unit (&Vu)[2], int t) {
         const int key0 = lo + (wave + kWaves * t) * kTileKeys;
@@ -365,7 +411,7 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
             for (int ms = 0; ms < 2; ms++) {
                 const int2v raw = *reinterpret_cast<const int2v *>(
                     tile_lds + (ms * 16 + lm) * kLdsRow + c * 32 + lg * 8);
-                const half8 A = bytes_to_f16_biased(raw);
+                const half8 A = bytes_to_f16_biased<Q4>(raw);
                 const half4 sk = *reinterpret_cast<const half4 *>(
                     sK + (c * kTileKeys + ms * 16 + lg * 4) * 2);
 #pragma unroll
@@ -480,7 +526,7 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
             for (int hf = 0; hf < 2; hf++) {
                 const int2v raw = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
                     (int2v __attribute__((address_space(3))) *)(vtr + c * 32 + hf * 16));
-                const half8 A = bytes_to_f16_biased(raw);
+                const half8 A = bytes_to_f16_biased<Q4>(raw);
 #pragma unroll
                 for (int nt = 0; nt < NT; nt++) {
                     float4v o = O[nt][c * 2 + hf];
@@ -586,13 +632,13 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
 // NT = 1: every slot has at most 16 (row, head) columns.  NT = 2: some slot has more (MTP
 // verify, 3-4 rows x 6 heads); slots that fit one column tile still take the NT = 1 body, so a
 // mixed batch pays the wider tile only where it is needed.  LDS is sized for the launch's NT.
-template <int NT, int DEPTH>
+template <int NT, int DEPTH, bool Q4 = false>
 __global__ void __launch_bounds__(kThreads, DECODE_MIN_WAVES) decode_q8_kernel(const DecodeArgs a)
 {
     if (NT == 1 || a.cols[blockIdx.y] * a.group <= 16)
-        decode_body<1, DEPTH>(a);
+        decode_body<1, DEPTH, Q4>(a);
     else
-        decode_body<NT, DEPTH>(a);
+        decode_body<NT, DEPTH, Q4>(a);
 }
 
 // Wave-wide reductions without LDS: DPP inside a row of 16 lanes, then the two row-swap
@@ -726,6 +772,12 @@ int decode_init()
     if (e == hipSuccess)
         e = hipFuncSetAttribute(reinterpret_cast<const void *>(&decode_q8_kernel<2, kDepth>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, decode_lds_bytes(2));
+    if (e == hipSuccess)
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&decode_q8_kernel<1, kDepth, true>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, decode_lds_bytes(1));
+    if (e == hipSuccess)
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&decode_q8_kernel<2, kDepth, true>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, decode_lds_bytes(2));
     if (e != hipSuccess)
         return fail((int)e, "hipFuncSetAttribute(decode LDS) failed: %d (%s)", (int)e,
                     hipGetErrorString(e));
@@ -755,11 +807,17 @@ int launch_decode_q8(hipStream_t st, const DecodeLaunch &L)
         a.cols[s] = s < L.slots ? L.cols[s] : 0;
     }
     const dim3 grid((unsigned)(L.n_kv * L.splits), (unsigned)L.slots, 1);
-    if (L.max_cols * a.group <= 16)
+    const bool narrow = L.max_cols * a.group <= 16;
+    if (L.q4) {
+        if (narrow)
+            hipLaunchKernelGGL((decode_q8_kernel<1, kDepth, true>), grid, dim3(kThreads, 1, 1), decode_lds_bytes(1), st, a);
+        else
+            hipLaunchKernelGGL((decode_q8_kernel<2, kDepth, true>), grid, dim3(kThreads, 1, 1), decode_lds_bytes(2), st, a);
+    } else if (narrow)
         hipLaunchKernelGGL((decode_q8_kernel<1, kDepth>), grid, dim3(kThreads, 1, 1), decode_lds_bytes(1), st, a);
     else
         hipLaunchKernelGGL((decode_q8_kernel<2, kDepth>), grid, dim3(kThreads, 1, 1), decode_lds_bytes(2), st, a);
-    int rc = launched("attn_decode_kv_q8");
+    int rc = launched(L.q4 ? "attn_decode_kv_q4" : "attn_decode_kv_q8");
     if (rc)
         return rc;
     hipLaunchKernelGGL(decode_reduce_kernel,

@@ -66,9 +66,72 @@ __global__ void __launch_bounds__(256) kv_encode_q8_kernel(
     q8_encode_store(v[src], vc + off, lane32);
 }
 
-int launch_kv_encode_q8(hipStream_t st, const float *k, const float *v, uint8_t *kc, uint8_t *vc,
-                        int n_kv, int head_dim, int stride, const int32_t *pos, int pos_stride,
-                        size_t slot_bytes, int units, int start, int src0, int /*rows*/)
+// ---- q4_0 quantize + append (crates/hipml-core/src/kv.rs:201-218) ---------------------------
+//
+// The scale takes the sign of the value of largest magnitude, the FIRST such value when several
+// tie (the reference folds left with a strict `>`; NaN never wins that comparison); d = -vmax/8,
+// id = 1/d or 0, q = clamp(round(x*id) + 8, 0, 15); byte j of the block holds q[j] in its low and
+// q[j+16] in its high nibble.  Same thread layout as the q8_0 kernel: 32 lanes per block.
+
+__device__ __forceinline__ float half_wave_vmax(float x, int lane32)
+{
+    float mag = fabsf(x);
+    if (!(mag == mag))
+        mag = -1.0f; // NaN: below every real magnitude, like a failed `>`
+    float val = x;
+    int idx = lane32;
+#pragma unroll
+    for (int bit = 16; bit > 0; bit >>= 1) {
+        const float om = __shfl_xor(mag, bit);
+        const float ov = __shfl_xor(val, bit);
+        const int oi = __shfl_xor(idx, bit);
+        const bool take = om > mag || (om == mag && oi < idx);
+        mag = take ? om : mag;
+        val = take ? ov : val;
+        idx = take ? oi : idx;
+    }
+    return mag > 0.0f ? val : 0.0f; // nothing beat the fold's initial +0
+}
+
+__device__ __forceinline__ void q4_encode_store(float x, uint8_t *dst_block, int lane32)
+{
+    const float vmax = half_wave_vmax(x, lane32);
+    const float d = -vmax / 8.0f;
+    const float id = d != 0.0f ? 1.0f / d : 0.0f;
+    const float t = roundf(x * id) + 8.0f;
+    const float c = fminf(15.0f, fmaxf(0.0f, t));
+    const int q = (t != t) ? 0 : (int)c; // NaN encodes as 0, like Rust's `as u8`
+    const int hi = __shfl_xor(q, 16);
+    if (lane32 == 0)
+        *reinterpret_cast<__half *>(dst_block) = __float2half_rn(d);
+    if (lane32 < 16)
+        dst_block[2 + lane32] = (uint8_t)(q | (hi << 4));
+}
+
+__global__ void __launch_bounds__(256) kv_encode_q4_kernel(
+    const float *__restrict__ k, const float *__restrict__ v, uint8_t *__restrict__ kc,
+    uint8_t *__restrict__ vc, int n_kv, int head_dim, int stride, const int32_t *__restrict__ pos,
+    int pos_stride, size_t slot_bytes, int start, int src0)
+{
+    const int h = blockIdx.x;
+    const int u = blockIdx.y;
+    const int t = threadIdx.x;
+    if (t >= head_dim)
+        return;
+    const int chunk = t >> 5;
+    const int lane32 = t & 31;
+    const int nchunk = head_dim >> 5;
+    const int p = pos ? pos[(size_t)u * pos_stride] : start + u;
+    const size_t src = ((size_t)(src0 + u) * n_kv + h) * head_dim + t;
+    const size_t off = (size_t)u * slot_bytes +
+                       (((size_t)h * stride + p) * nchunk + chunk) * kQ4BlockBytes;
+    q4_encode_store(k[src], kc + off, lane32);
+    q4_encode_store(v[src], vc + off, lane32);
+}
+
+int launch_kv_encode(hipStream_t st, int q4, const float *k, const float *v, uint8_t *kc, uint8_t *vc,
+                     int n_kv, int head_dim, int stride, const int32_t *pos, int pos_stride,
+                     size_t slot_bytes, int units, int start, int src0, int /*rows*/)
 {
     if (units == 0)
         return 0;
@@ -76,11 +139,12 @@ int launch_kv_encode_q8(hipStream_t st, const float *k, const float *v, uint8_t 
     // grid.y is limited to 65535: walk long chunks in slices.
     for (int u0 = 0; u0 < units; u0 += 32768) {
         const int n = units - u0 < 32768 ? units - u0 : 32768;
-        hipLaunchKernelGGL(kv_encode_q8_kernel, dim3(n_kv, n, 1), dim3(block, 1, 1), 0, st, k, v,
-                           kc + (size_t)u0 * slot_bytes, vc + (size_t)u0 * slot_bytes, n_kv,
-                           head_dim, stride, pos ? pos + (size_t)u0 * pos_stride : nullptr,
-                           pos_stride, slot_bytes, start + u0, src0 + u0);
-        int rc = launched("kv_encode_q8");
+        hipLaunchKernelGGL(q4 ? kv_encode_q4_kernel : kv_encode_q8_kernel, dim3(n_kv, n, 1),
+                           dim3(block, 1, 1), 0, st, k, v, kc + (size_t)u0 * slot_bytes,
+                           vc + (size_t)u0 * slot_bytes, n_kv, head_dim, stride,
+                           pos ? pos + (size_t)u0 * pos_stride : nullptr, pos_stride, slot_bytes,
+                           start + u0, src0 + u0);
+        int rc = launched(q4 ? "kv_encode_q4" : "kv_encode_q8");
         if (rc)
             return rc;
     }

@@ -100,17 +100,43 @@ __device__ __forceinline__ void load_half1(Half &h, const uint8_t *u)
     h.q = *reinterpret_cast<const uint4a4 *>(u + 52);
 }
 
+// q4_0: a unit is 36 bytes [s0 | 16 bytes | s1 | 16 bytes] at a dword boundary; one block is the
+// five dwords 0..4 (scale in the low half of dword 0) or 4..8 (scale in the high half of dword 4,
+// payload dword-aligned behind it).  Byte j of a block carries element j in its low nibble and
+// element j + 16 in its high nibble (crates/hipml-core/src/kv.rs:201-218).
+struct Half4 {
+    uint4v p;
+    uint32_t r; // dword 4 of the unit, in both halves
+};
+
+__device__ __forceinline__ void load_half0(Half4 &h, const uint8_t *u)
+{
+    h.p = *reinterpret_cast<const uint4a4 *>(u);
+    h.r = *reinterpret_cast<const uint32_t *>(u + 16);
+}
+
+__device__ __forceinline__ void load_half1(Half4 &h, const uint8_t *u)
+{
+    h.r = *reinterpret_cast<const uint32_t *>(u + 16);
+    h.p = *reinterpret_cast<const uint4a4 *>(u + 20);
+}
+
+template <bool Q4> struct HalfOf { typedef Half type; };
+template <> struct HalfOf<true> { typedef Half4 type; };
+
 // 16 int8 -> 16 f16 (value * d), d an f16 scale: the bytes become 1024 + (b+128)
 // in f16 by bit tricks, the bias is subtracted exactly, then one packed multiply
 // rounds d*b once -- the same value as (f16)((float)d * (float)b).
+// (OFFSET 128: int8 bytes, sign bit flipped first; OFFSET 8: unsigned nibbles 0..15, one per byte.)
+template <int OFFSET = 128>
 __device__ __forceinline__ void dequant16(uint4v raw, _Float16 d, uint4v &lo, uint4v &hi)
 {
-    const half2v bias = {(_Float16)1152.0f, (_Float16)1152.0f};
+    const half2v bias = {(_Float16)(1024.0f + OFFSET), (_Float16)(1024.0f + OFFSET)};
     const half2v dd = {d, d};
     uint32_t o[8];
 #pragma unroll
     for (int w = 0; w < 4; w++) {
-        const uint32_t x = raw[w] ^ 0x80808080u;
+        const uint32_t x = OFFSET == 128 ? raw[w] ^ 0x80808080u : raw[w];
         const uint32_t a = __builtin_amdgcn_perm(0x64646464u, x, 0x04010400u); // [0x64,b1,0x64,b0]
         const uint32_t b = __builtin_amdgcn_perm(0x64646464u, x, 0x04030402u); // [0x64,b3,0x64,b2]
         o[2 * w] = __builtin_bit_cast(uint32_t, (__builtin_bit_cast(half2v, a) - bias) * dd);
@@ -153,6 +179,39 @@ __device__ __forceinline__ void stage_block1(const Half &h, uint8_t *dst)
     d4[4] = x0;
     d4[5] = x1;
     dequant16(h.q, s1, x0, x1);
+    d4[6] = x0;
+    d4[7] = x1;
+}
+
+__device__ __forceinline__ void stage_block0(const Half4 &h, uint8_t *dst)
+{
+    uint4v e;
+    e[0] = __builtin_amdgcn_alignbit(h.p[1], h.p[0], 16);
+    e[1] = __builtin_amdgcn_alignbit(h.p[2], h.p[1], 16);
+    e[2] = __builtin_amdgcn_alignbit(h.p[3], h.p[2], 16);
+    e[3] = __builtin_amdgcn_alignbit(h.r, h.p[3], 16);
+    const uint4v mask = {0x0f0f0f0fu, 0x0f0f0f0fu, 0x0f0f0f0fu, 0x0f0f0f0fu};
+    const _Float16 s0 = __builtin_bit_cast(_Float16, (uint16_t)(h.p[0] & 0xffffu));
+    uint4v *d4 = reinterpret_cast<uint4v *>(dst);
+    uint4v x0, x1;
+    dequant16<8>(e & mask, s0, x0, x1);        // elements 0..15
+    d4[0] = x0;
+    d4[1] = x1;
+    dequant16<8>((e >> 4) & mask, s0, x0, x1); // elements 16..31
+    d4[2] = x0;
+    d4[3] = x1;
+}
+
+__device__ __forceinline__ void stage_block1(const Half4 &h, uint8_t *dst)
+{
+    const uint4v mask = {0x0f0f0f0fu, 0x0f0f0f0fu, 0x0f0f0f0fu, 0x0f0f0f0fu};
+    const _Float16 s1 = __builtin_bit_cast(_Float16, (uint16_t)(h.r >> 16));
+    uint4v *d4 = reinterpret_cast<uint4v *>(dst);
+    uint4v x0, x1;
+    dequant16<8>(h.p & mask, s1, x0, x1);
+    d4[4] = x0;
+    d4[5] = x1;
+    dequant16<8>((h.p >> 4) & mask, s1, x0, x1);
     d4[6] = x0;
     d4[7] = x1;
 }
@@ -219,9 +278,12 @@ __device__ __forceinline__ void lds_barrier()
     __builtin_amdgcn_sched_barrier(0);
 }
 
-template <bool SPLIT>
+template <bool SPLIT, bool Q4 = false>
 __global__ void __launch_bounds__(kPfThreads, 2) chunk_q8_kernel(const ChunkArgs a)
 {
+    typedef typename HalfOf<Q4>::type Half;
+    constexpr int kRowBytes = Q4 ? hipml::kRowBytesQ4 : hipml::kRowBytes;
+    constexpr int kUnitBytes = Q4 ? 36 : 68;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
     const int wave = threadIdx.x >> 6;
@@ -309,7 +371,7 @@ __global__ void __launch_bounds__(kPfThreads, 2) chunk_q8_kernel(const ChunkArgs
     const int su = threadIdx.x & 255;
     const int srow = (su >> 6) * 16 + ((su >> 1) & 7) + ((su >> 5) & 1) * 8;
     const int spr = (su & 1) | ((su >> 3) & 2);
-    const uint8_t *sbase = (set ? a.vc : a.kc) + (size_t)kvh * a.stride * kRowBytes + spr * 68;
+    const uint8_t *sbase = (set ? a.vc : a.kc) + (size_t)kvh * a.stride * kRowBytes + spr * kUnitBytes;
     const int sdst = set ? kVOff + srow * kVRow + spr * 128 : srow * kKRow + spr * 128;
     // One block of the unit is in flight at a time: block 0 of tile t+1 travels during the MFMA slot
     // M2(t-1) and is dequantized in V1(t), block 1 travels during M1(t) and is dequantized in V2(t).
@@ -678,6 +740,12 @@ int prefill_init()
     if (e == hipSuccess)
         e = hipFuncSetAttribute(reinterpret_cast<const void *>(&chunk_q8_kernel<true>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, kPfLds);
+    if (e == hipSuccess)
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&chunk_q8_kernel<false, true>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, kPfLds);
+    if (e == hipSuccess)
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&chunk_q8_kernel<true, true>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, kPfLds);
     if (e != hipSuccess)
         return fail((int)e, "hipFuncSetAttribute(prefill LDS) failed: %d (%s)", (int)e,
                     hipGetErrorString(e));
@@ -686,7 +754,7 @@ int prefill_init()
 
 int launch_chunk_q8(hipStream_t st, const float *q, const uint8_t *kc, const uint8_t *vc,
                     float *out, int n_head, int n_kv, int pos0, int tokens, int stride,
-                    float *part_acc, float *part_ml, int splits, const float *gate)
+                    float *part_acc, float *part_ml, int splits, const float *gate, int q4)
 {
     ChunkArgs a;
     a.gate = gate;
@@ -732,11 +800,17 @@ int launch_chunk_q8(hipStream_t st, const float *q, const uint8_t *kc, const uin
             grid = (unsigned)(combos * a.nblock);
     }
     if (splits < 2) {
-        hipLaunchKernelGGL(chunk_q8_kernel<false>, dim3(grid, 1, 1), block, kPfLds, st, a);
-        return launched("attn_chunk_q8");
+        if (q4)
+            hipLaunchKernelGGL((chunk_q8_kernel<false, true>), dim3(grid, 1, 1), block, kPfLds, st, a);
+        else
+            hipLaunchKernelGGL(chunk_q8_kernel<false>, dim3(grid, 1, 1), block, kPfLds, st, a);
+        return launched(q4 ? "attn_chunk_q4" : "attn_chunk_q8");
     }
-    hipLaunchKernelGGL(chunk_q8_kernel<true>, dim3(grid, 1, 1), block, kPfLds, st, a);
-    int rc = launched("attn_chunk_q8_split");
+    if (q4)
+        hipLaunchKernelGGL((chunk_q8_kernel<true, true>), dim3(grid, 1, 1), block, kPfLds, st, a);
+    else
+        hipLaunchKernelGGL(chunk_q8_kernel<true>, dim3(grid, 1, 1), block, kPfLds, st, a);
+    int rc = launched(q4 ? "attn_chunk_q4_split" : "attn_chunk_q8_split");
     if (rc)
         return rc;
     hipLaunchKernelGGL(chunk_combine_kernel, dim3((unsigned)tokens, (unsigned)((n_head + 3) / 4), 1),

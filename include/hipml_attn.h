@@ -20,8 +20,13 @@
  *     is two byte arrays K and V of [n_kv][stride][head_dim/32] 34-byte blocks
  *     (f16 scale, 32 x int8): block (kvh,pos,c) starts at byte
  *     ((kvh*stride + pos)*(head_dim/32) + c)*34      (crates/hipml-core/src/kv.rs:22-40).
- *   - `dtype` for cache entry points is the reference's KvDtype id (0 = q8_0).
- *     q4_0 (1) is rejected with HIPML_ATTN_E_UNSUPPORTED.
+ *     A q4_0 cache has the same shape with 18-byte blocks (f16 scale, 16 bytes whose low /
+ *     high nibbles are elements j / j+16; value = (nibble - 8) * scale, kv.rs:201-218).
+ *   - `dtype` of the append entry points is the reference's KvDtype id: 0 = q8_0, 1 = q4_0.
+ *     The decode entry points take the reference's kernel selector: 0 or 4 = q8_0, 1 or 5 =
+ *     q4_0 (crates/hipml-kernels/src/launch_kv.rs:146-170,329-334; its other values pick
+ *     variants of the reference's own kernels and are rejected).  The chunk entry points
+ *     take 1 = q8_0, 2 = q4_0 (attn_gpu/imp/attn_chunk_kv.rs:41-60).
  */
 #ifndef HIPML_ATTN_H
 #define HIPML_ATTN_H
@@ -128,7 +133,7 @@ int hipml_attn_chunk_front_f32(hipml_stream_t stream, const float *qg, float *k,
                                int n_kv, int head_dim, int n_rot, float theta_base, float eps,
                                int pos0, int tokens);
 
-/* ---- q8_0 KV append ------------------------------------------------------- */
+/* ---- q8_0 / q4_0 KV append ------------------------------------------------------- */
 
 /* One token: quantize k_in/v_in [n_kv][head_dim] into row step[0] of the cache.
  * Replaces Launcher::kv_encode_ptr_on -> kv_encode_q8,
@@ -149,7 +154,7 @@ int hipml_kv_encode_rows(hipml_stream_t stream, int dtype, const float *k_f32, c
                          void *k_cache, void *v_cache, int n_kv, int head_dim, int stride,
                          const int32_t *pos, size_t slot_bytes, int slots);
 
-/* ---- decode attention over a q8_0 cache ----------------------------------- */
+/* ---- decode attention over a q8_0 / q4_0 cache ----------------------------------- */
 
 /* One query row, live length step[1].  Split pass + merge.
  * part_acc: f32 [n_heads][splits][head_dim]; part_ml: f32 [n_heads][splits][2].
@@ -204,11 +209,11 @@ int hipml_attn_decode_batch_cols(hipml_stream_t stream, int dtype, const int32_t
                                  size_t kv_slot_bytes, size_t acc_slot, size_t ml_slot,
                                  size_t q_slot, int slots, const int32_t *cols_per_slot_host);
 
-/* ---- causal chunk prefill over a q8_0 cache -------------------------------- */
+/* ---- causal chunk prefill over a q8_0 / q4_0 cache -------------------------------- */
 
 /* tokens query rows at positions pos0..pos0+tokens-1 attend keys [0, pos0+t]
  * of a cache that already holds the chunk's own rows.  `dtype` follows the
- * reference's chunk launcher: 1 = q8_0.  splits < 2 runs the single-pass kernel
+ * reference's chunk launcher: 1 = q8_0, 2 = q4_0.  splits < 2 runs the single-pass kernel
  * and ignores the scratch; otherwise part_acc is f32
  * [splits][ceil32(tokens)][n_head][head_dim] and part_ml [..][2].
  * Replaces AttnLayer::chunk_attention_q8_split -> attn_chunk_wmma_f16 /
