@@ -438,7 +438,7 @@ def main() -> int:
         torch.cuda.empty_cache()
         also["decode_32768"] = bench_decode(torch, attn, 32768, d_steps, max(W // 4, 2), LAYERS)
         torch.cuda.empty_cache()
-        # beyond the BASELINE depths: shows what the same kernel does once launch and ramp-up
+        # beyond the two benchmark depths: shows what the same kernel does once launch and ramp-up
         # stop dominating (285 MB per layer)
         also["decode_131072"] = bench_decode(torch, attn, 131072, max(d_steps // 4, 5), 2, LAYERS)
         torch.cuda.empty_cache()

@@ -303,16 +303,19 @@ def q_gate(x, gate, y, n=None, stream=None):
 # ---- cache owner ------------------------------------------------------------------------------------
 
 class DeepKv:
-    """One layer's q8_0 cache plus its decode scratch: the role of the reference's
+    """One layer's quantized cache plus its decode scratch: the role of the reference's
     `DeepKv` (crates/hipml-model/src/gpu/deep_kv.rs:11-83).  K and V are separate
-    uint8 tensors of [n_kv][stride][272]."""
+    uint8 tensors of [n_kv][stride][row bytes]: 272 for q8_0 (dtype 0), 144 for q4_0 (dtype 1)."""
 
     def __init__(self, n_heads=24, n_kv=4, head_dim=HEAD_DIM, stride=4096, max_cols=1,
-                 device="cuda"):
+                 device="cuda", dtype=0):
         assert head_dim == HEAD_DIM
+        assert dtype in (0, 1), "KvDtype id: 0 = q8_0, 1 = q4_0"
+        self.dtype = dtype
+        self.row_bytes = ROW_BYTES if dtype == 0 else head_dim // 32 * 18
         self.n_heads, self.n_kv, self.head_dim, self.seq = n_heads, n_kv, head_dim, stride
-        self.k = torch.zeros((n_kv, stride, ROW_BYTES), dtype=torch.uint8, device=device)
-        self.v = torch.zeros((n_kv, stride, ROW_BYTES), dtype=torch.uint8, device=device)
+        self.k = torch.zeros((n_kv, stride, self.row_bytes), dtype=torch.uint8, device=device)
+        self.v = torch.zeros((n_kv, stride, self.row_bytes), dtype=torch.uint8, device=device)
         self.max_splits = max(decode_splits(stride, n_kv), 1)
         self.max_cols = max_cols
         self.part_acc = torch.empty((max_cols, n_heads, self.max_splits, head_dim),
@@ -324,4 +327,4 @@ class DeepKv:
         return min(decode_splits(seq, self.n_kv), self.max_splits)
 
     def bytes(self) -> int:
-        return 2 * self.n_kv * self.seq * ROW_BYTES
+        return 2 * self.n_kv * self.seq * self.row_bytes

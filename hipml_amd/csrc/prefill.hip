@@ -52,11 +52,6 @@ constexpr float kLog2e = 1.4426950408889634f;
 #ifndef PF_SKEW
 #define PF_SKEW 1
 #endif
-#ifdef PF_PRIO
-#define PRIO(n) __builtin_amdgcn_s_setprio(n)
-#else
-#define PRIO(n) do { } while (0)
-#endif
 
 struct ChunkArgs {
     const float *q;
@@ -380,9 +375,6 @@ __global__ void __launch_bounds__(kPfThreads, 2) chunk_q8_kernel(const ChunkArgs
     // for memory to do it.)
     Half half;
     auto unit_ptr = [&](int t) {
-#ifdef PF_DBG_SAMETILE
-        t = t & 7; // debug: keep re-reading the first tiles (cache hits)
-#endif
         int key = klo + t * kKTile + srow;
         key = key < khi ? key : khi - 1;
         return sbase + (size_t)key * kRowBytes;

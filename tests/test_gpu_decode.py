@@ -60,7 +60,7 @@ def test_deep_case_100k_one_head():
 
 @pytest.mark.parametrize("seq,stride", [(673, 680), (8192, 8192), (32768, 32768), (5000, 32768)])
 def test_decode_full_geometry(seq, stride):
-    # BASELINE configs 1 (depth 672 -> seq 673) and 3 (8,192 / 32,768): 24 q heads on 4 kv heads
+    # the benchmark depths (672 -> seq 673; 8,192; 32,768): 24 q heads on 4 kv heads
     r = orc.Rng(0x5EED_0003 + seq)
     q = r.normal_array((N_HEADS, HD))
     kf = r.normal_array((N_KV, seq, HD))
@@ -196,7 +196,7 @@ def test_batched_decode_uniform_rows():
 
 
 def test_batched_decode_with_mtp_slots_in_one_launch():
-    # BASELINE config 5: 16 slots, depths uniform in [512, 16384] under seed, slots 0..3 carry
+    # the batched benchmark case: 16 slots, depths uniform in [512, 16384] under seed, slots 0..3 carry
     # 3 query rows (causal within the draft), the rest 1.
     r = orc.Rng(0x5EED_0005)
     depths = [512 + int(float(r.uniform()) * (16384 - 512 + 1)) for _ in range(16)]

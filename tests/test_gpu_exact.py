@@ -32,7 +32,7 @@ def adversarial_rows(rng, rows, width):
 
 
 def test_kv_encode_bulk_bytes_equal_oracle():
-    # BASELINE config 2: 672 tokens x 4 kv heads x 256, appended at position 0 of a
+    # the headline benchmark shape: 672 tokens x 4 kv heads x 256, appended at position 0 of a
     # cache with stride > live length.
     rows, stride, start = 672, 680, 0
     r = orc.Rng(0xDDDD_EEEE_FFFF_0003)

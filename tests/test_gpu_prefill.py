@@ -1,6 +1,6 @@
 """Causal chunk prefill over a q8_0 cache: HIP path vs the oracle's row-by-row
 attn_causal_f32 over the dequantized cache.  Tolerance: max-abs 2e-3 / rel 1e-2
-(BASELINE gate; the reference's chunk class is 2e-3 / 2e-2,
+(the parity gate of this build; the reference's chunk class is 2e-3 / 2e-2,
 crates/hipml-cli/src/attn_chunk_parity.rs:18-20): fp16 operands, fp32 accumulation."""
 import numpy as np
 import pytest
@@ -59,7 +59,7 @@ def test_reference_chunk_case(tok, pos0, pad, splits):
 
 @pytest.mark.parametrize("splits", [1, 3])
 def test_prefill_672_at_0(splits):
-    # BASELINE config 2
+    # the headline benchmark shape: 672 tokens at depth 0
     tok, pos0 = 672, 0
     q, kb, vb, stride = chunk_inputs(0x5EED_0002, tok, pos0, 8)
     want = orc.attn_chunk_kv(q, kb, vb, N_HEADS, N_KV, HD, pos0, tok, stride, SCALE, n_threads=16)
@@ -81,7 +81,7 @@ def test_split_and_mono_agree_and_splits_above_diagonal_are_ignored():
 
 
 def test_deep_chunk_sampled_rows():
-    # BASELINE config 4 at reduced depth for the CPU side: 256 tokens at depth 20,000,
+    # the long-context benchmark shape at reduced depth for the CPU side: 256 tokens at depth 20,000,
     # every 37th row checked; exercises long-KV tiling and the split merge.
     tok, pos0 = 256, 20_000
     q, kb, vb, stride = chunk_inputs(0x5EED_0004, tok, pos0, 16)
