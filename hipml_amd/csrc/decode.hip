@@ -125,8 +125,10 @@ __device__ __forceinline__ void load_unit(Unit &u, const uint8_t *p)
 
 // Realign one unit and store it: payloads of blocks (2*pr, 2*pr+1) of tile row r to the padded
 // tile, their scales to the transposed table.
+// A row past the live length (`live` false) gets zero scales: its bytes are whatever the cache
+// holds there, and a non-finite scale would turn its zero weight into NaN.
 __device__ __forceinline__ void store_unit(const Unit &u, uint8_t *tile, uint8_t *scales, int r,
-                                           int pr)
+                                           int pr, bool live)
 {
     uint4v e0, e1;
     e0[0] = __builtin_amdgcn_alignbit(u.a[1], u.a[0], 16);
@@ -143,8 +145,8 @@ __device__ __forceinline__ void store_unit(const Unit &u, uint8_t *tile, uint8_t
     dst[2] = u.c;
     dst[3] = u.d;
     uint16_t *sc = reinterpret_cast<uint16_t *>(scales) + (2 * pr) * kTileKeys + r;
-    sc[0] = (uint16_t)(u.a[0] & 0xffffu);
-    sc[kTileKeys] = (uint16_t)(u.m >> 16);
+    sc[0] = live ? (uint16_t)(u.a[0] & 0xffffu) : (uint16_t)0;
+    sc[kTileKeys] = live ? (uint16_t)(u.m >> 16) : (uint16_t)0;
 }
 
 // q4_0: a unit is two 18-byte blocks of one key, 36 bytes at a dword boundary:
@@ -166,7 +168,7 @@ __device__ __forceinline__ void load_unit(Unit4 &u, const uint8_t *p)
 // Nibbles widened to one byte per element (values 0..15), element order, so the tile has the
 // q8_0 tile's shape and everything after staging is shared; the offset to remove is 8, not 128.
 __device__ __forceinline__ void store_unit(const Unit4 &u, uint8_t *tile, uint8_t *scales, int r,
-                                           int pr)
+                                           int pr, bool live)
 {
     uint4v e0;
     e0[0] = __builtin_amdgcn_alignbit(u.a[1], u.a[0], 16);
@@ -180,8 +182,8 @@ __device__ __forceinline__ void store_unit(const Unit4 &u, uint8_t *tile, uint8_
     dst[2] = u.b & mask;
     dst[3] = (u.b >> 4) & mask;
     uint16_t *sc = reinterpret_cast<uint16_t *>(scales) + (2 * pr) * kTileKeys + r;
-    sc[0] = (uint16_t)(u.a[0] & 0xffffu);
-    sc[kTileKeys] = (uint16_t)(u.m >> 16);
+    sc[0] = live ? (uint16_t)(u.a[0] & 0xffffu) : (uint16_t)0;
+    sc[kTileKeys] = live ? (uint16_t)(u.m >> 16) : (uint16_t)0;
 }
 
 template <bool Q4> struct UnitOf { typedef Unit type; };
@@ -245,9 +247,38 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
     const int group = a.group;
     const int nvalid = ncols * group;
 
-    // ---- Q rows first: their addresses need nothing from device memory, and issued ahead of
-    // the K/V stream they are not queued behind it.  Entry (nt, c, l) of the LDS operand table
-    // = Q[col n = nt*16 + l%16][c*32 + (l/16)*8 .. +8]; a thread owns entries tid + kThreads*k.
+    uint8_t *tile_lds = wave_base + wave * kWaveLds;
+    uint8_t *sK = tile_lds + kTileBytes;
+    uint8_t *sV = sK + kScaleBytes;
+
+    const uint8_t *kbase = a.k + (size_t)slot * a.kv_slot_bytes + (size_t)kvh * a.stride * kRowBytes;
+    const uint8_t *vbase = a.v + (size_t)slot * a.kv_slot_bytes + (size_t)kvh * a.stride * kRowBytes;
+
+    // ---- key tiles of this wave ---------------------------------------------------------------
+    // The 32-key tiles of a KV head are dealt round-robin: tile g belongs to split (g / kWaves)
+    // % splits, wave g % kWaves, so wave `wave` of split `split` owns tiles
+    // (t * splits + split) * kWaves + wave, t = 0, 1, ...  The addresses depend on the launch only,
+    // not on the live length, which lives in device memory: the first tile is requested before that
+    // length has been read (a tile past the live rows costs one load of rows inside the cache's
+    // stride and is masked out), and neighbouring workgroups stream neighbouring rows.
+    auto tile_key0 = [&](int t) { return ((t * a.splits + split) * kWaves + wave) * kTileKeys; };
+
+    // ---- staging registers: DEPTH tiles in flight, each 2 K units + 2 V units per lane -------
+    Unit Kst[DEPTH][2], Vst[DEPTH][2];
+    // unit j of a tile: u = lane + 64*j -> tile row u/4, block pair u%4
+    const int ur0 = lane >> 2, ur1 = 16 + (lane >> 2), upr = lane & 3;
+    const int last_row = a.stride - 1;
+    auto issue = [&](Unit (&dst)[2], const uint8_t *base, int t) {
+        const int key0 = tile_key0(t);
+        int ka = key0 + ur0, kb = key0 + ur1;
+        ka = ka < last_row ? ka : last_row; // never leave the cache; rows past the live length are
+        kb = kb < last_row ? kb : last_row; // neutralised when they are staged
+        load_unit(dst[0], base + (size_t)ka * kRowBytes + upr * kUnitBytes);
+        load_unit(dst[1], base + (size_t)kb * kRowBytes + upr * kUnitBytes);
+    };
+
+    // ---- Q rows first: their addresses need nothing from device memory.  Entry (nt, c, l) of the
+    // LDS operand table = Q[col n = nt*16 + l%16][c*32 + (l/16)*8 .. +8]; a thread owns entries tid + kThreads*k.
     constexpr int kQEntries = NT * 8 * 64 / kThreads;
     float4v qf[kQEntries][2];
 #pragma unroll
@@ -267,6 +298,12 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
         }
     }
 
+    // ... and right behind them the first tile: loads return in order, so the few Q rows are not
+    // queued behind 17 KB of K/V, and the tile is on its way before the live length is known
+    issue(Kst[0], kbase, 0);
+    issue(Vst[0], vbase, 0);
+    STAMP(5); // first tile requested
+
     // live lengths of this slot's rows
     int seqc[kMaxCols];
     int seq_max = 0;
@@ -277,34 +314,12 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
         seqc[c] = s;
         seq_max = s > seq_max ? s : seq_max;
     }
-    const int per = (seq_max + a.splits - 1) / a.splits;
-    const int lo = split * per;
-    const int hi = lo + per < seq_max ? lo + per : seq_max;
-    const int ntile_wg = hi > lo ? (hi - lo + kTileKeys - 1) / kTileKeys : 0;
-    // this wave's tiles: wave, wave + kWaves, ...
-    const int ntile = ntile_wg > wave ? (ntile_wg - wave + kWaves - 1) / kWaves : 0;
-
-    uint8_t *tile_lds = wave_base + wave * kWaveLds;
-    uint8_t *sK = tile_lds + kTileBytes;
-    uint8_t *sV = sK + kScaleBytes;
-
-    const uint8_t *kbase = a.k + (size_t)slot * a.kv_slot_bytes + (size_t)kvh * a.stride * kRowBytes;
-    const uint8_t *vbase = a.v + (size_t)slot * a.kv_slot_bytes + (size_t)kvh * a.stride * kRowBytes;
-
-    // ---- staging registers: DEPTH tiles in flight, each 2 K units + 2 V units per lane -------
-    Unit Kst[DEPTH][2], Vst[DEPTH][2];
-    // unit j of a tile: u = lane + 64*j -> tile row u/4, block pair u%4
-    const int ur0 = lane >> 2, ur1 = 16 + (lane >> 2), upr = lane & 3;
-    auto issue = [&](Unit (&dst)[2], const uint8_t *base, int t) {
-        const int key0 = lo + (wave + kWaves * t) * kTileKeys;
-        int ka = key0 + ur0, kb = key0 + ur1;
-        ka = ka < hi ? ka : hi - 1; // never touch rows past the live range
-        kb = kb < hi ? kb : hi - 1;
-        load_unit(dst[0], base + (size_t)ka * kRowBytes + upr * kUnitBytes);
-        load_unit(dst[1], base + (size_t)kb * kRowBytes + upr * kUnitBytes);
-    };
+    const int hi = seq_max; // keys at or past it are masked
+    STAMP(6); // live length known
+    const int first_key = tile_key0(0), step_keys = a.splits * kWaves * kTileKeys;
+    const int ntile = first_key < hi ? (hi - first_key + step_keys - 1) / step_keys : 0;
 #pragma unroll
-    for (int st = 0; st < DEPTH; st++)
+    for (int st = 1; st < DEPTH; st++)
         if (ntile > st) {
             issue(Kst[st], kbase, st);
             issue(Vst[st], vbase, st);
@@ -327,6 +342,7 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
         *reinterpret_cast<half8 *>(Qs + (((nt * 2 + 0) * 8 + c) * 64 + l) * 16) = h8;
         *reinterpret_cast<half8 *>(Qs + (((nt * 2 + 1) * 8 + c) * 64 + l) * 16) = l8;
     }
+    STAMP(7); // Q values arrived and written to LDS
     __syncthreads();
     // Bias table: the K bytes enter the MFMA as (b + 128) * 2^-24, so every score of block c
     // carries +128 * 2^-24 * sum_k q[k][n]; its negative is the C operand the block's MFMA starts
@@ -378,12 +394,12 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
     const half8 Abias = __builtin_bit_cast(half8, bias_bits); // eight times -offset * 2^-24
 
     auto process = [&](Unit (&Ku)[2], Unit (&Vu)[2], int t) {
-        const int key0 = lo + (wave + kWaves * t) * kTileKeys;
+        const int key0 = tile_key0(t);
         const bool more = t + DEPTH < ntile;
 
         // ---- K tile to LDS, refill the registers ------------------------------------------
-        store_unit(Ku[0], tile_lds, sK, ur0, upr);
-        store_unit(Ku[1], tile_lds, sK, ur1, upr);
+        store_unit(Ku[0], tile_lds, sK, ur0, upr, key0 + ur0 < hi);
+        store_unit(Ku[1], tile_lds, sK, ur1, upr, key0 + ur1 < hi);
         if (more)
             issue(Ku, kbase, t + DEPTH);
 
@@ -437,8 +453,8 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
 #endif
 
         // ---- V tile over the K tile, refill -----------------------------------------------
-        store_unit(Vu[0], tile_lds, sV, ur0, upr);
-        store_unit(Vu[1], tile_lds, sV, ur1, upr);
+        store_unit(Vu[0], tile_lds, sV, ur0, upr, key0 + ur0 < hi);
+        store_unit(Vu[1], tile_lds, sV, ur1, upr, key0 + ur1 < hi);
         if (more)
             issue(Vu, vbase, t + DEPTH);
 

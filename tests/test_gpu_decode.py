@@ -2,7 +2,9 @@
 on identical seeded inputs.  Gate: max-abs 2e-3 / rel 1e-2 (OR rule).  The kernel keeps K, V
 and the block scales exact and Q to ~22 bits, but rounds the softmax weight times the V block
 scale to f16 once (as the reference's chunk kernel rounds P), so its own class is a few 1e-4:
-KERNEL_CLASS below is asserted everywhere, a quarter of the gate."""
+KERNEL_CLASS below is asserted everywhere, half of the gate: the weights enter the PV product as
+f16 (relative 2^-11 = 4.9e-4 of a value of magnitude up to ~3 when one or two keys carry all the
+weight); at depths of hundreds of keys and more the observed error is below 1e-4."""
 import numpy as np
 import pytest
 import torch
@@ -15,7 +17,7 @@ from gpu_util import (N_HEADS, N_KV, HD, SCALE, ROW, dev, host, quantized_cache,
                       decode_scratch, run_decode, report)
 
 GATE = (2e-3, 1e-2)
-KERNEL_CLASS = (5e-4, 5e-3)
+KERNEL_CLASS = (1e-3, 5e-3)
 
 
 @pytest.fixture(scope="module", autouse=True)

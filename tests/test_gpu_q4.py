@@ -15,7 +15,7 @@ from gpu_util import N_HEADS, N_KV, HD, SCALE, dev, host, step_buffer, report  #
 Q4 = 1
 ROW4 = 144
 GATE = (2e-3, 1e-2)
-KERNEL_CLASS = (5e-4, 5e-3)
+KERNEL_CLASS = (1e-3, 5e-3)
 
 
 @pytest.fixture(scope="module", autouse=True)
