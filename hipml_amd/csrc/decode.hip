@@ -1,6 +1,6 @@
 // Split-K decode attention over a q8_0 KV cache for gfx950 (wave64, MFMA).
 //
-// One workgroup (4 waves) owns one (kv head, key split, slot).  Each wave walks
+// One workgroup (4 waves) owns one (kv head, key split, work item = slot or half of its heads).  Each wave walks
 // its own 32-key tiles of the split with a private online softmax and no
 // workgroup barrier in the loop; the four waves merge in LDS at the end and
 // write one unnormalised partial per (row, head, split).  A second kernel
@@ -19,8 +19,8 @@
 //   S^T[key][n]  = K[key][:] . Q^T[:][n]      A = K bytes as f16, B = Q (hi + lo f16, from LDS)
 //   O^T[d][n]   += V^T[d][key] . P'[key][n]   A = V bytes as f16 (LDS transpose read),
 //                                              B = P' = p * scale_of_block(key, d/32), hi + lo f16
-// n runs over (query row, head of the GQA group): up to 4 rows x 8 heads, in
-// tiles of 16 columns.  The C layout of S^T (row = 4*(lane/16)+i, col = lane%16)
+// n runs over (query row, head) pairs, at most 16 per workgroup: a slot with more (3-4 MTP
+// rows x 6-8 heads) is cut by heads into two work items.  The C layout of S^T (row = 4*(lane/16)+i, col = lane%16)
 // is exactly the B layout the PV product needs, so probabilities never leave
 // their lane, and every per-column scalar (max, sum, rescale) lives in lane%16.
 //
@@ -35,6 +35,8 @@
 
 #include "common.h"
 
+#include <string.h>
+
 namespace hipml {
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
@@ -45,6 +47,7 @@ typedef int int2v __attribute__((ext_vector_type(2)));
 typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
 typedef uint32_t uint4a4 __attribute__((ext_vector_type(4), aligned(4)));
 
+constexpr int kMaxItems = 2 * kMaxSlots;               // work items of one launch (see DecodeArgs)
 constexpr int kTileKeys = 32;                         // keys per wave tile
 constexpr int kLdsRow = 288;                          // 256 payload bytes + 32 pad (bank spread)
 constexpr int kTileBytes = kTileKeys * kLdsRow;       // 9216: payload tile (K, then V)
@@ -101,8 +104,15 @@ struct DecodeArgs {
     int n_kv, group, stride, splits;
     float scale_log2; // scale * log2(e) * 2^24
     size_t kv_slot_bytes, acc_slot, ml_slot, q_slot;
-    uint16_t row0[kMaxSlots];
-    uint8_t cols[kMaxSlots];
+    // Work items (grid.y).  A slot whose rows x heads fit one 16-column MFMA tile is one item; a
+    // wider one (3-4 MTP rows x 6 heads) is cut by heads into items of at most 16 columns that
+    // stream the same cache rows: their workgroups are gridDim.x apart in launch order, a multiple
+    // of the 8 XCDs here, so the second reader finds the rows in the first one's L2.
+    uint16_t row0[kMaxItems];  // first query row of the item's slot
+    uint8_t cols[kMaxItems];   // query rows of the slot (1..kMaxCols)
+    uint8_t kvslot[kMaxItems]; // slot index, for the cache base
+    uint8_t head0[kMaxItems];  // first head (within the GQA group) of the item
+    uint8_t nhead[kMaxItems];  // heads of the item
 };
 
 // 68 bytes of a key row starting at a block-pair boundary: [s0 | 32 x i8 | s1 | 32 x i8].
@@ -241,10 +251,12 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
     const int lg = lane >> 4; // k-group
     const int kvh = blockIdx.x / a.splits;
     const int split = blockIdx.x - kvh * a.splits;
-    const int slot = blockIdx.y;
-    const int row0 = a.row0[slot];
-    const int ncols = a.cols[slot];
-    const int group = a.group;
+    const int item = blockIdx.y;
+    const int slot = a.kvslot[item];
+    const int row0 = a.row0[item];
+    const int ncols = a.cols[item];
+    const int group = a.nhead[item]; // heads of this item: columns are (row, head) pairs over them
+    const int hbase = kvh * a.group + a.head0[item];
     const int nvalid = ncols * group;
 
     uint8_t *tile_lds = wave_base + wave * kWaveLds;
@@ -261,7 +273,8 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
     // not on the live length, which lives in device memory: the first tile is requested before that
     // length has been read (a tile past the live rows costs one load of rows inside the cache's
     // stride and is masked out), and neighbouring workgroups stream neighbouring rows.
-    auto tile_key0 = [&](int t) { return ((t * a.splits + split) * kWaves + wave) * kTileKeys; };
+    const int nsp = a.splits;
+    auto tile_key0 = [&](int t) { return ((t * nsp + split) * kWaves + wave) * kTileKeys; };
 
     // ---- staging registers: DEPTH tiles in flight, each 2 K units + 2 V units per lane -------
     Unit Kst[DEPTH][2], Vst[DEPTH][2];
@@ -292,7 +305,7 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
             const int col = n / group;
             const int head = n - col * group;
             const float *qp = a.q + (size_t)(row0 + col) * a.q_slot +
-                              (size_t)(kvh * group + head) * kHeadDim + c * 32 + (l >> 4) * 8;
+                              (size_t)(hbase + head) * kHeadDim + c * 32 + (l >> 4) * 8;
             qf[k][0] = *reinterpret_cast<const float4v *>(qp);
             qf[k][1] = *reinterpret_cast<const float4v *>(qp + 4);
         }
@@ -316,7 +329,7 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
     }
     const int hi = seq_max; // keys at or past it are masked
     STAMP(6); // live length known
-    const int first_key = tile_key0(0), step_keys = a.splits * kWaves * kTileKeys;
+    const int first_key = tile_key0(0), step_keys = nsp * kWaves * kTileKeys;
     const int ntile = first_key < hi ? (hi - first_key + step_keys - 1) / step_keys : 0;
 #pragma unroll
     for (int st = 1; st < DEPTH; st++)
@@ -620,7 +633,7 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
                     wgt[w] *= kTwo24;
                 }
                 const int col = ng / group;
-                const int head = kvh * group + (ng - col * group);
+                const int head = hbase + (ng - col * group);
                 const size_t slice = (size_t)head * a.splits + split;
                 float *pa = a.part_acc + (size_t)(row0 + col) * a.acc_slot + slice * kHeadDim + d0;
 #pragma unroll
@@ -645,16 +658,11 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
     STAMP(4);
 }
 
-// NT = 1: every slot has at most 16 (row, head) columns.  NT = 2: some slot has more (MTP
-// verify, 3-4 rows x 6 heads); slots that fit one column tile still take the NT = 1 body, so a
-// mixed batch pays the wider tile only where it is needed.  LDS is sized for the launch's NT.
-template <int NT, int DEPTH, bool Q4 = false>
+// One 16-column tile per workgroup (NT = 1): wider slots arrive as several work items.
+template <int DEPTH, bool Q4 = false>
 __global__ void __launch_bounds__(kThreads, DECODE_MIN_WAVES) decode_q8_kernel(const DecodeArgs a)
 {
-    if (NT == 1 || a.cols[blockIdx.y] * a.group <= 16)
-        decode_body<1, DEPTH, Q4>(a);
-    else
-        decode_body<NT, DEPTH, Q4>(a);
+    decode_body<1, DEPTH, Q4>(a);
 }
 
 // Wave-wide reductions without LDS: DPP inside a row of 16 lanes, then the two row-swap
@@ -782,18 +790,12 @@ extern "C" int hipml_dbg_read_stamps(unsigned long long *host, size_t n)
 
 int decode_init()
 {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&decode_q8_kernel<1, kDepth>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&decode_q8_kernel<kDepth, false>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize,
                                        decode_lds_bytes(1));
     if (e == hipSuccess)
-        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&decode_q8_kernel<2, kDepth>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, decode_lds_bytes(2));
-    if (e == hipSuccess)
-        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&decode_q8_kernel<1, kDepth, true>),
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&decode_q8_kernel<kDepth, true>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, decode_lds_bytes(1));
-    if (e == hipSuccess)
-        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&decode_q8_kernel<2, kDepth, true>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, decode_lds_bytes(2));
     if (e != hipSuccess)
         return fail((int)e, "hipFuncSetAttribute(decode LDS) failed: %d (%s)", (int)e,
                     hipGetErrorString(e));
@@ -818,21 +820,30 @@ int launch_decode_q8(hipStream_t st, const DecodeLaunch &L)
     a.acc_slot = L.acc_slot;
     a.ml_slot = L.ml_slot;
     a.q_slot = L.q_slot;
-    for (int s = 0; s < kMaxSlots; s++) {
-        a.row0[s] = s < L.slots ? L.row0[s] : 0;
-        a.cols[s] = s < L.slots ? L.cols[s] : 0;
+    memset(a.row0, 0, sizeof(a.row0));
+    memset(a.cols, 0, sizeof(a.cols));
+    memset(a.kvslot, 0, sizeof(a.kvslot));
+    memset(a.head0, 0, sizeof(a.head0));
+    memset(a.nhead, 0, sizeof(a.nhead));
+    int items = 0;
+    for (int s = 0; s < L.slots; s++) {
+        const int columns = L.cols[s] * a.group;
+        const int parts = (columns + 15) / 16;                  // 1 or 2 (cols <= 4, group <= 8)
+        const int per = (a.group + parts - 1) / parts;          // heads per item
+        for (int h0 = 0; h0 < a.group; h0 += per) {
+            a.row0[items] = L.row0[s];
+            a.cols[items] = L.cols[s];
+            a.kvslot[items] = (uint8_t)s;
+            a.head0[items] = (uint8_t)h0;
+            a.nhead[items] = (uint8_t)(a.group - h0 < per ? a.group - h0 : per);
+            items++;
+        }
     }
-    const dim3 grid((unsigned)(L.n_kv * L.splits), (unsigned)L.slots, 1);
-    const bool narrow = L.max_cols * a.group <= 16;
-    if (L.q4) {
-        if (narrow)
-            hipLaunchKernelGGL((decode_q8_kernel<1, kDepth, true>), grid, dim3(kThreads, 1, 1), decode_lds_bytes(1), st, a);
-        else
-            hipLaunchKernelGGL((decode_q8_kernel<2, kDepth, true>), grid, dim3(kThreads, 1, 1), decode_lds_bytes(2), st, a);
-    } else if (narrow)
-        hipLaunchKernelGGL((decode_q8_kernel<1, kDepth>), grid, dim3(kThreads, 1, 1), decode_lds_bytes(1), st, a);
+    const dim3 grid((unsigned)(L.n_kv * L.splits), (unsigned)items, 1);
+    if (L.q4)
+        hipLaunchKernelGGL((decode_q8_kernel<kDepth, true>), grid, dim3(kThreads, 1, 1), decode_lds_bytes(1), st, a);
     else
-        hipLaunchKernelGGL((decode_q8_kernel<2, kDepth>), grid, dim3(kThreads, 1, 1), decode_lds_bytes(2), st, a);
+        hipLaunchKernelGGL((decode_q8_kernel<kDepth, false>), grid, dim3(kThreads, 1, 1), decode_lds_bytes(1), st, a);
     int rc = launched(L.q4 ? "attn_decode_kv_q4" : "attn_decode_kv_q8");
     if (rc)
         return rc;
