@@ -214,18 +214,23 @@ __global__ void __launch_bounds__(64) mrope_kernel(
     }
 }
 
-// grid (n_head + n_kv, tokens); 64 threads.  Token t rotates at pos0 + t.
-__global__ void __launch_bounds__(64) rope_chunk_kernel(
+// 256 threads = 8 head rows x 32 lanes; head row r of the chunk = (token r / (n_head + n_kv),
+// q head or k head); token t rotates at pos0 + t.
+__global__ void __launch_bounds__(256) rope_chunk_kernel(
     float *__restrict__ q, float *__restrict__ kx, int n_head, int n_kv, int head_dim, int n_rot,
-    float theta, int pos0, const float *__restrict__ tab, int tab_rows)
+    float theta, int pos0, int tokens, const float *__restrict__ tab, int tab_rows)
 {
-    const int h = blockIdx.x;
-    const int t = blockIdx.y;
+    const int per = n_head + n_kv;
+    const long long r = (long long)blockIdx.x * 8 + (threadIdx.x >> 5);
+    if (r >= (long long)tokens * per)
+        return;
+    const int t = (int)(r / per);
+    const int h = (int)(r - (long long)t * per);
     const int half = n_rot >> 1;
     const int p = pos0 + t;
     float *row = h < n_head ? q + ((size_t)t * n_head + h) * head_dim
                             : kx + ((size_t)t * n_kv + (h - n_head)) * head_dim;
-    for (int k = threadIdx.x; k < half; k += blockDim.x) {
+    for (int k = threadIdx.x & 31; k < half; k += 32) {
         float cs, sn;
         rope_cs(tab, tab_rows, half, k, p, n_rot, theta, cs, sn);
         const float x1 = row[k];
@@ -270,11 +275,13 @@ int launch_rope_chunk(hipStream_t st, float *q, float *k, int n_head, int n_kv, 
 {
     int tab_rows = 0;
     const float *t = table_for(tab, theta, n_rot, &tab_rows);
-    for (int t0 = 0; t0 < tokens; t0 += 32768) {
-        const int n = tokens - t0 < 32768 ? tokens - t0 : 32768;
-        hipLaunchKernelGGL(rope_chunk_kernel, dim3(n_head + n_kv, n, 1), dim3(64, 1, 1), 0, st,
-                           q + (size_t)t0 * n_head * head_dim, k + (size_t)t0 * n_kv * head_dim,
-                           n_head, n_kv, head_dim, n_rot, theta, pos0 + t0, t, tab_rows);
+    const int slab = 1 << 20; // tokens per launch: keeps the row count inside the grid limit
+    for (int t0 = 0; t0 < tokens; t0 += slab) {
+        const int n = tokens - t0 < slab ? tokens - t0 : slab;
+        const long long rows = (long long)n * (n_head + n_kv);
+        hipLaunchKernelGGL(rope_chunk_kernel, dim3((unsigned)((rows + 7) / 8), 1, 1), dim3(256, 1, 1), 0,
+                           st, q + (size_t)t0 * n_head * head_dim, k + (size_t)t0 * n_kv * head_dim,
+                           n_head, n_kv, head_dim, n_rot, theta, pos0 + t0, n, t, tab_rows);
         int rc = launched("rope_chunk_f32");
         if (rc)
             return rc;
