@@ -393,27 +393,46 @@ __global__ void __launch_bounds__(kPfThreads, 2) chunk_q8_kernel(const ChunkArgs
     // Steps 0..kQLdsSteps-1 are parked in this wave's corner of LDS and re-read per use: 256
     // registers do not hold O (128), all of Q (64), the scores, the tile prefetch and the operand
     // pipeline at once, and what the compiler would spill instead goes to scratch memory.
+    //
+    // The rows are fetched whole (one instruction = one token's 256 floats of this head, 1 KB
+    // contiguous), converted and transposed through this wave's 16.5 KB corner of the tile buffers,
+    // which are still unused: a lane-per-token fetch of 16-byte pieces from rows 24 KB apart took
+    // several times longer to arrive.  The operand is then read back with the K tile's pattern.
     half8 qf[16];
     uint8_t *qlds = lds + kQLdsOff + wave * kQLdsSteps * 1024 + lane * 16;
     {
-        const int tq = tok < a.tokens ? tok : a.tokens - 1;
-        const float *qp = a.q + ((size_t)tq * a.n_head + head) * kHeadDim + lh * 8;
+        uint8_t *qt = lds + wave * (kQTile * kKRow);
+        const float *qh = a.q + (size_t)head * kHeadDim + lane * 4;
+        const size_t tok_stride = (size_t)a.n_head * kHeadDim;
+#pragma unroll
+        for (int b = 0; b < 2; b++) {
+            float4v f[16];
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const int tr = t0 + b * 16 + i;
+                f[i] = *reinterpret_cast<const float4v *>(qh + (size_t)(tr < a.tokens ? tr : a.tokens - 1) * tok_stride);
+            }
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                half4 h;
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    h[j] = (_Float16)f[i][j];
+                *reinterpret_cast<half4 *>(qt + (b * 16 + i) * kKRow + lane * 8) = h;
+            }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // this wave's own writes
+        __builtin_amdgcn_wave_barrier();
 #pragma unroll
         for (int ks = 0; ks < 16; ks++) {
-            const float4v f0 = *reinterpret_cast<const float4v *>(qp + ks * 16);
-            const float4v f1 = *reinterpret_cast<const float4v *>(qp + ks * 16 + 4);
-            half8 h;
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                h[j] = (_Float16)f0[j];
-                h[4 + j] = (_Float16)f1[j];
-            }
+            const half8 h = *reinterpret_cast<const half8 *>(qt + ln * kKRow + ks * 32 + lh * 16);
             if (ks < kQLdsSteps)
                 *reinterpret_cast<half8 *>(qlds + ks * 1024) = h;
             else
                 qf[ks] = h;
         }
     }
+    __syncthreads(); // every wave has its Q: the tile buffers may now take the first tile
 
     float16v O[8];
 #pragma unroll
