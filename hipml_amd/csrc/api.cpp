@@ -202,6 +202,11 @@ int hipml_attn_batch_splits(int stride, int n_kv, int slots)
 {
     if (stride < 1 || n_kv < 1 || slots < 1)
         return 1;
+    // Two resident rounds of workgroups (two per CU, 512 on the chip).  Measured on 16 slots, stride
+    // 16,448: one round (8 splits) is best when all slots are deep (108 vs 116 us) but loses where
+    // depths are skewed, because a slot never gets more than `splits` workgroups (one deep + 15
+    // shallow: 68 vs 44 us; 4 deep + 12 shallow: 68 vs 49 us); counts in between leave a partial
+    // round behind (10: 135 us, 12: 128 us on the all-deep case).
     int by_work = (stride + 127) / 128;
     int by_cus = 1024 / (n_kv * slots);
     if (by_cus < 1)

@@ -329,6 +329,18 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
     }
     const int hi = seq_max; // keys at or past it are masked
     STAMP(6); // live length known
+    if (split * kWaves * kTileKeys >= hi) {
+        // not one live tile for any wave of this workgroup (a shallow slot of a batch, or more
+        // splits than tiles): leave an empty partial and go, the merge skips it
+        if ((int)threadIdx.x < nvalid) {
+            const int col = threadIdx.x / group;
+            const int head = hbase + (threadIdx.x - col * group);
+            float *pm = a.part_ml + (size_t)(row0 + col) * a.ml_slot + ((size_t)head * a.splits + split) * 2;
+            pm[0] = -INFINITY;
+            pm[1] = 0.0f;
+        }
+        return; // uniform over the workgroup
+    }
     const int first_key = tile_key0(0), step_keys = nsp * kWaves * kTileKeys;
     const int ntile = first_key < hi ? (hi - first_key + step_keys - 1) / step_keys : 0;
 #pragma unroll
