@@ -202,13 +202,17 @@ int hipml_attn_batch_splits(int stride, int n_kv, int slots)
 {
     if (stride < 1 || n_kv < 1 || slots < 1)
         return 1;
-    // Two resident rounds of workgroups (two per CU, 512 on the chip).  Measured on 16 slots, stride
-    // 16,448: one round (8 splits) is best when all slots are deep (108 vs 116 us) but loses where
-    // depths are skewed, because a slot never gets more than `splits` workgroups (one deep + 15
-    // shallow: 68 vs 44 us; 4 deep + 12 shallow: 68 vs 49 us); counts in between leave a partial
-    // round behind (10: 135 us, 12: 128 us on the all-deep case).
+    // Batches of up to a quarter of the chip's workgroup window in slots run as one window of workers
+    // that share the slots by depth (see the decode kernel); `splits` is then only the cap on one
+    // slot's workers and the width of its partials, and a generous cap lets a deep slot among
+    // shallow ones take more of the chip (16 slots, one of depth 16,384 and fifteen of 512: 51 us at
+    // cap 16, 37 us at cap 32).  Larger batches launch every split of every slot; there two windows
+    // of workgroups were the best compromise between all-deep and skewed batches.
     int by_work = (stride + 127) / 128;
-    int by_cus = 1024 / (n_kv * slots);
+    const int window = 512 / n_kv;
+    int by_cus = (4 * slots <= window ? 2048 : 1024) / (n_kv * slots);
+    if (by_cus > 64)
+        by_cus = 64;
     if (by_cus < 1)
         by_cus = 1;
     int s = by_work < by_cus ? by_work : by_cus;

@@ -35,6 +35,7 @@
 
 #include "common.h"
 
+#include <stddef.h>
 #include <string.h>
 
 namespace hipml {
@@ -102,6 +103,8 @@ struct DecodeArgs {
     float *part_ml;
     const int32_t *pos;
     int n_kv, group, stride, splits;
+    int items;     // work items (grid.y of a plain launch)
+    int workers;   // > 0: worker launch, workgroups per KV head (see decode_body)
     float scale_log2; // scale * log2(e) * 2^24
     size_t kv_slot_bytes, acc_slot, ml_slot, q_slot;
     // Work items (grid.y).  A slot whose rows x heads fit one 16-column MFMA tile is one item; a
@@ -249,15 +252,105 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
     const int lane = threadIdx.x & 63;
     const int lm = lane & 15; // MFMA row/col within the 16-tile
     const int lg = lane >> 4; // k-group
-    const int kvh = blockIdx.x / a.splits;
-    const int split = blockIdx.x - kvh * a.splits;
-    const int item = blockIdx.y;
+    // ---- which (kv head, item, split) this workgroup is ---------------------------------------
+    // Plain launches: grid (n_kv * splits, items), every split of every item gets tiles.
+    // Worker launches (batches, a.workers > 0): grid (n_kv * workers).  The hardware starts the
+    // workgroups of a launch in windows of as many as fit the chip (512 here) and opens the next
+    // window only when the whole previous one has finished, so a workgroup with little or nothing to
+    // do still holds its place for as long as the longest one of its window.  A batch has items of
+    // very different depth: its launch is therefore exactly one window of workers, and each worker
+    // derives its (item, split) from the live lengths in device memory: item i gets
+    // nsp_i = clamp(floor(tiles_i * (workers - items) / sum of tiles), 1, splits) consecutive
+    // workers (their sum cannot exceed `workers`; what the rounding leaves is handed out one by
+    // one), i.e. about equal work per worker.
+    int kvh, split, item, nsp;
+    if (a.workers > 0) {
+        kvh = blockIdx.x / a.workers;
+        const int w = blockIdx.x - kvh * a.workers;
+        // lane i looks at item i (the launcher uses this mode for at most 64 items); item tables
+        // are read through the kernel-argument pointer: a lane-indexed read of the by-value
+        // argument struct would make the compiler copy its arrays to scratch
+        typedef const __attribute__((address_space(4))) uint8_t *KargBytes;
+        typedef const __attribute__((address_space(4))) uint16_t *KargHalves;
+        const KargBytes ka = (KargBytes)__builtin_amdgcn_kernarg_segment_ptr();
+        const KargHalves t_row0 = (KargHalves)(ka + offsetof(DecodeArgs, row0));
+        const KargBytes t_cols = ka + offsetof(DecodeArgs, cols);
+        int tiles = 0;
+        if (lane < a.items) {
+            const int r0 = t_row0[lane], nc = t_cols[lane];
+            int sm = 0;
+            for (int c = 0; c < nc; c++) {
+                int v = a.pos[(size_t)(r0 + c) * 2 + 1];
+                v = v < 0 ? 0 : (v > a.stride ? a.stride : v);
+                sm = v > sm ? v : sm;
+            }
+            tiles = (sm + kTileKeys - 1) / kTileKeys;
+        }
+        int total = tiles;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1)
+            total += __shfl_xor(total, off);
+        total = total > 0 ? total : 1;
+        int share = 0;
+        if (lane < a.items) {
+            share = (int)((long long)tiles * (a.workers - a.items) / total);
+            share = share < 1 ? 1 : (share < a.splits ? share : a.splits);
+        }
+        // the shares are rounded down: hand the workers left over to the items in turn, one each per
+        // pass, while they are below their cap
+        int used = share;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1)
+            used += __shfl_xor(used, off);
+        int left = a.workers - used; // >= 0 by construction
+        for (int pass = 0; pass < 3 && left > 0; pass++) {
+            const bool want = lane < a.items && tiles > share * kWaves && share < a.splits;
+            const unsigned long long m = __ballot(want);
+            const int rank = __builtin_popcountll(m & ((1ull << lane) - 1ull));
+            if (want && rank < left)
+                share++;
+            const int given = __builtin_popcountll(m);
+            left -= given < left ? given : left;
+        }
+        int end = share; // inclusive prefix sum over lanes
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const int up = __shfl_up(end, off);
+            end += lane >= off ? up : 0;
+        }
+        const unsigned long long hit = __ballot(lane < a.items && w >= end - share && w < end);
+        if (hit == 0)
+            return; // more workers than the shares add up to (uniform over the workgroup)
+        item = __builtin_ctzll(hit);
+        nsp = __shfl(share, item);
+        split = w - (__shfl(end, item) - nsp);
+        item = __builtin_amdgcn_readfirstlane(item);
+        nsp = __builtin_amdgcn_readfirstlane(nsp);
+        split = __builtin_amdgcn_readfirstlane(split);
+    } else {
+        kvh = blockIdx.x / a.splits;
+        split = blockIdx.x - kvh * a.splits;
+        item = blockIdx.y;
+        nsp = a.splits;
+    }
     const int slot = a.kvslot[item];
     const int row0 = a.row0[item];
     const int ncols = a.cols[item];
     const int group = a.nhead[item]; // heads of this item: columns are (row, head) pairs over them
     const int hbase = kvh * a.group + a.head0[item];
     const int nvalid = ncols * group;
+    if (a.workers > 0 && split == 0 && nsp < a.splits) {
+        // the splits of this item that no worker takes: empty partials, which the merge skips
+        const int empty = a.splits - nsp;
+        for (int e = threadIdx.x; e < nvalid * empty; e += kThreads) {
+            const int n = e / empty, sp = nsp + (e - n * empty);
+            const int col = n / group;
+            const int head = hbase + (n - col * group);
+            float *pm = a.part_ml + (size_t)(row0 + col) * a.ml_slot + ((size_t)head * a.splits + sp) * 2;
+            pm[0] = -INFINITY;
+            pm[1] = 0.0f;
+        }
+    }
 
     uint8_t *tile_lds = wave_base + wave * kWaveLds;
     uint8_t *sK = tile_lds + kTileBytes;
@@ -268,12 +361,11 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
 
     // ---- key tiles of this wave ---------------------------------------------------------------
     // The 32-key tiles of a KV head are dealt round-robin: tile g belongs to split (g / kWaves)
-    // % splits, wave g % kWaves, so wave `wave` of split `split` owns tiles
-    // (t * splits + split) * kWaves + wave, t = 0, 1, ...  The addresses depend on the launch only,
-    // not on the live length, which lives in device memory: the first tile is requested before that
-    // length has been read (a tile past the live rows costs one load of rows inside the cache's
-    // stride and is masked out), and neighbouring workgroups stream neighbouring rows.
-    const int nsp = a.splits;
+    // % nsp, wave g % kWaves, so wave `wave` of split `split` owns tiles
+    // (t * nsp + split) * kWaves + wave, t = 0, 1, ...  In a plain launch the addresses depend on
+    // the launch only, not on the live length, which lives in device memory: the first tile is
+    // requested before that length has been read (a tile past the live rows costs one load of rows
+    // inside the cache's stride and is masked out), and neighbouring workgroups stream neighbouring rows.
     auto tile_key0 = [&](int t) { return ((t * nsp + split) * kWaves + wave) * kTileKeys; };
 
     // ---- staging registers: DEPTH tiles in flight, each 2 K units + 2 V units per lane -------
@@ -851,7 +943,13 @@ int launch_decode_q8(hipStream_t st, const DecodeLaunch &L)
             items++;
         }
     }
-    const dim3 grid((unsigned)(L.n_kv * L.splits), (unsigned)items, 1);
+    a.items = items;
+    // batches: one window of workers (two workgroups per CU over 256 CUs), as long as every item can
+    // have a worker of its own and lane i of a wave can look at item i
+    const int window = 512 / L.n_kv;
+    a.workers = items > 1 && items <= 64 && 2 * items <= window ? window : 0;
+    const dim3 grid = a.workers > 0 ? dim3((unsigned)(L.n_kv * a.workers), 1, 1)
+                                    : dim3((unsigned)(L.n_kv * L.splits), (unsigned)items, 1);
     if (L.q4)
         hipLaunchKernelGGL((decode_q8_kernel<kDepth, true>), grid, dim3(kThreads, 1, 1), decode_lds_bytes(1), st, a);
     else
