@@ -1,0 +1,92 @@
+"""The C ABI without a GPU: libhipml_attn.so loads, exports every function include/hipml_attn.h
+declares, the host-only entry points (split policies, RoPE table) compute, and argument errors
+are reported before anything is launched."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from hipml_amd import attn
+    return attn.lib()
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "hipml_attn.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(hipml_\w+)\s*\(", text)))
+
+
+def test_every_declared_function_is_exported(lib):
+    names = declared_functions()
+    assert len(names) >= 25
+    missing = [n for n in names if not hasattr(lib, n)]
+    assert not missing, missing
+
+
+def test_python_mirror_lists_every_declared_function():
+    from hipml_amd import attn
+    assert sorted(attn.EXPORTS) == declared_functions()
+
+
+def test_split_policies(lib):
+    from hipml_amd import attn
+    # decode: 128 keys per split, at most two workgroups per CU over the KV heads
+    assert attn.decode_splits(1, 4) == 1
+    assert attn.decode_splits(8192, 4) == 64
+    assert attn.decode_splits(32768, 4) == 128
+    assert attn.decode_splits(1 << 20, 4) == 128
+    # batches: a cap on one slot's workers, never below 1
+    assert 1 <= attn.batch_splits(16448, 4, 16) <= 64
+    assert attn.batch_splits(16448, 4, 128) >= 1
+    assert attn.batch_splits(100, 4, 16) == 1
+    # prefill: no key slices once the task blocks fill the chip; slices keep n_kv*splits on the XCDs
+    assert attn.chunk_splits(0, 8192, 4) == 1
+    s = attn.chunk_splits(100_000, 2048, 4)
+    assert s > 1 and (4 * s) % 8 == 0
+    assert attn.chunk_splits(0, 1, 4) >= 1
+
+
+def test_rope_table_on_the_host_is_the_f64_definition(lib):
+    theta, n_rot, max_pos = 1e7, 64, 300
+    nbytes = lib.hipml_rope_table_bytes(n_rot, max_pos)
+    assert nbytes == max_pos * (n_rot // 2) * 2 * 4
+    tab = np.empty(nbytes // 4, dtype=np.float32)
+    assert lib.hipml_rope_table_fill_host(tab.ctypes.data_as(C.c_void_p), C.c_float(theta), n_rot, max_pos) == 0
+    tab = tab.reshape(max_pos, n_rot // 2, 2)
+    k = np.arange(n_rot // 2, dtype=np.float64)
+    freq = np.float64(np.float32(theta)) ** (-2.0 * k / n_rot)
+    ang = np.arange(max_pos, dtype=np.float64)[:, None] * freq[None, :]
+    assert np.array_equal(tab[..., 0], np.cos(ang).astype(np.float32))
+    assert np.array_equal(tab[..., 1], np.sin(ang).astype(np.float32))
+
+
+def test_argument_errors_come_before_any_launch(lib):
+    from hipml_amd import attn
+    null = C.c_void_p(0)
+    one = C.c_void_p(16)  # a non-null, 16-byte aligned value that is never dereferenced on these paths
+    # NULL buffers
+    rc = lib.hipml_attn_decode_kv(null, null, 0, null, one, one, one, one, one, 24, 4, 256, 64, C.c_float(0.0625), 1, 0, 0)
+    assert rc < 0 and b"NULL" in lib.hipml_attn_last_error()
+    # unknown cache format
+    rc = lib.hipml_attn_decode_kv(null, one, 9, one, one, one, one, one, one, 24, 4, 256, 64, C.c_float(0.0625), 1, 0, 0)
+    assert rc == -2 and b"dtype" in lib.hipml_attn_last_error()
+    # head geometry the kernels are not built for
+    rc = lib.hipml_attn_decode_kv(null, one, 0, one, one, one, one, one, one, 24, 4, 128, 64, C.c_float(0.0625), 1, 0, 0)
+    assert rc < 0 and b"head_dim" in lib.hipml_attn_last_error()
+    # a chunk that does not fit the cache
+    rc = lib.hipml_attn_chunk_q8_split(null, one, one, one, one, 24, 4, 256, 60, 10, 1, 64, null, null, 1)
+    assert rc < 0 and b"does not fit" in lib.hipml_attn_last_error()
+    # key slices without scratch
+    rc = lib.hipml_attn_chunk_q8_split(null, one, one, one, one, 24, 4, 256, 0, 10, 1, 64, null, null, 4)
+    assert rc < 0 and b"NULL" in lib.hipml_attn_last_error()
+    # the Python mirror raises where the reference's launcher returns Err(String)
+    with pytest.raises(attn.HipmlError) as e:
+        attn._check(rc)
+    assert e.value.code == rc
