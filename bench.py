@@ -216,6 +216,21 @@ def bench_decode(torch, attn, seq, steps, warmup, layers, dtype=0):
         for _ in range(steps):
             one_pass()
     us = t.ms * 1e3 / (steps * layers)
+    # the same with the sigmoid output gate: in the merge kernel, and as the separate launch it replaces
+    gate = torch.randn((H, HD), device="cuda", generator=gen)
+    for _ in range(warmup):
+        for k, v in caches:
+            attn.attn_decode_kv_gate(stepbuf, dtype, q, k, v, acc, ml, out, gate, H, KV, HD, stride, SCALE, splits)
+    with Timer(torch) as tg:
+        for _ in range(steps):
+            for k, v in caches:
+                attn.attn_decode_kv_gate(stepbuf, dtype, q, k, v, acc, ml, out, gate, H, KV, HD, stride, SCALE,
+                                         splits)
+    with Timer(torch) as ts:
+        for _ in range(steps):
+            for k, v in caches:
+                attn.attn_decode_kv(stepbuf, dtype, q, k, v, acc, ml, out, H, KV, HD, stride, SCALE, splits)
+                attn.q_gate(out, gate, out, H * HD)
     nbytes = decode_bytes(seq) * row // ROW
     gbs = nbytes / (us * 1e-6) / 1e9
     traffic = measured_traffic({8192: "decode8k", 32768: "decode32k"}.get(seq, "") if dtype == 0 else "",
@@ -225,6 +240,8 @@ def bench_decode(torch, attn, seq, steps, warmup, layers, dtype=0):
                     f"split-K {splits} + merge",
         "seq": seq, "splits": splits, "layers_rotated": layers,
         "us_per_layer": us,
+        "us_per_layer_gate_fused": tg.ms * 1e3 / (steps * layers),
+        "us_per_layer_gate_separate": ts.ms * 1e3 / (steps * layers),
         "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": gbs / HBM_PEAK_GBS, "traffic": traffic,
                      "kernel": "decode_q8_kernel + decode_reduce_kernel",
@@ -286,6 +303,8 @@ def bench_batch(torch, attn, orc, steps, warmup, layers):
                     f"slots 0..3 carry 3 query rows (MTP verify), one launch",
         "slots": slots, "rows": rows, "live_rows": live, "splits": splits, "layers_rotated": layers,
         "us_per_layer": us,
+        "us_per_layer_gate_fused": tg.ms * 1e3 / (steps * layers),
+        "us_per_layer_gate_separate": ts.ms * 1e3 / (steps * layers),
         "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": gbs / HBM_PEAK_GBS, "traffic": traffic,
                      "kernel": "decode_q8_kernel + decode_reduce_kernel",

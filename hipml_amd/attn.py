@@ -32,6 +32,7 @@ EXPORTS = [
     "hipml_kv_encode", "hipml_kv_encode_bulk", "hipml_kv_encode_rows",
     "hipml_attn_decode_kv", "hipml_attn_decode_kv_cols", "hipml_attn_decode_rows",
     "hipml_attn_decode_batch", "hipml_attn_decode_batch_cols",
+    "hipml_attn_decode_kv_gate", "hipml_attn_decode_batch_cols_gate",
     "hipml_attn_chunk_q8_split", "hipml_attn_chunk_q8_split_gate", "hipml_q_gate_f32",
     "hipml_attn_front_f32", "hipml_attn_chunk_front_f32",
 ]
@@ -85,6 +86,10 @@ def lib() -> C.CDLL:
                                             sz, sz, sz, sz, i, i]),
             "hipml_attn_decode_batch_cols": (i, [vp, i, vp, vp, vp, vp, vp, vp, vp, i, i, i, i, f,
                                                  i, sz, sz, sz, sz, i, vp]),
+            "hipml_attn_decode_kv_gate": (i, [vp, vp, i, vp, vp, vp, vp, vp, vp, vp, i, i, i, i, f, i,
+                                              sz, sz]),
+            "hipml_attn_decode_batch_cols_gate": (i, [vp, i, vp, vp, vp, vp, vp, vp, vp, vp, i, i, i,
+                                                      i, f, i, sz, sz, sz, sz, i, vp]),
             "hipml_attn_chunk_q8_split": (i, [vp, vp, vp, vp, vp, i, i, i, i, i, i, i, vp, vp, i]),
             "hipml_attn_chunk_q8_split_gate": (i, [vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, i, vp, vp, i]),
             "hipml_q_gate_f32": (i, [vp, vp, vp, vp, sz]),
@@ -265,6 +270,25 @@ def attn_decode_batch_cols(dtype, pos, q, k_cache, v_cache, part_acc, part_ml, o
         _stream(stream), dtype, _p(pos), _p(q), _p(k_cache), _p(v_cache), _p(part_acc),
         _p(part_ml), _p(out), n_heads, n_kv, head_dim, stride, scale, splits, kv_slot_bytes,
         acc_slot, ml_slot, q_slot, len(cols_per_slot), C.addressof(arr)))
+
+
+def attn_decode_kv_gate(step, dtype, q, k, v, part_acc, part_ml, out, gate, n_heads, n_kv, head_dim,
+                        stride, scale, splits, k_off=0, v_off=0, stream=None):
+    """`launch_kv::launch_ptrs` followed by `AttnLayer::q_gate_only`, in the merge kernel."""
+    _check(lib().hipml_attn_decode_kv_gate(_stream(stream), _p(step), dtype, _p(q), _p(k), _p(v),
+                                           _p(part_acc), _p(part_ml), _p(out), _p(gate), n_heads,
+                                           n_kv, head_dim, stride, scale, splits, k_off, v_off))
+
+
+def attn_decode_batch_cols_gate(dtype, pos, q, k_cache, v_cache, part_acc, part_ml, out, gate,
+                                n_heads, n_kv, head_dim, stride, scale, splits, kv_slot_bytes,
+                                acc_slot, ml_slot, q_slot, cols_per_slot, stream=None):
+    """`attn_decode_batch_cols` with the gate half of `output_rows` applied in the merge kernel."""
+    arr = (C.c_int32 * len(cols_per_slot))(*[int(c) for c in cols_per_slot])
+    _check(lib().hipml_attn_decode_batch_cols_gate(
+        _stream(stream), dtype, _p(pos), _p(q), _p(k_cache), _p(v_cache), _p(part_acc),
+        _p(part_ml), _p(out), _p(gate), n_heads, n_kv, head_dim, stride, scale, splits,
+        kv_slot_bytes, acc_slot, ml_slot, q_slot, len(cols_per_slot), C.addressof(arr)))
 
 
 # ---- chunk prefill ---------------------------------------------------------------------------

@@ -92,7 +92,7 @@ static int decode_common(hipStream_t st, int dtype, const int32_t *pos, const fl
                          const void *v, float *part_acc, float *part_ml, float *out, int n_heads,
                          int n_kv, int head_dim, int stride, float scale, int splits,
                          size_t kv_slot_bytes, size_t acc_slot, size_t ml_slot, size_t q_slot,
-                         int slots, const int32_t *cols_per_slot)
+                         int slots, const int32_t *cols_per_slot, const float *gate = nullptr)
 {
     REQUIRE_PTR(pos);
     REQUIRE_PTR(q);
@@ -111,7 +111,8 @@ static int decode_common(hipStream_t st, int dtype, const int32_t *pos, const fl
     if (slots < 1 || slots > kMaxSlots)
         return fail(HIPML_ATTN_E_RANGE, "slots %d outside 1..%d", slots, kMaxSlots);
     if ((rc = check_aligned16(k, "k cache")) || (rc = check_aligned16(v, "v cache")) ||
-        (rc = check_aligned16(q, "q")) || (rc = check_aligned16(part_acc, "part_acc")))
+        (rc = check_aligned16(q, "q")) || (rc = check_aligned16(part_acc, "part_acc")) ||
+        (rc = check_aligned16(out, "out")) || (rc = check_aligned16(gate, "gate")))
         return rc;
     if (kv_slot_bytes % 16 != 0 || q_slot % 4 != 0 || acc_slot % 4 != 0)
         return fail(HIPML_ATTN_E_RANGE, "slot strides must keep 16-byte alignment");
@@ -124,6 +125,7 @@ static int decode_common(hipStream_t st, int dtype, const int32_t *pos, const fl
     L.part_acc = part_acc;
     L.part_ml = part_ml;
     L.out = out;
+    L.gate = gate;
     L.pos = pos;
     L.n_heads = n_heads;
     L.n_kv = n_kv;
@@ -582,6 +584,46 @@ int hipml_attn_decode_batch_cols(hipml_stream_t stream, int dtype, const int32_t
     return decode_common(as_stream(stream), fmt, pos, q, k_cache, v_cache, part_acc, part_ml, out,
                          n_heads, n_kv, head_dim, stride, scale, splits, kv_slot_bytes, acc_slot,
                          ml_slot, q_slot, slots, cols_per_slot_host);
+}
+
+int hipml_attn_decode_kv_gate(hipml_stream_t stream, const int32_t *step, int dtype, const float *q,
+                              const void *k, const void *v, float *part_acc, float *part_ml,
+                              float *out, const float *gate, int n_heads, int n_kv, int head_dim,
+                              int stride, float scale, int splits, size_t k_off, size_t v_off)
+{
+    clear_error();
+    int fmt = 0;
+    int rc = decode_format(dtype, &fmt);
+    if (rc)
+        return rc;
+    REQUIRE_PTR(k);
+    REQUIRE_PTR(v);
+    REQUIRE_PTR(gate);
+    const size_t slice = (size_t)(n_heads > 0 ? n_heads : 0) * (size_t)(splits > 0 ? splits : 0);
+    return decode_common(as_stream(stream), fmt, step, q, static_cast<const uint8_t *>(k) + k_off,
+                         static_cast<const uint8_t *>(v) + v_off, part_acc, part_ml, out, n_heads,
+                         n_kv, head_dim, stride, scale, splits, 0, slice * kHeadDim, slice * 2,
+                         (size_t)n_heads * kHeadDim, 1, nullptr, gate);
+}
+
+int hipml_attn_decode_batch_cols_gate(hipml_stream_t stream, int dtype, const int32_t *pos,
+                                      const float *q, const void *k_cache, const void *v_cache,
+                                      float *part_acc, float *part_ml, float *out,
+                                      const float *gate, int n_heads, int n_kv, int head_dim,
+                                      int stride, float scale, int splits, size_t kv_slot_bytes,
+                                      size_t acc_slot, size_t ml_slot, size_t q_slot, int slots,
+                                      const int32_t *cols_per_slot_host)
+{
+    clear_error();
+    int fmt = 0;
+    int rc = decode_format(dtype, &fmt);
+    if (rc)
+        return rc;
+    REQUIRE_PTR(cols_per_slot_host);
+    REQUIRE_PTR(gate);
+    return decode_common(as_stream(stream), fmt, pos, q, k_cache, v_cache, part_acc, part_ml, out,
+                         n_heads, n_kv, head_dim, stride, scale, splits, kv_slot_bytes, acc_slot,
+                         ml_slot, q_slot, slots, cols_per_slot_host, gate);
 }
 
 // ---- chunk prefill ---------------------------------------------------------------------------------

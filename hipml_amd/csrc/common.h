@@ -25,6 +25,16 @@ int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
 int launched(const char *what);
 void clear_error();
 
+#ifdef __HIPCC__
+// The sigmoid output gate (crates/hipml-core/src/ops.rs:354-360).  Every kernel that gates writes it
+// through this one expression, so a fused call and the attention followed by the stand-alone gate
+// kernel give the same bits.
+__device__ __forceinline__ float gated(float x, float g)
+{
+    return x * (1.0f / (1.0f + expf(-g)));
+}
+#endif
+
 inline hipStream_t as_stream(hipml_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
 
 // n_heads / n_kv / head_dim rules shared by the attention launchers
@@ -60,6 +70,7 @@ struct DecodeLaunch {
     float *part_acc;
     float *part_ml;
     float *out;
+    const float *gate;  // rows laid out like `out`, or nullptr: out *= sigmoid(gate) in the merge
     const int32_t *pos; // (pos, seq) pairs, one per row
     int n_heads, n_kv, stride, splits, slots;
     int q4; // cache format: 0 = q8_0, 1 = q4_0

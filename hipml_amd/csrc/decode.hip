@@ -801,7 +801,7 @@ constexpr int kReduceMaxSplits = 4096;
 
 __global__ void __launch_bounds__(256) decode_reduce_kernel(
     const float *__restrict__ part_acc, const float *__restrict__ part_ml, float *__restrict__ out,
-    int splits, size_t acc_slot, size_t ml_slot, size_t q_slot)
+    const float *__restrict__ gate, int splits, size_t acc_slot, size_t ml_slot, size_t q_slot)
 {
     __shared__ float w_s[kReduceMaxSplits];
     __shared__ float red_m[4], red_l[4];
@@ -824,6 +824,11 @@ __global__ void __launch_bounds__(256) decode_reduce_kernel(
         if (s < splits)
             x0[k] = *reinterpret_cast<const float4v *>(acc + (size_t)s * kHeadDim);
     }
+    // the output gate of the row (optional), fetched by the threads that write the result
+    const size_t out_at = (size_t)row * q_slot + (size_t)head * kHeadDim + dq * 64 + (tid & 15) * 4;
+    float4v gt = {0, 0, 0, 0};
+    if (gate != nullptr && tid < 16)
+        gt = *reinterpret_cast<const float4v *>(gate + out_at);
 
     // weights: w_s = 2^(m_s - m) for splits that saw a key, else 0
     float m = -INFINITY;
@@ -880,8 +885,9 @@ __global__ void __launch_bounds__(256) decode_reduce_kernel(
         float4v r = t * inv;
         if (!(den > 0.0f))
             r = (float4v){0, 0, 0, 0};
-        *reinterpret_cast<float4v *>(out + (size_t)row * q_slot + (size_t)head * kHeadDim + dq * 64 +
-                                     tid * 4) = r;
+        if (gate != nullptr)
+            r = (float4v){gated(r[0], gt[0]), gated(r[1], gt[1]), gated(r[2], gt[2]), gated(r[3], gt[3])};
+        *reinterpret_cast<float4v *>(out + out_at) = r;
     }
 }
 
@@ -959,7 +965,7 @@ int launch_decode_q8(hipStream_t st, const DecodeLaunch &L)
         return rc;
     hipLaunchKernelGGL(decode_reduce_kernel,
                        dim3((unsigned)L.n_heads * 4, (unsigned)L.total_rows, 1), dim3(256, 1, 1), 0,
-                       st, L.part_acc, L.part_ml, L.out, L.splits, L.acc_slot, L.ml_slot, L.q_slot);
+                       st, L.part_acc, L.part_ml, L.out, L.gate, L.splits, L.acc_slot, L.ml_slot, L.q_slot);
     return launched("attn_decode_kv_reduce");
 }
 

@@ -410,10 +410,10 @@ __global__ void __launch_bounds__(256) q_gate_kernel4(const float4 *x, const flo
     const float4 a = x[i];
     const float4 b = g[i];
     float4 r;
-    r.x = a.x * (1.0f / (1.0f + expf(-b.x)));
-    r.y = a.y * (1.0f / (1.0f + expf(-b.y)));
-    r.z = a.z * (1.0f / (1.0f + expf(-b.z)));
-    r.w = a.w * (1.0f / (1.0f + expf(-b.w)));
+    r.x = gated(a.x, b.x);
+    r.y = gated(a.y, b.y);
+    r.z = gated(a.z, b.z);
+    r.w = gated(a.w, b.w);
     y[i] = r;
 }
 
@@ -423,7 +423,7 @@ __global__ void __launch_bounds__(256) q_gate_kernel1(const float *x, const floa
     const size_t i = first + (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n)
         return;
-    y[i] = x[i] * (1.0f / (1.0f + expf(-g[i])));
+    y[i] = gated(x[i], g[i]);
 }
 
 int launch_q_gate(hipStream_t st, const float *x, const float *gate, float *y, size_t n)

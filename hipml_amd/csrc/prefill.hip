@@ -211,13 +211,6 @@ __device__ __forceinline__ void stage_block1(const Half4 &h, uint8_t *dst)
     d4[7] = x1;
 }
 
-// The output gate, written exactly as the stand-alone gate kernel writes it, so a fused call and
-// the attention followed by that kernel give the same bits.
-__device__ __forceinline__ float gated(float x, float g)
-{
-    return x * (1.0f / (1.0f + expf(-g)));
-}
-
 // Number of key slices of task block tb (see ChunkArgs::slice_tiles); *seq_block receives the number
 // of keys its last token sees.
 __device__ __host__ __forceinline__ int block_slices(int tb, int ntask, int group, int tokens, int pos0,

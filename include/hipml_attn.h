@@ -209,6 +209,26 @@ int hipml_attn_decode_batch_cols(hipml_stream_t stream, int dtype, const int32_t
                                  size_t kv_slot_bytes, size_t acc_slot, size_t ml_slot,
                                  size_t q_slot, int slots, const int32_t *cols_per_slot_host);
 
+/* Decode with the sigmoid output gate applied where the splits are merged:
+ * out = attention * sigmoid(gate), `gate` laid out like `out` (f32 [n_heads][head_dim] per row,
+ * rows q_slot apart).  The result has the bits of the ungated call followed by hipml_q_gate_f32
+ * on the same rows; it saves that launch.  hipml_attn_decode_kv_gate is
+ * hipml_attn_decode_kv (one row, position from the step buffer) and
+ * hipml_attn_decode_batch_cols_gate is hipml_attn_decode_batch_cols, each with `gate` after `out`.
+ * Replaces launch_kv::launch_ptrs / attn_decode_batch followed by AttnLayer::q_gate_only or the
+ * gate half of output_rows, crates/hipml-kernels/src/attn_gpu.rs:822-840,967-990. */
+int hipml_attn_decode_kv_gate(hipml_stream_t stream, const int32_t *step, int dtype, const float *q,
+                              const void *k, const void *v, float *part_acc, float *part_ml,
+                              float *out, const float *gate, int n_heads, int n_kv, int head_dim,
+                              int stride, float scale, int splits, size_t k_off, size_t v_off);
+int hipml_attn_decode_batch_cols_gate(hipml_stream_t stream, int dtype, const int32_t *pos,
+                                      const float *q, const void *k_cache, const void *v_cache,
+                                      float *part_acc, float *part_ml, float *out,
+                                      const float *gate, int n_heads, int n_kv, int head_dim,
+                                      int stride, float scale, int splits, size_t kv_slot_bytes,
+                                      size_t acc_slot, size_t ml_slot, size_t q_slot, int slots,
+                                      const int32_t *cols_per_slot_host);
+
 /* ---- causal chunk prefill over a q8_0 / q4_0 cache -------------------------------- */
 
 /* tokens query rows at positions pos0..pos0+tokens-1 attend keys [0, pos0+t]

@@ -13,7 +13,7 @@ pytestmark = pytest.mark.gpu
 
 from oracle import binding as orc  # noqa: E402
 from hipml_amd import attn  # noqa: E402
-from gpu_util import (N_HEADS, N_KV, HD, SCALE, ROW, dev, host, quantized_cache,  # noqa: E402
+from gpu_util import (N_HEADS, N_KV, HD, SCALE, ROW, dev, host, quantized_cache, step_buffer,  # noqa: E402
                       decode_scratch, run_decode, report)
 
 GATE = (2e-3, 1e-2)
@@ -248,3 +248,59 @@ def test_verify_group_through_rows_entry_shares_the_cache():
     for c in range(cols):
         want = orc.attn_decode_kv(q[c], kb, vb, N_HEADS, N_KV, HD, pos0 + c + 1, SCALE, stride=stride)
         assert orc.compare(want, host(out)[c], *KERNEL_CLASS)[0]
+
+
+def test_gated_decode_has_the_bits_of_decode_then_gate():
+    # launch_kv::launch_ptrs + AttnLayer::q_gate_only (attn_gpu.rs:822-840) in one call: same bits as
+    # the two calls, and out * sigmoid(gate) of the oracle
+    seq, stride = 5000, 8192
+    r = orc.Rng(0x6A7E_0001)
+    q = r.normal_array((N_HEADS, HD))
+    gate = r.normal_array((N_HEADS, HD))
+    kf = r.normal_array((N_KV, seq, HD))
+    vf = r.normal_array((N_KV, seq, HD))
+    kb, vb = quantized_cache(kf, vf, stride)
+    splits = attn.decode_splits(seq, N_KV)
+    acc, ml = decode_scratch(N_HEADS, splits)
+    step = step_buffer(seq - 1, seq)
+    two = torch.full((N_HEADS, HD), float("nan"), dtype=torch.float32, device="cuda")
+    attn.attn_decode_kv(step, 0, dev(q), dev(kb), dev(vb), acc, ml, two, N_HEADS, N_KV, HD, stride,
+                        SCALE, splits)
+    attn.q_gate(two, dev(gate), two, N_HEADS * HD)
+    one = torch.full((N_HEADS, HD), float("nan"), dtype=torch.float32, device="cuda")
+    attn.attn_decode_kv_gate(step, 0, dev(q), dev(kb), dev(vb), acc, ml, one, dev(gate), N_HEADS, N_KV,
+                             HD, stride, SCALE, splits)
+    torch.cuda.synchronize()
+    assert torch.equal(one, two)
+    want = orc.q_gate(orc.attn_decode_kv(q, kb, vb, N_HEADS, N_KV, HD, seq, SCALE, stride=stride),
+                      gate.ravel())
+    ok, _, _ = report("gated decode seq 5000", want, host(one).ravel(), *KERNEL_CLASS)
+    assert ok
+
+
+def test_gated_batch_with_mtp_slots():
+    depths = [700, 33, 4000, 1]
+    cols = [3, 1, 2, 1]
+    stride = 4352
+    q, kc, vc, pos = make_slots(depths, cols, stride, 0x6A7E_0002)
+    rows = len(pos)
+    gate = orc.Rng(0x6A7E_0003).normal_array((rows, N_HEADS, HD))
+    splits = attn.batch_splits(stride, N_KV, len(depths))
+    acc, ml = decode_scratch(N_HEADS, splits, rows)
+    args = (N_HEADS, N_KV, HD, stride, SCALE, splits, N_KV * stride * ROW, N_HEADS * splits * HD,
+            N_HEADS * splits * 2, N_HEADS * HD, cols)
+    p = torch.tensor(pos, dtype=torch.int32, device="cuda")
+    two = torch.full((rows, N_HEADS, HD), float("nan"), dtype=torch.float32, device="cuda")
+    attn.attn_decode_batch_cols(0, p, dev(q), dev(kc), dev(vc), acc, ml, two, *args)
+    attn.q_gate(two, dev(gate), two, rows * N_HEADS * HD)
+    one = torch.full((rows, N_HEADS, HD), float("nan"), dtype=torch.float32, device="cuda")
+    attn.attn_decode_batch_cols_gate(0, p, dev(q), dev(kc), dev(vc), acc, ml, one, dev(gate), *args)
+    torch.cuda.synchronize()
+    assert torch.equal(one, two)
+    row = 0
+    for s, c in enumerate(cols):
+        for j in range(c):
+            want = orc.q_gate(orc.attn_decode_kv(q[row], kc[s], vc[s], N_HEADS, N_KV, HD, pos[row][1], SCALE,
+                                                 stride=stride), gate[row].ravel())
+            assert orc.compare(want, host(one)[row].ravel(), *KERNEL_CLASS)[0], (s, j)
+            row += 1
