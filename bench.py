@@ -338,6 +338,38 @@ def bench_front(torch, attn, tokens, steps):
                          "frac": gbs / HBM_PEAK_GBS, "traffic": None, "kernel": "front_kernel"}}
 
 
+def random_q8_0_weights(torch, m, k, gen):
+    """[m][k/32] Q8_0 blocks with random payloads and the reference's case scale 2^-10 (f16 0x1400)."""
+    w = torch.randint(0, 256, (m * (k // 32), 34), dtype=torch.uint8, device="cuda", generator=gen)
+    w[:, 0] = 0x00
+    w[:, 1] = 0x14
+    return w.reshape(-1)
+
+
+def bench_gemv(torch, attn, rows, steps, layers, m=5120, k=6144):
+    """Output projection W_o (Q8_0, 6144 -> 5120) over `rows` activation rows, rotating over
+    `layers` distinct matrices (33.4 MB each) so the weights come from HBM."""
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(0x5EED0007)
+    ws = [random_q8_0_weights(torch, m, k, gen) for _ in range(layers)]
+    x = torch.randn((rows, k), device="cuda", generator=gen) * 0.5
+    y = torch.empty((rows, m), device="cuda")
+    for w in ws:
+        attn.gemv_q8_0_rows(w, x, y, m, k, rows)
+    with Timer(torch) as t:
+        for _ in range(steps):
+            for w in ws:
+                attn.gemv_q8_0_rows(w, x, y, m, k, rows)
+    us = t.ms * 1e3 / (steps * layers)
+    nbytes = m * (k // 32) * 34 * ((rows + 15) // 16)
+    gbs = nbytes / (us * 1e-6) / 1e9
+    return {"workload": f"W_o projection, Q8_0 {m}x{k}, {rows} activation rows",
+            "us_per_layer": us, "weight_bytes": m * (k // 32) * 34, "layers_rotated": layers,
+            "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": gbs / HBM_PEAK_GBS, "traffic": None, "kernel": "gemv_q8_rows_kernel",
+                         "bytes_per_launch": nbytes, "launch_us": us}}
+
+
 def bench_copycal(torch, steps):
     """Plain device copy of a known size: the yardstick the HBM traffic counters
     (FETCH_SIZE / WRITE_SIZE) are scaled by."""
@@ -398,7 +430,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--main-only", action="store_true", help="skip the 'also' workloads")
     ap.add_argument("--only", default="", help="run one workload alone (prefill672, decode8k, "
-                    "decode32k, decode128k, chunk100k, batch16, front672, copycal) for profiling; prints its object")
+                    "decode32k, decode128k, chunk100k, batch16, front672, decode32k_q4, gemv1, gemv4, gemv16, copycal) for profiling; prints its object")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -428,6 +460,9 @@ def main() -> int:
             "copycal": lambda: bench_copycal(torch, K),
             "front672": lambda: bench_front(torch, attn, 672, max(K, 20)),
             "decode32k_q4": lambda: bench_decode(torch, attn, 32768, max(K, 20), 3, LAYERS, 1),
+            "gemv1": lambda: bench_gemv(torch, attn, 1, max(K // 4, 10), LAYERS),
+            "gemv4": lambda: bench_gemv(torch, attn, 4, max(K // 4, 10), LAYERS),
+            "gemv16": lambda: bench_gemv(torch, attn, 16, max(K // 4, 10), LAYERS),
         }[args.only]
         print(json.dumps(fn()))
         return 0

@@ -35,6 +35,7 @@ EXPORTS = [
     "hipml_attn_decode_kv_gate", "hipml_attn_decode_batch_cols_gate",
     "hipml_attn_chunk_q8_split", "hipml_attn_chunk_q8_split_gate", "hipml_q_gate_f32",
     "hipml_attn_front_f32", "hipml_attn_chunk_front_f32",
+    "hipml_gemv_q8_0_rows",
 ]
 
 
@@ -95,6 +96,7 @@ def lib() -> C.CDLL:
             "hipml_q_gate_f32": (i, [vp, vp, vp, vp, sz]),
             "hipml_attn_front_f32": (i, [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, i, i, vp, f, f]),
             "hipml_attn_chunk_front_f32": (i, [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, f, f, i, i]),
+            "hipml_gemv_q8_0_rows": (i, [vp, vp, vp, vp, i, i, i]),
         }
         for name, (res, args) in sig.items():
             fn = getattr(l, name)
@@ -322,6 +324,13 @@ def chunk_scratch(tokens: int, n_head: int, splits: int, device="cuda"):
 def q_gate(x, gate, y, n=None, stream=None):
     n = x.numel() if n is None else n
     _check(lib().hipml_q_gate_f32(_stream(stream), _p(x), _p(gate), _p(y), n))
+
+
+# ---- projections over Q8_0 weights ------------------------------------------------------------------
+
+def gemv_q8_0_rows(w, x, y, m, k, rows, stream=None):
+    """`AttnLayer::gemv` / `gemv_rows` / `gemv_batched` over a Q8_0 weight matrix: y[rows][m]."""
+    _check(lib().hipml_gemv_q8_0_rows(_stream(stream), _p(w), _p(x), _p(y), m, k, rows))
 
 
 # ---- cache owner ------------------------------------------------------------------------------------

@@ -19,6 +19,7 @@ SOURCES = [
     ("exact.hip", ["-ffp-contract=off"]),
     ("decode.hip", []),
     ("prefill.hip", []),
+    ("proj.hip", []),
     ("api.cpp", ["-x", "hip"]),
 ]
 

@@ -700,4 +700,28 @@ int hipml_q_gate_f32(hipml_stream_t stream, const float *x, const float *gate, f
     return launch_q_gate(as_stream(stream), x, gate, y, n);
 }
 
+// ---- projections over Q8_0 weights ----------------------------------------------------------------
+
+int hipml_gemv_q8_0_rows(hipml_stream_t stream, const void *w, const float *x, float *y, int m, int k,
+                         int rows)
+{
+    clear_error();
+    REQUIRE_PTR(w);
+    REQUIRE_PTR(x);
+    REQUIRE_PTR(y);
+    if (m < 1)
+        return fail(HIPML_ATTN_E_RANGE, "m %d must be positive", m);
+    if (k < 64 || k % 64 != 0)
+        return fail(HIPML_ATTN_E_RANGE, "k %d must be a positive multiple of 64 (two Q8_0 blocks: rows "
+                                        "stay dword aligned)", k);
+    if (rows < 1 || rows > 128)
+        return fail(HIPML_ATTN_E_RANGE, "rows %d outside 1..128", rows);
+    if (((uintptr_t)w & 3) != 0)
+        return fail(HIPML_ATTN_E_RANGE, "w must be 4-byte aligned");
+    int rc = check_aligned16(x, "x");
+    if (rc)
+        return rc;
+    return launch_gemv_q8_rows(as_stream(stream), static_cast<const uint8_t *>(w), x, y, m, k, rows);
+}
+
 } // extern "C"

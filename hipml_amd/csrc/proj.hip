@@ -1,0 +1,370 @@
+// Projections over Q8_0 weight matrices for gfx950 (wave64, MFMA): the step after the attention
+// core (the output projection W_o) and, with other shapes, the one before it (W_q, W_k, W_v).
+//
+// W is [m][k/32] blocks of 34 bytes (f16 scale d, 32 int8), row-major; y[r][row] = sum_k W[row][k] x[r][k]
+// (crates/hipml-core/src/quant.rs:653-675, crates/hipml-core/src/ops.rs:102-104,136-176).
+//
+// gemv_q8_rows_kernel: up to 4 activation rows per pass, bound by streaming W once from HBM.
+//   All MFMAs are v_mfma_f32_16x16x32_f16 with A = x (activation rows), B = W (16 weight rows),
+//   one q8 block = one contraction, so the f16 block scale multiplies an exact integer dot product
+//   in fp32: acc += d * (x . q), as the CPU definition's d*q products summed in fp32.
+//   Fetch: a step is a pair of blocks of one weight row, 68 bytes at a dword boundary.  Lane 4*r + g
+//   requests, with dword-aligned loads only, the 12 bytes that hold quarter g of the even block
+//   (2 bytes in, realigned with alignbit) and the 8 of the odd block's quarter; the scales ride
+//   along in lanes g = 0 and g = 3.  The four lanes of a quad read contiguous bytes.  (The MFMA's own
+//   lane order, row = lane % 16, with 2-byte aligned 64-bit loads made every lane several requests
+//   of its own: 9.5 M cache accesses per call and 1.0 TB/s.)  One ds_bpermute per register then
+//   moves the data to the MFMA lane (row lm, quarter lg).  The C
+//   tile puts weight row lm back in lane lm (rows of C are activation rows), where its scale is.
+//   int8 -> f16 exactly: byte b^0x80 = b+128 under a high byte 0x64 is the f16 1024 + (b+128);
+//   one packed f16 subtract of 1152 leaves b.  x enters as hi + lo f16 halves (two MFMAs, ~22 bits),
+//   converted once per workgroup into LDS in operand order: that is what limits a pass to 4 rows.
+//   The waves of a workgroup split k; a wave requests the activations first, then two chunks of
+//   its weight blocks (all of them for k = 6144) before it waits for anything, and the partial sums
+//   meet in LDS in a fixed order (no atomics: the result does not depend on timing).
+
+#include "common.h"
+
+namespace hipml {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
+typedef uint32_t uint2a4 __attribute__((ext_vector_type(2), aligned(4)));
+typedef uint32_t uint3a4 __attribute__((ext_vector_type(3), aligned(4)));
+
+constexpr int kQ8Block = 34;
+
+#ifdef GEMV_TIMING
+// debug builds: per-workgroup phase timestamps (100 MHz wall clock), 8 slots per workgroup
+__device__ unsigned long long g_gemv_t[8 * 1024];
+#define GSTAMP(i) do { if ((threadIdx.x & 63) == 0 && blockIdx.y == 0 && blockIdx.x < 1024 && (threadIdx.x >> 6) == ((i) >> 3)) g_gemv_t[blockIdx.x * 8 + ((i) & 7)] = wall_clock64(); } while (0)
+extern "C" int hipml_dbg_read_gemv(unsigned long long *host, size_t n)
+{
+    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_gemv_t), n * 8);
+}
+#else
+#define GSTAMP(i) do { } while (0)
+#endif
+
+// 8 int8 (two dwords) -> 8 f16 holding the same integers, exactly.
+__device__ __forceinline__ half8 int8x8_to_f16(uint32_t w0, uint32_t w1)
+{
+    const uint32_t x0 = w0 ^ 0x80808080u, x1 = w1 ^ 0x80808080u;
+    const uint32_t hi = 0x64646464u;
+    uint4v r;
+    r[0] = __builtin_amdgcn_perm(hi, x0, 0x04010400u);
+    r[1] = __builtin_amdgcn_perm(hi, x0, 0x04030402u);
+    r[2] = __builtin_amdgcn_perm(hi, x1, 0x04010400u);
+    r[3] = __builtin_amdgcn_perm(hi, x1, 0x04030402u);
+    half8 h = __builtin_bit_cast(half8, r);
+    const half8 off = {1152, 1152, 1152, 1152, 1152, 1152, 1152, 1152};
+    return h - off;
+}
+
+// 8 f32 -> hi and lo f16 halves with hi + lo = x to ~22 bits.
+__device__ __forceinline__ void split_hi_lo(const float4v &a, const float4v &b, half8 &hi, half8 &lo)
+{
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const float x0 = j < 2 ? a[2 * j] : b[2 * j - 4];
+        const float x1 = j < 2 ? a[2 * j + 1] : b[2 * j - 3];
+        const half2v h = __builtin_bit_cast(half2v, __builtin_amdgcn_cvt_pkrtz(x0, x1));
+        const half2v l =
+            __builtin_bit_cast(half2v, __builtin_amdgcn_cvt_pkrtz(x0 - (float)h[0], x1 - (float)h[1]));
+        hi[2 * j] = h[0];
+        hi[2 * j + 1] = h[1];
+        lo[2 * j] = l[0];
+        lo[2 * j + 1] = l[1];
+    }
+}
+
+// One chunk of a wave's steps, as fetched.  A step is a pair of blocks of one weight row (68 bytes,
+// dword aligned): the fetch lane of k quarter g holds bytes 8g..8g+11 of the pair (the even block's
+// quarter sits 2 bytes in; g = 0 also catches the even scale, g = 3 the odd one) and the odd block's
+// quarter, which is aligned.
+template <int TILES, int CH>
+struct GemvChunk {
+    uint3a4 e[CH][TILES];
+    uint2a4 o[CH][TILES];
+};
+
+constexpr int kGemvMaxRows = 4;        // activation rows per pass (their operands live in LDS)
+constexpr int kGemvLdsBudget = 128 << 10;
+
+// Activation rows per pass for a given k: as many (up to kGemvMaxRows) as keep the hi/lo operands of
+// the whole rows, 4 bytes per element, inside the LDS budget; 0 = k too large.
+__host__ __device__ inline int gemv_rows_per_pass(int k)
+{
+    const int fit = kGemvLdsBudget / (4 * k);
+    return fit > kGemvMaxRows ? kGemvMaxRows : fit;
+}
+static_assert(kGemvLdsBudget / 4 / 8 / 256 <= 16, "a pass is staged in one round of at most 16 groups per thread");
+
+// LDS: x operands [k/32 blocks][2*rp A rows: hi of rows 0..rp-1, then lo][4 quarters][8 x f16], then
+// the partial sums [WAVES][TILES][32 lanes] float4.  The hi and the lo halves are different rows of
+// ONE A operand: A rows 0..3 carry hi, rows 4..7 lo, so a block is one MFMA and the two partial
+// products come out in lanes 0..15 (hi) and 16..31 (lo) of the C tile.
+template <int WAVES, int TILES, int CH, int XG>
+__global__ void __launch_bounds__(64 * WAVES, TILES == 1 ? 2 : 1) gemv_q8_rows_kernel(const uint8_t *__restrict__ w,
+                                                                const float *__restrict__ x,
+                                                                float *__restrict__ y, int m, int k,
+                                                                int rows, int rp)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int lm = lane & 15, lg = lane >> 4; // MFMA operand lane: weight row lm, k quarter lg
+    const int fr = lane >> 2, fg = lane & 3;  // fetch lane: weight row fr, k quarter fg
+    const int pull = (lm * 4 + lg) * 4;       // byte address of the fetch lane that holds this lane's operand
+    const int nb = k >> 5;
+    const size_t row_bytes = (size_t)nb * kQ8Block;
+    const int m0 = blockIdx.x * (16 * TILES);
+    const int r0 = blockIdx.y * rp;
+    const int nrows = rows - r0 < rp ? rows - r0 : rp;
+    const int nu = nb >> 1; // steps: pairs of blocks
+    const int u_lo = (int)((long)wave * nu / WAVES), u_hi = (int)((long)(wave + 1) * nu / WAVES);
+    float4v *red = reinterpret_cast<float4v *>(lds + (size_t)nb * rp * 128);
+    const int per_row = k >> 3; // 8-element groups of one activation row
+
+    // ---- 1. this thread's share of the activations, requested first (they are waited for first) --
+    // group e = 8 consecutive k of one row; (row, e) pairs are dealt round-robin to the threads
+    const int groups = nrows * (k >> 3);
+    // XG groups in flight per thread and round; a thread with fewer left wraps around to groups that
+    // are not its own (loaded, not stored) rather than all such threads asking for one address
+    float4v xa[XG], xb[XG];
+    auto x_issue = [&](int g0) {
+#pragma unroll
+        for (int i = 0; i < XG; i++) {
+            int g = g0 + i * 64 * WAVES;
+            g = g < groups ? g : g % groups;
+            const float *p = x + (size_t)r0 * k + (size_t)g * 8; // rows are contiguous: group g of the pass
+
+            xa[i] = *reinterpret_cast<const float4v *>(p);
+            xb[i] = *reinterpret_cast<const float4v *>(p + 4);
+        }
+    };
+    auto x_store = [&](int g0) {
+#pragma unroll
+        for (int i = 0; i < XG; i++) {
+            const int g = g0 + i * 64 * WAVES;
+            if (g < groups) {
+                const int r = rp == 1 ? 0 : g / per_row, e = g - r * per_row;
+                half8 hi, lo;
+                split_hi_lo(xa[i], xb[i], hi, lo);
+                uint8_t *blk = lds + (size_t)(e >> 2) * rp * 128 + (e & 3) * 16;
+                *reinterpret_cast<half8 *>(blk + r * 64) = hi;
+                *reinterpret_cast<half8 *>(blk + (rp + r) * 64) = lo;
+            }
+        }
+    };
+    GSTAMP(0);
+    x_issue(threadIdx.x);
+    // every wave's activation requests enter the CU's memory pipeline before any wave's weight
+    // requests: the pipeline serves them in order, and the first barrier below waits for the last
+    // wave's activations
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- 2. the first two chunks of this wave's weight blocks ------------------------------------
+    // rows past the end are clamped: they load (and compute) a duplicate that is never stored
+    const uint8_t *wp[TILES];
+#pragma unroll
+    for (int t = 0; t < TILES; t++) {
+        const int row = m0 + t * 16 + fr < m ? m0 + t * 16 + fr : m - 1;
+        wp[t] = w + (size_t)row * row_bytes;
+    }
+    typedef GemvChunk<TILES, CH> Chunk;
+    auto fetch = [&](Chunk &c, int u0) {
+#pragma unroll
+        for (int i = 0; i < CH; i++) {
+            int uc = u0 + i < u_hi ? u0 + i : u_hi - 1;
+            uc = uc < 0 ? 0 : uc;
+#pragma unroll
+            for (int t = 0; t < TILES; t++) {
+                const uint8_t *unit = wp[t] + (size_t)uc * (2 * kQ8Block);
+                c.e[i][t] = *reinterpret_cast<const uint3a4 *>(unit + fg * 8);
+                c.o[i][t] = *reinterpret_cast<const uint2a4 *>(unit + 36 + fg * 8);
+            }
+        }
+    };
+    Chunk A, B;
+    fetch(A, u_lo);
+    fetch(B, u_lo + CH);
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- 3. activations to LDS as MFMA operands -----------------------------------------------
+    GSTAMP(1);
+    x_store(threadIdx.x); // XG covers every group: the launcher sizes the pass for that
+    GSTAMP(2);
+    __syncthreads();
+    GSTAMP(3);
+
+    // ---- 4. the block steps --------------------------------------------------------------------
+    float4v acc[TILES];
+#pragma unroll
+    for (int t = 0; t < TILES; t++)
+        acc[t] = (float4v){0, 0, 0, 0};
+    // A row lm: hi of activation row lm for lm < 4, lo of row lm - 4 for 4 <= lm < 8; the rest, and
+    // rows past the live ones, repeat a valid slot (their products are never read)
+    const int ar = (lm & 3) < nrows ? (lm & 3) : nrows - 1;
+    const uint8_t *xop = lds + ((size_t)(((lm >> 2) & 1) * rp + ar) * 4 + lg) * 16;
+    // One step = operands staged (realign, gather scales, move to the MFMA lanes, read x), then the
+    // arithmetic; a step's staging is issued before the previous step's arithmetic so the LDS
+    // round trips are covered, and the scheduler may not move anything across a step: a step waits
+    // for its own two loads only.
+    struct Staged {
+        uint32_t q[TILES][4];
+        uint32_t ds[TILES];
+        half8 x0, x1;
+    };
+    auto stage = [&](Staged &s, const Chunk &c, int i, int u) {
+        const int uc = u < u_hi ? u : u_hi - 1;
+#pragma unroll
+        for (int t = 0; t < TILES; t++) {
+            const uint3a4 e = c.e[i][t];
+            // in the fetch lane: the even quarter realigned; both scales gathered in the quad's lane 0
+            const int e2_of_g3 = __builtin_amdgcn_update_dpp(0, (int)e[2], 0xFF, 0xf, 0xf, true);
+            const int sc = (int)((e[0] & 0xffffu) | ((uint32_t)e2_of_g3 & 0xffff0000u));
+            s.q[t][0] = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)__builtin_amdgcn_alignbit(e[1], e[0], 16));
+            s.q[t][1] = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)__builtin_amdgcn_alignbit(e[2], e[1], 16));
+            s.q[t][2] = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)c.o[i][t][0]);
+            s.q[t][3] = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)c.o[i][t][1]);
+            s.ds[t] = (uint32_t)__builtin_amdgcn_ds_bpermute(lm * 16, sc);
+        }
+        s.x0 = *reinterpret_cast<const half8 *>(xop + (size_t)uc * rp * 256);
+        s.x1 = *reinterpret_cast<const half8 *>(xop + (size_t)uc * rp * 256 + rp * 128);
+    };
+    auto math = [&](const Staged &s, int u) {
+#pragma unroll
+        for (int t = 0; t < TILES; t++) {
+            const float d0 = u < u_hi ? (float)__builtin_bit_cast(_Float16, (uint16_t)(s.ds[t] & 0xffffu)) : 0.0f;
+            const float d1 = u < u_hi ? (float)__builtin_bit_cast(_Float16, (uint16_t)(s.ds[t] >> 16)) : 0.0f;
+            const half8 w0 = int8x8_to_f16(s.q[t][0], s.q[t][1]), w1 = int8x8_to_f16(s.q[t][2], s.q[t][3]);
+            float4v p0 = {0, 0, 0, 0}, p1 = {0, 0, 0, 0};
+            p0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(s.x0, w0, p0, 0, 0, 0);
+            p1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(s.x1, w1, p1, 0, 0, 0);
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                acc[t][j] = fmaf(d1, p1[j], fmaf(d0, p0[j], acc[t][j]));
+        }
+    };
+    auto compute = [&](const Chunk &c, int u0) {
+        Staged s0, s1;
+        stage(s0, c, 0, u0);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < CH; i += 2) {
+            if (i + 1 < CH)
+                stage(s1, c, i + 1, u0 + i + 1);
+            __builtin_amdgcn_sched_barrier(0);
+            math(s0, u0 + i);
+            __builtin_amdgcn_sched_barrier(0);
+            if (i + 1 < CH) {
+                if (i + 2 < CH)
+                    stage(s0, c, i + 2, u0 + i + 2);
+                __builtin_amdgcn_sched_barrier(0);
+                math(s1, u0 + i + 1);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    };
+    // The first two chunks (all of a wave's steps up to k = 64 * 2 * CH * WAVES) are straight-line
+    // code, so each step waits for exactly its own loads while the rest are still in flight.
+    // Longer rows continue in a loop that fetches and consumes two chunks per turn; nothing is
+    // carried in registers from one turn to the next (carried chunks made the compiler copy them at
+    // the loop head, behind a wait for every outstanding load).
+    if (u_hi > u_lo) {
+        compute(A, u_lo);
+        GSTAMP(4);
+        compute(B, u_lo + CH);
+        GSTAMP(5);
+        for (int u = u_lo + 2 * CH; u < u_hi; u += 2 * CH) {
+            fetch(A, u);
+            fetch(B, u + CH);
+            compute(A, u);
+            compute(B, u + CH);
+        }
+    }
+
+    // ---- 5. the k slices meet in a fixed order: lanes 0..15 hold the hi products of activation
+    // rows 0..3, lanes 16..31 the lo products ---------------------------------------------------
+    if (lg < 2) {
+#pragma unroll
+        for (int t = 0; t < TILES; t++)
+            red[(wave * TILES + t) * 32 + lane] = acc[t];
+    }
+    __syncthreads();
+    GSTAMP(6);
+    if (threadIdx.x < 16 * TILES) {
+        const int t = threadIdx.x >> 4, l = threadIdx.x & 15;
+        float4v hi = red[t * 32 + l], lo = red[t * 32 + 16 + l];
+#pragma unroll
+        for (int u = 1; u < WAVES; u++) {
+            hi += red[(u * TILES + t) * 32 + l];
+            lo += red[(u * TILES + t) * 32 + 16 + l];
+        }
+        const float4v s = hi + lo;
+        const int row = m0 + t * 16 + l;
+        if (row < m) {
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                if (j < nrows)
+                    y[(size_t)(r0 + j) * m + row] = s[j];
+        }
+    }
+}
+
+template <int WAVES, int TILES, int CH, int XG>
+static int launch_gemv_xg(hipStream_t st, const uint8_t *w, const float *x, float *y, int m, int k,
+                          int rows, int rp)
+{
+    const size_t lds = (size_t)(k >> 5) * rp * 128 + (size_t)WAVES * TILES * 32 * sizeof(float4v);
+    auto kern = gemv_q8_rows_kernel<WAVES, TILES, CH, XG>;
+    static bool raised = false; // the limit is a property of the function: set once per process
+    if (!raised) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 << 10);
+        if (e != hipSuccess)
+            return fail((int)e, "hipFuncSetAttribute(gemv LDS) failed: %d (%s)", (int)e, hipGetErrorString(e));
+        raised = true;
+    }
+    const dim3 grid((unsigned)((m + 16 * TILES - 1) / (16 * TILES)), (unsigned)((rows + rp - 1) / rp), 1);
+    hipLaunchKernelGGL(kern, grid, dim3(64 * WAVES, 1, 1), lds, st, w, x, y, m, k, rows, rp);
+    return launched("gemv_q8_0_rows");
+}
+
+template <int WAVES, int TILES, int CH>
+static int launch_gemv_variant(hipStream_t st, const uint8_t *w, const float *x, float *y, int m, int k,
+                               int rows, int rp)
+{
+    // 8-element groups of the activations per thread
+    const int need = (rp * (k >> 3) + 64 * WAVES - 1) / (64 * WAVES);
+    if (need <= 2)
+        return launch_gemv_xg<WAVES, TILES, CH, 2>(st, w, x, y, m, k, rows, rp);
+    if (need <= 4)
+        return launch_gemv_xg<WAVES, TILES, CH, 4>(st, w, x, y, m, k, rows, rp);
+    if (need <= 8)
+        return launch_gemv_xg<WAVES, TILES, CH, 8>(st, w, x, y, m, k, rows, rp);
+    return launch_gemv_xg<WAVES, TILES, CH, 16>(st, w, x, y, m, k, rows, rp);
+}
+
+int launch_gemv_q8_rows(hipStream_t st, const uint8_t *w, const float *x, float *y, int m, int k, int rows)
+{
+    int rp = gemv_rows_per_pass(k);
+    if (rp < 1)
+        return fail(HIPML_ATTN_E_RANGE, "k %d: one activation row does not fit the LDS operand buffer", k);
+    rp = rows < rp ? rows : rp;
+    // One 16-row weight tile per workgroup keeps the kernel inside 128 registers, so two workgroups
+    // share a CU and the 320 workgroups of a 5120-row matrix start together (workgroups start in
+    // windows of as many as fit the chip; a second window opens when the first has drained).  With
+    // 3-4 rows per pass the activations' staging needs more registers: two tiles per workgroup,
+    // half as many workgroups, one per CU (measured at 5120 x 6144: 1 row 12.2 vs 15.0 us, 4 rows
+    // 18.5 vs 16.7 us).
+    if (rp <= 2)
+        return launch_gemv_variant<8, 1, 6>(st, w, x, y, m, k, rows, rp);
+    return launch_gemv_variant<8, 2, 6>(st, w, x, y, m, k, rows, rp);
+}
+
+} // namespace hipml

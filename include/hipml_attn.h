@@ -265,6 +265,21 @@ int hipml_attn_chunk_q8_split_gate(hipml_stream_t stream, const float *q, const 
 int hipml_q_gate_f32(hipml_stream_t stream, const float *x, const float *gate, float *y,
                      size_t n);
 
+/* ---- projections over Q8_0 weight matrices (the steps either side of the attention core) ---- */
+
+/* y[r][row] = sum_k W[row][k] * x[r][k] for r < rows: W is m rows of k/32 Q8_0 blocks (34 bytes:
+ * f16 scale, 32 int8) at a 4-byte aligned address, x is f32 [rows][k] (16-byte aligned), y is f32
+ * [rows][m]; k a multiple of 64 up to 32768, 1 <= rows <= 128.
+ * W streams from memory once per 4 rows; fp32 accumulation of exact integer block products (the
+ * activations enter as hi + lo f16 halves), so every row has the precision class of the
+ * reference's f32 GEMV kernels and row r does not depend on `rows`.
+ * Replaces AttnLayer::gemv / gemv_rows / gemv_batched over a Q8_0 ResidentMat (the output
+ * projection of apply_output / output_rows, and W_q, W_k, W_v in prepare_rows),
+ * crates/hipml-kernels/src/attn_gpu.rs:843-846,967-1023,1066-1117 -> gemv_q8_0 / gemv_q8_0_b,
+ * crates/hipml-kernels/kernels/gemv_q8_0.hip:20-66. */
+int hipml_gemv_q8_0_rows(hipml_stream_t stream, const void *w, const float *x, float *y, int m,
+                         int k, int rows);
+
 #ifdef __cplusplus
 }
 #endif

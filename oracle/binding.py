@@ -83,6 +83,10 @@ def _declare(l: C.CDLL) -> None:
                                            sz, sz, _szp, sz, f32, _f32p]),
         "orc_attn_chunk_kv": (None, [_f32p, _u8p, _u8p, sz, sz, sz, sz, sz, sz, f32, i, _i32p, sz,
                                      i, _f32p]),
+        "orc_dequant_q8_0": (None, [_u8p, _f32p]),
+        "orc_gemv_q8_0": (None, [_u8p, _f32p, sz, sz, _f32p]),
+        "orc_gemm_q8_0": (None, [_u8p, _f32p, sz, sz, sz, i, _f32p]),
+        "orc_random_q8_0_bytes": (None, [C.POINTER(_Rng), sz, _u8p]),
         "orc_compare": (i, [_f32p, _f32p, sz, f32, f32, _f32p, _f32p]),
     }
     for name, (res, args) in sig.items():
@@ -323,6 +327,40 @@ def attn_chunk_kv(q, k, v, n_heads, n_kv, head_dim, pos0, tokens, stride, scale,
     out = np.empty((n_rows, n_heads, head_dim), dtype=np.float32)
     lib().orc_attn_chunk_kv(_pf(q), _pb(k), _pb(v), n_heads, n_kv, head_dim, pos0, tokens, stride,
                             scale, dtype, rp, n_rows, n_threads, _pf(out))
+    return out
+
+
+# ---- Q8_0 weight matrices ---------------------------------------------------------
+
+def dequant_q8_0(block) -> np.ndarray:
+    block = _b(block)
+    assert block.size == 34
+    out = np.empty(32, dtype=np.float32)
+    lib().orc_dequant_q8_0(_pb(block), _pf(out))
+    return out
+
+
+def gemv_q8_0(w, x, m, k) -> np.ndarray:
+    w, x = _b(w), _f(x)
+    assert w.size == m * (k // 32) * 34 and x.size == k
+    y = np.empty(m, dtype=np.float32)
+    lib().orc_gemv_q8_0(_pb(w), _pf(x), m, k, _pf(y))
+    return y
+
+
+def gemm_q8_0(w, x, tokens, m, k, n_threads=1) -> np.ndarray:
+    """y[tokens][m]; n_threads > 1 spreads weight rows over OpenMP threads (each output is still the
+    scalar in-order sum)."""
+    w, x = _b(w), _f(x)
+    assert w.size == m * (k // 32) * 34 and x.size == tokens * k
+    y = np.empty((tokens, m), dtype=np.float32)
+    lib().orc_gemm_q8_0(_pb(w), _pf(x), tokens, m, k, n_threads, _pf(y))
+    return y
+
+
+def random_q8_0_bytes(rng: "Rng", nblocks: int) -> np.ndarray:
+    out = np.empty(nblocks * 34, dtype=np.uint8)
+    lib().orc_random_q8_0_bytes(C.byref(rng._r), nblocks, _pb(out))
     return out
 
 

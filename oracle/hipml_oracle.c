@@ -591,3 +591,69 @@ int orc_compare(const float *expected, const float *actual, size_t n, float abs_
         *max_rel_out = max_rel;
     return (max_abs <= abs_tol || max_rel <= rel_tol) ? 1 : 0;
 }
+
+/* ---- Q8_0 weight matrices: quant.rs:433-443, 653-675, 785-796, 846-854; ops.rs:102-104, 136-176 -- */
+
+void orc_dequant_q8_0(const uint8_t *block, float *out)
+{
+    const float d = orc_f16_to_f32((uint16_t)(block[0] | (block[1] << 8)));
+    for (int i = 0; i < 32; i++)
+        out[i] = d * (float)(int8_t)block[2 + i];
+}
+
+void orc_gemv_q8_0(const uint8_t *w, const float *x, size_t m, size_t k, float *y)
+{
+    const size_t nb = k / 32, row_bytes = nb * 34;
+    float tmp[32];
+    for (size_t row = 0; row < m; row++) {
+        const uint8_t *rd = w + row * row_bytes;
+        float acc = 0.0f;
+        for (size_t b = 0; b < nb; b++) {
+            orc_dequant_q8_0(rd + b * 34, tmp);
+            const float *xb = x + b * 32;
+            for (int l = 0; l < 32; l++)
+                acc += tmp[l] * xb[l];
+        }
+        y[row] = acc;
+    }
+}
+
+void orc_gemm_q8_0(const uint8_t *w, const float *x, size_t tokens, size_t m, size_t k,
+                   int n_threads, float *y)
+{
+    const size_t nb = k / 32, row_bytes = nb * 34;
+#pragma omp parallel for schedule(static) num_threads(n_threads > 1 ? n_threads : 1)
+    for (long r = 0; r < (long)m; r++) {
+        float *row = (float *)malloc(k * sizeof(float));
+        const uint8_t *rd = w + (size_t)r * row_bytes;
+        for (size_t b = 0; b < nb; b++)
+            orc_dequant_q8_0(rd + b * 34, row + b * 32);
+        for (size_t t = 0; t < tokens; t++) {
+            const float *xr = x + t * k;
+            float acc = 0.0f;
+            for (size_t j = 0; j < k; j++)
+                acc += row[j] * xr[j];
+            y[t * m + (size_t)r] = acc;
+        }
+        free(row);
+    }
+}
+
+void orc_random_q8_0_bytes(orc_rng *r, size_t nblocks, uint8_t *out)
+{
+    for (size_t blk = 0; blk < nblocks; blk++) {
+        uint8_t *b = out + blk * 34;
+        size_t i = 0;
+        while (i + 8 <= 34) {
+            uint64_t v = orc_rng_next_u64(r);
+            for (int j = 0; j < 8; j++)
+                b[i + j] = (uint8_t)(v >> (8 * j));
+            i += 8;
+        }
+        uint64_t tail = orc_rng_next_u64(r);
+        for (int j = 0; i + j < 34; j++)
+            b[i + j] = (uint8_t)(tail >> (8 * j));
+        b[0] = 0x00;
+        b[1] = 0x14;
+    }
+}

@@ -103,6 +103,19 @@ void orc_attn_chunk_kv(const float *q, const uint8_t *k, const uint8_t *v, size_
                        size_t n_kv, size_t head_dim, size_t pos0, size_t tokens, size_t stride,
                        float scale, int dtype, const int32_t *rows, size_t n_rows,
                        int n_threads, float *out);
+/* ---- Q8_0 weight matrices (the projections either side of the attention core) ------------
+ * crates/hipml-core/src/quant.rs:433-443 (dequant_q8_0), :653-675 (gemv_q8_0),
+ * crates/hipml-core/src/ops.rs:102-104,136-176 (gemm_q8_0), quant.rs:785-796,846-854
+ * (random_q8_0_bytes: eight bytes per next_u64 little-endian, then the scale bytes overwritten
+ * with f16 0x1400 = 2^-10). */
+void orc_dequant_q8_0(const uint8_t *block, float *out);
+/* y[m] = sum over blocks in order, within a block l = 0..31: acc += (d * q_l) * x_l. */
+void orc_gemv_q8_0(const uint8_t *w, const float *x, size_t m, size_t k, float *y);
+/* y[t][m]: the row is dequantized once, then acc += row[j] * x[t][j] for j ascending. */
+void orc_gemm_q8_0(const uint8_t *w, const float *x, size_t tokens, size_t m, size_t k,
+                   int n_threads, float *y);
+void orc_random_q8_0_bytes(orc_rng *r, size_t nblocks, uint8_t *out);
+
 /* crates/hipml-core/src/parity.rs:44-80.  Returns 1 when within tolerance
  * (max_abs <= abs_tol OR max_rel <= rel_tol). */
 int orc_compare(const float *expected, const float *actual, size_t n, float abs_tol,

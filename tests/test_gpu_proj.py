@@ -1,0 +1,115 @@
+"""Projections over Q8_0 weight matrices (the step after the attention core): HIP path through the
+C ABI vs the CPU oracle on the reference's case recipes (raw random block bytes with scale 2^-10,
+N(0,1) activations; crates/hipml-core/src/quant_parity.rs:80-86,125-133,
+crates/hipml-core/src/prefill_parity.rs:114-119,209-219).  Tolerance: the reference's Tol::DEFAULT
+(1e-4 abs OR 1e-3 rel) for its small cases; its LARGE_TOL (2e-3 / 3e-2) bounds the production
+shape, where the kernel is asserted at 2e-4 abs (outputs of magnitude ~10, both sides fp32 sums of
+6144 terms in different orders)."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+from oracle import binding as orc  # noqa: E402
+from hipml_amd import attn  # noqa: E402
+from gpu_util import dev, host, report  # noqa: E402
+
+DEFAULT = (1e-4, 1e-3)
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _init():
+    attn.init(0)
+
+
+def run_gemv(w, x, m, k, rows):
+    y = torch.full((rows, m), float("nan"), dtype=torch.float32, device="cuda")
+    attn.gemv_q8_0_rows(dev(w), dev(x), y, m, k, rows)
+    torch.cuda.synchronize()
+    return host(y)
+
+
+def test_reference_gemv_case_64x512():
+    r = orc.Rng(0x4B51_0005)
+    m, k = 64, 512
+    w = orc.random_q8_0_bytes(r, m * k // 32)
+    x = r.normal_array(k)
+    want = orc.gemv_q8_0(w, x, m, k)
+    got = run_gemv(w, x, m, k, 1)[0]
+    ok, _, _ = report("gemv_q8_0 64x512", want, got, *DEFAULT)
+    assert ok
+
+
+def test_reference_gemm_case_64x512_t4_and_skinny_200x512():
+    for seed, m, k, t in ((0x9F11_0003, 64, 512, 4), (0x5C11_0006, 200, 512, 4)):
+        r = orc.Rng(seed)
+        w = orc.random_q8_0_bytes(r, m * k // 32)
+        x = r.normal_array((t, k))
+        want = orc.gemm_q8_0(w, x, t, m, k)
+        got = run_gemv(w, x, m, k, t)
+        ok, _, _ = report(f"q8_0 rows {m}x{k} t={t}", want, got, *DEFAULT)
+        assert ok
+
+
+def test_integer_case_is_exact():
+    # d = 1 and small integer activations: every partial sum is an integer below 2^24, so any
+    # summation order gives the same f32 and the result must equal the oracle's bit for bit
+    r = orc.Rng(0x1234)
+    m, k, rows = 80, 1024, 5
+    w = orc.random_q8_0_bytes(r, m * k // 32).reshape(-1, 34)
+    w[:, 0], w[:, 1] = 0x00, 0x3C
+    x = np.round(r.normal_array((rows, k)) * 2).astype(np.float32)
+    want = orc.gemm_q8_0(w.ravel(), x, rows, m, k)
+    assert np.array_equal(run_gemv(w.ravel(), x, m, k, rows), want)
+
+
+@pytest.mark.parametrize("rows", [1, 3, 16, 17, 24])
+def test_output_projection_shape(rows):
+    # W_o of the model: 6144 -> 5120; activations of the size the gated attention output has
+    r = orc.Rng(0x0E00 + rows)
+    m, k = 5120, 6144
+    w = orc.random_q8_0_bytes(r, m * k // 32)
+    x = r.normal_array((rows, k), 0.5)
+    want = orc.gemm_q8_0(w, x, rows, m, k, n_threads=8)
+    got = run_gemv(w, x, m, k, rows)
+    ok, ma, _ = report(f"W_o 5120x6144 rows={rows}", want, got, 2e-4, 1e-3)
+    assert ok
+    # a row does not depend on how many rows travel with it
+    if rows == 3:
+        alone = run_gemv(w, x[1], m, k, 1)[0]
+        assert np.array_equal(alone, got[1])
+
+
+def test_ragged_shapes_and_scales():
+    # m not a multiple of the workgroup's row tile, k with fewer block pairs than k slices, real
+    # scales.  Outputs reach magnitude ~200 here, where two fp32 summation orders differ by ~1e-3: the
+    # reference bounds such cases with LARGE_TOL (2e-3 / 3e-2, quant_parity.rs:20-25); on top of that
+    # the kernel must be as close to the float64 value as the sequential fp32 sum is.
+    r = orc.Rng(0x7A66)
+    for m, k, rows in ((1, 64, 1), (33, 192, 2), (1000, 320, 7), (50, 4096, 16)):
+        w = orc.random_q8_0_bytes(r, m * k // 32).reshape(-1, 34)
+        scales = (r.uniform_array(w.shape[0]) * 0.05 + 0.001).astype(np.float16)
+        w[:, :2] = scales.view(np.uint8).reshape(-1, 2)
+        x = r.normal_array((rows, k))
+        want = orc.gemm_q8_0(w.ravel(), x, rows, m, k)
+        got = run_gemv(w.ravel(), x, m, k, rows)
+        ok, _, _ = report(f"q8_0 rows {m}x{k} t={rows}", want, got, 2e-3, 3e-2)
+        assert ok
+        blocks = w.reshape(m, k // 32, 34)
+        dense = (blocks[:, :, :2].copy().view(np.float16).astype(np.float64)
+                 * blocks[:, :, 2:].view(np.int8).astype(np.float64)).reshape(m, k)
+        exact = x.astype(np.float64) @ dense.T
+        assert np.max(np.abs(got - exact)) <= max(2 * np.max(np.abs(want - exact)), 1e-5)
+
+
+def test_argument_errors():
+    w = torch.zeros(34 * 4, dtype=torch.uint8, device="cuda")
+    x = torch.zeros(64, device="cuda")
+    y = torch.zeros(2, device="cuda")
+    with pytest.raises(attn.HipmlError):
+        attn.gemv_q8_0_rows(w, x, y, 2, 96, 1)     # k not a multiple of 64
+    with pytest.raises(attn.HipmlError):
+        attn.gemv_q8_0_rows(w, x, y, 2, 64, 129)   # too many rows
+    with pytest.raises(attn.HipmlError):
+        attn.gemv_q8_0_rows(w, x, y, 0, 64, 1)

@@ -358,3 +358,58 @@ def test_qg_split_layout(orc):
     q, g = orc.qg_split(qg, nh, hd)
     assert np.array_equal(q, [0, 1, 2, 3, 8, 9, 10, 11, 16, 17, 18, 19])
     assert np.array_equal(g, [4, 5, 6, 7, 12, 13, 14, 15, 20, 21, 22, 23])
+
+
+# ---- Q8_0 weight matrices (the output projection after the attention core) ----------------------
+
+def test_q8_0_weight_block_hand_vector(orc):
+    # crates/hipml-core/tests/quant_reference.rs:144-156: d = 0.5 (0x3800), q_i = i + 1
+    b = np.zeros(34, dtype=np.uint8)
+    b[0], b[1] = 0x00, 0x38
+    b[2:] = np.arange(1, 33, dtype=np.uint8)
+    assert np.array_equal(orc.dequant_q8_0(b), 0.5 * np.arange(1, 33, dtype=np.float32))
+    # negative payloads are two's-complement int8
+    b[2] = 0x80
+    assert orc.dequant_q8_0(b)[0] == -64.0
+
+
+def test_random_q8_0_bytes_layout(orc):
+    # quant.rs:785-796,846-854: the byte stream is next_u64() little-endian, five draws per block
+    # (8+8+8+8 and a 2-byte tail), scale bytes overwritten with 0x1400 = 2^-10
+    r, r2 = orc.Rng(0x4B51_0005), orc.Rng(0x4B51_0005)
+    w = orc.random_q8_0_bytes(r, 3).reshape(3, 34)
+    for blk in range(3):
+        draws = [r2.next_u64() for _ in range(5)]
+        want = b"".join(int(d).to_bytes(8, "little") for d in draws)[:34]
+        assert bytes(w[blk][2:]) == want[2:]
+        assert w[blk][0] == 0x00 and w[blk][1] == 0x14
+    assert orc.f16_to_f32(0x1400) == np.float32(2.0 ** -10)
+
+
+def test_gemv_and_gemm_q8_0_against_float64(orc):
+    # the reference's case shapes: gemv 64x512 (quant_parity.rs:125-133), gemm 64x512 t=4
+    # (prefill_parity.rs:209-219); the definition is a plain dot product over dequantized weights
+    r = orc.Rng(0x4B51_0005)
+    m, k = 64, 512
+    w = orc.random_q8_0_bytes(r, m * k // 32)
+    x = r.normal_array(k)
+    blocks = w.reshape(m, k // 32, 34)
+    d = blocks[:, :, :2].copy().view(np.float16).astype(np.float64)
+    dense = (d * blocks[:, :, 2:].view(np.int8).astype(np.float64)).reshape(m, k)
+    y = orc.gemv_q8_0(w, x, m, k)
+    assert np.max(np.abs(y - dense @ x.astype(np.float64))) < 1e-4
+    # an integer case is exact in f32 whatever the order: d = 1, x = small integers
+    wi = w.copy().reshape(-1, 34)
+    wi[:, 0], wi[:, 1] = 0x00, 0x3C
+    xi = np.round(x * 3).astype(np.float32)
+    dense_i = wi[:, 2:].view(np.int8).astype(np.float64).reshape(m, k)
+    assert np.array_equal(orc.gemv_q8_0(wi.ravel(), xi, m, k), (dense_i @ xi).astype(np.float32))
+    # gemm row t equals the gemv of x[t] (ops.rs:136-176 keeps the same j-ascending sum) ...
+    r = orc.Rng(0x9F11_0003)
+    w = orc.random_q8_0_bytes(r, m * k // 32)
+    xs = r.normal_array((4, k))
+    y = orc.gemm_q8_0(w, xs, 4, m, k)
+    for t in range(4):
+        assert np.array_equal(y[t], orc.gemv_q8_0(w, xs[t], m, k))
+    # ... whatever the thread count
+    assert np.array_equal(y, orc.gemm_q8_0(w, xs, 4, m, k, n_threads=4))
