@@ -370,6 +370,29 @@ def bench_gemv(torch, attn, rows, steps, layers, m=5120, k=6144):
                          "bytes_per_launch": nbytes, "launch_us": us}}
 
 
+def bench_gemm(torch, attn, tokens, steps, layers, m=5120, k=6144):
+    """Output projection of a prefill chunk: [tokens][6144] x W_o^T (Q8_0) on MFMA, f16 operands."""
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(0x5EED0008)
+    ws = [random_q8_0_weights(torch, m, k, gen) for _ in range(layers)]
+    x = torch.randn((tokens, k), device="cuda", generator=gen) * 0.5
+    y = torch.empty((tokens, m), device="cuda")
+    for w in ws:
+        attn.gemm_q8_0_f16(w, x, y, m, k, tokens)
+    with Timer(torch) as t:
+        for _ in range(steps):
+            for w in ws:
+                attn.gemm_q8_0_f16(w, x, y, m, k, tokens)
+    us = t.ms * 1e3 / (steps * layers)
+    flop = 2.0 * tokens * m * k
+    tf = flop / (us * 1e-6) / 1e12
+    return {"workload": f"W_o projection of a chunk, Q8_0 {m}x{k}, {tokens} tokens",
+            "us_per_layer": us, "flop": flop, "layers_rotated": layers,
+            "roofline": {"bound": "mfma", "achieved": tf, "peak": MFMA_F16_PEAK_TF, "unit": "TFLOP/s",
+                         "frac": tf / MFMA_F16_PEAK_TF, "traffic": None, "kernel": "gemm_q8_f16_kernel",
+                         "flop_per_launch": flop, "launch_us": us}}
+
+
 def bench_copycal(torch, steps):
     """Plain device copy of a known size: the yardstick the HBM traffic counters
     (FETCH_SIZE / WRITE_SIZE) are scaled by."""
@@ -430,7 +453,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--main-only", action="store_true", help="skip the 'also' workloads")
     ap.add_argument("--only", default="", help="run one workload alone (prefill672, decode8k, "
-                    "decode32k, decode128k, chunk100k, batch16, front672, decode32k_q4, gemv1, gemv4, gemv16, copycal) for profiling; prints its object")
+                    "decode32k, decode128k, chunk100k, batch16, front672, decode32k_q4, gemv1, gemv4, gemv16, gemm672, gemm2048, copycal) for profiling; prints its object")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -463,6 +486,8 @@ def main() -> int:
             "gemv1": lambda: bench_gemv(torch, attn, 1, max(K // 4, 10), LAYERS),
             "gemv4": lambda: bench_gemv(torch, attn, 4, max(K // 4, 10), LAYERS),
             "gemv16": lambda: bench_gemv(torch, attn, 16, max(K // 4, 10), LAYERS),
+            "gemm672": lambda: bench_gemm(torch, attn, 672, max(K // 10, 5), 4),
+            "gemm2048": lambda: bench_gemm(torch, attn, 2048, max(K // 20, 3), 4),
         }[args.only]
         print(json.dumps(fn()))
         return 0

@@ -35,7 +35,7 @@ EXPORTS = [
     "hipml_attn_decode_kv_gate", "hipml_attn_decode_batch_cols_gate",
     "hipml_attn_chunk_q8_split", "hipml_attn_chunk_q8_split_gate", "hipml_q_gate_f32",
     "hipml_attn_front_f32", "hipml_attn_chunk_front_f32",
-    "hipml_gemv_q8_0_rows",
+    "hipml_gemv_q8_0_rows", "hipml_gemm_q8_0_f16",
 ]
 
 
@@ -97,6 +97,7 @@ def lib() -> C.CDLL:
             "hipml_attn_front_f32": (i, [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, i, i, vp, f, f]),
             "hipml_attn_chunk_front_f32": (i, [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, f, f, i, i]),
             "hipml_gemv_q8_0_rows": (i, [vp, vp, vp, vp, i, i, i]),
+            "hipml_gemm_q8_0_f16": (i, [vp, vp, vp, vp, i, i, i]),
         }
         for name, (res, args) in sig.items():
             fn = getattr(l, name)
@@ -331,6 +332,12 @@ def q_gate(x, gate, y, n=None, stream=None):
 def gemv_q8_0_rows(w, x, y, m, k, rows, stream=None):
     """`AttnLayer::gemv` / `gemv_rows` / `gemv_batched` over a Q8_0 weight matrix: y[rows][m]."""
     _check(lib().hipml_gemv_q8_0_rows(_stream(stream), _p(w), _p(x), _p(y), m, k, rows))
+
+
+def gemm_q8_0_f16(w, x, y, m, k, tokens, stream=None):
+    """`AttnLayer::apply_output_chunk`'s tiled GEMM (after the gate) over a Q8_0 weight matrix:
+    y[tokens][m], f16 operands."""
+    _check(lib().hipml_gemm_q8_0_f16(_stream(stream), _p(w), _p(x), _p(y), m, k, tokens))
 
 
 # ---- cache owner ------------------------------------------------------------------------------------

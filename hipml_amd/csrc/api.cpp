@@ -174,6 +174,8 @@ int hipml_attn_init(int device)
     int rc = decode_init();
     if (rc == 0)
         rc = prefill_init();
+    if (rc == 0)
+        rc = proj_init();
     if (rc)
         return rc;
     g_inited = true;
@@ -722,6 +724,28 @@ int hipml_gemv_q8_0_rows(hipml_stream_t stream, const void *w, const float *x, f
     if (rc)
         return rc;
     return launch_gemv_q8_rows(as_stream(stream), static_cast<const uint8_t *>(w), x, y, m, k, rows);
+}
+
+int hipml_gemm_q8_0_f16(hipml_stream_t stream, const void *w, const float *x, float *y, int m, int k,
+                        int tokens)
+{
+    clear_error();
+    REQUIRE_PTR(w);
+    REQUIRE_PTR(x);
+    REQUIRE_PTR(y);
+    if (m < 1)
+        return fail(HIPML_ATTN_E_RANGE, "m %d must be positive", m);
+    if (k < 64 || k % 64 != 0)
+        return fail(HIPML_ATTN_E_RANGE, "k %d must be a positive multiple of 64 (two Q8_0 blocks: rows "
+                                        "stay dword aligned)", k);
+    if (tokens < 1)
+        return fail(HIPML_ATTN_E_RANGE, "tokens %d must be positive", tokens);
+    if (((uintptr_t)w & 3) != 0)
+        return fail(HIPML_ATTN_E_RANGE, "w must be 4-byte aligned");
+    int rc = check_aligned16(x, "x");
+    if (rc)
+        return rc;
+    return launch_gemm_q8_f16(as_stream(stream), static_cast<const uint8_t *>(w), x, y, m, k, tokens);
 }
 
 } // extern "C"

@@ -322,14 +322,6 @@ static int launch_gemv_xg(hipStream_t st, const uint8_t *w, const float *x, floa
 {
     const size_t lds = (size_t)(k >> 5) * rp * 128 + (size_t)WAVES * TILES * 32 * sizeof(float4v);
     auto kern = gemv_q8_rows_kernel<WAVES, TILES, CH, XG>;
-    static bool raised = false; // the limit is a property of the function: set once per process
-    if (!raised) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 << 10);
-        if (e != hipSuccess)
-            return fail((int)e, "hipFuncSetAttribute(gemv LDS) failed: %d (%s)", (int)e, hipGetErrorString(e));
-        raised = true;
-    }
     const dim3 grid((unsigned)((m + 16 * TILES - 1) / (16 * TILES)), (unsigned)((rows + rp - 1) / rp), 1);
     hipLaunchKernelGGL(kern, grid, dim3(64 * WAVES, 1, 1), lds, st, w, x, y, m, k, rows, rp);
     return launched("gemv_q8_0_rows");
@@ -365,6 +357,213 @@ int launch_gemv_q8_rows(hipStream_t st, const uint8_t *w, const float *x, float 
     if (rp <= 2)
         return launch_gemv_variant<8, 1, 6>(st, w, x, y, m, k, rows, rp);
     return launch_gemv_variant<8, 2, 6>(st, w, x, y, m, k, rows, rp);
+}
+
+
+// ---- gemm_q8_f16_kernel: many activation rows (a prefill chunk) ---------------------------------
+//
+// y[t][row] for a 128 (tokens) x 128 (weight rows) tile per workgroup, MFMA-bound:
+// v_mfma_f32_32x32x16_f16 with A = x (f32 -> f16, round to nearest), B = W dequantized to f16 (d*q, one
+// rounding: the precision class of the reference's f16-operand prefill kernels and of this library's
+// chunk attention), fp32 accumulation.  Four waves, each a 64 x 64 quarter (2 x 2 MFMA tiles: every
+// operand read from LDS feeds two MFMAs).  A k step is 64 values = one 68-byte pair of blocks per
+// weight row; both operand tiles are staged as [128 rows][64 f16] with a 144-byte row pitch (128-bit
+// reads and writes of 16 consecutive rows then touch every bank once), double buffered, one barrier
+// per step.  Fetch for step s+2 is issued, step s+1 (fetched during the previous step) is converted
+// and written to the other buffer, step s is multiplied: the three run in one wave's instruction
+// stream so that its VALU work sits in the shadow of its MFMAs.
+// Weight fetch uses the lane order of the row kernel above (quad = the four quarters of a pair of
+// blocks, dword-aligned loads); a thread handles rows r and r + 64.
+
+typedef float float16v __attribute__((ext_vector_type(16)));
+typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+
+constexpr int kGemmT = 128, kGemmM = 128, kGemmK = 64;
+constexpr int kGemmPitch = 144;
+constexpr int kGemmTile = 128 * kGemmPitch;   // one operand tile
+constexpr int kGemmBuf = 2 * kGemmTile;       // x tile + w tile
+constexpr int kGemmLds = 2 * kGemmBuf;        // double buffered: 73,728 bytes
+
+struct GemmFetch {
+    uint3a4 e[2];   // even-block quarter (+ scales in quad lanes 0 and 3), rows r and r + 64
+    uint2a4 o[2];   // odd-block quarter
+    float4v x[8];   // 4 activations of rows xr + 16 i
+};
+
+// 8 exact integer f16 times the block scale (f16): the product has at most 19 significant bits and
+// is rounded once, as f16(d * q) is.
+__device__ __forceinline__ half8 dequant8(uint32_t w0, uint32_t w1, _Float16 d)
+{
+    const half8 q = int8x8_to_f16(w0, w1);
+    const half8 dv = {d, d, d, d, d, d, d, d};
+    return q * dv;
+}
+
+__global__ void __launch_bounds__(256) gemm_q8_f16_kernel(const uint8_t *__restrict__ w,
+                                                         const float *__restrict__ x,
+                                                         float *__restrict__ y, int m, int k, int tokens)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int m0 = blockIdx.x * kGemmM, t0 = blockIdx.y * kGemmT;
+    const int nsteps = k / kGemmK;
+    const size_t row_bytes = (size_t)(k >> 5) * kQ8Block;
+
+    // fetch roles
+    const int fr = tid >> 2, fg = tid & 3; // weight rows fr and fr + 64, k quarter fg of each block
+    const uint8_t *wp[2];
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        const int row = m0 + fr + 64 * h < m ? m0 + fr + 64 * h : m - 1;
+        wp[h] = w + (size_t)row * row_bytes + fg * 8;
+    }
+    const int xr = tid >> 4, xc = tid & 15; // activation rows xr + 16 i, floats xc*4.. of the step
+    const float *xp[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const int t = t0 + xr + 16 * i < tokens ? t0 + xr + 16 * i : tokens - 1;
+        xp[i] = x + (size_t)t * k + xc * 4;
+    }
+    auto fetch = [&](GemmFetch &f, int s) {
+        const int sc = s < nsteps ? s : nsteps - 1;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const uint8_t *unit = wp[h] + (size_t)sc * (2 * kQ8Block);
+            f.e[h] = *reinterpret_cast<const uint3a4 *>(unit);
+            f.o[h] = *reinterpret_cast<const uint2a4 *>(unit + 36);
+        }
+#pragma unroll
+        for (int i = 0; i < 8; i++)
+            f.x[i] = *reinterpret_cast<const float4v *>(xp[i] + (size_t)sc * kGemmK);
+    };
+    auto stage = [&](const GemmFetch &f, uint8_t *buf) {
+        uint8_t *xt = buf, *wt = buf + kGemmTile;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            // round to nearest even (v_cvt_pk_f16_f32): truncation would bias every product the same way
+            const half4v v = __builtin_convertvector(f.x[i], half4v);
+            *reinterpret_cast<half4v *>(xt + (xr + 16 * i) * kGemmPitch + xc * 8) = v;
+        }
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const uint3a4 e = f.e[h];
+            const uint32_t s0 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)e[0], 0x00, 0xf, 0xf, true);
+            const uint32_t s1 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)e[2], 0xFF, 0xf, 0xf, true);
+            const _Float16 d0 = __builtin_bit_cast(_Float16, (uint16_t)(s0 & 0xffffu));
+            const _Float16 d1 = __builtin_bit_cast(_Float16, (uint16_t)(s1 >> 16));
+            const half8 v0 = dequant8(__builtin_amdgcn_alignbit(e[1], e[0], 16),
+                                      __builtin_amdgcn_alignbit(e[2], e[1], 16), d0);
+            const half8 v1 = dequant8(f.o[h][0], f.o[h][1], d1);
+            uint8_t *dst = wt + (fr + 64 * h) * kGemmPitch + fg * 16;
+            *reinterpret_cast<half8 *>(dst) = v0;        // k = fg*8 .. of the even block
+            *reinterpret_cast<half8 *>(dst + 64) = v1;   // k = 32 + fg*8 .. (the odd block)
+        }
+    };
+
+    // MFMA roles: wave (wt, wm) owns tokens wt*64.. and weight rows wm*64..
+    const int wt_ = wave >> 1, wm_ = wave & 1;
+    const int ln = lane & 31, lh = lane >> 5;
+    float16v acc[2][2];
+#pragma unroll
+    for (int a = 0; a < 2; a++)
+#pragma unroll
+        for (int b = 0; b < 2; b++)
+#pragma unroll
+            for (int i = 0; i < 16; i++)
+                acc[a][b][i] = 0.0f;
+    auto multiply = [&](const uint8_t *buf) {
+        const uint8_t *xa = buf + (wt_ * 64 + ln) * kGemmPitch + lh * 16;
+        const uint8_t *wb = buf + kGemmTile + (wm_ * 64 + ln) * kGemmPitch + lh * 16;
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++) {
+            half8 A[2], B[2];
+#pragma unroll
+            for (int a = 0; a < 2; a++)
+                A[a] = *reinterpret_cast<const half8 *>(xa + a * 32 * kGemmPitch + kk * 32);
+#pragma unroll
+            for (int b = 0; b < 2; b++)
+                B[b] = *reinterpret_cast<const half8 *>(wb + b * 32 * kGemmPitch + kk * 32);
+#pragma unroll
+            for (int a = 0; a < 2; a++)
+#pragma unroll
+                for (int b = 0; b < 2; b++)
+                    acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[a], B[b], acc[a][b], 0, 0, 0);
+        }
+    };
+
+    GemmFetch f0, f1;
+    fetch(f0, 0);
+    fetch(f1, 1);
+    stage(f0, lds);
+    __syncthreads();
+    // step s: f1 holds step s+1 (s even) or f0 does (s odd); the loop body is written twice so the
+    // two fetch records keep their registers
+    int s = 0;
+    while (true) {
+        fetch(f0, s + 2);
+        if (s + 1 < nsteps)
+            stage(f1, lds + kGemmBuf);
+        multiply(lds);
+        __syncthreads();
+        if (++s >= nsteps)
+            break;
+        fetch(f1, s + 2);
+        if (s + 1 < nsteps)
+            stage(f0, lds);
+        multiply(lds + kGemmBuf);
+        __syncthreads();
+        if (++s >= nsteps)
+            break;
+    }
+
+    // C tile: lane holds column ln (weight row), rows (i/4)*8 + lh*4 + i%4 (tokens)
+#pragma unroll
+    for (int a = 0; a < 2; a++)
+#pragma unroll
+        for (int b = 0; b < 2; b++) {
+            const int row = m0 + wm_ * 64 + b * 32 + ln;
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const int t = t0 + wt_ * 64 + a * 32 + (i >> 2) * 8 + lh * 4 + (i & 3);
+                if (t < tokens && row < m)
+                    y[(size_t)t * m + row] = acc[a][b][i];
+            }
+        }
+}
+
+template <int WAVES, int TILES, int CH>
+static hipError_t raise_gemv_lds()
+{
+    hipError_t e = hipSuccess;
+    auto raise = [&](const void *f) {
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, 160 << 10);
+    };
+    raise(reinterpret_cast<const void *>(&gemv_q8_rows_kernel<WAVES, TILES, CH, 2>));
+    raise(reinterpret_cast<const void *>(&gemv_q8_rows_kernel<WAVES, TILES, CH, 4>));
+    raise(reinterpret_cast<const void *>(&gemv_q8_rows_kernel<WAVES, TILES, CH, 8>));
+    raise(reinterpret_cast<const void *>(&gemv_q8_rows_kernel<WAVES, TILES, CH, 16>));
+    return e;
+}
+
+int proj_init()
+{
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q8_f16_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLds);
+    if (e == hipSuccess)
+        e = raise_gemv_lds<8, 1, 6>();
+    if (e == hipSuccess)
+        e = raise_gemv_lds<8, 2, 6>();
+    if (e != hipSuccess)
+        return fail((int)e, "hipFuncSetAttribute(projection LDS) failed: %d (%s)", (int)e, hipGetErrorString(e));
+    return 0;
+}
+
+int launch_gemm_q8_f16(hipStream_t st, const uint8_t *w, const float *x, float *y, int m, int k, int tokens)
+{
+    const dim3 grid((unsigned)((m + kGemmM - 1) / kGemmM), (unsigned)((tokens + kGemmT - 1) / kGemmT), 1);
+    hipLaunchKernelGGL(gemm_q8_f16_kernel, grid, dim3(256, 1, 1), kGemmLds, st, w, x, y, m, k, tokens);
+    return launched("gemm_q8_0_f16");
 }
 
 } // namespace hipml

@@ -280,6 +280,17 @@ int hipml_q_gate_f32(hipml_stream_t stream, const float *x, const float *gate, f
 int hipml_gemv_q8_0_rows(hipml_stream_t stream, const void *w, const float *x, float *y, int m,
                          int k, int rows);
 
+/* The same product for a prefill chunk (any number of tokens): y[t][row] = W[row][:] . x[t][:] on
+ * MFMA with f16 operands -- x rounded to f16, W dequantized to f16(d*q) -- and fp32 accumulation:
+ * the precision class of the reference's f16-operand prefill kernels (its f32 tile kernel for Q8_0
+ * is bounded by 1e-4 on small cases; this one by 2e-3 abs / 3e-2 rel, the reference's LARGE_TOL, at
+ * the model's shape).  Same layouts and argument rules as hipml_gemv_q8_0_rows.
+ * Replaces AttnLayer::apply_output_chunk -> prefill_resident(prefill_q8_0) after the gate, and the
+ * chunk's Q/K/V projections, crates/hipml-kernels/src/attn_gpu/imp/attn_chunk.rs:343-397,
+ * crates/hipml-kernels/kernels/prefill_q8_0.hip:44-60. */
+int hipml_gemm_q8_0_f16(hipml_stream_t stream, const void *w, const float *x, float *y, int m, int k,
+                        int tokens);
+
 #ifdef __cplusplus
 }
 #endif

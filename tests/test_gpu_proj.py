@@ -113,3 +113,59 @@ def test_argument_errors():
         attn.gemv_q8_0_rows(w, x, y, 2, 64, 129)   # too many rows
     with pytest.raises(attn.HipmlError):
         attn.gemv_q8_0_rows(w, x, y, 0, 64, 1)
+
+
+# ---- the chunk GEMM (f16 operands) ---------------------------------------------------------------
+
+# f16 operands: the reference budgets its own f16-operand kernels on these case shapes with
+# 5e-2 abs / 5e-1 rel (k = 512) and 2.5e-1 / 5e-2 (k = 5120) (prefill_parity.rs:318-326); asserted here
+# five and twenty-five times tighter.  Expected error: two roundings of 2^-11 per product, i.e.
+# ~4e-4 of the root-sum-square of a row's terms (1.6 at k = 512 with N(0,1) activations).
+F16_SMALL = (1e-2, 1e-1)
+F16_LARGE = (1e-2, 5e-2)
+
+
+def run_gemm(w, x, m, k, tokens):
+    y = torch.full((tokens, m), float("nan"), dtype=torch.float32, device="cuda")
+    attn.gemm_q8_0_f16(dev(w), dev(x), y, m, k, tokens)
+    torch.cuda.synchronize()
+    return host(y)
+
+
+def f16_operand_reference(w, x, m, k):
+    """What the kernel is meant to compute, in float64: x rounded to f16, W as f16(d*q)."""
+    blocks = w.reshape(m, k // 32, 34)
+    d = blocks[:, :, :2].copy().view(np.float16).astype(np.float32)
+    q = blocks[:, :, 2:].view(np.int8).astype(np.float32)
+    dense = (d * q).astype(np.float16).astype(np.float64).reshape(m, k)
+    return x.astype(np.float16).astype(np.float64) @ dense.T
+
+
+@pytest.mark.parametrize("seed,m,k,t", [(0x9F11_0003, 64, 512, 4), (0x5C11_0006, 200, 512, 4),
+                                        (0xA001, 128, 64, 128), (0xA002, 300, 1024, 37), (0xA003, 129, 192, 257)])
+def test_gemm_reference_cases_and_ragged_tiles(seed, m, k, t):
+    r = orc.Rng(seed)
+    w = orc.random_q8_0_bytes(r, m * k // 32)
+    x = r.normal_array((t, k))
+    want = orc.gemm_q8_0(w, x, t, m, k)
+    got = run_gemm(w, x, m, k, t)
+    ok, _, _ = report(f"gemm_q8_0_f16 {m}x{k} t={t}", want, got, *F16_SMALL)
+    assert ok
+    # against its own definition the kernel is at fp32-accumulation level
+    assert np.max(np.abs(got - f16_operand_reference(w, x, m, k))) < 2e-5 * np.sqrt(k)
+
+
+def test_gemm_output_projection_672_tokens():
+    r = orc.Rng(0x0E67)
+    m, k, t = 5120, 6144, 672
+    w = orc.random_q8_0_bytes(r, m * k // 32)
+    x = r.normal_array((t, k), 0.5)
+    got = run_gemm(w, x, m, k, t)
+    rows = [0, 1, 127, 128, 300, 671]
+    want = orc.gemm_q8_0(w, x[rows], len(rows), m, k, n_threads=8)
+    ok, _, _ = report("W_o 5120x6144 t=672 (6 rows checked)", want, got[rows], *F16_LARGE)
+    assert ok
+    assert np.isfinite(got).all()
+    # linearity over tokens holds bit for bit: a token's row does not depend on its tile neighbours
+    alone = run_gemm(w, x[300:301], m, k, 1)
+    assert np.array_equal(alone[0], got[300])
