@@ -371,25 +371,35 @@ def bench_gemv(torch, attn, rows, steps, layers, m=5120, k=6144):
 
 
 def bench_gemm(torch, attn, tokens, steps, layers, m=5120, k=6144):
-    """Output projection of a prefill chunk: [tokens][6144] x W_o^T (Q8_0) on MFMA, f16 operands."""
+    """Output side of a prefill chunk: y = W_o (out * sigmoid(gate)), [tokens][6144] x W_o^T (Q8_0) on
+    MFMA with f16 operands."""
     gen = torch.Generator(device="cuda")
     gen.manual_seed(0x5EED0008)
     ws = [random_q8_0_weights(torch, m, k, gen) for _ in range(layers)]
     x = torch.randn((tokens, k), device="cuda", generator=gen) * 0.5
     y = torch.empty((tokens, m), device="cuda")
+    gate = torch.randn((tokens, k), device="cuda", generator=gen)
+    x16 = torch.empty((tokens, k), dtype=torch.float16, device="cuda")
     for w in ws:
         attn.gemm_q8_0_f16(w, x, y, m, k, tokens)
-    with Timer(torch) as t:
+        attn.output_chunk_q8_0(w, x, gate, y, m, k, tokens, x16)
+    with Timer(torch) as t32:
         for _ in range(steps):
             for w in ws:
                 attn.gemm_q8_0_f16(w, x, y, m, k, tokens)
+    # the whole output side: gate + rounding to f16 in one pass, then the GEMM over f16 rows
+    with Timer(torch) as t:
+        for _ in range(steps):
+            for w in ws:
+                attn.output_chunk_q8_0(w, x, gate, y, m, k, tokens, x16)
     us = t.ms * 1e3 / (steps * layers)
     flop = 2.0 * tokens * m * k
     tf = flop / (us * 1e-6) / 1e12
     return {"workload": f"W_o projection of a chunk, Q8_0 {m}x{k}, {tokens} tokens",
-            "us_per_layer": us, "flop": flop, "layers_rotated": layers,
+            "us_per_layer": us, "us_per_layer_f32_rows_no_gate": t32.ms * 1e3 / (steps * layers),
+            "flop": flop, "layers_rotated": layers,
             "roofline": {"bound": "mfma", "achieved": tf, "peak": MFMA_F16_PEAK_TF, "unit": "TFLOP/s",
-                         "frac": tf / MFMA_F16_PEAK_TF, "traffic": None, "kernel": "gemm_q8_f16_kernel",
+                         "frac": tf / MFMA_F16_PEAK_TF, "traffic": None, "kernel": "gate_f16_kernel + gemm_q8_f16_kernel",
                          "flop_per_launch": flop, "launch_us": us}}
 
 

@@ -35,7 +35,7 @@ EXPORTS = [
     "hipml_attn_decode_kv_gate", "hipml_attn_decode_batch_cols_gate",
     "hipml_attn_chunk_q8_split", "hipml_attn_chunk_q8_split_gate", "hipml_q_gate_f32",
     "hipml_attn_front_f32", "hipml_attn_chunk_front_f32",
-    "hipml_gemv_q8_0_rows", "hipml_gemm_q8_0_f16",
+    "hipml_gemv_q8_0_rows", "hipml_gemm_q8_0_f16", "hipml_attn_output_chunk_q8_0",
 ]
 
 
@@ -98,6 +98,7 @@ def lib() -> C.CDLL:
             "hipml_attn_chunk_front_f32": (i, [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, f, f, i, i]),
             "hipml_gemv_q8_0_rows": (i, [vp, vp, vp, vp, i, i, i]),
             "hipml_gemm_q8_0_f16": (i, [vp, vp, vp, vp, i, i, i]),
+            "hipml_attn_output_chunk_q8_0": (i, [vp, vp, vp, vp, vp, i, i, i, vp]),
         }
         for name, (res, args) in sig.items():
             fn = getattr(l, name)
@@ -338,6 +339,14 @@ def gemm_q8_0_f16(w, x, y, m, k, tokens, stream=None):
     """`AttnLayer::apply_output_chunk`'s tiled GEMM (after the gate) over a Q8_0 weight matrix:
     y[tokens][m], f16 operands."""
     _check(lib().hipml_gemm_q8_0_f16(_stream(stream), _p(w), _p(x), _p(y), m, k, tokens))
+
+
+def output_chunk_q8_0(wo, attn_out, gate, y, m, k, tokens, x16, stream=None):
+    """`AttnLayer::apply_output_chunk`: y = W_o (attn_out * sigmoid(gate)); gate may be None; x16 is
+    scratch of tokens*k f16."""
+    _check(lib().hipml_attn_output_chunk_q8_0(_stream(stream), _p(wo), _p(attn_out),
+                                              _p(gate) if gate is not None else None, _p(y), m, k,
+                                              tokens, _p(x16)))
 
 
 # ---- cache owner ------------------------------------------------------------------------------------

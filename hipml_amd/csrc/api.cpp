@@ -726,10 +726,8 @@ int hipml_gemv_q8_0_rows(hipml_stream_t stream, const void *w, const float *x, f
     return launch_gemv_q8_rows(as_stream(stream), static_cast<const uint8_t *>(w), x, y, m, k, rows);
 }
 
-int hipml_gemm_q8_0_f16(hipml_stream_t stream, const void *w, const float *x, float *y, int m, int k,
-                        int tokens)
+static int check_gemm(const void *w, const float *x, const float *y, int m, int k, int tokens)
 {
-    clear_error();
     REQUIRE_PTR(w);
     REQUIRE_PTR(x);
     REQUIRE_PTR(y);
@@ -742,10 +740,32 @@ int hipml_gemm_q8_0_f16(hipml_stream_t stream, const void *w, const float *x, fl
         return fail(HIPML_ATTN_E_RANGE, "tokens %d must be positive", tokens);
     if (((uintptr_t)w & 3) != 0)
         return fail(HIPML_ATTN_E_RANGE, "w must be 4-byte aligned");
-    int rc = check_aligned16(x, "x");
+    return check_aligned16(x, "x");
+}
+
+int hipml_gemm_q8_0_f16(hipml_stream_t stream, const void *w, const float *x, float *y, int m, int k,
+                        int tokens)
+{
+    clear_error();
+    int rc = check_gemm(w, x, y, m, k, tokens);
     if (rc)
         return rc;
-    return launch_gemm_q8_f16(as_stream(stream), static_cast<const uint8_t *>(w), x, y, m, k, tokens);
+    return launch_gemm_q8_f16(as_stream(stream), static_cast<const uint8_t *>(w), x, nullptr, y, m, k,
+                              tokens, nullptr);
+}
+
+int hipml_attn_output_chunk_q8_0(hipml_stream_t stream, const void *wo, const float *attn_out,
+                                 const float *gate, float *y, int m, int k, int tokens, void *x16)
+{
+    clear_error();
+    int rc = check_gemm(wo, attn_out, y, m, k, tokens);
+    if (rc)
+        return rc;
+    REQUIRE_PTR(x16);
+    if ((rc = check_aligned16(gate, "gate")) || (rc = check_aligned16(x16, "x16")))
+        return rc;
+    return launch_gemm_q8_f16(as_stream(stream), static_cast<const uint8_t *>(wo), attn_out, gate, y, m, k,
+                              tokens, x16);
 }
 
 } // extern "C"

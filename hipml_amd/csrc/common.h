@@ -94,7 +94,10 @@ int launch_chunk_q8(hipStream_t st, const float *q, const uint8_t *kc, const uin
 // y[r][row] = W[row][:] . x[r][:] over a Q8_0 weight matrix, rows <= 128 activation rows (proj.hip).
 int launch_gemv_q8_rows(hipStream_t st, const uint8_t *w, const float *x, float *y, int m, int k, int rows);
 // The same product for a prefill chunk: f16 operands on MFMA, fp32 accumulation (proj.hip).
-int launch_gemm_q8_f16(hipStream_t st, const uint8_t *w, const float *x, float *y, int m, int k, int tokens);
+// With a scratch of tokens*k f16 (x16) the activations are gated (gate may be null) and converted once
+// by a first kernel; without it the GEMM converts the f32 activations itself (gate must be null).
+int launch_gemm_q8_f16(hipStream_t st, const uint8_t *w, const float *x, const float *gate, float *y, int m,
+                       int k, int tokens, void *x16);
 // Raise the projection kernels' dynamic LDS limit (once per process; called by hipml_attn_init).
 int proj_init();
 

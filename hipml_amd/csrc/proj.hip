@@ -369,11 +369,14 @@ int launch_gemv_q8_rows(hipStream_t st, const uint8_t *w, const float *x, float 
 // operand read from LDS feeds two MFMAs).  A k step is 64 values = one 68-byte pair of blocks per
 // weight row; both operand tiles are staged as [128 rows][64 f16] with a 144-byte row pitch (128-bit
 // reads and writes of 16 consecutive rows then touch every bank once), double buffered, one barrier
-// per step.  Fetch for step s+2 is issued, step s+1 (fetched during the previous step) is converted
-// and written to the other buffer, step s is multiplied: the three run in one wave's instruction
-// stream so that its VALU work sits in the shadow of its MFMAs.
+// per step.  A fetch record is refilled as soon as it has been staged.
 // Weight fetch uses the lane order of the row kernel above (quad = the four quarters of a pair of
 // blocks, dword-aligned loads); a thread handles rows r and r + 64.
+// X16: the activations arrive as f16 (written by gate_f16_kernel below).  With f32 activations a
+// step moves 32 KB of them through the CU's 64-byte-per-cycle vector memory path -- more cycles
+// than the step's MFMAs take (measured: 700 of a step's 2,200 cycles are spent issuing loads) -- and
+// every one of the m/128 workgroups of a token tile repeats that; f16 halves it and drops the
+// conversion.
 
 typedef float float16v __attribute__((ext_vector_type(16)));
 typedef _Float16 half4v __attribute__((ext_vector_type(4)));
@@ -384,10 +387,11 @@ constexpr int kGemmTile = 128 * kGemmPitch;   // one operand tile
 constexpr int kGemmBuf = 2 * kGemmTile;       // x tile + w tile
 constexpr int kGemmLds = 2 * kGemmBuf;        // double buffered: 73,728 bytes
 
+template <bool X16>
 struct GemmFetch {
-    uint3a4 e[2];   // even-block quarter (+ scales in quad lanes 0 and 3), rows r and r + 64
-    uint2a4 o[2];   // odd-block quarter
-    float4v x[8];   // 4 activations of rows xr + 16 i
+    uint3a4 e[2];            // even-block quarter (+ scales in quad lanes 0 and 3), rows r and r + 64
+    uint2a4 o[2];            // odd-block quarter
+    float4v x[X16 ? 4 : 8];  // f32: 4 activations of rows xr + 16 i; f16: 8 of rows xr + 32 i
 };
 
 // 8 exact integer f16 times the block scale (f16): the product has at most 19 significant bits and
@@ -399,8 +403,9 @@ __device__ __forceinline__ half8 dequant8(uint32_t w0, uint32_t w1, _Float16 d)
     return q * dv;
 }
 
+template <bool X16>
 __global__ void __launch_bounds__(256) gemm_q8_f16_kernel(const uint8_t *__restrict__ w,
-                                                         const float *__restrict__ x,
+                                                         const void *__restrict__ xv,
                                                          float *__restrict__ y, int m, int k, int tokens)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -408,6 +413,9 @@ __global__ void __launch_bounds__(256) gemm_q8_f16_kernel(const uint8_t *__restr
     const int m0 = blockIdx.x * kGemmM, t0 = blockIdx.y * kGemmT;
     const int nsteps = k / kGemmK;
     const size_t row_bytes = (size_t)(k >> 5) * kQ8Block;
+    constexpr int XN = X16 ? 4 : 8;          // activation loads per thread and step
+    constexpr int XROWS = X16 ? 32 : 16;     // rows covered by one such load of the workgroup
+    constexpr int XELT = X16 ? 2 : 4;        // bytes per activation
 
     // fetch roles
     const int fr = tid >> 2, fg = tid & 3; // weight rows fr and fr + 64, k quarter fg of each block
@@ -417,14 +425,16 @@ __global__ void __launch_bounds__(256) gemm_q8_f16_kernel(const uint8_t *__restr
         const int row = m0 + fr + 64 * h < m ? m0 + fr + 64 * h : m - 1;
         wp[h] = w + (size_t)row * row_bytes + fg * 8;
     }
-    const int xr = tid >> 4, xc = tid & 15; // activation rows xr + 16 i, floats xc*4.. of the step
-    const float *xp[8];
+    // activations: 16 bytes per load; a row's 64 values of the step are 16 (f32) or 8 (f16) lanes
+    const int xr = X16 ? tid >> 3 : tid >> 4, xc = X16 ? tid & 7 : tid & 15;
+    const uint8_t *xp[XN];
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-        const int t = t0 + xr + 16 * i < tokens ? t0 + xr + 16 * i : tokens - 1;
-        xp[i] = x + (size_t)t * k + xc * 4;
+    for (int i = 0; i < XN; i++) {
+        const int t = t0 + xr + XROWS * i < tokens ? t0 + xr + XROWS * i : tokens - 1;
+        xp[i] = static_cast<const uint8_t *>(xv) + ((size_t)t * k) * XELT + xc * 16;
     }
-    auto fetch = [&](GemmFetch &f, int s) {
+    typedef GemmFetch<X16> Fetch;
+    auto fetch = [&](Fetch &f, int s) {
         const int sc = s < nsteps ? s : nsteps - 1;
 #pragma unroll
         for (int h = 0; h < 2; h++) {
@@ -433,16 +443,20 @@ __global__ void __launch_bounds__(256) gemm_q8_f16_kernel(const uint8_t *__restr
             f.o[h] = *reinterpret_cast<const uint2a4 *>(unit + 36);
         }
 #pragma unroll
-        for (int i = 0; i < 8; i++)
-            f.x[i] = *reinterpret_cast<const float4v *>(xp[i] + (size_t)sc * kGemmK);
+        for (int i = 0; i < XN; i++)
+            f.x[i] = *reinterpret_cast<const float4v *>(xp[i] + (size_t)sc * (kGemmK * XELT));
     };
-    auto stage = [&](const GemmFetch &f, uint8_t *buf) {
+    auto stage = [&](const Fetch &f, uint8_t *buf) {
         uint8_t *xt = buf, *wt = buf + kGemmTile;
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-            // round to nearest even (v_cvt_pk_f16_f32): truncation would bias every product the same way
-            const half4v v = __builtin_convertvector(f.x[i], half4v);
-            *reinterpret_cast<half4v *>(xt + (xr + 16 * i) * kGemmPitch + xc * 8) = v;
+        for (int i = 0; i < XN; i++) {
+            if (X16) {
+                *reinterpret_cast<float4v *>(xt + (xr + XROWS * i) * kGemmPitch + xc * 16) = f.x[i];
+            } else {
+                // round to nearest even (v_cvt_pk_f16_f32): truncation would bias every product the same way
+                const half4v v = __builtin_convertvector(f.x[i], half4v);
+                *reinterpret_cast<half4v *>(xt + (xr + XROWS * i) * kGemmPitch + xc * 8) = v;
+            }
         }
 #pragma unroll
         for (int h = 0; h < 2; h++) {
@@ -491,30 +505,27 @@ __global__ void __launch_bounds__(256) gemm_q8_f16_kernel(const uint8_t *__restr
         }
     };
 
-    GemmFetch f0, f1;
+    // Two steps per turn keep the two records and the two buffers in the same registers through
+    // the loop; a fetch past the last step repeats it and is never multiplied.
+    Fetch f0, f1;
     fetch(f0, 0);
     fetch(f1, 1);
     stage(f0, lds);
+    fetch(f0, 2);
     __syncthreads();
-    // step s: f1 holds step s+1 (s even) or f0 does (s odd); the loop body is written twice so the
-    // two fetch records keep their registers
     int s = 0;
-    while (true) {
-        fetch(f0, s + 2);
-        if (s + 1 < nsteps)
-            stage(f1, lds + kGemmBuf);
-        multiply(lds);
+    for (; s + 2 <= nsteps; s += 2) {
+        stage(f1, lds + kGemmBuf); // step s + 1
+        fetch(f1, s + 3);
+        multiply(lds);             // step s
         __syncthreads();
-        if (++s >= nsteps)
-            break;
-        fetch(f1, s + 2);
-        if (s + 1 < nsteps)
-            stage(f0, lds);
-        multiply(lds + kGemmBuf);
+        stage(f0, lds);            // step s + 2
+        fetch(f0, s + 4);
+        multiply(lds + kGemmBuf);  // step s + 1
         __syncthreads();
-        if (++s >= nsteps)
-            break;
     }
+    if (nsteps & 1)
+        multiply(lds);
 
     // C tile: lane holds column ln (weight row), rows (i/4)*8 + lh*4 + i%4 (tokens)
 #pragma unroll
@@ -529,6 +540,35 @@ __global__ void __launch_bounds__(256) gemm_q8_f16_kernel(const uint8_t *__restr
                     y[(size_t)t * m + row] = acc[a][b][i];
             }
         }
+}
+
+// x16[i] = f16(x[i] * sigmoid(gate[i])) (gate may be null: plain conversion), 8 values per thread.
+// The gate is the expression every gating kernel of this library uses, the rounding the one the
+// f32-activation GEMM applies when it stages x: the two routes give the same bits.
+__global__ void __launch_bounds__(256) gate_f16_kernel(const float4v *__restrict__ x,
+                                                      const float4v *__restrict__ gate,
+                                                      half8 *__restrict__ x16, size_t n8)
+{
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n8)
+        return;
+    float4v a = x[2 * i], b = x[2 * i + 1];
+    if (gate != nullptr) {
+        const float4v ga = gate[2 * i], gb = gate[2 * i + 1];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            a[j] = gated(a[j], ga[j]);
+            b[j] = gated(b[j], gb[j]);
+        }
+    }
+    const half4v ha = __builtin_convertvector(a, half4v), hb = __builtin_convertvector(b, half4v);
+    half8 h;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        h[j] = ha[j];
+        h[4 + j] = hb[j];
+    }
+    x16[i] = h;
 }
 
 template <int WAVES, int TILES, int CH>
@@ -548,8 +588,11 @@ static hipError_t raise_gemv_lds()
 
 int proj_init()
 {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q8_f16_kernel),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q8_f16_kernel<false>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLds);
+    if (e == hipSuccess)
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q8_f16_kernel<true>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLds);
     if (e == hipSuccess)
         e = raise_gemv_lds<8, 1, 6>();
     if (e == hipSuccess)
@@ -559,10 +602,23 @@ int proj_init()
     return 0;
 }
 
-int launch_gemm_q8_f16(hipStream_t st, const uint8_t *w, const float *x, float *y, int m, int k, int tokens)
+// x16 != nullptr: gate (optional) and convert into x16 first, then the GEMM over f16 activations.
+int launch_gemm_q8_f16(hipStream_t st, const uint8_t *w, const float *x, const float *gate, float *y, int m,
+                       int k, int tokens, void *x16)
 {
     const dim3 grid((unsigned)((m + kGemmM - 1) / kGemmM), (unsigned)((tokens + kGemmT - 1) / kGemmT), 1);
-    hipLaunchKernelGGL(gemm_q8_f16_kernel, grid, dim3(256, 1, 1), kGemmLds, st, w, x, y, m, k, tokens);
+    if (x16 == nullptr) {
+        hipLaunchKernelGGL(gemm_q8_f16_kernel<false>, grid, dim3(256, 1, 1), kGemmLds, st, w, x, y, m, k, tokens);
+        return launched("gemm_q8_0_f16");
+    }
+    const size_t n8 = (size_t)tokens * k / 8;
+    hipLaunchKernelGGL(gate_f16_kernel, dim3((unsigned)((n8 + 255) / 256), 1, 1), dim3(256, 1, 1), 0, st,
+                       reinterpret_cast<const float4v *>(x), reinterpret_cast<const float4v *>(gate),
+                       static_cast<half8 *>(x16), n8);
+    int rc = launched("gate_f16");
+    if (rc)
+        return rc;
+    hipLaunchKernelGGL(gemm_q8_f16_kernel<true>, grid, dim3(256, 1, 1), kGemmLds, st, w, x16, y, m, k, tokens);
     return launched("gemm_q8_0_f16");
 }
 

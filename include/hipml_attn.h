@@ -291,6 +291,16 @@ int hipml_gemv_q8_0_rows(hipml_stream_t stream, const void *w, const float *x, f
 int hipml_gemm_q8_0_f16(hipml_stream_t stream, const void *w, const float *x, float *y, int m, int k,
                         int tokens);
 
+/* The output side of a chunk in one call: y = W_o (attn_out * sigmoid(gate)), gate may be NULL (the
+ * rows are already gated, e.g. by hipml_attn_chunk_q8_split_gate).  x16 is caller scratch of
+ * tokens*k f16 (2 bytes each, 16-byte aligned; the attention's split scratch is free by then): a
+ * first kernel gates and rounds the rows to f16 once, the GEMM then reads half the bytes per
+ * workgroup.  Same bits as hipml_q_gate_f32 followed by hipml_gemm_q8_0_f16, faster.
+ * Replaces AttnLayer::apply_output_chunk (q_gate_f32 + the tiled GEMM),
+ * crates/hipml-kernels/src/attn_gpu/imp/attn_chunk.rs:343-397. */
+int hipml_attn_output_chunk_q8_0(hipml_stream_t stream, const void *wo, const float *attn_out,
+                                 const float *gate, float *y, int m, int k, int tokens, void *x16);
+
 #ifdef __cplusplus
 }
 #endif

@@ -169,3 +169,32 @@ def test_gemm_output_projection_672_tokens():
     # linearity over tokens holds bit for bit: a token's row does not depend on its tile neighbours
     alone = run_gemm(w, x[300:301], m, k, 1)
     assert np.array_equal(alone[0], got[300])
+
+
+def test_output_chunk_equals_gate_then_gemm():
+    # AttnLayer::apply_output_chunk (attn_chunk.rs:343-397) in one call: same bits as the gate kernel
+    # followed by the f32-activation GEMM, with and without a gate; ragged token count
+    r = orc.Rng(0x0C47)
+    m, k, t = 384, 1024, 203
+    w = orc.random_q8_0_bytes(r, m * k // 32)
+    a = r.normal_array((t, k))
+    g = r.normal_array((t, k))
+    wd, ad, gd = dev(w), dev(a), dev(g)
+    x16 = torch.empty((t, k), dtype=torch.float16, device="cuda")
+    one = torch.full((t, m), float("nan"), dtype=torch.float32, device="cuda")
+    attn.output_chunk_q8_0(wd, ad, gd, one, m, k, t, x16)
+    gated = torch.empty_like(ad)
+    attn.q_gate(ad, gd, gated, t * k)
+    two = torch.full((t, m), float("nan"), dtype=torch.float32, device="cuda")
+    attn.gemm_q8_0_f16(wd, gated, two, m, k, t)
+    torch.cuda.synchronize()
+    assert torch.equal(one, two)
+    want = orc.gemm_q8_0(w, orc.q_gate(a.ravel(), g.ravel()).reshape(t, k), t, m, k)
+    ok, _, _ = report("output chunk 384x1024 t=203", want, host(one), *F16_SMALL)
+    assert ok
+    plain = torch.full((t, m), float("nan"), dtype=torch.float32, device="cuda")
+    attn.output_chunk_q8_0(wd, ad, None, plain, m, k, t, x16)
+    ref = torch.full((t, m), float("nan"), dtype=torch.float32, device="cuda")
+    attn.gemm_q8_0_f16(wd, ad, ref, m, k, t)
+    torch.cuda.synchronize()
+    assert torch.equal(plain, ref)
