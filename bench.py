@@ -539,6 +539,12 @@ def main() -> int:
         from oracle import binding as orc  # only for the seeded depth recipe and the CPU leg
         also["batch16_mtp"] = bench_batch(torch, attn, orc, d_steps, max(W // 4, 2), 4)
         torch.cuda.empty_cache()
+        # the step after the path: output projection over Q8_0 weights (decode rows, then a chunk)
+        also["wo_rows_1"] = bench_gemv(torch, attn, 1, d_steps, LAYERS)
+        also["wo_rows_4"] = bench_gemv(torch, attn, 4, d_steps, LAYERS)
+        torch.cuda.empty_cache()
+        also["wo_chunk_672"] = bench_gemm(torch, attn, 672, max(K // 20, 5), 4)
+        torch.cuda.empty_cache()
         line["also"] = also
 
     if not args.no_cpu:

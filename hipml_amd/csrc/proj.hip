@@ -365,11 +365,13 @@ int launch_gemv_q8_rows(hipStream_t st, const uint8_t *w, const float *x, float 
 // y[t][row] for a 128 (tokens) x 128 (weight rows) tile per workgroup, MFMA-bound:
 // v_mfma_f32_32x32x16_f16 with A = x (f32 -> f16, round to nearest), B = W dequantized to f16 (d*q, one
 // rounding: the precision class of the reference's f16-operand prefill kernels and of this library's
-// chunk attention), fp32 accumulation.  Four waves, each a 64 x 64 quarter (2 x 2 MFMA tiles: every
-// operand read from LDS feeds two MFMAs).  A k step is 64 values = one 68-byte pair of blocks per
+// chunk attention), fp32 accumulation.  Four consumer waves, each a 64 x 64 quarter (2 x 2 MFMA tiles:
+// every operand read from LDS feeds two MFMAs), and four producer waves that fetch and stage.  A k step is 64 values = one 68-byte pair of blocks per
 // weight row; both operand tiles are staged as [128 rows][64 f16] with a 144-byte row pitch (128-bit
 // reads and writes of 16 consecutive rows then touch every bank once), double buffered, one barrier
-// per step.  A fetch record is refilled as soon as it has been staged.
+// per step.  A fetch record is refilled as soon as it has been staged.  (One set of four waves doing
+// both, interleaved by hand MFMA by MFMA, took 1,600 cycles per step with a single workgroup on the
+// CU: every wait left its SIMD idle.)
 // Weight fetch uses the lane order of the row kernel above (quad = the four quarters of a pair of
 // blocks, dword-aligned loads); a thread handles rows r and r + 64.
 // X16: the activations arrive as f16 (written by gate_f16_kernel below).  With f32 activations a
@@ -377,6 +379,20 @@ int launch_gemv_q8_rows(hipStream_t st, const uint8_t *w, const float *x, float 
 // than the step's MFMAs take (measured: 700 of a step's 2,200 cycles are spent issuing loads) -- and
 // every one of the m/128 workgroups of a token tile repeats that; f16 halves it and drops the
 // conversion.
+
+#ifdef GEMM_TIMING
+// debug builds: cycles spent between marks, summed over the steps, per wave of the first workgroups
+__device__ unsigned long long g_gemm_t[16 * 8 * 8];
+#define GT(i) do { __builtin_amdgcn_sched_barrier(0); const unsigned long long now_ = __builtin_readcyclecounter(); if ((i) > 0) gt_sum[(i)] += now_ - gt_last; gt_last = now_; __builtin_amdgcn_sched_barrier(0); } while (0)
+#define GTDUMP() do { if ((threadIdx.x & 63) == 0 && blockIdx.x < 4 && blockIdx.y < 4) for (int i_ = 0; i_ < 8; i_++) g_gemm_t[((blockIdx.y * 4 + blockIdx.x) * 8 + (threadIdx.x >> 6)) * 8 + i_] = gt_sum[i_]; } while (0)
+extern "C" int hipml_dbg_read_gemm(unsigned long long *host, size_t n)
+{
+    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_gemm_t), n * 8);
+}
+#else
+#define GT(i) do { } while (0)
+#define GTDUMP() do { } while (0)
+#endif
 
 typedef float float16v __attribute__((ext_vector_type(16)));
 typedef _Float16 half4v __attribute__((ext_vector_type(4)));
@@ -404,12 +420,13 @@ __device__ __forceinline__ half8 dequant8(uint32_t w0, uint32_t w1, _Float16 d)
 }
 
 template <bool X16>
-__global__ void __launch_bounds__(256) gemm_q8_f16_kernel(const uint8_t *__restrict__ w,
+__global__ void __launch_bounds__(512) gemm_q8_f16_kernel(const uint8_t *__restrict__ w,
                                                          const void *__restrict__ xv,
                                                          float *__restrict__ y, int m, int k, int tokens)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const bool producer = threadIdx.x >= 256;
+    const int tid = threadIdx.x & 255, wave = tid >> 6, lane = tid & 63; // within the role
     const int m0 = blockIdx.x * kGemmM, t0 = blockIdx.y * kGemmT;
     const int nsteps = k / kGemmK;
     const size_t row_bytes = (size_t)(k >> 5) * kQ8Block;
@@ -505,27 +522,78 @@ __global__ void __launch_bounds__(256) gemm_q8_f16_kernel(const uint8_t *__restr
         }
     };
 
+    // Waves 4..7 produce (fetch, dequantize, write the next step's tiles), waves 0..3 consume (operand
+    // reads and MFMAs of the current step); one barrier per step hands a buffer over.  A SIMD holds
+    // one wave of each kind, and a VALU wave and an MFMA wave of one SIMD issue side by side.
     // Two steps per turn keep the two records and the two buffers in the same registers through
     // the loop; a fetch past the last step repeats it and is never multiplied.
-    Fetch f0, f1;
-    fetch(f0, 0);
-    fetch(f1, 1);
-    stage(f0, lds);
-    fetch(f0, 2);
-    __syncthreads();
-    int s = 0;
-    for (; s + 2 <= nsteps; s += 2) {
-        stage(f1, lds + kGemmBuf); // step s + 1
-        fetch(f1, s + 3);
-        multiply(lds);             // step s
+#ifdef GEMM_TIMING
+    unsigned long long gt_sum[8] = {0, 0, 0, 0, 0, 0, 0, 0}, gt_last = 0;
+#endif
+    if (producer) {
+        // Four fetch records in rotation: a record is refilled as soon as it has been staged and is
+        // staged again four steps later, so its loads have three steps to arrive (with two records the
+        // producers spent 860 cycles of a 1,400-cycle step waiting for them).  Four steps per turn keep
+        // the records in the same registers; a fetch past the last step repeats it.
+        Fetch r0, r1, r2, r3;
+        fetch(r0, 0);
+        fetch(r1, 1);
+        fetch(r2, 2);
+        fetch(r3, 3);
+        stage(r0, lds);
+        fetch(r0, 4);
         __syncthreads();
-        stage(f0, lds);            // step s + 2
-        fetch(f0, s + 4);
-        multiply(lds + kGemmBuf);  // step s + 1
+        int s = 0;
+        for (; s + 4 <= nsteps; s += 4) {
+            GT(0);
+            stage(r1, lds + kGemmBuf); // step s + 1, while step s is multiplied
+            GT(1);
+            fetch(r1, s + 5);
+            GT(2);
+            __syncthreads();
+            GT(3);
+            stage(r2, lds);
+            fetch(r2, s + 6);
+            __syncthreads();
+            stage(r3, lds + kGemmBuf);
+            fetch(r3, s + 7);
+            __syncthreads();
+            stage(r0, lds);            // step s + 4
+            fetch(r0, s + 8);
+            __syncthreads();
+        }
+        GTDUMP();
+        // the last one to three steps: their records are already on the way
+        const int rest = nsteps - s;
+        if (rest >= 1) {
+            if (rest >= 2)
+                stage(r1, lds + kGemmBuf);
+            __syncthreads();
+        }
+        if (rest >= 2) {
+            if (rest >= 3)
+                stage(r2, lds);
+            __syncthreads();
+        }
+        if (rest >= 3)
+            __syncthreads();
+        return;
+    }
+    __syncthreads();
+    for (int s = 0; s + 2 <= nsteps; s += 2) {
+        GT(0);
+        multiply(lds);
+        GT(1);
+        __syncthreads();
+        GT(3);
+        multiply(lds + kGemmBuf);
         __syncthreads();
     }
-    if (nsteps & 1)
+    GTDUMP();
+    if (nsteps & 1) {
         multiply(lds);
+        __syncthreads();
+    }
 
     // C tile: lane holds column ln (weight row), rows (i/4)*8 + lh*4 + i%4 (tokens)
 #pragma unroll
@@ -608,7 +676,7 @@ int launch_gemm_q8_f16(hipStream_t st, const uint8_t *w, const float *x, const f
 {
     const dim3 grid((unsigned)((m + kGemmM - 1) / kGemmM), (unsigned)((tokens + kGemmT - 1) / kGemmT), 1);
     if (x16 == nullptr) {
-        hipLaunchKernelGGL(gemm_q8_f16_kernel<false>, grid, dim3(256, 1, 1), kGemmLds, st, w, x, y, m, k, tokens);
+        hipLaunchKernelGGL(gemm_q8_f16_kernel<false>, grid, dim3(512, 1, 1), kGemmLds, st, w, x, y, m, k, tokens);
         return launched("gemm_q8_0_f16");
     }
     const size_t n8 = (size_t)tokens * k / 8;
@@ -618,7 +686,7 @@ int launch_gemm_q8_f16(hipStream_t st, const uint8_t *w, const float *x, const f
     int rc = launched("gate_f16");
     if (rc)
         return rc;
-    hipLaunchKernelGGL(gemm_q8_f16_kernel<true>, grid, dim3(256, 1, 1), kGemmLds, st, w, x16, y, m, k, tokens);
+    hipLaunchKernelGGL(gemm_q8_f16_kernel<true>, grid, dim3(512, 1, 1), kGemmLds, st, w, x16, y, m, k, tokens);
     return launched("gemm_q8_0_f16");
 }
 
