@@ -366,7 +366,9 @@ def bench_gemv(torch, attn, rows, steps, layers, m=5120, k=6144):
     return {"workload": f"W_o projection, Q8_0 {m}x{k}, {rows} activation rows",
             "us_per_layer": us, "weight_bytes": m * (k // 32) * 34, "layers_rotated": layers,
             "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": gbs / HBM_PEAK_GBS, "traffic": None, "kernel": "gemv_q8_rows_kernel",
+                         "frac": gbs / HBM_PEAK_GBS,
+                         "traffic": measured_traffic("gemv1" if rows == 1 else "", ["gemv_q8_rows_kernel"]),
+                         "kernel": "gemv_q8_rows_kernel",
                          "bytes_per_launch": nbytes, "launch_us": us}}
 
 
@@ -399,7 +401,10 @@ def bench_gemm(torch, attn, tokens, steps, layers, m=5120, k=6144):
             "us_per_layer": us, "us_per_layer_f32_rows_no_gate": t32.ms * 1e3 / (steps * layers),
             "flop": flop, "layers_rotated": layers,
             "roofline": {"bound": "mfma", "achieved": tf, "peak": MFMA_F16_PEAK_TF, "unit": "TFLOP/s",
-                         "frac": tf / MFMA_F16_PEAK_TF, "traffic": None, "kernel": "gate_f16_kernel + gemm_q8_f16_kernel",
+                         "frac": tf / MFMA_F16_PEAK_TF,
+                         "traffic": measured_traffic("gemm672" if tokens == 672 else "",
+                                                     ["gate_f16_kernel", "gemm_q8_f16_kernel"]),
+                         "kernel": "gate_f16_kernel + gemm_q8_f16_kernel",
                          "flop_per_launch": flop, "launch_us": us}}
 
 

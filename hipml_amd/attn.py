@@ -36,6 +36,7 @@ EXPORTS = [
     "hipml_attn_chunk_q8_split", "hipml_attn_chunk_q8_split_gate", "hipml_q_gate_f32",
     "hipml_attn_front_f32", "hipml_attn_chunk_front_f32",
     "hipml_gemv_q8_0_rows", "hipml_gemm_q8_0_f16", "hipml_attn_output_chunk_q8_0",
+    "hipml_kv_rows_copy",
 ]
 
 
@@ -96,6 +97,7 @@ def lib() -> C.CDLL:
             "hipml_q_gate_f32": (i, [vp, vp, vp, vp, sz]),
             "hipml_attn_front_f32": (i, [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, i, i, vp, f, f]),
             "hipml_attn_chunk_front_f32": (i, [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, f, f, i, i]),
+            "hipml_kv_rows_copy": (i, [vp, i, vp, vp, vp, vp, i, i, i, i, i]),
             "hipml_gemv_q8_0_rows": (i, [vp, vp, vp, vp, i, i, i]),
             "hipml_gemm_q8_0_f16": (i, [vp, vp, vp, vp, i, i, i]),
             "hipml_attn_output_chunk_q8_0": (i, [vp, vp, vp, vp, vp, i, i, i, vp]),
@@ -224,6 +226,13 @@ def kv_encode_rows(dtype, k_f32, v_f32, k_cache, v_cache, n_kv, head_dim, stride
     _check(lib().hipml_kv_encode_rows(_stream(stream), dtype, _p(k_f32), _p(v_f32), _p(k_cache),
                                       _p(v_cache), n_kv, head_dim, stride, _p(pos), slot_bytes,
                                       slots))
+
+
+def kv_rows_copy(dtype, k_src, v_src, k_dst, v_dst, n_kv, head_dim, src_stride, dst_stride, rows,
+                 stream=None):
+    """Prefix snapshot / restore of cache rows (`GpuEngine::prefix_capture` / `prefix_restore`)."""
+    _check(lib().hipml_kv_rows_copy(_stream(stream), dtype, _p(k_src), _p(v_src), _p(k_dst), _p(v_dst),
+                                    n_kv, head_dim, src_stride, dst_stride, rows))
 
 
 # ---- decode -------------------------------------------------------------------------------
@@ -377,3 +386,22 @@ class DeepKv:
 
     def bytes(self) -> int:
         return 2 * self.n_kv * self.seq * self.row_bytes
+
+    def snapshot(self, pos: int, stream=None):
+        """Rows [0, pos) of every head, packed [n_kv][pos][row bytes] (K, V): the quantized half of a
+        prefix snapshot (crates/hipml-model/src/gpu/prefix.rs:214-239)."""
+        k = torch.empty((self.n_kv, pos, self.row_bytes), dtype=torch.uint8, device=self.k.device)
+        v = torch.empty_like(k)
+        if pos > 0:
+            kv_rows_copy(self.dtype, self.k, self.v, k, v, self.n_kv, self.head_dim, self.seq, pos, pos,
+                         stream)
+        return k, v
+
+    def restore(self, k, v, stream=None):
+        """Write a packed snapshot back as rows [0, pos) of this cache; rows past pos keep their bytes
+        (they are never read: the live length says so)."""
+        pos = k.shape[1]
+        assert pos <= self.seq and k.shape == v.shape == (self.n_kv, pos, self.row_bytes)
+        if pos > 0:
+            kv_rows_copy(self.dtype, k, v, self.k, self.v, self.n_kv, self.head_dim, pos, self.seq, pos,
+                         stream)

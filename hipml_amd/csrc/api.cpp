@@ -490,6 +490,31 @@ int hipml_kv_encode_rows(hipml_stream_t stream, int dtype, const float *k_f32, c
                                slot_bytes, slots, 0, 0, slots);
 }
 
+int hipml_kv_rows_copy(hipml_stream_t stream, int dtype, const void *k_src, const void *v_src, void *k_dst,
+                       void *v_dst, int n_kv, int head_dim, int src_stride, int dst_stride, int rows)
+{
+    clear_error();
+    int rc = check_kv_dtype(dtype);
+    if (rc)
+        return rc;
+    REQUIRE_PTR(k_src);
+    REQUIRE_PTR(v_src);
+    REQUIRE_PTR(k_dst);
+    REQUIRE_PTR(v_dst);
+    if (head_dim != kHeadDim)
+        return fail(HIPML_ATTN_E_UNSUPPORTED, "head_dim %d: this library is built for %d", head_dim, kHeadDim);
+    if (n_kv < 1 || n_kv > 64)
+        return fail(HIPML_ATTN_E_RANGE, "n_kv %d outside 1..64", n_kv);
+    if (rows < 0 || rows > src_stride || rows > dst_stride)
+        return fail(HIPML_ATTN_E_RANGE, "rows %d do not fit strides %d -> %d", rows, src_stride, dst_stride);
+    if ((rc = check_aligned16(k_src, "k_src")) || (rc = check_aligned16(v_src, "v_src")) ||
+        (rc = check_aligned16(k_dst, "k_dst")) || (rc = check_aligned16(v_dst, "v_dst")))
+        return rc;
+    return launch_kv_rows_copy(as_stream(stream), dtype, static_cast<const uint8_t *>(k_src),
+                               static_cast<const uint8_t *>(v_src), static_cast<uint8_t *>(k_dst),
+                               static_cast<uint8_t *>(v_dst), n_kv, src_stride, dst_stride, rows);
+}
+
 // ---- decode ------------------------------------------------------------------------------------
 
 int hipml_attn_decode_kv(hipml_stream_t stream, const int32_t *step, int dtype, const float *q,

@@ -452,4 +452,39 @@ int launch_q_gate(hipStream_t st, const float *x, const float *gate, float *y, s
     return 0;
 }
 
+// ---- prefix snapshot / restore of cache rows ------------------------------------------
+//
+// Rows [0, rows) of every KV head, K and V, between two caches that differ only in their rows per
+// head (crates/hipml-model/src/gpu/prefix.rs:214-239 packs a prefix as [head][pos][row] with one
+// device copy per head and array; this is one launch, legal under capture).  16 bytes per thread
+// and turn: a row is 272 or 144 bytes, so every head's span starts and ends on a 16-byte boundary.
+
+__global__ void __launch_bounds__(256) kv_rows_copy_kernel(const uint4 *__restrict__ k_src,
+                                                          const uint4 *__restrict__ v_src,
+                                                          uint4 *__restrict__ k_dst, uint4 *__restrict__ v_dst,
+                                                          size_t src_head16, size_t dst_head16, size_t span16)
+{
+    const uint4 *src = (blockIdx.z ? v_src : k_src) + blockIdx.y * src_head16;
+    uint4 *dst = (blockIdx.z ? v_dst : k_dst) + blockIdx.y * dst_head16;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < span16; i += (size_t)gridDim.x * 256)
+        dst[i] = src[i];
+}
+
+int launch_kv_rows_copy(hipStream_t st, int q4, const uint8_t *k_src, const uint8_t *v_src, uint8_t *k_dst,
+                        uint8_t *v_dst, int n_kv, int src_stride, int dst_stride, int rows)
+{
+    const size_t row16 = (size_t)(q4 ? kRowBytesQ4 : kRowBytes) / 16;
+    const size_t span16 = (size_t)rows * row16;
+    if (span16 == 0)
+        return 0;
+    size_t blocks = (span16 + 255) / 256;
+    if (blocks > 512)
+        blocks = 512; // 2,048 workgroups over K, V and four heads fill the chip; the rest is the loop
+    hipLaunchKernelGGL(kv_rows_copy_kernel, dim3((unsigned)blocks, (unsigned)n_kv, 2), dim3(256, 1, 1), 0, st,
+                       reinterpret_cast<const uint4 *>(k_src), reinterpret_cast<const uint4 *>(v_src),
+                       reinterpret_cast<uint4 *>(k_dst), reinterpret_cast<uint4 *>(v_dst),
+                       (size_t)src_stride * row16, (size_t)dst_stride * row16, span16);
+    return launched("kv_rows_copy");
+}
+
 } // namespace hipml

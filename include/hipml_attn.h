@@ -265,6 +265,15 @@ int hipml_attn_chunk_q8_split_gate(hipml_stream_t stream, const float *q, const 
 int hipml_q_gate_f32(hipml_stream_t stream, const float *x, const float *gate, float *y,
                      size_t n);
 
+/* Prefix snapshot / restore: rows [0, rows) of every KV head of K and V, from a cache with
+ * src_stride rows per head to one with dst_stride rows per head (same format; dtype 0 = q8_0,
+ * 1 = q4_0).  dst_stride = rows packs a prefix as [head][rows][row bytes]; swapping the roles
+ * restores it.  One launch, asynchronous, legal under capture.
+ * Replaces the per-head copy_range_on loop of GpuEngine::prefix_capture / prefix_restore over a
+ * DeepKv, crates/hipml-model/src/gpu/prefix.rs:214-239. */
+int hipml_kv_rows_copy(hipml_stream_t stream, int dtype, const void *k_src, const void *v_src, void *k_dst,
+                       void *v_dst, int n_kv, int head_dim, int src_stride, int dst_stride, int rows);
+
 /* ---- projections over Q8_0 weight matrices (the steps either side of the attention core) ---- */
 
 /* y[r][row] = sum_k W[row][k] * x[r][k] for r < rows: W is m rows of k/32 Q8_0 blocks (34 bytes:

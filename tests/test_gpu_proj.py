@@ -198,3 +198,17 @@ def test_output_chunk_equals_gate_then_gemm():
     attn.gemm_q8_0_f16(wd, ad, ref, m, k, t)
     torch.cuda.synchronize()
     assert torch.equal(plain, ref)
+
+
+@pytest.mark.parametrize("m,k", [(1024, 5120), (12288, 5120)])
+def test_qkv_projection_shapes(m, k):
+    # the projections before the path use the same entry points: W_k / W_v 5120 -> 1024 and
+    # W_q (q|gate) 5120 -> 12288 (attn_gpu.rs:490-498, prepare_rows :948-966)
+    r = orc.Rng(0x0AB0 + m)
+    w = orc.random_q8_0_bytes(r, m * k // 32)
+    x = r.normal_array((3, k), 0.5)
+    want = orc.gemm_q8_0(w, x, 3, m, k, n_threads=8)
+    ok, _, _ = report(f"rows {m}x{k} t=3", want, run_gemv(w, x, m, k, 3), 2e-4, 1e-3)
+    assert ok
+    ok, _, _ = report(f"chunk {m}x{k} t=3", want, run_gemm(w, x, m, k, 3), *F16_LARGE)
+    assert ok
