@@ -303,8 +303,6 @@ def bench_batch(torch, attn, orc, steps, warmup, layers):
                     f"slots 0..3 carry 3 query rows (MTP verify), one launch",
         "slots": slots, "rows": rows, "live_rows": live, "splits": splits, "layers_rotated": layers,
         "us_per_layer": us,
-        "us_per_layer_gate_fused": tg.ms * 1e3 / (steps * layers),
-        "us_per_layer_gate_separate": ts.ms * 1e3 / (steps * layers),
         "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": gbs / HBM_PEAK_GBS, "traffic": traffic,
                      "kernel": "decode_q8_kernel + decode_reduce_kernel",
