@@ -128,11 +128,10 @@ def bench_prefill(torch, attn, tokens, pos0, steps, warmup, layers, prefix_fill=
                                       splits)
 
     def step(i):
-        # the gate is applied where the attention result is written (same bits as the separate
-        # gate kernel, one pass over the rows less)
+        # RoPE and the append share one launch; the gate is applied where the attention result is
+        # written (same bits as the separate kernels, two launches and one pass over the rows less)
         k, v = caches[i % layers]
-        attn.rope_chunk(q, kx, H, KV, HD, NROT, THETA, pos0, tokens)
-        attn.kv_encode_bulk(0, kx, vx, k, v, KV, HD, stride, pos0, 0, tokens)
+        attn.rope_encode_chunk(q, kx, vx, k, v, H, KV, HD, NROT, THETA, pos0, tokens, 0, stride)
         attn.chunk_attention_q8_split_gate(q, k, v, gate, out, H, KV, HD, pos0, tokens, 1, stride,
                                            acc, ml, splits)
 
@@ -173,7 +172,7 @@ def bench_prefill(torch, attn, tokens, pos0, steps, warmup, layers, prefix_fill=
         "tokens": tokens, "pos0": pos0, "splits": splits, "layers_rotated": layers,
         "ms_per_step": wall_ms,
         "tok_per_s": tokens / (wall_ms * 1e-3),
-        "ms_per_step_separate_gate": unfused_ms,
+        "ms_per_step_separate_launches": unfused_ms,
         "attn_ms": attn_ms,
         "attn_tok_per_s": tokens / (attn_ms * 1e-3),
         "roofline": {"bound": "mfma", "achieved": tf, "peak": MFMA_F16_PEAK_TF, "unit": "TFLOP/s",

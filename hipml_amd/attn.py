@@ -36,7 +36,7 @@ EXPORTS = [
     "hipml_attn_chunk_q8_split", "hipml_attn_chunk_q8_split_gate", "hipml_q_gate_f32",
     "hipml_attn_front_f32", "hipml_attn_chunk_front_f32",
     "hipml_gemv_q8_0_rows", "hipml_gemm_q8_0_f16", "hipml_attn_output_chunk_q8_0",
-    "hipml_kv_rows_copy",
+    "hipml_kv_rows_copy", "hipml_rope_encode_chunk_f32",
 ]
 
 
@@ -98,6 +98,7 @@ def lib() -> C.CDLL:
             "hipml_attn_front_f32": (i, [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, i, i, vp, f, f]),
             "hipml_attn_chunk_front_f32": (i, [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, f, f, i, i]),
             "hipml_kv_rows_copy": (i, [vp, i, vp, vp, vp, vp, i, i, i, i, i]),
+            "hipml_rope_encode_chunk_f32": (i, [vp, vp, vp, vp, vp, vp, i, i, i, i, f, i, i, i, i]),
             "hipml_gemv_q8_0_rows": (i, [vp, vp, vp, vp, i, i, i]),
             "hipml_gemm_q8_0_f16": (i, [vp, vp, vp, vp, i, i, i]),
             "hipml_attn_output_chunk_q8_0": (i, [vp, vp, vp, vp, vp, i, i, i, vp]),
@@ -226,6 +227,14 @@ def kv_encode_rows(dtype, k_f32, v_f32, k_cache, v_cache, n_kv, head_dim, stride
     _check(lib().hipml_kv_encode_rows(_stream(stream), dtype, _p(k_f32), _p(v_f32), _p(k_cache),
                                       _p(v_cache), n_kv, head_dim, stride, _p(pos), slot_bytes,
                                       slots))
+
+
+def rope_encode_chunk(q, k, v, k_cache, v_cache, n_head, n_kv, head_dim, n_rot, theta, pos0, tokens,
+                      dtype, stride, stream=None):
+    """`rope_chunk` + `kv_encode_bulk(start=pos0, src0=0, rows=tokens)` in one launch."""
+    _check(lib().hipml_rope_encode_chunk_f32(_stream(stream), _p(q), _p(k), _p(v), _p(k_cache),
+                                             _p(v_cache), n_head, n_kv, head_dim, n_rot, theta, pos0,
+                                             tokens, dtype, stride))
 
 
 def kv_rows_copy(dtype, k_src, v_src, k_dst, v_dst, n_kv, head_dim, src_stride, dst_stride, rows,

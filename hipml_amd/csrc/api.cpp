@@ -474,6 +474,32 @@ int hipml_kv_encode_bulk(hipml_stream_t stream, int dtype, const float *k_f32, c
                                0, rows, start, src0, rows);
 }
 
+int hipml_rope_encode_chunk_f32(hipml_stream_t stream, float *q, float *k, const float *v, void *k_cache,
+                                void *v_cache, int n_head, int n_kv, int head_dim, int n_rot,
+                                float theta_base, int pos0, int tokens, int dtype, int stride)
+{
+    clear_error();
+    REQUIRE_PTR(q);
+    int rc = check_rope(n_head, head_dim, n_rot, theta_base);
+    if (rc == 0)
+        rc = check_encode(dtype, k, v, k_cache, v_cache, n_kv, head_dim, stride);
+    if (rc)
+        return rc;
+    if (head_dim != kHeadDim || n_rot != 64)
+        return fail(HIPML_ATTN_E_UNSUPPORTED, "head_dim %d / n_rot %d: the fused kernel is built for %d / 64",
+                    head_dim, n_rot, kHeadDim);
+    if (pos0 < 0 || tokens < 0)
+        return fail(HIPML_ATTN_E_RANGE, "pos0 %d / tokens %d must be non-negative", pos0, tokens);
+    if ((long long)pos0 + tokens > stride)
+        return fail(HIPML_ATTN_E_RANGE, "rows [%d, %d) do not fit a cache of %d rows per head", pos0,
+                    pos0 + tokens, stride);
+    if (tokens == 0)
+        return 0;
+    return launch_rope_encode_chunk(as_stream(stream), dtype, q, k, v, static_cast<uint8_t *>(k_cache),
+                                    static_cast<uint8_t *>(v_cache), n_head, n_kv, n_rot, theta_base, pos0,
+                                    tokens, stride, g_rope);
+}
+
 int hipml_kv_encode_rows(hipml_stream_t stream, int dtype, const float *k_f32, const float *v_f32,
                          void *k_cache, void *v_cache, int n_kv, int head_dim, int stride,
                          const int32_t *pos, size_t slot_bytes, int slots)

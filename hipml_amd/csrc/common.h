@@ -58,6 +58,10 @@ int launch_rope_chunk(hipStream_t st, float *q, float *k, int n_head, int n_kv, 
 int launch_kv_encode(hipStream_t st, int q4, const float *k, const float *v, uint8_t *kc, uint8_t *vc,
                      int n_kv, int head_dim, int stride, const int32_t *pos, int pos_stride,
                      size_t slot_bytes, int slots, int start, int src0, int rows);
+// rope_chunk + kv_encode_bulk(start = pos0, src0 = 0, rows = tokens) in one launch (n_rot must be 64).
+int launch_rope_encode_chunk(hipStream_t st, int q4, float *q, float *k, const float *v, uint8_t *kc,
+                             uint8_t *vc, int n_head, int n_kv, int n_rot, float theta, int pos0,
+                             int tokens, int stride, const RopeTable &tab);
 int launch_kv_rows_copy(hipStream_t st, int q4, const uint8_t *k_src, const uint8_t *v_src, uint8_t *k_dst,
                         uint8_t *v_dst, int n_kv, int src_stride, int dst_stride, int rows);
 int launch_front(hipStream_t st, const float *qg, float *q, float *gate, float *k, const float *qw,

@@ -289,6 +289,88 @@ int launch_rope_chunk(hipStream_t st, float *q, float *k, int n_head, int n_kv, 
     return 0;
 }
 
+// RoPE of a chunk and the append of its K/V rows in one launch: the first `q_blocks` workgroups
+// rotate 8 query head rows each (as rope_chunk_kernel does), the others take one (token, kv head)
+// each: thread t holds value t of the K row, pair partners (t, t + 32 for t < 32) meet through a
+// lane exchange inside wave 0, the rotated row is written back and quantized together with the V
+// row (as kv_encode_*_kernel does).  Same expressions, same bits as the two separate launches.
+template <bool Q4>
+__global__ void __launch_bounds__(256) rope_encode_chunk_kernel(
+    float *__restrict__ q, float *__restrict__ kx, const float *__restrict__ vx, uint8_t *__restrict__ kc,
+    uint8_t *__restrict__ vc, int n_head, int n_kv, int n_rot, float theta, int pos0, int tokens,
+    int stride, int q_blocks, const float *__restrict__ tab, int tab_rows)
+{
+    const int half = n_rot >> 1;
+    if ((int)blockIdx.x < q_blocks) {
+        const long long r = (long long)blockIdx.x * 8 + (threadIdx.x >> 5);
+        if (r >= (long long)tokens * n_head)
+            return;
+        const int t = (int)(r / n_head);
+        float *row = q + (size_t)r * kHeadDim;
+        for (int k = threadIdx.x & 31; k < half; k += 32) {
+            float cs, sn;
+            rope_cs(tab, tab_rows, half, k, pos0 + t, n_rot, theta, cs, sn);
+            const float x1 = row[k];
+            const float x2 = row[half + k];
+            row[k] = x1 * cs - x2 * sn;
+            row[half + k] = x1 * sn + x2 * cs;
+        }
+        return;
+    }
+    const int u = (int)blockIdx.x - q_blocks; // (token, kv head)
+    const int tok = u / n_kv, h = u - tok * n_kv;
+    const int t = threadIdx.x;
+    const size_t src = (size_t)u * kHeadDim + t;
+    float xk = kx[src];
+    const float xv = vx[src];
+    if (t < 64) { // wave 0: the rotated channels are 0 .. n_rot-1 <= 64
+        const float other = __shfl_xor(xk, half); // half is 32 here (checked by the launcher)
+        if (t < n_rot) {
+            const int k = t < half ? t : t - half;
+            float cs, sn;
+            rope_cs(tab, tab_rows, half, k, pos0 + tok, n_rot, theta, cs, sn);
+            xk = t < half ? xk * cs - other * sn : other * sn + xk * cs;
+            kx[src] = xk;
+        }
+    }
+    const int chunk = t >> 5, lane32 = t & 31;
+    const size_t blk = ((size_t)h * stride + (pos0 + tok)) * (kHeadDim / 32) + chunk;
+    if (Q4) {
+        q4_encode_store(xk, kc + blk * kQ4BlockBytes, lane32);
+        q4_encode_store(xv, vc + blk * kQ4BlockBytes, lane32);
+    } else {
+        q8_encode_store(xk, kc + blk * kQ8BlockBytes, lane32);
+        q8_encode_store(xv, vc + blk * kQ8BlockBytes, lane32);
+    }
+}
+
+int launch_rope_encode_chunk(hipStream_t st, int q4, float *q, float *k, const float *v, uint8_t *kc,
+                             uint8_t *vc, int n_head, int n_kv, int n_rot, float theta, int pos0,
+                             int tokens, int stride, const RopeTable &tab)
+{
+    int tab_rows = 0;
+    const float *t = table_for(tab, theta, n_rot, &tab_rows);
+    const int slab = 1 << 18; // tokens per launch: keeps the grid inside 2^31 workgroups
+    for (int t0 = 0; t0 < tokens; t0 += slab) {
+        const int n = tokens - t0 < slab ? tokens - t0 : slab;
+        const int q_blocks = (int)(((long long)n * n_head + 7) / 8);
+        const dim3 grid((unsigned)(q_blocks + n * n_kv), 1, 1);
+        float *qq = q + (size_t)t0 * n_head * kHeadDim;
+        float *kk = k + (size_t)t0 * n_kv * kHeadDim;
+        const float *vv = v + (size_t)t0 * n_kv * kHeadDim;
+        if (q4)
+            hipLaunchKernelGGL(rope_encode_chunk_kernel<true>, grid, dim3(256, 1, 1), 0, st, qq, kk, vv, kc, vc,
+                               n_head, n_kv, n_rot, theta, pos0 + t0, n, stride, q_blocks, t, tab_rows);
+        else
+            hipLaunchKernelGGL(rope_encode_chunk_kernel<false>, grid, dim3(256, 1, 1), 0, st, qq, kk, vv, kc, vc,
+                               n_head, n_kv, n_rot, theta, pos0 + t0, n, stride, q_blocks, t, tab_rows);
+        int rc = launched("rope_encode_chunk");
+        if (rc)
+            return rc;
+    }
+    return 0;
+}
+
 // ---- attention front end ------------------------------------------------------------
 //
 // q|gate split, per-head RMS norm of q and k, M-RoPE of both, one wave per (row, head):

@@ -147,6 +147,15 @@ int hipml_kv_encode(hipml_stream_t stream, const int32_t *step, int dtype, const
 int hipml_kv_encode_bulk(hipml_stream_t stream, int dtype, const float *k_f32, const float *v_f32,
                          void *k_cache, void *v_cache, int n_kv, int head_dim, int stride,
                          int start, int src0, int rows);
+/* RoPE of a chunk and the append of its K/V rows in one launch: hipml_rope_chunk_f32(q, k, ...)
+ * followed by hipml_kv_encode_bulk(dtype, k, v, ..., start = pos0, src0 = 0, rows = tokens), with the
+ * same bits in q, k and both caches.  v is f32 [tokens][n_kv][head_dim].  head_dim 256, n_rot 64.
+ * Replaces the RoPE half of AttnLayer::chunk_front + Launcher::kv_encode_bulk as issued per chunk,
+ * crates/hipml-model/src/gpu/attn_tile.rs:53-68. */
+int hipml_rope_encode_chunk_f32(hipml_stream_t stream, float *q, float *k, const float *v, void *k_cache,
+                                void *v_cache, int n_head, int n_kv, int head_dim, int n_rot,
+                                float theta_base, int pos0, int tokens, int dtype, int stride);
+
 /* One row per slot: row s of k_f32/v_f32 goes to cache (base + s*slot_bytes) at
  * position pos[s*2].  Replaces Launcher::kv_encode_rows_ptr -> kv_encode_q8_b,
  * crates/hipml-kernels/src/launch/device/batch_launch.rs:59-105. */

@@ -173,6 +173,35 @@ def test_rope_chunk_bits_equal_oracle(pos0, tokens):
     assert np.array_equal(qg.view(np.uint32), want_q.view(np.uint32))
 
 
+@pytest.mark.parametrize("dtype", [0, 1])
+@pytest.mark.parametrize("pos0,tokens", [(0, 672), (29, 37), (100_000, 300)])
+def test_fused_rope_and_append_has_the_bits_of_the_two_launches(pos0, tokens, dtype):
+    # rope_chunk + kv_encode_bulk in one launch: q, k and both caches byte for byte, and the cache
+    # bytes against the oracle (rope in f64 trig, then the format's quantizer)
+    stride = pos0 + tokens + 5
+    row = 272 if dtype == 0 else 144
+    r = orc.Rng(4321 + pos0 + dtype)
+    q = r.normal_array((tokens, N_HEADS, HD))
+    k = r.normal_array((tokens, N_KV, HD))
+    v = r.normal_array((tokens, N_KV, HD))
+    q1, k1, q2, k2, vd = dev(q), dev(k), dev(q), dev(k), dev(v)
+    kc1 = torch.full((N_KV, stride, row), 0x5A, dtype=torch.uint8, device="cuda")
+    vc1, kc2, vc2 = kc1.clone(), kc1.clone(), kc1.clone()
+    attn.rope_chunk(q1, k1, N_HEADS, N_KV, HD, N_ROT, THETA, pos0, tokens)
+    attn.kv_encode_bulk(dtype, k1, vd, kc1, vc1, N_KV, HD, stride, pos0, 0, tokens)
+    attn.rope_encode_chunk(q2, k2, vd, kc2, vc2, N_HEADS, N_KV, HD, N_ROT, THETA, pos0, tokens, dtype, stride)
+    torch.cuda.synchronize()
+    assert torch.equal(q1, q2) and torch.equal(k1, k2)
+    assert torch.equal(kc1, kc2) and torch.equal(vc1, vc2)
+    kr = np.stack([orc.rope_multi(k[t], N_KV, HD, N_ROT, SECTIONS, [pos0 + t] * 4, THETA).reshape(N_KV, HD)
+                   for t in range(tokens)])
+    want_k = orc.quantize(dtype, np.ascontiguousarray(kr.transpose(1, 0, 2))).reshape(N_KV, tokens, row)
+    want_v = orc.quantize(dtype, np.ascontiguousarray(v.transpose(1, 0, 2))).reshape(N_KV, tokens, row)
+    assert np.array_equal(host(kc2)[:, pos0:pos0 + tokens], want_k)
+    assert np.array_equal(host(vc2)[:, pos0:pos0 + tokens], want_v)
+    assert bool((kc2[:, :pos0] == 0x5A).all()) and bool((kc2[:, pos0 + tokens:] == 0x5A).all())
+
+
 def test_rope_beyond_table_falls_back_to_device_math():
     # positions past the table are computed on the device: within one f32 ulp of the
     # host definition (not guaranteed identical), so this is a tolerance check.
