@@ -75,6 +75,14 @@ static int decode_format(int dtype, int *kv_dtype)
                 "KV dtype selector %d: 0/4 (q8_0) and 1/5 (q4_0) are built", dtype);
 }
 
+// The MFMA kernels keep more LDS than a launch may use by default; hipml_attn_init raises the limit.
+static int require_init()
+{
+    if (!g_inited)
+        return fail(HIPML_ATTN_E_STATE, "hipml_attn_init has not been called in this process");
+    return 0;
+}
+
 static int check_aligned16(const void *p, const char *name)
 {
     if (((uintptr_t)p & 15) != 0)
@@ -151,6 +159,8 @@ static int decode_common(hipStream_t st, int dtype, const int32_t *pos, const fl
     }
     L.total_rows = rows;
     L.max_cols = max_cols;
+    if ((rc = require_init()))
+        return rc;
     return launch_decode_q8(st, L);
 }
 
@@ -719,6 +729,8 @@ static int chunk_q8_common(hipml_stream_t stream, const float *q, const void *kc
         return rc;
     if (tokens == 0)
         return 0;
+    if ((rc = require_init()))
+        return rc;
     return launch_chunk_q8(as_stream(stream), q, static_cast<const uint8_t *>(kc),
                            static_cast<const uint8_t *>(vc), out, n_head, n_kv, pos0, tokens,
                            stride, part_acc, part_ml, splits, want_gate ? gate : nullptr, dtype == 2 ? 1 : 0);
@@ -772,6 +784,8 @@ int hipml_gemv_q8_0_rows(hipml_stream_t stream, const void *w, const float *x, f
     if (((uintptr_t)w & 3) != 0)
         return fail(HIPML_ATTN_E_RANGE, "w must be 4-byte aligned");
     int rc = check_aligned16(x, "x");
+    if (rc == 0)
+        rc = require_init();
     if (rc)
         return rc;
     return launch_gemv_q8_rows(as_stream(stream), static_cast<const uint8_t *>(w), x, y, m, k, rows);
@@ -791,7 +805,8 @@ static int check_gemm(const void *w, const float *x, const float *y, int m, int 
         return fail(HIPML_ATTN_E_RANGE, "tokens %d must be positive", tokens);
     if (((uintptr_t)w & 3) != 0)
         return fail(HIPML_ATTN_E_RANGE, "w must be 4-byte aligned");
-    return check_aligned16(x, "x");
+    int rc = check_aligned16(x, "x");
+    return rc ? rc : require_init();
 }
 
 int hipml_gemm_q8_0_f16(hipml_stream_t stream, const void *w, const float *x, float *y, int m, int k,

@@ -100,7 +100,7 @@ __host__ __device__ inline int gemv_rows_per_pass(int k)
     const int fit = kGemvLdsBudget / (4 * k);
     return fit > kGemvMaxRows ? kGemvMaxRows : fit;
 }
-static_assert(kGemvLdsBudget / 4 / 8 / 256 <= 16, "a pass is staged in one round of at most 16 groups per thread");
+static_assert(kGemvLdsBudget / 4 / 8 / 512 <= 8, "a pass is staged in one round of at most 8 groups per thread");
 
 // LDS: x operands [k/32 blocks][2*rp A rows: hi of rows 0..rp-1, then lo][4 quarters][8 x f16], then
 // the partial sums [WAVES][TILES][32 lanes] float4.  The hi and the lo halves are different rows of
@@ -337,9 +337,8 @@ static int launch_gemv_variant(hipStream_t st, const uint8_t *w, const float *x,
         return launch_gemv_xg<WAVES, TILES, CH, 2>(st, w, x, y, m, k, rows, rp);
     if (need <= 4)
         return launch_gemv_xg<WAVES, TILES, CH, 4>(st, w, x, y, m, k, rows, rp);
-    if (need <= 8)
-        return launch_gemv_xg<WAVES, TILES, CH, 8>(st, w, x, y, m, k, rows, rp);
-    return launch_gemv_xg<WAVES, TILES, CH, 16>(st, w, x, y, m, k, rows, rp);
+    // rp * k <= 32,768 (the LDS budget), so 8 groups per thread always cover a pass
+    return launch_gemv_xg<WAVES, TILES, CH, 8>(st, w, x, y, m, k, rows, rp);
 }
 
 int launch_gemv_q8_rows(hipStream_t st, const uint8_t *w, const float *x, float *y, int m, int k, int rows)
@@ -650,7 +649,6 @@ static hipError_t raise_gemv_lds()
     raise(reinterpret_cast<const void *>(&gemv_q8_rows_kernel<WAVES, TILES, CH, 2>));
     raise(reinterpret_cast<const void *>(&gemv_q8_rows_kernel<WAVES, TILES, CH, 4>));
     raise(reinterpret_cast<const void *>(&gemv_q8_rows_kernel<WAVES, TILES, CH, 8>));
-    raise(reinterpret_cast<const void *>(&gemv_q8_rows_kernel<WAVES, TILES, CH, 16>));
     return e;
 }
 

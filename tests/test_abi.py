@@ -90,3 +90,22 @@ def test_argument_errors_come_before_any_launch(lib):
     with pytest.raises(attn.HipmlError) as e:
         attn._check(rc)
     assert e.value.code == rc
+
+
+def test_launching_entry_points_ask_for_init_first(lib):
+    # the MFMA kernels need the LDS limit that hipml_attn_init raises; without it a call with valid
+    # arguments is refused with a message instead of failing inside the launch
+    from hipml_amd import attn
+    if attn_inited():
+        pytest.skip("the library was initialised earlier in this process")
+    one = C.c_void_p(16)
+    rc = lib.hipml_gemv_q8_0_rows(None, one, one, one, 64, 64, 1)
+    assert rc == -6 and b"hipml_attn_init" in lib.hipml_attn_last_error()
+    rc = lib.hipml_attn_decode_kv(None, one, 0, one, one, one, one, one, one, 24, 4, 256, 64,
+                                  C.c_float(0.0625), 1, 0, 0)
+    assert rc == -6 and b"hipml_attn_init" in lib.hipml_attn_last_error()
+
+
+def attn_inited():
+    import torch
+    return torch.cuda.is_available()
