@@ -157,3 +157,149 @@ def test_greedy_argmax_of_a_synthetic_projection_agrees():
     # every disagreement must be explained by a margin below twice the logit noise
     assert all(agree[i] or margin[i] <= 2 * noise[i] for i in range(len(agree)))
     assert agree.mean() >= 0.98
+
+
+def test_layer_tail_with_projection_replays_under_a_captured_graph():
+    # decode step with the fused entry points: append, attention + gate in the merge, then the output
+    # projection over Q8_0 weights -- captured once, replayed at growing positions, every replay
+    # against the eager result of the same calls (bit for bit) and against the oracle.
+    stride, pos0, steps = 512, 300, 3
+    m, k = 320, N_HEADS * HD
+    r = orc.Rng(0x6AA0)
+    kf = r.normal_array((N_KV, pos0, HD))
+    vf = r.normal_array((N_KV, pos0, HD))
+    kb0, vb0 = quantized_cache(kf, vf, stride)
+    wo = orc.random_q8_0_bytes(r, m * k // 32)
+    qs = r.normal_array((steps, N_HEADS, HD))
+    ks = r.normal_array((steps, N_KV, HD))
+    vs = r.normal_array((steps, N_KV, HD))
+    gs = r.normal_array((steps, N_HEADS, HD))
+
+    kc, vc, wd = dev(kb0), dev(vb0), dev(wo)
+    splits = attn.decode_splits(stride, N_KV)
+    acc = torch.empty((N_HEADS, splits, HD), device="cuda")
+    ml = torch.empty((N_HEADS, splits, 2), device="cuda")
+    step = torch.zeros(8, dtype=torch.int32, device="cuda")
+    q_in = torch.empty((N_HEADS, HD), device="cuda")
+    k_in = torch.empty((N_KV, HD), device="cuda")
+    v_in = torch.empty((N_KV, HD), device="cuda")
+    g_in = torch.empty((N_HEADS, HD), device="cuda")
+    out = torch.empty((N_HEADS, HD), device="cuda")
+    y = torch.empty((1, m), device="cuda")
+
+    def one_step():
+        attn.kv_encode(step, 0, k_in, v_in, kc, vc, N_KV, HD, stride)
+        attn.attn_decode_kv_gate(step, 0, q_in, kc, vc, acc, ml, out, g_in, N_HEADS, N_KV, HD, stride, SCALE,
+                                 splits)
+        attn.gemv_q8_0_rows(wd, out, y, m, k, 1)
+
+    def set_inputs(i):
+        p = pos0 + i
+        step.copy_(torch.tensor([p, p + 1, 0, 0, p, p, p, p], dtype=torch.int32))
+        q_in.copy_(torch.from_numpy(qs[i]))
+        k_in.copy_(torch.from_numpy(ks[i]))
+        v_in.copy_(torch.from_numpy(vs[i]))
+        g_in.copy_(torch.from_numpy(gs[i]))
+
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        set_inputs(0)
+        one_step()
+    torch.cuda.current_stream().wait_stream(s)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        one_step()
+
+    kb, vb = kb0.copy(), vb0.copy()
+    for i in range(steps):
+        p = pos0 + i
+        kc.copy_(dev(kb))
+        vc.copy_(dev(vb))
+        set_inputs(i)
+        one_step()                 # eager
+        torch.cuda.synchronize()
+        eager = y.clone()
+        kc.copy_(dev(kb))
+        vc.copy_(dev(vb))
+        y.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, eager), f"replay {i} differs from the eager calls"
+        kb[:, p] = orc.quantize(0, ks[i]).reshape(N_KV, ROW)
+        vb[:, p] = orc.quantize(0, vs[i]).reshape(N_KV, ROW)
+        a = orc.q_gate(orc.attn_decode_kv(qs[i], kb, vb, N_HEADS, N_KV, HD, p + 1, SCALE, stride=stride),
+                       gs[i].ravel())
+        want = orc.gemv_q8_0(wo, a, m, k)
+        # the attention result carries the decode kernel's 1e-3 class into 6,144-term sums
+        ok, _, _ = report(f"graph replay {i}: gated decode + W_o", want, host(y).ravel(), 2e-3, 1e-2)
+        assert ok
+
+
+def test_chunk_layer_with_fused_launches_replays_under_a_captured_graph():
+    # rope + append in one launch, chunk attention with the gate in the merge, output projection over
+    # f16 rows: captured once, replayed three times with eager work in between
+    tok, pos0, pad = 70, 40, 18
+    stride = pos0 + tok + pad
+    m, k = 256, N_HEADS * HD
+    r = orc.Rng(0x6AA1)
+    wo = orc.random_q8_0_bytes(r, m * k // 32)
+    kf = r.normal_array((N_KV, pos0, HD))
+    vf = r.normal_array((N_KV, pos0, HD))
+    kb0, vb0 = quantized_cache(kf, vf, stride)
+    attn.rope_table(THETA, N_ROT, 2048)
+    wd = dev(wo)
+    kc, vc = dev(kb0), dev(vb0)
+    q_in = torch.empty((tok, N_HEADS, HD), device="cuda")
+    k_in = torch.empty((tok, N_KV, HD), device="cuda")
+    v_in = torch.empty((tok, N_KV, HD), device="cuda")
+    g_in = torch.empty((tok, N_HEADS, HD), device="cuda")
+    out = torch.empty((tok, N_HEADS, HD), device="cuda")
+    y = torch.empty((tok, m), device="cuda")
+    splits = 3
+    acc, ml = attn.chunk_scratch(tok, N_HEADS, splits)
+    x16 = torch.empty((tok, k), dtype=torch.float16, device="cuda")
+
+    def layer():
+        attn.rope_encode_chunk(q_in, k_in, v_in, kc, vc, N_HEADS, N_KV, HD, N_ROT, THETA, pos0, tok, 0, stride)
+        attn.chunk_attention_q8_split_gate(q_in, kc, vc, g_in, out, N_HEADS, N_KV, HD, pos0, tok, 1, stride,
+                                           acc, ml, splits)
+        attn.output_chunk_q8_0(wd, out, None, y, m, k, tok, x16)
+
+    def set_inputs(seed):
+        rr = orc.Rng(seed)
+        q_in.copy_(torch.from_numpy(rr.normal_array((tok, N_HEADS, HD))))
+        k_in.copy_(torch.from_numpy(rr.normal_array((tok, N_KV, HD))))
+        v_in.copy_(torch.from_numpy(rr.normal_array((tok, N_KV, HD))))
+        g_in.copy_(torch.from_numpy(rr.normal_array((tok, N_HEADS, HD))))
+
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        set_inputs(1)
+        layer()
+    torch.cuda.current_stream().wait_stream(s)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        layer()
+    for i in range(3):
+        set_inputs(100 + i)
+        kc.copy_(dev(kb0))
+        vc.copy_(dev(vb0))
+        q_keep, k_keep = q_in.clone(), k_in.clone()
+        layer()
+        torch.cuda.synchronize()
+        eager_y, eager_k = y.clone(), kc.clone()
+        q_in.copy_(q_keep)         # the layer ropes q and k in place: start the replay from the same inputs
+        k_in.copy_(k_keep)
+        kc.copy_(dev(kb0))
+        vc.copy_(dev(vb0))
+        y.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, eager_y) and torch.equal(kc, eager_k), f"replay {i} differs from the eager calls"
+        assert bool(torch.isfinite(y).all())
