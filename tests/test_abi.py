@@ -109,3 +109,40 @@ def test_launching_entry_points_ask_for_init_first(lib):
 def attn_inited():
     import torch
     return torch.cuda.is_available()
+
+
+def test_header_is_plain_c_and_links_from_c(tmp_path):
+    # the boundary is a C ABI: a C (not C++) translation unit includes the header, references every
+    # declared function and links against the library; it runs the host-only entry points
+    import shutil
+    import subprocess
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no C compiler")
+    names = declared_functions()
+    refs = "\n".join(f"    p[{i}] = (fn)&{n};" for i, n in enumerate(names))
+    src = tmp_path / "abi_check.c"
+    src.write_text(f"""
+#include <stdio.h>
+#include <string.h>
+#include "hipml_attn.h"
+typedef void (*fn)(void);
+int main(void) {{
+    fn p[{len(names)}];
+{refs}
+    for (int i = 0; i < {len(names)}; i++) if (!p[i]) return 2;
+    if (strstr(hipml_attn_version(), "gfx950") == NULL) return 3;
+    if (hipml_attn_decode_splits(32768, 4) != 128) return 4;
+    if (hipml_rope_table_bytes(64, 10) != 10 * 32 * 2 * sizeof(float)) return 5;
+    if (hipml_gemv_q8_0_rows(NULL, NULL, NULL, NULL, 1, 64, 1) != HIPML_ATTN_E_NULL) return 6;
+    printf("%d functions\\n", {len(names)});
+    return 0;
+}}
+""")
+    exe = tmp_path / "abi_check"
+    libdir = os.path.join(ROOT, "hipml_amd")
+    subprocess.run([gcc, "-std=c99", "-Wall", "-Werror", "-pedantic", "-I", os.path.join(ROOT, "include"),
+                    str(src), "-o", str(exe), "-L", libdir, "-lhipml_attn", f"-Wl,-rpath,{libdir}",
+                    "-Wl,-rpath,/opt/rocm/lib"], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout
+    assert out.strip() == f"{len(names)} functions"
