@@ -335,6 +335,68 @@ def bench_front(torch, attn, tokens, steps):
                          "frac": gbs / HBM_PEAK_GBS, "traffic": None, "kernel": "front_kernel"}}
 
 
+def bench_decode_layer(torch, attn, seq, steps, layers):
+    """One decode token through the attention block of `layers` layers: front end (q|gate split, head
+    norms, RoPE), append, split-K attention with the gate in the merge, output projection -- issued
+    eagerly, and captured once in a HIP graph and replayed (positions live in the device step buffer)."""
+    m, k = 5120, H * HD
+    stride = seq + 64
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(0x5EED0009)
+    caches, ws = [], []
+    for _ in range(layers):
+        kc = torch.empty((KV, stride, ROW), dtype=torch.uint8, device="cuda")
+        vc = torch.empty((KV, stride, ROW), dtype=torch.uint8, device="cuda")
+        fill_cache_normal(torch, attn, kc, vc, stride, seq, gen)
+        caches.append((kc, vc))
+        ws.append(random_q8_0_weights(torch, m, k, gen))
+    qg = torch.randn((H, 2 * HD), device="cuda", generator=gen)
+    kx0 = torch.randn((KV, HD), device="cuda", generator=gen)
+    kx = kx0.clone()
+    vx = torch.randn((KV, HD), device="cuda", generator=gen)
+    qw = torch.ones(HD, device="cuda")
+    kw = torch.ones(HD, device="cuda")
+    q = torch.empty((H, HD), device="cuda")
+    gate = torch.empty((H, HD), device="cuda")
+    out = torch.empty((H, HD), device="cuda")
+    y = torch.empty((1, m), device="cuda")
+    splits = attn.decode_splits(stride, KV)
+    acc = torch.empty((H, splits, HD), device="cuda")
+    ml = torch.empty((H, splits, 2), device="cuda")
+    step = torch.tensor([seq, seq + 1, 0, 0, seq, seq, seq, seq], dtype=torch.int32, device="cuda")
+    attn.rope_table(THETA, NROT, stride + 64)
+
+    def one_pass():
+        for (kc, vc), w in zip(caches, ws):
+            attn.attn_front(qg, q, gate, kx, qw, kw, H, KV, HD, NROT, (11, 11, 10, 0), step[4:], THETA, 1e-6)
+            attn.kv_encode(step, 0, kx, vx, kc, vc, KV, HD, stride)
+            attn.attn_decode_kv_gate(step, 0, q, kc, vc, acc, ml, out, gate, H, KV, HD, stride, SCALE, splits)
+            attn.gemv_q8_0_rows(w, out, y, m, k, 1)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        one_pass()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        one_pass()
+    for _ in range(3):
+        one_pass()
+        graph.replay()
+    with Timer(torch) as te:
+        for _ in range(steps):
+            one_pass()
+    with Timer(torch) as tg:
+        for _ in range(steps):
+            graph.replay()
+    return {"workload": f"decode token @ depth {seq}: front end + append + attention with gate + W_o, "
+                        f"{layers} layers per pass (5 launches per layer)",
+            "us_per_layer_eager": te.ms * 1e3 / (steps * layers),
+            "us_per_layer_graph_replay": tg.ms * 1e3 / (steps * layers)}
+
+
 def random_q8_0_weights(torch, m, k, gen):
     """[m][k/32] Q8_0 blocks with random payloads and the reference's case scale 2^-10 (f16 0x1400)."""
     w = torch.randint(0, 256, (m * (k // 32), 34), dtype=torch.uint8, device="cuda", generator=gen)
@@ -470,7 +532,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--main-only", action="store_true", help="skip the 'also' workloads")
     ap.add_argument("--only", default="", help="run one workload alone (prefill672, decode8k, "
-                    "decode32k, decode128k, chunk100k, batch16, front672, decode32k_q4, gemv1, gemv4, gemv16, gemm672, gemm2048, copycal) for profiling; prints its object")
+                    "decode32k, decode128k, chunk100k, batch16, front672, decode32k_q4, gemv1, gemv4, gemv16, gemm672, gemm2048, layer32k, copycal) for profiling; prints its object")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -503,6 +565,7 @@ def main() -> int:
             "gemv1": lambda: bench_gemv(torch, attn, 1, max(K // 4, 10), LAYERS),
             "gemv4": lambda: bench_gemv(torch, attn, 4, max(K // 4, 10), LAYERS),
             "gemv16": lambda: bench_gemv(torch, attn, 16, max(K // 4, 10), LAYERS),
+            "layer32k": lambda: bench_decode_layer(torch, attn, 32768, max(K // 4, 10), LAYERS),
             "gemm672": lambda: bench_gemm(torch, attn, 672, max(K // 10, 5), 4),
             "gemm2048": lambda: bench_gemm(torch, attn, 2048, max(K // 20, 3), 4),
         }[args.only]
@@ -551,6 +614,8 @@ def main() -> int:
         also["wo_rows_4"] = bench_gemv(torch, attn, 4, d_steps, LAYERS)
         torch.cuda.empty_cache()
         also["wo_chunk_672"] = bench_gemm(torch, attn, 672, max(K // 20, 5), 4)
+        torch.cuda.empty_cache()
+        also["decode_layer_32768"] = bench_decode_layer(torch, attn, 32768, d_steps, LAYERS)
         torch.cuda.empty_cache()
         line["also"] = also
 
