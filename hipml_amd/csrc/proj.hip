@@ -381,9 +381,9 @@ int launch_gemv_q8_rows(hipStream_t st, const uint8_t *w, const float *x, float 
 
 #ifdef GEMM_TIMING
 // debug builds: cycles spent between marks, summed over the steps, per wave of the first workgroups
-__device__ unsigned long long g_gemm_t[16 * 8 * 8];
+__device__ unsigned long long g_gemm_t[16 * 16 * 8];
 #define GT(i) do { __builtin_amdgcn_sched_barrier(0); const unsigned long long now_ = __builtin_readcyclecounter(); if ((i) > 0) gt_sum[(i)] += now_ - gt_last; gt_last = now_; __builtin_amdgcn_sched_barrier(0); } while (0)
-#define GTDUMP() do { if ((threadIdx.x & 63) == 0 && blockIdx.x < 4 && blockIdx.y < 4) for (int i_ = 0; i_ < 8; i_++) g_gemm_t[((blockIdx.y * 4 + blockIdx.x) * 8 + (threadIdx.x >> 6)) * 8 + i_] = gt_sum[i_]; } while (0)
+#define GTDUMP() do { if ((threadIdx.x & 63) == 0 && blockIdx.x < 4 && blockIdx.y < 4) for (int i_ = 0; i_ < 8; i_++) g_gemm_t[((blockIdx.y * 4 + blockIdx.x) * 16 + (threadIdx.x >> 6)) * 8 + i_] = gt_sum[i_]; } while (0)
 extern "C" int hipml_dbg_read_gemm(unsigned long long *host, size_t n)
 {
     return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_gemm_t), n * 8);
@@ -396,17 +396,25 @@ extern "C" int hipml_dbg_read_gemm(unsigned long long *host, size_t n)
 typedef float float16v __attribute__((ext_vector_type(16)));
 typedef _Float16 half4v __attribute__((ext_vector_type(4)));
 
-constexpr int kGemmT = 128, kGemmM = 128, kGemmK = 64;
-constexpr int kGemmPitch = 144;
-constexpr int kGemmTile = 128 * kGemmPitch;   // one operand tile
-constexpr int kGemmBuf = 2 * kGemmTile;       // x tile + w tile
-constexpr int kGemmLds = 2 * kGemmBuf;        // double buffered: 73,728 bytes
+constexpr int kGemmT = 128, kGemmM = 128;
+constexpr int kGemmUnits = 1;                     // 64-value units (pairs of blocks) per step
+constexpr int kGemmK = 64 * kGemmUnits;           // values per step
+constexpr int kGemmPitch = kGemmK * 2 + 16;       // 144: an odd number of 16-byte groups
+constexpr int kGemmTile = 128 * kGemmPitch;       // one operand tile
+constexpr int kGemmBuf = 2 * kGemmTile;           // x tile + w tile
+constexpr int kGemmLds = 2 * kGemmBuf;            // double buffered: 73,728 bytes
+#ifndef GEMM_WAVES
+#define GEMM_WAVES 8
+#endif
+constexpr int kGemmWaves = GEMM_WAVES;            // waves per role
 
-template <bool X16>
+// What one producer thread fetches for one step: per unit WN weight (row, quarter) pairs, and XN
+// 16-byte pieces of the activation tile.
+template <int WN, int XN>
 struct GemmFetch {
-    uint3a4 e[2];            // even-block quarter (+ scales in quad lanes 0 and 3), rows r and r + 64
-    uint2a4 o[2];            // odd-block quarter
-    float4v x[X16 ? 4 : 8];  // f32: 4 activations of rows xr + 16 i; f16: 8 of rows xr + 32 i
+    uint3a4 e[kGemmUnits][WN];   // even-block quarter (+ scales in quad lanes 0 and 3)
+    uint2a4 o[kGemmUnits][WN];   // odd-block quarter
+    float4v x[XN];               // f32: 4 activations; f16: 8
 };
 
 // 8 exact integer f16 times the block scale (f16): the product has at most 19 significant bits and
@@ -418,51 +426,71 @@ __device__ __forceinline__ half8 dequant8(uint32_t w0, uint32_t w1, _Float16 d)
     return q * dv;
 }
 
-template <bool X16>
-__global__ void __launch_bounds__(512) gemm_q8_f16_kernel(const uint8_t *__restrict__ w,
-                                                         const void *__restrict__ xv,
-                                                         float *__restrict__ y, int m, int k, int tokens)
+// NW waves per role (consumers first, then producers): 4 + 4 or 8 + 8.  LDS serves a wave at about
+// 34 B/clk for 128-bit reads and 16-20 B/clk for 128-bit writes whatever the others do, up to well
+// over 128 B/clk in all (measured), so eight waves per role move the same tiles in less time.
+template <bool X16, int NW>
+__global__ void __launch_bounds__(128 * NW) gemm_q8_f16_kernel(const uint8_t *__restrict__ w,
+                                                              const void *__restrict__ xv,
+                                                              float *__restrict__ y, int m, int k, int tokens)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    const bool producer = threadIdx.x >= 256;
-    const int tid = threadIdx.x & 255, wave = tid >> 6, lane = tid & 63; // within the role
+    constexpr int NT = 64 * NW; // threads per role
+    constexpr int KU = kGemmUnits;
+    const bool producer = threadIdx.x >= NT;
+    const int tid = producer ? threadIdx.x - NT : threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63; // within the role
     const int m0 = blockIdx.x * kGemmM, t0 = blockIdx.y * kGemmT;
-    const int nsteps = k / kGemmK;
+    const int nunits = k >> 6;
+    const int nsteps = (nunits + KU - 1) / KU;   // the last step may hold fewer units: zero weights
     const size_t row_bytes = (size_t)(k >> 5) * kQ8Block;
-    constexpr int XN = X16 ? 4 : 8;          // activation loads per thread and step
-    constexpr int XROWS = X16 ? 32 : 16;     // rows covered by one such load of the workgroup
-    constexpr int XELT = X16 ? 2 : 4;        // bytes per activation
+    constexpr int WN = 512 / NT;                 // weight (row, quarter) pairs per producer thread and unit
+    constexpr int WROWS = NT / 4;                // rows covered by one such pair of the workgroup
+    constexpr int XELT = X16 ? 2 : 4;            // bytes per activation
+    constexpr int XV = 16 / XELT;                // activations per 16-byte piece
+    constexpr int XPR = kGemmK / XV;             // pieces per tile row
+    constexpr int XN = 128 * XPR / NT;           // pieces per producer thread
+    constexpr int XROWS = NT / XPR;              // rows covered by one piece of the workgroup
 
     // fetch roles
-    const int fr = tid >> 2, fg = tid & 3; // weight rows fr and fr + 64, k quarter fg of each block
-    const uint8_t *wp[2];
+    const int fr = tid >> 2, fg = tid & 3; // weight rows fr + WROWS h, k quarter fg of each block
+    const uint8_t *wp[WN];
 #pragma unroll
-    for (int h = 0; h < 2; h++) {
-        const int row = m0 + fr + 64 * h < m ? m0 + fr + 64 * h : m - 1;
+    for (int h = 0; h < WN; h++) {
+        const int row = m0 + fr + WROWS * h < m ? m0 + fr + WROWS * h : m - 1;
         wp[h] = w + (size_t)row * row_bytes + fg * 8;
     }
-    // activations: 16 bytes per load; a row's 64 values of the step are 16 (f32) or 8 (f16) lanes
-    const int xr = X16 ? tid >> 3 : tid >> 4, xc = X16 ? tid & 7 : tid & 15;
+    // activations: 16 bytes per load, XPR consecutive lanes cover a tile row
+    const int xr = tid / XPR, xc = tid % XPR;
     const uint8_t *xp[XN];
 #pragma unroll
     for (int i = 0; i < XN; i++) {
         const int t = t0 + xr + XROWS * i < tokens ? t0 + xr + XROWS * i : tokens - 1;
-        xp[i] = static_cast<const uint8_t *>(xv) + ((size_t)t * k) * XELT + xc * 16;
+        xp[i] = static_cast<const uint8_t *>(xv) + ((size_t)t * k) * XELT;
     }
-    typedef GemmFetch<X16> Fetch;
+    typedef GemmFetch<WN, XN> Fetch;
     auto fetch = [&](Fetch &f, int s) {
         const int sc = s < nsteps ? s : nsteps - 1;
 #pragma unroll
-        for (int h = 0; h < 2; h++) {
-            const uint8_t *unit = wp[h] + (size_t)sc * (2 * kQ8Block);
-            f.e[h] = *reinterpret_cast<const uint3a4 *>(unit);
-            f.o[h] = *reinterpret_cast<const uint2a4 *>(unit + 36);
+        for (int u = 0; u < KU; u++) {
+            const int g = sc * KU + u < nunits ? sc * KU + u : nunits - 1;
+#pragma unroll
+            for (int h = 0; h < WN; h++) {
+                const uint8_t *unit = wp[h] + (size_t)g * (2 * kQ8Block);
+                f.e[u][h] = *reinterpret_cast<const uint3a4 *>(unit);
+                f.o[u][h] = *reinterpret_cast<const uint2a4 *>(unit + 36);
+            }
         }
+        // a piece past the end of the row (second unit of a short last step) repeats the row's last
+        // piece: it meets zero weights
+        int kx = sc * kGemmK + xc * XV;
+        if (KU > 1)
+            kx = kx + XV <= k ? kx : k - XV;
 #pragma unroll
         for (int i = 0; i < XN; i++)
-            f.x[i] = *reinterpret_cast<const float4v *>(xp[i] + (size_t)sc * (kGemmK * XELT));
+            f.x[i] = *reinterpret_cast<const float4v *>(xp[i] + (size_t)kx * XELT);
     };
-    auto stage = [&](const Fetch &f, uint8_t *buf) {
+    auto stage = [&](const Fetch &f, uint8_t *buf, int s) {
         uint8_t *xt = buf, *wt = buf + kGemmTile;
 #pragma unroll
         for (int i = 0; i < XN; i++) {
@@ -475,57 +503,63 @@ __global__ void __launch_bounds__(512) gemm_q8_f16_kernel(const uint8_t *__restr
             }
         }
 #pragma unroll
-        for (int h = 0; h < 2; h++) {
-            const uint3a4 e = f.e[h];
-            const uint32_t s0 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)e[0], 0x00, 0xf, 0xf, true);
-            const uint32_t s1 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)e[2], 0xFF, 0xf, 0xf, true);
-            const _Float16 d0 = __builtin_bit_cast(_Float16, (uint16_t)(s0 & 0xffffu));
-            const _Float16 d1 = __builtin_bit_cast(_Float16, (uint16_t)(s1 >> 16));
-            const half8 v0 = dequant8(__builtin_amdgcn_alignbit(e[1], e[0], 16),
-                                      __builtin_amdgcn_alignbit(e[2], e[1], 16), d0);
-            const half8 v1 = dequant8(f.o[h][0], f.o[h][1], d1);
-            uint8_t *dst = wt + (fr + 64 * h) * kGemmPitch + fg * 16;
-            *reinterpret_cast<half8 *>(dst) = v0;        // k = fg*8 .. of the even block
-            *reinterpret_cast<half8 *>(dst + 64) = v1;   // k = 32 + fg*8 .. (the odd block)
+        for (int u = 0; u < KU; u++) {
+            const bool live = KU == 1 || s * KU + u < nunits;
+#pragma unroll
+            for (int h = 0; h < WN; h++) {
+                const uint3a4 e = f.e[u][h];
+                const uint32_t s0 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)e[0], 0x00, 0xf, 0xf, true);
+                const uint32_t s1 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)e[2], 0xFF, 0xf, 0xf, true);
+                const _Float16 d0 = __builtin_bit_cast(_Float16, (uint16_t)(live ? s0 & 0xffffu : 0u));
+                const _Float16 d1 = __builtin_bit_cast(_Float16, (uint16_t)(live ? s1 >> 16 : 0u));
+                const half8 v0 = dequant8(__builtin_amdgcn_alignbit(e[1], e[0], 16),
+                                          __builtin_amdgcn_alignbit(e[2], e[1], 16), d0);
+                const half8 v1 = dequant8(f.o[u][h][0], f.o[u][h][1], d1);
+                uint8_t *dst = wt + (fr + WROWS * h) * kGemmPitch + u * 128 + fg * 16;
+                *reinterpret_cast<half8 *>(dst) = v0;        // k = fg*8 .. of the even block
+                *reinterpret_cast<half8 *>(dst + 64) = v1;   // k = 32 + fg*8 .. (the odd block)
+            }
         }
     };
 
-    // MFMA roles: wave (wt, wm) owns tokens wt*64.. and weight rows wm*64..
+    // MFMA roles: consumer wave (wt, wm) owns AT 32-token tiles from token wt * 32 AT and weight rows
+    // wm*64..: 64 x 64 per wave with four consumers, 32 x 64 with eight
+    constexpr int AT = 8 / NW;
     const int wt_ = wave >> 1, wm_ = wave & 1;
     const int ln = lane & 31, lh = lane >> 5;
-    float16v acc[2][2];
+    float16v acc[AT][2];
 #pragma unroll
-    for (int a = 0; a < 2; a++)
+    for (int a = 0; a < AT; a++)
 #pragma unroll
         for (int b = 0; b < 2; b++)
 #pragma unroll
             for (int i = 0; i < 16; i++)
                 acc[a][b][i] = 0.0f;
     auto multiply = [&](const uint8_t *buf) {
-        const uint8_t *xa = buf + (wt_ * 64 + ln) * kGemmPitch + lh * 16;
+        const uint8_t *xa = buf + (wt_ * 32 * AT + ln) * kGemmPitch + lh * 16;
         const uint8_t *wb = buf + kGemmTile + (wm_ * 64 + ln) * kGemmPitch + lh * 16;
 #pragma unroll
-        for (int kk = 0; kk < 4; kk++) {
-            half8 A[2], B[2];
+        for (int kk = 0; kk < 4 * KU; kk++) {
+            half8 A[AT], B[2];
 #pragma unroll
-            for (int a = 0; a < 2; a++)
+            for (int a = 0; a < AT; a++)
                 A[a] = *reinterpret_cast<const half8 *>(xa + a * 32 * kGemmPitch + kk * 32);
 #pragma unroll
             for (int b = 0; b < 2; b++)
                 B[b] = *reinterpret_cast<const half8 *>(wb + b * 32 * kGemmPitch + kk * 32);
 #pragma unroll
-            for (int a = 0; a < 2; a++)
+            for (int a = 0; a < AT; a++)
 #pragma unroll
                 for (int b = 0; b < 2; b++)
                     acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[a], B[b], acc[a][b], 0, 0, 0);
         }
     };
 
-    // Waves 4..7 produce (fetch, dequantize, write the next step's tiles), waves 0..3 consume (operand
-    // reads and MFMAs of the current step); one barrier per step hands a buffer over.  A SIMD holds
-    // one wave of each kind, and a VALU wave and an MFMA wave of one SIMD issue side by side.
-    // Two steps per turn keep the two records and the two buffers in the same registers through
-    // the loop; a fetch past the last step repeats it and is never multiplied.
+    // The second half of the waves produce (fetch, dequantize, write the next step's tiles), the first
+    // half consume (operand reads and MFMAs of the current step); one barrier per step hands a buffer
+    // over.  A SIMD holds waves of both kinds, and a VALU wave and an MFMA wave of one SIMD issue side
+    // by side.  (Two units per step, half as many barriers, measured slower: 76.5 against 72.8 us at
+    // 672 tokens.)
 #ifdef GEMM_TIMING
     unsigned long long gt_sum[8] = {0, 0, 0, 0, 0, 0, 0, 0}, gt_last = 0;
 #endif
@@ -539,25 +573,25 @@ __global__ void __launch_bounds__(512) gemm_q8_f16_kernel(const uint8_t *__restr
         fetch(r1, 1);
         fetch(r2, 2);
         fetch(r3, 3);
-        stage(r0, lds);
+        stage(r0, lds, 0);
         fetch(r0, 4);
         __syncthreads();
         int s = 0;
         for (; s + 4 <= nsteps; s += 4) {
             GT(0);
-            stage(r1, lds + kGemmBuf); // step s + 1, while step s is multiplied
+            stage(r1, lds + kGemmBuf, s + 1); // step s + 1, while step s is multiplied
             GT(1);
             fetch(r1, s + 5);
             GT(2);
             __syncthreads();
             GT(3);
-            stage(r2, lds);
+            stage(r2, lds, s + 2);
             fetch(r2, s + 6);
             __syncthreads();
-            stage(r3, lds + kGemmBuf);
+            stage(r3, lds + kGemmBuf, s + 3);
             fetch(r3, s + 7);
             __syncthreads();
-            stage(r0, lds);            // step s + 4
+            stage(r0, lds, s + 4);            // step s + 4
             fetch(r0, s + 8);
             __syncthreads();
         }
@@ -566,12 +600,12 @@ __global__ void __launch_bounds__(512) gemm_q8_f16_kernel(const uint8_t *__restr
         const int rest = nsteps - s;
         if (rest >= 1) {
             if (rest >= 2)
-                stage(r1, lds + kGemmBuf);
+                stage(r1, lds + kGemmBuf, s + 1);
             __syncthreads();
         }
         if (rest >= 2) {
             if (rest >= 3)
-                stage(r2, lds);
+                stage(r2, lds, s + 2);
             __syncthreads();
         }
         if (rest >= 3)
@@ -596,13 +630,13 @@ __global__ void __launch_bounds__(512) gemm_q8_f16_kernel(const uint8_t *__restr
 
     // C tile: lane holds column ln (weight row), rows (i/4)*8 + lh*4 + i%4 (tokens)
 #pragma unroll
-    for (int a = 0; a < 2; a++)
+    for (int a = 0; a < AT; a++)
 #pragma unroll
         for (int b = 0; b < 2; b++) {
             const int row = m0 + wm_ * 64 + b * 32 + ln;
 #pragma unroll
             for (int i = 0; i < 16; i++) {
-                const int t = t0 + wt_ * 64 + a * 32 + (i >> 2) * 8 + lh * 4 + (i & 3);
+                const int t = t0 + wt_ * 32 * AT + a * 32 + (i >> 2) * 8 + lh * 4 + (i & 3);
                 if (t < tokens && row < m)
                     y[(size_t)t * m + row] = acc[a][b][i];
             }
@@ -654,10 +688,10 @@ static hipError_t raise_gemv_lds()
 
 int proj_init()
 {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q8_f16_kernel<false>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q8_f16_kernel<false, kGemmWaves>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLds);
     if (e == hipSuccess)
-        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q8_f16_kernel<true>),
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q8_f16_kernel<true, kGemmWaves>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLds);
     if (e == hipSuccess)
         e = raise_gemv_lds<8, 1, 6>();
@@ -674,7 +708,8 @@ int launch_gemm_q8_f16(hipStream_t st, const uint8_t *w, const float *x, const f
 {
     const dim3 grid((unsigned)((m + kGemmM - 1) / kGemmM), (unsigned)((tokens + kGemmT - 1) / kGemmT), 1);
     if (x16 == nullptr) {
-        hipLaunchKernelGGL(gemm_q8_f16_kernel<false>, grid, dim3(512, 1, 1), kGemmLds, st, w, x, y, m, k, tokens);
+        hipLaunchKernelGGL((gemm_q8_f16_kernel<false, kGemmWaves>), grid, dim3(128 * kGemmWaves, 1, 1), kGemmLds,
+                           st, w, x, y, m, k, tokens);
         return launched("gemm_q8_0_f16");
     }
     const size_t n8 = (size_t)tokens * k / 8;
@@ -684,7 +719,8 @@ int launch_gemm_q8_f16(hipStream_t st, const uint8_t *w, const float *x, const f
     int rc = launched("gate_f16");
     if (rc)
         return rc;
-    hipLaunchKernelGGL(gemm_q8_f16_kernel<true>, grid, dim3(512, 1, 1), kGemmLds, st, w, x16, y, m, k, tokens);
+    hipLaunchKernelGGL((gemm_q8_f16_kernel<true, kGemmWaves>), grid, dim3(128 * kGemmWaves, 1, 1), kGemmLds, st, w,
+                       x16, y, m, k, tokens);
     return launched("gemm_q8_0_f16");
 }
 
