@@ -565,6 +565,9 @@ def main() -> int:
             "gemv1": lambda: bench_gemv(torch, attn, 1, max(K // 4, 10), LAYERS),
             "gemv4": lambda: bench_gemv(torch, attn, 4, max(K // 4, 10), LAYERS),
             "gemv16": lambda: bench_gemv(torch, attn, 16, max(K // 4, 10), LAYERS),
+            "gemv24": lambda: bench_gemv(torch, attn, 24, max(K // 4, 10), LAYERS),
+            "gemm24": lambda: bench_gemm(torch, attn, 24, max(K // 4, 10), LAYERS),
+            "gemm128": lambda: bench_gemm(torch, attn, 128, max(K // 4, 10), LAYERS),
             "layer32k": lambda: bench_decode_layer(torch, attn, 32768, max(K // 4, 10), LAYERS),
             "gemm672": lambda: bench_gemm(torch, attn, 672, max(K // 10, 5), 4),
             "gemm2048": lambda: bench_gemm(torch, attn, 2048, max(K // 20, 3), 4),
@@ -612,6 +615,7 @@ def main() -> int:
         # the step after the path: output projection over Q8_0 weights (decode rows, then a chunk)
         also["wo_rows_1"] = bench_gemv(torch, attn, 1, d_steps, LAYERS)
         also["wo_rows_4"] = bench_gemv(torch, attn, 4, d_steps, LAYERS)
+        also["wo_rows_24"] = bench_gemv(torch, attn, 24, d_steps, LAYERS)  # the batch of 16 slots with 4 verify groups
         torch.cuda.empty_cache()
         also["wo_chunk_672"] = bench_gemm(torch, attn, 672, max(K // 20, 5), 4)
         torch.cuda.empty_cache()

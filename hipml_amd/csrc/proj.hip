@@ -316,6 +316,197 @@ __global__ void __launch_bounds__(64 * WAVES, TILES == 1 ? 2 : 1) gemv_q8_rows_k
     }
 }
 
+// ---- gemv_q8_tile_kernel: 5 to 128 activation rows (batched decode, verify groups) --------------
+//
+// The same streaming of W as above, with the activations as full 16-row A tiles: A row = activation
+// row, hi and lo halves as two chained MFMAs, XT tiles (16 or 32 rows) per pass.  The rows' operands
+// no longer fit LDS, and need not: the waves of a workgroup split k, so no two of them want the same
+// activations; lane (lm, lg) loads the 8 f32 of row lm, k quarter lg of each block straight from
+// global memory (L2: the rows are a few hundred KB that every workgroup reads) and splits them in
+// registers.  A step (a pair of blocks: 16 XT registers of activations, 5 TILES of weights) is one
+// record; four records rotate, each refilled as soon as it has been consumed, activations before
+// weights in request order (the loads complete in order: a step then waits for nothing younger than
+// itself).  What the time is made of at 5120 x 6144 and 16 rows: 13.1 us with the activation loads
+// taken out (the arithmetic is hidden behind the weight stream), 16.1 with all of them hitting L1,
+// 19.8 as it is: every workgroup reads every row (393 KB through its CU's L1 for 208 KB of weights).
+// Four weight tiles per workgroup halve that and leave 80 workgroups, too few to keep HBM busy (27.5 us).
+template <int TILES, int XT>
+struct TileRec {
+    float4v x[XT][2][2]; // [tile][block of the pair][half of the 8 values]
+    uint3a4 e[TILES];
+    uint2a4 o[TILES];
+};
+
+template <int WAVES, int TILES, int XT, int STEPS>
+__global__ void __launch_bounds__(64 * WAVES, 1) gemv_q8_tile_kernel(const uint8_t *__restrict__ w,
+                                                                   const float *__restrict__ x,
+                                                                   float *__restrict__ y, int m, int k, int rows)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int lm = lane & 15, lg = lane >> 4; // MFMA operand lane: A row / weight row lm, k quarter lg
+    const int fr = lane >> 2, fg = lane & 3;  // fetch lane: weight row fr, k quarter fg
+    const int pull = (lm * 4 + lg) * 4;
+    const int nb = k >> 5;
+    const size_t row_bytes = (size_t)nb * kQ8Block;
+    const int m0 = blockIdx.x * (16 * TILES);
+    const int r0 = blockIdx.y * (16 * XT);
+    const int nu = nb >> 1; // steps: pairs of blocks
+    // The steps are dealt to the waves round-robin: the activation rows are a multiple of the L2's
+    // channel interleave apart, so the 16 rows of one load meet in one channel, and only the k
+    // offsets of requests in flight spread the traffic; eight neighbouring steps are 2 KB of a row.
+    // (With a contiguous slice of k per wave the activation loads cost 10 us on top of 13.)
+    float4v *red = reinterpret_cast<float4v *>(lds);
+
+    // rows past the end are clamped: loaded and multiplied, never stored
+    const float *xp[XT];
+#pragma unroll
+    for (int t = 0; t < XT; t++) {
+        const int r = r0 + t * 16 + lm < rows ? r0 + t * 16 + lm : rows - 1;
+        xp[t] = x + (size_t)r * k + lg * 8;
+    }
+    const uint8_t *wp[TILES];
+#pragma unroll
+    for (int t = 0; t < TILES; t++) {
+        const int row = m0 + t * 16 + fr < m ? m0 + t * 16 + fr : m - 1;
+        wp[t] = w + (size_t)row * row_bytes;
+    }
+    typedef TileRec<TILES, XT> Rec;
+    auto fetch = [&](Rec &c, int u) {
+        const int uc = u < nu ? u : nu - 1;
+#pragma unroll
+        for (int t = 0; t < XT; t++)
+#pragma unroll
+            for (int b = 0; b < 2; b++) {
+                const float *p = xp[t] + (size_t)uc * 64 + b * 32;
+                c.x[t][b][0] = *reinterpret_cast<const float4v *>(p);
+                c.x[t][b][1] = *reinterpret_cast<const float4v *>(p + 4);
+            }
+#pragma unroll
+        for (int t = 0; t < TILES; t++) {
+            const uint8_t *unit = wp[t] + (size_t)uc * (2 * kQ8Block);
+            c.e[t] = *reinterpret_cast<const uint3a4 *>(unit + fg * 8);
+            c.o[t] = *reinterpret_cast<const uint2a4 *>(unit + 36 + fg * 8);
+        }
+    };
+    float4v acc[TILES][XT];
+#pragma unroll
+    for (int t = 0; t < TILES; t++)
+#pragma unroll
+        for (int a = 0; a < XT; a++)
+            acc[t][a] = (float4v){0, 0, 0, 0};
+    auto consume = [&](const Rec &c, int u) {
+        const bool live = u < nu;
+        half8 hi[XT][2], lo[XT][2];
+#pragma unroll
+        for (int a = 0; a < XT; a++)
+#pragma unroll
+            for (int b = 0; b < 2; b++)
+                split_hi_lo(c.x[a][b][0], c.x[a][b][1], hi[a][b], lo[a][b]);
+#pragma unroll
+        for (int t = 0; t < TILES; t++) {
+            const uint3a4 e = c.e[t];
+            const int e2_of_g3 = __builtin_amdgcn_update_dpp(0, (int)e[2], 0xFF, 0xf, 0xf, true);
+            const int sc = (int)((e[0] & 0xffffu) | ((uint32_t)e2_of_g3 & 0xffff0000u));
+            const uint32_t q0 = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)__builtin_amdgcn_alignbit(e[1], e[0], 16));
+            const uint32_t q1 = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)__builtin_amdgcn_alignbit(e[2], e[1], 16));
+            const uint32_t q2 = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)c.o[t][0]);
+            const uint32_t q3 = (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)c.o[t][1]);
+            const uint32_t ds = (uint32_t)__builtin_amdgcn_ds_bpermute(lm * 16, sc);
+            const float d0 = live ? (float)__builtin_bit_cast(_Float16, (uint16_t)(ds & 0xffffu)) : 0.0f;
+            const float d1 = live ? (float)__builtin_bit_cast(_Float16, (uint16_t)(ds >> 16)) : 0.0f;
+            const half8 w0 = int8x8_to_f16(q0, q1), w1 = int8x8_to_f16(q2, q3);
+#pragma unroll
+            for (int a = 0; a < XT; a++) {
+                float4v p0 = {0, 0, 0, 0}, p1 = {0, 0, 0, 0};
+                p0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(hi[a][0], w0, p0, 0, 0, 0);
+                p1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(hi[a][1], w1, p1, 0, 0, 0);
+                p0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(lo[a][0], w0, p0, 0, 0, 0);
+                p1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(lo[a][1], w1, p1, 0, 0, 0);
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    acc[t][a][j] = fmaf(d1, p1[j], fmaf(d0, p0[j], acc[t][a][j]));
+            }
+        }
+    };
+    // STEPS > 0: every wave has exactly STEPS steps (the launcher checks) and the code is straight
+    // line, so each step waits for exactly its own loads.  Otherwise a loop of four steps per turn
+    // (the records keep their registers; the compiler waits for every outstanding load at the head
+    // of a turn); a fetch past the wave's last step repeats it and a step past it multiplies by a
+    // zero scale.  The scheduler may not move a step's arithmetic past the refill behind it, or the
+    // other way round: either makes the wave wait for loads it has only just asked for.
+    Rec c[4];
+    const int u_lo = wave;
+    fetch(c[0], u_lo);
+    fetch(c[1], u_lo + WAVES);
+    fetch(c[2], u_lo + 2 * WAVES);
+    fetch(c[3], u_lo + 3 * WAVES);
+    if (STEPS > 0) {
+#pragma unroll
+        for (int i = 0; i < STEPS; i++) {
+            __builtin_amdgcn_sched_barrier(0);
+            consume(c[i & 3], u_lo + i * WAVES);
+            __builtin_amdgcn_sched_barrier(0);
+            if (i + 4 < STEPS)
+                fetch(c[i & 3], u_lo + (i + 4) * WAVES);
+        }
+    } else {
+        for (int u = u_lo; u < nu; u += 4 * WAVES) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                __builtin_amdgcn_sched_barrier(0);
+                consume(c[i], u + i * WAVES);
+                __builtin_amdgcn_sched_barrier(0);
+                fetch(c[i], u + (i + 4) * WAVES);
+            }
+        }
+    }
+
+    // the k slices meet in a fixed order: C row 4 lg + j = activation row, column lm = weight row
+#pragma unroll
+    for (int t = 0; t < TILES; t++)
+#pragma unroll
+        for (int a = 0; a < XT; a++)
+            red[((wave * TILES + t) * XT + a) * 64 + lane] = acc[t][a];
+    __syncthreads();
+    for (int i = threadIdx.x; i < TILES * XT * 64; i += 64 * WAVES) {
+        float4v s = red[i];
+#pragma unroll
+        for (int u = 1; u < WAVES; u++)
+            s += red[u * TILES * XT * 64 + i];
+        const int l = i & 63, a = (i >> 6) % XT, t = (i >> 6) / XT;
+        const int row = m0 + t * 16 + (l & 15);
+        const int r = r0 + a * 16 + 4 * (l >> 4);
+        if (row < m) {
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                if (r + j < rows)
+                    y[(size_t)(r + j) * m + row] = s[j];
+        }
+    }
+}
+
+template <int WAVES, int TILES, int XT, int STEPS>
+static int launch_gemv_tile_steps(hipStream_t st, const uint8_t *w, const float *x, float *y, int m, int k, int rows)
+{
+    const size_t lds = (size_t)WAVES * TILES * XT * 64 * sizeof(float4v);
+    auto kern = gemv_q8_tile_kernel<WAVES, TILES, XT, STEPS>;
+    const dim3 grid((unsigned)((m + 16 * TILES - 1) / (16 * TILES)), (unsigned)((rows + 16 * XT - 1) / (16 * XT)), 1);
+    hipLaunchKernelGGL(kern, grid, dim3(64 * WAVES, 1, 1), lds, st, w, x, y, m, k, rows);
+    return launched("gemv_q8_0_rows");
+}
+
+template <int WAVES, int TILES, int XT>
+static int launch_gemv_tile(hipStream_t st, const uint8_t *w, const float *x, float *y, int m, int k, int rows)
+{
+    // straight-line variants for the model's two inner sizes: 6144 (W_o) and 5120 (W_q, W_k, W_v)
+    if (k == 64 * WAVES * 12)
+        return launch_gemv_tile_steps<WAVES, TILES, XT, 12>(st, w, x, y, m, k, rows);
+    if (k == 64 * WAVES * 10)
+        return launch_gemv_tile_steps<WAVES, TILES, XT, 10>(st, w, x, y, m, k, rows);
+    return launch_gemv_tile_steps<WAVES, TILES, XT, 0>(st, w, x, y, m, k, rows);
+}
+
 template <int WAVES, int TILES, int CH, int XG>
 static int launch_gemv_xg(hipStream_t st, const uint8_t *w, const float *x, float *y, int m, int k,
                           int rows, int rp)
@@ -347,6 +538,10 @@ int launch_gemv_q8_rows(hipStream_t st, const uint8_t *w, const float *x, float 
     if (rp < 1)
         return fail(HIPML_ATTN_E_RANGE, "k %d: one activation row does not fit the LDS operand buffer", k);
     rp = rows < rp ? rows : rp;
+    // more than a pass of the row kernel: full A tiles of 16 or 32 rows
+    if (rows > kGemvMaxRows)
+        return rows > 16 ? launch_gemv_tile<8, 2, 2>(st, w, x, y, m, k, rows)
+                         : launch_gemv_tile<8, 2, 1>(st, w, x, y, m, k, rows);
     // One 16-row weight tile per workgroup keeps the kernel inside 128 registers, so two workgroups
     // share a CU and the 320 workgroups of a 5120-row matrix start together (workgroups start in
     // windows of as many as fit the chip; a second window opens when the first has drained).  With

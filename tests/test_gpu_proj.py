@@ -87,7 +87,10 @@ def test_ragged_shapes_and_scales():
     # reference bounds such cases with LARGE_TOL (2e-3 / 3e-2, quant_parity.rs:20-25); on top of that
     # the kernel must be as close to the float64 value as the sequential fp32 sum is.
     r = orc.Rng(0x7A66)
-    for m, k, rows in ((1, 64, 1), (33, 192, 2), (1000, 320, 7), (50, 4096, 16)):
+    # rows 1-4 take the row kernel; more rows take full 16- or 32-row tiles (k = 5120 and 6144 in
+    # straight-line code, any other k in a loop; k = 64 leaves seven of eight waves without a step)
+    for m, k, rows in ((1, 64, 1), (33, 192, 2), (1000, 320, 7), (50, 4096, 16), (7, 64, 5),
+                       (40, 5120, 9), (130, 704, 33), (64, 1024, 128), (20, 6144, 47)):
         w = orc.random_q8_0_bytes(r, m * k // 32).reshape(-1, 34)
         scales = (r.uniform_array(w.shape[0]) * 0.05 + 0.001).astype(np.float16)
         w[:, :2] = scales.view(np.uint8).reshape(-1, 2)
