@@ -22,6 +22,7 @@
 //   The waves of a workgroup split k; a wave requests the activations first, then two chunks of
 //   its weight blocks (all of them for k = 6144) before it waits for anything, and the partial sums
 //   meet in LDS in a fixed order (no atomics: the result does not depend on timing).
+// gemv_q8_tile_kernel (further down): the same stream for 5 to 128 rows, activations as full A tiles.
 
 #include "common.h"
 
@@ -559,15 +560,15 @@ int launch_gemv_q8_rows(hipStream_t st, const uint8_t *w, const float *x, float 
 // y[t][row] for a 128 (tokens) x 128 (weight rows) tile per workgroup, MFMA-bound:
 // v_mfma_f32_32x32x16_f16 with A = x (f32 -> f16, round to nearest), B = W dequantized to f16 (d*q, one
 // rounding: the precision class of the reference's f16-operand prefill kernels and of this library's
-// chunk attention), fp32 accumulation.  Four consumer waves, each a 64 x 64 quarter (2 x 2 MFMA tiles:
-// every operand read from LDS feeds two MFMAs), and four producer waves that fetch and stage.  A k step is 64 values = one 68-byte pair of blocks per
+// chunk attention), fp32 accumulation.  Eight consumer waves, each a 32 x 64 piece (1 x 2 MFMA tiles),
+// and eight producer waves that fetch and stage.  A k step is 64 values = one 68-byte pair of blocks per
 // weight row; both operand tiles are staged as [128 rows][64 f16] with a 144-byte row pitch (128-bit
 // reads and writes of 16 consecutive rows then touch every bank once), double buffered, one barrier
 // per step.  A fetch record is refilled as soon as it has been staged.  (One set of four waves doing
 // both, interleaved by hand MFMA by MFMA, took 1,600 cycles per step with a single workgroup on the
 // CU: every wait left its SIMD idle.)
 // Weight fetch uses the lane order of the row kernel above (quad = the four quarters of a pair of
-// blocks, dword-aligned loads); a thread handles rows r and r + 64.
+// blocks, dword-aligned loads).
 // X16: the activations arrive as f16 (written by gate_f16_kernel below).  With f32 activations a
 // step moves 32 KB of them through the CU's 64-byte-per-cycle vector memory path -- more cycles
 // than the step's MFMAs take (measured: 700 of a step's 2,200 cycles are spent issuing loads) -- and
