@@ -366,10 +366,14 @@ def bench_decode_layer(torch, attn, seq, steps, layers):
     step = torch.tensor([seq, seq + 1, 0, 0, seq, seq, seq, seq], dtype=torch.int32, device="cuda")
     attn.rope_table(THETA, NROT, stride + 64)
 
-    def one_pass():
+    def one_pass(fused=True):
         for (kc, vc), w in zip(caches, ws):
-            attn.attn_front(qg, q, gate, kx, qw, kw, H, KV, HD, NROT, (11, 11, 10, 0), step[4:], THETA, 1e-6)
-            attn.kv_encode(step, 0, kx, vx, kc, vc, KV, HD, stride)
+            if fused:
+                attn.attn_front_encode(step, 0, qg, q, gate, kx, vx, qw, kw, kc, vc, H, KV, HD, NROT,
+                                       (11, 11, 10, 0), THETA, 1e-6, stride)
+            else:
+                attn.attn_front(qg, q, gate, kx, qw, kw, H, KV, HD, NROT, (11, 11, 10, 0), step[4:], THETA, 1e-6)
+                attn.kv_encode(step, 0, kx, vx, kc, vc, KV, HD, stride)
             attn.attn_decode_kv_gate(step, 0, q, kc, vc, acc, ml, out, gate, H, KV, HD, stride, SCALE, splits)
             attn.gemv_q8_0_rows(w, out, y, m, k, 1)
 
@@ -384,17 +388,22 @@ def bench_decode_layer(torch, attn, seq, steps, layers):
         one_pass()
     for _ in range(3):
         one_pass()
+        one_pass(False)
         graph.replay()
     with Timer(torch) as te:
         for _ in range(steps):
             one_pass()
+    with Timer(torch) as ts:
+        for _ in range(steps):
+            one_pass(False)
     with Timer(torch) as tg:
         for _ in range(steps):
             graph.replay()
-    return {"workload": f"decode token @ depth {seq}: front end + append + attention with gate + W_o, "
-                        f"{layers} layers per pass (5 launches per layer)",
+    return {"workload": f"decode token @ depth {seq}: front end with append + attention with gate + W_o, "
+                        f"{layers} layers per pass (4 launches per layer)",
             "us_per_layer_eager": te.ms * 1e3 / (steps * layers),
-            "us_per_layer_graph_replay": tg.ms * 1e3 / (steps * layers)}
+            "us_per_layer_graph_replay": tg.ms * 1e3 / (steps * layers),
+            "us_per_layer_eager_front_and_append_apart": ts.ms * 1e3 / (steps * layers)}
 
 
 def random_q8_0_weights(torch, m, k, gen):

@@ -37,6 +37,7 @@ EXPORTS = [
     "hipml_attn_front_f32", "hipml_attn_chunk_front_f32",
     "hipml_gemv_q8_0_rows", "hipml_gemm_q8_0_f16", "hipml_attn_output_chunk_q8_0",
     "hipml_kv_rows_copy", "hipml_rope_encode_chunk_f32",
+    "hipml_attn_front_encode_f32", "hipml_attn_chunk_front_encode_f32",
 ]
 
 
@@ -97,6 +98,10 @@ def lib() -> C.CDLL:
             "hipml_q_gate_f32": (i, [vp, vp, vp, vp, sz]),
             "hipml_attn_front_f32": (i, [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, i, i, vp, f, f]),
             "hipml_attn_chunk_front_f32": (i, [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, f, f, i, i]),
+            "hipml_attn_front_encode_f32": (i, [vp, vp, i, vp, vp, vp, vp, vp, vp, vp, vp, vp,
+                                                i, i, i, i, i, i, i, i, f, f, i]),
+            "hipml_attn_chunk_front_encode_f32": (i, [vp, i, vp, vp, vp, vp, vp, vp, vp, vp, vp,
+                                                      i, i, i, i, f, f, i, i, i]),
             "hipml_kv_rows_copy": (i, [vp, i, vp, vp, vp, vp, i, i, i, i, i]),
             "hipml_rope_encode_chunk_f32": (i, [vp, vp, vp, vp, vp, vp, i, i, i, i, f, i, i, i, i]),
             "hipml_gemv_q8_0_rows": (i, [vp, vp, vp, vp, i, i, i]),
@@ -207,6 +212,26 @@ def chunk_front(qg, k, q, gate, q_norm, k_norm, n_heads, n_kv, head_dim, n_rot, 
     _check(lib().hipml_attn_chunk_front_f32(_stream(stream), _p(qg), _p(k), _p(q), _p(gate),
                                             _p(q_norm), _p(k_norm), n_heads, n_kv, head_dim, n_rot,
                                             theta, eps, pos0, tokens))
+
+
+def attn_front_encode(step, dtype, qg, q, gate, k, v, q_norm, k_norm, k_cache, v_cache, n_heads, n_kv,
+                      head_dim, n_rot, sections, theta, eps, stride, stream=None):
+    """`attn_front` and `kv_encode` of the same token in one launch (same bits): the row goes to
+    position step[0], the M-RoPE ids are step[4..7]."""
+    s0, s1, s2, s3 = sections
+    _check(lib().hipml_attn_front_encode_f32(_stream(stream), _p(step), dtype, _p(qg), _p(q), _p(gate),
+                                             _p(k), _p(v), _p(q_norm), _p(k_norm), _p(k_cache),
+                                             _p(v_cache), n_heads, n_kv, head_dim, n_rot, s0, s1, s2, s3,
+                                             theta, eps, stride))
+
+
+def chunk_front_encode(dtype, qg, k, v, q, gate, q_norm, k_norm, k_cache, v_cache, n_heads, n_kv,
+                       head_dim, n_rot, theta, eps, pos0, tokens, stride, stream=None):
+    """`chunk_front` and `kv_encode_bulk(start=pos0, src0=0, rows=tokens)` in one launch (same bits)."""
+    _check(lib().hipml_attn_chunk_front_encode_f32(_stream(stream), dtype, _p(qg), _p(k), _p(v), _p(q),
+                                                   _p(gate), _p(q_norm), _p(k_norm), _p(k_cache),
+                                                   _p(v_cache), n_heads, n_kv, head_dim, n_rot, theta,
+                                                   eps, pos0, tokens, stride))
 
 
 # ---- KV append ------------------------------------------------------------------------

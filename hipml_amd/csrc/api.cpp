@@ -451,6 +451,52 @@ static int check_encode(int dtype, const void *k, const void *v, const void *kc,
     return 0;
 }
 
+// The front end and the append of the finished K row and of the V row in one launch.
+int hipml_attn_front_encode_f32(hipml_stream_t stream, const int32_t *step, int dtype, const float *qg,
+                                float *q, float *gate, float *k, const float *v, const float *q_norm,
+                                const float *k_norm, void *k_cache, void *v_cache, int n_heads, int n_kv,
+                                int head_dim, int n_rot, int s0, int s1, int s2, int s3, float theta_base,
+                                float eps, int stride)
+{
+    clear_error();
+    REQUIRE_PTR(step);
+    int rc = check_front(qg, q, gate, k, q_norm, k_norm, n_heads, n_kv, head_dim, n_rot, theta_base, eps);
+    if (rc == 0)
+        rc = check_encode(dtype, k, v, k_cache, v_cache, n_kv, head_dim, stride);
+    if (rc)
+        return rc;
+    if (s0 < 0 || s1 < 0 || s2 < 0 || s3 < 0)
+        return fail(HIPML_ATTN_E_RANGE, "negative M-RoPE section");
+    return launch_front(as_stream(stream), qg, q, gate, k, q_norm, k_norm, n_heads, n_kv, n_rot, s0, s1,
+                        s2, s3, step + 4, 0, 1, theta_base, eps, g_rope, dtype, v,
+                        static_cast<uint8_t *>(k_cache), static_cast<uint8_t *>(v_cache), step, 0, stride);
+}
+
+int hipml_attn_chunk_front_encode_f32(hipml_stream_t stream, int dtype, const float *qg, float *k,
+                                      const float *v, float *q, float *gate, const float *q_norm,
+                                      const float *k_norm, void *k_cache, void *v_cache, int n_heads,
+                                      int n_kv, int head_dim, int n_rot, float theta_base, float eps,
+                                      int pos0, int tokens, int stride)
+{
+    clear_error();
+    int rc = check_front(qg, q, gate, k, q_norm, k_norm, n_heads, n_kv, head_dim, n_rot, theta_base, eps);
+    if (rc == 0)
+        rc = check_encode(dtype, k, v, k_cache, v_cache, n_kv, head_dim, stride);
+    if (rc)
+        return rc;
+    if (pos0 < 0 || tokens < 0)
+        return fail(HIPML_ATTN_E_RANGE, "pos0 %d / tokens %d must be non-negative", pos0, tokens);
+    if ((long long)pos0 + tokens > stride)
+        return fail(HIPML_ATTN_E_RANGE, "rows [%d, %d) do not fit a cache of %d rows per head", pos0,
+                    pos0 + tokens, stride);
+    if (tokens == 0)
+        return 0;
+    return launch_front(as_stream(stream), qg, q, gate, k, q_norm, k_norm, n_heads, n_kv, n_rot, 0, 0, 0,
+                        0, nullptr, pos0, tokens, theta_base, eps, g_rope, dtype, v,
+                        static_cast<uint8_t *>(k_cache), static_cast<uint8_t *>(v_cache), nullptr, pos0,
+                        stride);
+}
+
 int hipml_kv_encode(hipml_stream_t stream, const int32_t *step, int dtype, const float *k_in,
                     const float *v_in, void *k_cache, void *v_cache, int n_kv, int head_dim,
                     int stride)

@@ -66,7 +66,9 @@ int launch_kv_rows_copy(hipStream_t st, int q4, const uint8_t *k_src, const uint
                         uint8_t *v_dst, int n_kv, int src_stride, int dst_stride, int rows);
 int launch_front(hipStream_t st, const float *qg, float *q, float *gate, float *k, const float *qw,
                  const float *kw, int n_heads, int n_kv, int n_rot, int s0, int s1, int s2, int s3,
-                 const int32_t *pos, int pos0, int rows, float theta, float eps, const RopeTable &tab);
+                 const int32_t *pos, int pos0, int rows, float theta, float eps, const RopeTable &tab,
+                 int enc = -1, const float *v = nullptr, uint8_t *kc = nullptr, uint8_t *vc = nullptr,
+                 const int32_t *step = nullptr, int start = 0, int stride = 0);
 int launch_q_gate(hipStream_t st, const float *x, const float *gate, float *y, size_t n);
 
 struct DecodeLaunch {

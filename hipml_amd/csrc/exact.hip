@@ -384,18 +384,53 @@ int launch_rope_encode_chunk(hipStream_t st, int q4, float *q, float *k, const f
 // (x * scale) * w; the rotation reads cos/sin as the other RoPE kernels here do.
 // grid: ceil((n_heads + n_kv) * rows / 4) workgroups of 4 waves.  `pos` (device int32[4]) gives
 // the four M-RoPE position ids of a single row; when it is null, row t rotates at pos0 + t.
+// What the append half of a fused launch needs (kv == nullptr: front end only).
+struct FrontAppend {
+    const float *v;      // [rows][n_kv][256]
+    uint8_t *kc, *vc;    // caches
+    const int32_t *step; // row 0 goes to position step[0]; null: row r goes to start + r
+    int start, stride;
+};
+
+// ENC: 0 = front end only, 1 = also quantize the finished K row and the V row to q8_0 and append
+// them, 2 = the same to q4_0 -- the K wave keeps its row in registers (element lane + 64 j in slot
+// j, so a half-wave holds one block of 32, as the append kernels' 32-lane groups do) and n_kv more
+// waves per row take the V rows.  Same expressions on the same values: the bits of the two launches.
+template <int ENC>
 __global__ void __launch_bounds__(256) front_kernel(
     const float *__restrict__ qg, float *__restrict__ q, float *__restrict__ gate, float *k,
     const float *__restrict__ qw, const float *__restrict__ kw, int n_heads, int n_kv, int n_rot,
     int s0, int s1, int s2, int s3, const int32_t *__restrict__ pos, int pos0, int rows, float theta,
-    float eps, const float *__restrict__ tab, int tab_rows)
+    float eps, const float *__restrict__ tab, int tab_rows, const FrontAppend ap)
 {
     __shared__ float buf[4][kHeadDim];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int per_row = n_heads + n_kv;
     const int idx = blockIdx.x * 4 + wave;
-    if (idx >= per_row * rows)
+    const int nfront = per_row * rows;
+    if (idx >= nfront + (ENC ? n_kv * rows : 0))
         return; // no workgroup-wide barrier below: waves are independent
+    const int lane32 = lane & 31;
+    if (ENC && idx >= nfront) {
+        // a V row: quantize and append
+        const int u = idx - nfront;
+        const int row = u / n_kv, h = u - row * n_kv;
+        const int p = ap.step ? ap.step[0] : ap.start + row;
+        const float *src = ap.v + (size_t)u * kHeadDim;
+        float x[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            x[j] = src[lane + 64 * j];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const size_t blk = ((size_t)h * ap.stride + p) * (kHeadDim / 32) + 2 * j + (lane >> 5);
+            if (ENC == 2)
+                q4_encode_store(x[j], ap.vc + blk * kQ4BlockBytes, lane32);
+            else
+                q8_encode_store(x[j], ap.vc + blk * kQ8BlockBytes, lane32);
+        }
+        return;
+    }
     const int row = idx / per_row;
     const int hb = idx - row * per_row;
     const bool is_q = hb < n_heads;
@@ -430,48 +465,72 @@ __global__ void __launch_bounds__(256) front_kernel(
     __builtin_amdgcn_wave_barrier();
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 
+    // element e = lane + 64 j: rotated with its partner when e < n_rot (the first half of the pairs
+    // takes x1 c - x2 s, the second x1 s + x2 c), passed through otherwise
     const int half = n_rot >> 1;
     const int sect = s0 + s1 + s2 + s3;
-    for (int c = lane; c < half; c += 64) {
-        int p = pos ? pos[0] : pos0 + row;
-        if (pos && sect > 0) {
-            const int s = c % sect;
-            if (s < s0)
-                p = pos[0];
-            else if (s < s0 + s1)
-                p = pos[1];
-            else if (s < s0 + s1 + s2)
-                p = pos[2];
-            else
-                p = pos[3];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int e = lane + 64 * j;
+        float out = buf[wave][e];
+        if (e < n_rot) {
+            const bool first = e < half;
+            const int c = first ? e : e - half;
+            int p = pos ? pos[0] : pos0 + row;
+            if (pos && sect > 0) {
+                const int sc = c % sect;
+                if (sc < s0)
+                    p = pos[0];
+                else if (sc < s0 + s1)
+                    p = pos[1];
+                else if (sc < s0 + s1 + s2)
+                    p = pos[2];
+                else
+                    p = pos[3];
+            }
+            float cs, sn;
+            rope_cs(tab, tab_rows, half, c, p, n_rot, theta, cs, sn);
+            const float x1 = buf[wave][c];
+            const float x2 = buf[wave][c + half];
+            out = first ? x1 * cs - x2 * sn : x1 * sn + x2 * cs;
         }
-        float cs, sn;
-        rope_cs(tab, tab_rows, half, c, p, n_rot, theta, cs, sn);
-        const float x1 = buf[wave][c];
-        const float x2 = buf[wave][c + half];
-        dst[c] = x1 * cs - x2 * sn;
-        dst[c + half] = x1 * sn + x2 * cs;
+        dst[e] = out;
+        x[j] = out;
     }
-    for (int d = n_rot + lane; d < kHeadDim; d += 64)
-        dst[d] = buf[wave][d];
+    if (ENC && !is_q) {
+        const int p = ap.step ? ap.step[0] : ap.start + row;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const size_t blk = ((size_t)h * ap.stride + p) * (kHeadDim / 32) + 2 * j + (lane >> 5);
+            if (ENC == 2)
+                q4_encode_store(x[j], ap.kc + blk * kQ4BlockBytes, lane32);
+            else
+                q8_encode_store(x[j], ap.kc + blk * kQ8BlockBytes, lane32);
+        }
+    }
 }
 
+// enc: -1 = front end only (v, kc, vc unused), 0 = q8_0, 1 = q4_0 append of the K and V rows.
 int launch_front(hipStream_t st, const float *qg, float *q, float *gate, float *k, const float *qw,
                  const float *kw, int n_heads, int n_kv, int n_rot, int s0, int s1, int s2, int s3,
-                 const int32_t *pos, int pos0, int rows, float theta, float eps, const RopeTable &tab)
+                 const int32_t *pos, int pos0, int rows, float theta, float eps, const RopeTable &tab,
+                 int enc, const float *v, uint8_t *kc, uint8_t *vc, const int32_t *step, int start,
+                 int stride)
 {
     int tab_rows = 0;
     const float *t = table_for(tab, theta, n_rot, &tab_rows);
-    const int per_row = n_heads + n_kv;
+    const int per_row = n_heads + n_kv + (enc >= 0 ? n_kv : 0);
     const int max_rows = 1 << 22; // keeps (rows * per_row) far inside int
     for (int r0 = 0; r0 < rows; r0 += max_rows) {
         const int n = rows - r0 < max_rows ? rows - r0 : max_rows;
         const unsigned grid = (unsigned)(((long long)per_row * n + 3) / 4);
-        hipLaunchKernelGGL(front_kernel, dim3(grid, 1, 1), dim3(256, 1, 1), 0, st,
+        const FrontAppend ap = {v ? v + (size_t)r0 * n_kv * kHeadDim : nullptr, kc, vc, step, start + r0, stride};
+        auto kern = enc < 0 ? front_kernel<0> : enc == 0 ? front_kernel<1> : front_kernel<2>;
+        hipLaunchKernelGGL(kern, dim3(grid, 1, 1), dim3(256, 1, 1), 0, st,
                            qg + (size_t)r0 * n_heads * 2 * kHeadDim, q + (size_t)r0 * n_heads * kHeadDim,
                            gate + (size_t)r0 * n_heads * kHeadDim, k + (size_t)r0 * n_kv * kHeadDim, qw, kw,
-                           n_heads, n_kv, n_rot, s0, s1, s2, s3, pos, pos0 + r0, n, theta, eps, t, tab_rows);
-        int rc = launched("attn_front_f32");
+                           n_heads, n_kv, n_rot, s0, s1, s2, s3, pos, pos0 + r0, n, theta, eps, t, tab_rows, ap);
+        int rc = launched(enc < 0 ? "attn_front_f32" : "attn_front_encode_f32");
         if (rc)
             return rc;
     }

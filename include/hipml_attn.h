@@ -133,6 +133,29 @@ int hipml_attn_chunk_front_f32(hipml_stream_t stream, const float *qg, float *k,
                                int n_kv, int head_dim, int n_rot, float theta_base, float eps,
                                int pos0, int tokens);
 
+/* hipml_attn_front_f32 and hipml_kv_encode (below) of the same token in one launch: the K row is
+ * quantized from the registers that hold it after the rotation, the V row [n_kv][head_dim] by n_kv
+ * more waves; q, gate, k and both caches end with the bits of the two calls.  `step` is the step
+ * buffer (int32[8]): the row goes to position step[0], the M-RoPE position ids are step[4..7].
+ * Replaces AttnLayer::front followed by Launcher::kv_encode_ptr_on
+ * (crates/hipml-kernels/src/attn_gpu.rs:549-609, launch/device/graph_launch.rs:878-966; call site
+ * crates/hipml-model/src/gpu.rs:576-592). */
+int hipml_attn_front_encode_f32(hipml_stream_t stream, const int32_t *step, int dtype, const float *qg,
+                                float *q, float *gate, float *k, const float *v, const float *q_norm,
+                                const float *k_norm, void *k_cache, void *v_cache, int n_heads, int n_kv,
+                                int head_dim, int n_rot, int s0, int s1, int s2, int s3, float theta_base,
+                                float eps, int stride);
+
+/* hipml_attn_chunk_front_f32 and hipml_kv_encode_bulk(start = pos0, src0 = 0, rows = tokens) in one
+ * launch, same bits.  Replaces AttnLayer::chunk_front followed by Launcher::kv_encode_bulk
+ * (crates/hipml-kernels/src/attn_gpu/imp/attn_chunk.rs:129-205,
+ * launch/device/graph_launch.rs:980-1028; call site crates/hipml-model/src/gpu/attn_tile.rs:53-68). */
+int hipml_attn_chunk_front_encode_f32(hipml_stream_t stream, int dtype, const float *qg, float *k,
+                                      const float *v, float *q, float *gate, const float *q_norm,
+                                      const float *k_norm, void *k_cache, void *v_cache, int n_heads,
+                                      int n_kv, int head_dim, int n_rot, float theta_base, float eps,
+                                      int pos0, int tokens, int stride);
+
 /* ---- q8_0 / q4_0 KV append ------------------------------------------------------- */
 
 /* One token: quantize k_in/v_in [n_kv][head_dim] into row step[0] of the cache.

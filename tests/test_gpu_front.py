@@ -101,3 +101,87 @@ def test_front_rejects_other_head_dims():
     with pytest.raises(attn.HipmlError) as e:
         attn.attn_front(x, x, x, x, x, x, 4, 1, 128, 64, SECTIONS, pos, THETA, EPS)
     assert "head_dim" in str(e.value)
+
+
+@pytest.mark.parametrize("dtype", [0, 1])
+def test_decode_front_with_append_has_the_bits_of_the_two_launches(dtype):
+    # one token: front end, then the append of its K and V rows at step[0], against one fused launch;
+    # stride > position, caches pre-filled so that a stray write shows
+    qg, k, qw, kw = front_inputs(0xF30A + dtype, 1)
+    r = orc.Rng(0xF30B + dtype)
+    v = r.normal_array((N_KV, HD))
+    stride, p = 300, 257
+    row_bytes = 272 if dtype == 0 else 144
+    step = torch.tensor([p, p + 1, 0, 0, p, 77, 9999, 5], dtype=torch.int32, device="cuda")
+
+    def run(fused):
+        q = torch.full((N_HEADS, HD), float("nan"), device="cuda")
+        gate = torch.full((N_HEADS, HD), float("nan"), device="cuda")
+        kd, vd = dev(k[0]), dev(v)
+        kc = torch.full((N_KV * stride * row_bytes,), 0x5A, dtype=torch.uint8, device="cuda")
+        vc = torch.full((N_KV * stride * row_bytes,), 0xA5, dtype=torch.uint8, device="cuda")
+        if fused:
+            attn.attn_front_encode(step, dtype, dev(qg[0]), q, gate, kd, vd, dev(qw), dev(kw), kc, vc,
+                                   N_HEADS, N_KV, HD, N_ROT, SECTIONS, THETA, EPS, stride)
+        else:
+            attn.attn_front(dev(qg[0]), q, gate, kd, dev(qw), dev(kw), N_HEADS, N_KV, HD, N_ROT, SECTIONS,
+                            step[4:], THETA, EPS)
+            attn.kv_encode(step, dtype, kd, vd, kc, vc, N_KV, HD, stride)
+        torch.cuda.synchronize()
+        return [host(t) for t in (q, gate, kd, kc, vc)]
+
+    two, one = run(False), run(True)
+    for name, a, b in zip(("q", "gate", "k", "k cache", "v cache"), two, one):
+        assert np.array_equal(a, b), name
+    # the appended row is the oracle's encoding of the oracle's front end, everything else untouched
+    _, _, wk = orc.attn_front(qg[0], k[0], qw, kw, N_HEADS, N_KV, HD, N_ROT, SECTIONS,
+                              (p, 77, 9999, 5), THETA, EPS, tree=True)
+    enc = lambda x: orc.quantize(dtype, x)  # noqa: E731
+    kc = one[3].reshape(N_KV, stride, row_bytes)
+    assert np.array_equal(kc[:, p].ravel(), enc(wk)), "appended K row"
+    assert np.array_equal(one[4].reshape(N_KV, stride, row_bytes)[:, p].ravel(), enc(v.ravel())), "appended V row"
+    mask = np.ones(stride, dtype=bool)
+    mask[p] = False
+    assert (kc[:, mask] == 0x5A).all() and (one[4].reshape(N_KV, stride, row_bytes)[:, mask] == 0xA5).all()
+
+
+@pytest.mark.parametrize("dtype,rows,pos0", [(0, 37, 29), (0, 672, 0), (1, 5, 100_000)])
+def test_chunk_front_with_append_has_the_bits_of_the_two_launches(dtype, rows, pos0):
+    qg, k, qw, kw = front_inputs(0xF40C + rows, rows)
+    r = orc.Rng(0xF40D + rows)
+    v = r.normal_array((rows, N_KV, HD))
+    stride = pos0 + rows + 3
+    row_bytes = 272 if dtype == 0 else 144
+
+    def run(fused):
+        q = torch.full((rows, N_HEADS, HD), float("nan"), device="cuda")
+        gate = torch.full((rows, N_HEADS, HD), float("nan"), device="cuda")
+        kd, vd = dev(k), dev(v)
+        kc = torch.zeros((N_KV * stride * row_bytes,), dtype=torch.uint8, device="cuda")
+        vc = torch.zeros((N_KV * stride * row_bytes,), dtype=torch.uint8, device="cuda")
+        if fused:
+            attn.chunk_front_encode(dtype, dev(qg), kd, vd, q, gate, dev(qw), dev(kw), kc, vc, N_HEADS,
+                                    N_KV, HD, N_ROT, THETA, EPS, pos0, rows, stride)
+        else:
+            attn.chunk_front(dev(qg), kd, q, gate, dev(qw), dev(kw), N_HEADS, N_KV, HD, N_ROT, THETA, EPS,
+                             pos0, rows)
+            attn.kv_encode_bulk(dtype, kd, vd, kc, vc, N_KV, HD, stride, pos0, 0, rows)
+        torch.cuda.synchronize()
+        return [host(t) for t in (q, gate, kd, kc, vc)]
+
+    two, one = run(False), run(True)
+    for name, a, b in zip(("q", "gate", "k", "k cache", "v cache"), two, one):
+        assert np.array_equal(a, b), name
+    assert one[3].any() and one[4].any()
+
+
+def test_front_with_append_rejects_bad_arguments():
+    t = torch.zeros(16, device="cuda")
+    b = torch.zeros(16, dtype=torch.uint8, device="cuda")
+    with pytest.raises(attn.HipmlError):   # rows do not fit the cache
+        attn.chunk_front_encode(0, t, t, t, t, t, t, t, b, b, N_HEADS, N_KV, HD, N_ROT, THETA, EPS, 10, 5, 12)
+    with pytest.raises(attn.HipmlError):   # unknown cache format
+        attn.chunk_front_encode(7, t, t, t, t, t, t, t, b, b, N_HEADS, N_KV, HD, N_ROT, THETA, EPS, 0, 1, 12)
+    with pytest.raises(attn.HipmlError):   # no step buffer
+        attn.attn_front_encode(None, 0, t, t, t, t, t, t, t, b, b, N_HEADS, N_KV, HD, N_ROT, SECTIONS,
+                               THETA, EPS, 12)
