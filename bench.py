@@ -406,6 +406,67 @@ def bench_decode_layer(torch, attn, seq, steps, layers):
             "us_per_layer_eager_front_and_append_apart": ts.ms * 1e3 / (steps * layers)}
 
 
+def bench_chunk_layer(torch, attn, tokens, pos0, steps, layers):
+    """A chunk through the attention block: front end (q|gate split, head norms, RoPE) with the append,
+    gated attention delivering f16 rows, W_o GEMM over them -- 4 launches -- beside the same work as
+    the separate calls (front end, append, attention with gate, gate/convert pass, GEMM)."""
+    m, k = 5120, H * HD
+    stride = (pos0 + tokens + 63) // 64 * 64
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(0x5EED000A)
+    caches, ws = [], []
+    for _ in range(layers):
+        kc = torch.zeros((KV, stride, ROW), dtype=torch.uint8, device="cuda")
+        vc = torch.zeros((KV, stride, ROW), dtype=torch.uint8, device="cuda")
+        if pos0 > 0:
+            fill_cache_normal(torch, attn, kc, vc, stride, pos0, gen)
+        caches.append((kc, vc))
+        ws.append(random_q8_0_weights(torch, m, k, gen))
+    qg = torch.randn((tokens, H, 2 * HD), device="cuda", generator=gen)
+    kx = torch.randn((tokens, KV, HD), device="cuda", generator=gen)
+    vx = torch.randn((tokens, KV, HD), device="cuda", generator=gen)
+    qw = torch.ones(HD, device="cuda")
+    kw = torch.ones(HD, device="cuda")
+    q = torch.empty((tokens, H, HD), device="cuda")
+    gate = torch.empty((tokens, H, HD), device="cuda")
+    out = torch.empty((tokens, H, HD), device="cuda")
+    out16 = torch.empty((tokens, H, HD), dtype=torch.float16, device="cuda")
+    y = torch.empty((tokens, m), device="cuda")
+    splits = attn.chunk_splits(pos0, tokens, KV)
+    acc = ml = None
+    if splits >= 2:
+        acc, ml = attn.chunk_scratch(tokens, H, splits)
+    attn.rope_table(THETA, NROT, max(pos0 + tokens, 1024))
+
+    def fused(i):
+        (kc, vc), w = caches[i % layers], ws[i % layers]
+        attn.chunk_front_encode(0, qg, kx, vx, q, gate, qw, kw, kc, vc, H, KV, HD, NROT, THETA, 1e-6,
+                                pos0, tokens, stride)
+        attn.chunk_attention_q8_split_gate_f16(q, kc, vc, gate, out, out16, H, KV, HD, pos0, tokens, 1,
+                                               stride, acc, ml, splits)
+        attn.output_chunk_q8_0(w, None, None, y, m, k, tokens, out16)
+
+    def apart(i):
+        (kc, vc), w = caches[i % layers], ws[i % layers]
+        attn.chunk_front(qg, kx, q, gate, qw, kw, H, KV, HD, NROT, THETA, 1e-6, pos0, tokens)
+        attn.kv_encode_bulk(0, kx, vx, kc, vc, KV, HD, stride, pos0, 0, tokens)
+        attn.chunk_attention_q8_split_gate(q, kc, vc, gate, out, H, KV, HD, pos0, tokens, 1, stride,
+                                           acc, ml, splits)
+        attn.output_chunk_q8_0(w, out, None, y, m, k, tokens, out16)
+
+    res = {}
+    for name, fn in (("us_per_layer", fused), ("us_per_layer_separate_calls", apart)):
+        for i in range(3):
+            fn(i)
+        with Timer(torch) as t:
+            for i in range(steps):
+                fn(i)
+        res[name] = t.ms * 1e3 / steps
+    return {"workload": f"chunk {tokens}@{pos0} through front end with append + gated attention (f16 rows) "
+                        f"+ W_o GEMM, {layers} layers rotated (4 launches per layer)", **res,
+            "tok_per_s": tokens / (res["us_per_layer"] * 1e-6)}
+
+
 def random_q8_0_weights(torch, m, k, gen):
     """[m][k/32] Q8_0 blocks with random payloads and the reference's case scale 2^-10 (f16 0x1400)."""
     w = torch.randint(0, 256, (m * (k // 32), 34), dtype=torch.uint8, device="cuda", generator=gen)
@@ -541,7 +602,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--main-only", action="store_true", help="skip the 'also' workloads")
     ap.add_argument("--only", default="", help="run one workload alone (prefill672, decode8k, "
-                    "decode32k, decode128k, chunk100k, batch16, front672, decode32k_q4, gemv1, gemv4, gemv16, gemm672, gemm2048, layer32k, copycal) for profiling; prints its object")
+                    "decode32k, decode128k, chunk100k, batch16, front672, decode32k_q4, gemv1, gemv4, gemv16, gemm672, gemm2048, layer32k, layer672, copycal) for profiling; prints its object")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -578,6 +639,7 @@ def main() -> int:
             "gemm24": lambda: bench_gemm(torch, attn, 24, max(K // 4, 10), LAYERS),
             "gemm128": lambda: bench_gemm(torch, attn, 128, max(K // 4, 10), LAYERS),
             "layer32k": lambda: bench_decode_layer(torch, attn, 32768, max(K // 4, 10), LAYERS),
+            "layer672": lambda: bench_chunk_layer(torch, attn, 672, 0, max(K // 10, 5), 4),
             "gemm672": lambda: bench_gemm(torch, attn, 672, max(K // 10, 5), 4),
             "gemm2048": lambda: bench_gemm(torch, attn, 2048, max(K // 20, 3), 4),
         }[args.only]
@@ -629,6 +691,8 @@ def main() -> int:
         also["wo_chunk_672"] = bench_gemm(torch, attn, 672, max(K // 20, 5), 4)
         torch.cuda.empty_cache()
         also["decode_layer_32768"] = bench_decode_layer(torch, attn, 32768, d_steps, LAYERS)
+        torch.cuda.empty_cache()
+        also["chunk_layer_672"] = bench_chunk_layer(torch, attn, 672, 0, max(K // 10, 5), 4)
         torch.cuda.empty_cache()
         line["also"] = also
 

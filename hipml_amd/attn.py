@@ -38,6 +38,7 @@ EXPORTS = [
     "hipml_gemv_q8_0_rows", "hipml_gemm_q8_0_f16", "hipml_attn_output_chunk_q8_0",
     "hipml_kv_rows_copy", "hipml_rope_encode_chunk_f32",
     "hipml_attn_front_encode_f32", "hipml_attn_chunk_front_encode_f32",
+    "hipml_attn_chunk_q8_split_gate_f16",
 ]
 
 
@@ -95,6 +96,7 @@ def lib() -> C.CDLL:
                                                       i, f, i, sz, sz, sz, sz, i, vp]),
             "hipml_attn_chunk_q8_split": (i, [vp, vp, vp, vp, vp, i, i, i, i, i, i, i, vp, vp, i]),
             "hipml_attn_chunk_q8_split_gate": (i, [vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, i, vp, vp, i]),
+            "hipml_attn_chunk_q8_split_gate_f16": (i, [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, i, vp, vp, i]),
             "hipml_q_gate_f32": (i, [vp, vp, vp, vp, sz]),
             "hipml_attn_front_f32": (i, [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, i, i, vp, f, f]),
             "hipml_attn_chunk_front_f32": (i, [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, f, f, i, i]),
@@ -356,6 +358,16 @@ def chunk_attention_q8_split_gate(q, kc, vc, gate, out, n_head, n_kv, head_dim, 
                                                 stride, _p(part_acc), _p(part_ml), splits))
 
 
+def chunk_attention_q8_split_gate_f16(q, kc, vc, gate, out, out16, n_head, n_kv, head_dim, pos0, tokens,
+                                      dtype, stride, part_acc, part_ml, splits, stream=None):
+    """The gated chunk attention with its rows delivered as f16 in `out16` (what the output projection
+    reads); `out` is working memory."""
+    _check(lib().hipml_attn_chunk_q8_split_gate_f16(_stream(stream), _p(q), _p(kc), _p(vc), _p(gate),
+                                                    _p(out), _p(out16), n_head, n_kv, head_dim, pos0,
+                                                    tokens, dtype, stride, _p(part_acc), _p(part_ml),
+                                                    splits))
+
+
 def chunk_scratch(tokens: int, n_head: int, splits: int, device="cuda"):
     """Split-K scratch sized as the reference's prefill path sizes it."""
     qslots = (tokens + 31) // 32 * 32
@@ -386,7 +398,7 @@ def gemm_q8_0_f16(w, x, y, m, k, tokens, stream=None):
 
 def output_chunk_q8_0(wo, attn_out, gate, y, m, k, tokens, x16, stream=None):
     """`AttnLayer::apply_output_chunk`: y = W_o (attn_out * sigmoid(gate)); gate may be None; x16 is
-    scratch of tokens*k f16."""
+    scratch of tokens*k f16.  attn_out None: x16 already holds the rows as f16."""
     _check(lib().hipml_attn_output_chunk_q8_0(_stream(stream), _p(wo), _p(attn_out),
                                               _p(gate) if gate is not None else None, _p(y), m, k,
                                               tokens, _p(x16)))

@@ -740,13 +740,18 @@ int hipml_attn_decode_batch_cols_gate(hipml_stream_t stream, int dtype, const in
 static int chunk_q8_common(hipml_stream_t stream, const float *q, const void *kc, const void *vc,
                            float *out, const float *gate, bool want_gate, int n_head, int n_kv,
                            int head_dim, int pos0, int tokens, int dtype, int stride, float *part_acc,
-                           float *part_ml, int splits)
+                           float *part_ml, int splits, void *out16 = nullptr, bool want_f16 = false)
 {
     clear_error();
     REQUIRE_PTR(q);
     REQUIRE_PTR(kc);
     REQUIRE_PTR(vc);
     REQUIRE_PTR(out);
+    if (want_f16) {
+        REQUIRE_PTR(out16);
+        if (int rc16 = check_aligned16(out16, "out16"))
+            return rc16;
+    }
     if (want_gate)
         REQUIRE_PTR(gate);
     // the reference's chunk launcher numbers the formats 1 = q8_0, 2 = q4_0
@@ -779,7 +784,8 @@ static int chunk_q8_common(hipml_stream_t stream, const float *q, const void *kc
         return rc;
     return launch_chunk_q8(as_stream(stream), q, static_cast<const uint8_t *>(kc),
                            static_cast<const uint8_t *>(vc), out, n_head, n_kv, pos0, tokens,
-                           stride, part_acc, part_ml, splits, want_gate ? gate : nullptr, dtype == 2 ? 1 : 0);
+                           stride, part_acc, part_ml, splits, want_gate ? gate : nullptr, dtype == 2 ? 1 : 0,
+                           want_f16 ? out16 : nullptr);
 }
 
 int hipml_attn_chunk_q8_split(hipml_stream_t stream, const float *q, const void *kc,
@@ -798,6 +804,15 @@ int hipml_attn_chunk_q8_split_gate(hipml_stream_t stream, const float *q, const 
 {
     return chunk_q8_common(stream, q, kc, vc, out, gate, true, n_head, n_kv, head_dim, pos0, tokens,
                            dtype, stride, part_acc, part_ml, splits);
+}
+
+int hipml_attn_chunk_q8_split_gate_f16(hipml_stream_t stream, const float *q, const void *kc,
+                                       const void *vc, const float *gate, float *out, void *out16,
+                                       int n_head, int n_kv, int head_dim, int pos0, int tokens, int dtype,
+                                       int stride, float *part_acc, float *part_ml, int splits)
+{
+    return chunk_q8_common(stream, q, kc, vc, out, gate, true, n_head, n_kv, head_dim, pos0, tokens,
+                           dtype, stride, part_acc, part_ml, splits, out16, true);
 }
 
 // ---- gate ---------------------------------------------------------------------------------------------
@@ -870,10 +885,13 @@ int hipml_attn_output_chunk_q8_0(hipml_stream_t stream, const void *wo, const fl
                                  const float *gate, float *y, int m, int k, int tokens, void *x16)
 {
     clear_error();
-    int rc = check_gemm(wo, attn_out, y, m, k, tokens);
+    REQUIRE_PTR(x16);
+    // attn_out == NULL: x16 already holds the rows (hipml_attn_chunk_q8_split_gate_f16 wrote them)
+    int rc = check_gemm(wo, attn_out ? attn_out : static_cast<const float *>(x16), y, m, k, tokens);
     if (rc)
         return rc;
-    REQUIRE_PTR(x16);
+    if (attn_out == nullptr && gate != nullptr)
+        return fail(HIPML_ATTN_E_NULL, "a gate needs the f32 rows it applies to (attn_out is NULL)");
     if ((rc = check_aligned16(gate, "gate")) || (rc = check_aligned16(x16, "x16")))
         return rc;
     return launch_gemm_q8_f16(as_stream(stream), static_cast<const uint8_t *>(wo), attn_out, gate, y, m, k,

@@ -97,7 +97,7 @@ int decode_init();
 int prefill_init();
 int launch_chunk_q8(hipStream_t st, const float *q, const uint8_t *kc, const uint8_t *vc,
                     float *out, int n_head, int n_kv, int pos0, int tokens, int stride,
-                    float *part_acc, float *part_ml, int splits, const float *gate, int q4);
+                    float *part_acc, float *part_ml, int splits, const float *gate, int q4, void *out16 = nullptr);
 
 // y[r][row] = W[row][:] . x[r][:] over a Q8_0 weight matrix, rows <= 128 activation rows (proj.hip).
 int launch_gemv_q8_rows(hipStream_t st, const uint8_t *w, const float *x, float *y, int m, int k, int rows);

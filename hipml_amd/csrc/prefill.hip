@@ -676,10 +676,12 @@ __global__ void __launch_bounds__(kPfThreads, 2) chunk_q8_kernel(const ChunkArgs
 
 // Fold the key slices: one workgroup per (token, 4 heads); thread = (head, float4 of d).  A (token,
 // head) whose task block has a single slice was written by the attention kernel itself.
+// out16 != nullptr: the finished rows go there as f16 (round to nearest even), the operand form of
+// the output projection, and `out` only carries the single-slice rows in from the attention kernel.
 __global__ void __launch_bounds__(256) chunk_combine_kernel(
     const float *__restrict__ part_acc, const float *__restrict__ part_ml, float *out,
     const float *__restrict__ gate, int n_head, int qslots, int splits, int group, int ntask, int tokens,
-    int pos0, int slice_tiles, int uniform)
+    int pos0, int slice_tiles, int uniform, _Float16 *__restrict__ out16)
 {
     const int tok = blockIdx.x;
     const int head = blockIdx.y * 4 + (threadIdx.x >> 6);
@@ -692,11 +694,16 @@ __global__ void __launch_bounds__(256) chunk_combine_kernel(
         const int task = (tok / kQTile) * group + head % group;
         nsp = block_slices(task / kTasks, ntask, group, tokens, pos0, splits, slice_tiles, nullptr);
         if (nsp == 1) {
-            if (gate) {
-                const float4v x = *reinterpret_cast<const float4v *>(out + o);
-                const float4v gt = *reinterpret_cast<const float4v *>(gate + o);
-                *reinterpret_cast<float4v *>(out + o) =
-                    (float4v){gated(x[0], gt[0]), gated(x[1], gt[1]), gated(x[2], gt[2]), gated(x[3], gt[3])};
+            if (gate || out16) {
+                float4v x = *reinterpret_cast<const float4v *>(out + o);
+                if (gate) {
+                    const float4v gt = *reinterpret_cast<const float4v *>(gate + o);
+                    x = (float4v){gated(x[0], gt[0]), gated(x[1], gt[1]), gated(x[2], gt[2]), gated(x[3], gt[3])};
+                }
+                if (out16)
+                    *reinterpret_cast<half4 *>(out16 + o) = __builtin_convertvector(x, half4);
+                else
+                    *reinterpret_cast<float4v *>(out + o) = x;
             }
             return;
         }
@@ -727,7 +734,18 @@ __global__ void __launch_bounds__(256) chunk_combine_kernel(
         const float4v gt = *reinterpret_cast<const float4v *>(gate + o);
         r = (float4v){gated(r[0], gt[0]), gated(r[1], gt[1]), gated(r[2], gt[2]), gated(r[3], gt[3])};
     }
-    *reinterpret_cast<float4v *>(out + o) = r;
+    if (out16)
+        *reinterpret_cast<half4 *>(out16 + o) = __builtin_convertvector(r, half4);
+    else
+        *reinterpret_cast<float4v *>(out + o) = r;
+}
+
+// f16 copy of finished f32 rows (the unsplit path with an f16 destination), 4 values per thread.
+__global__ void __launch_bounds__(256) rows_f16_kernel(const float4v *__restrict__ x, half4 *__restrict__ y, size_t n4)
+{
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n4)
+        y[i] = __builtin_convertvector(x[i], half4);
 }
 
 #ifdef PF_TIMING
@@ -758,7 +776,7 @@ int prefill_init()
 
 int launch_chunk_q8(hipStream_t st, const float *q, const uint8_t *kc, const uint8_t *vc,
                     float *out, int n_head, int n_kv, int pos0, int tokens, int stride,
-                    float *part_acc, float *part_ml, int splits, const float *gate, int q4)
+                    float *part_acc, float *part_ml, int splits, const float *gate, int q4, void *out16)
 {
     ChunkArgs a;
     a.gate = gate;
@@ -808,7 +826,13 @@ int launch_chunk_q8(hipStream_t st, const float *q, const uint8_t *kc, const uin
             hipLaunchKernelGGL((chunk_q8_kernel<false, true>), dim3(grid, 1, 1), block, kPfLds, st, a);
         else
             hipLaunchKernelGGL(chunk_q8_kernel<false>, dim3(grid, 1, 1), block, kPfLds, st, a);
-        return launched(q4 ? "attn_chunk_q4" : "attn_chunk_q8");
+        int rc = launched(q4 ? "attn_chunk_q4" : "attn_chunk_q8");
+        if (rc || out16 == nullptr)
+            return rc;
+        const size_t n4 = (size_t)tokens * n_head * kHeadDim / 4;
+        hipLaunchKernelGGL(rows_f16_kernel, dim3((unsigned)((n4 + 255) / 256), 1, 1), dim3(256, 1, 1), 0, st,
+                           reinterpret_cast<const float4v *>(out), static_cast<half4 *>(out16), n4);
+        return launched("attn_chunk_rows_f16");
     }
     if (q4)
         hipLaunchKernelGGL((chunk_q8_kernel<true, true>), dim3(grid, 1, 1), block, kPfLds, st, a);
@@ -819,7 +843,7 @@ int launch_chunk_q8(hipStream_t st, const float *q, const uint8_t *kc, const uin
         return rc;
     hipLaunchKernelGGL(chunk_combine_kernel, dim3((unsigned)tokens, (unsigned)((n_head + 3) / 4), 1),
                        dim3(256, 1, 1), 0, st, part_acc, part_ml, out, gate, n_head, a.qslots, a.splits, a.group,
-                       a.ntask, tokens, pos0, a.slice_tiles, a.uniform);
+                       a.ntask, tokens, pos0, a.slice_tiles, a.uniform, static_cast<_Float16 *>(out16));
     return launched("attn_chunk_combine");
 }
 

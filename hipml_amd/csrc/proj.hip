@@ -898,7 +898,8 @@ int proj_init()
     return 0;
 }
 
-// x16 != nullptr: gate (optional) and convert into x16 first, then the GEMM over f16 activations.
+// x16 != nullptr: gate (optional) and convert into x16 first, then the GEMM over f16 activations;
+// x == nullptr: x16 already holds them.
 int launch_gemm_q8_f16(hipStream_t st, const uint8_t *w, const float *x, const float *gate, float *y, int m,
                        int k, int tokens, void *x16)
 {
@@ -908,13 +909,15 @@ int launch_gemm_q8_f16(hipStream_t st, const uint8_t *w, const float *x, const f
                            st, w, x, y, m, k, tokens);
         return launched("gemm_q8_0_f16");
     }
-    const size_t n8 = (size_t)tokens * k / 8;
-    hipLaunchKernelGGL(gate_f16_kernel, dim3((unsigned)((n8 + 255) / 256), 1, 1), dim3(256, 1, 1), 0, st,
-                       reinterpret_cast<const float4v *>(x), reinterpret_cast<const float4v *>(gate),
-                       static_cast<half8 *>(x16), n8);
-    int rc = launched("gate_f16");
-    if (rc)
-        return rc;
+    if (x != nullptr) {
+        const size_t n8 = (size_t)tokens * k / 8;
+        hipLaunchKernelGGL(gate_f16_kernel, dim3((unsigned)((n8 + 255) / 256), 1, 1), dim3(256, 1, 1), 0, st,
+                           reinterpret_cast<const float4v *>(x), reinterpret_cast<const float4v *>(gate),
+                           static_cast<half8 *>(x16), n8);
+        int rc = launched("gate_f16");
+        if (rc)
+            return rc;
+    }
     hipLaunchKernelGGL((gemm_q8_f16_kernel<true, kGemmWaves>), grid, dim3(128 * kGemmWaves, 1, 1), kGemmLds, st, w,
                        x16, y, m, k, tokens);
     return launched("gemm_q8_0_f16");

@@ -288,6 +288,18 @@ int hipml_attn_chunk_q8_split_gate(hipml_stream_t stream, const float *q, const 
                                    int n_kv, int head_dim, int pos0, int tokens, int dtype,
                                    int stride, float *part_acc, float *part_ml, int splits);
 
+/* The same with the finished rows delivered as f16 (round to nearest even) in out16
+ * [tokens][n_head][head_dim], 16-byte aligned: the operand form of the output projection, so
+ * hipml_attn_output_chunk_q8_0(attn_out = NULL, gate = NULL, x16 = out16) can follow without its
+ * conversion pass.  out16 holds exactly f16(what hipml_attn_chunk_q8_split_gate writes to out);
+ * `out` (same size as there) is working memory here and holds nothing defined afterwards.
+ * Replaces chunk_attention_q8_split + apply_output_chunk's gate
+ * (attn_chunk_kv.rs:72-107, crates/hipml-kernels/src/attn_gpu/imp/attn_chunk.rs:343-364). */
+int hipml_attn_chunk_q8_split_gate_f16(hipml_stream_t stream, const float *q, const void *kc,
+                                       const void *vc, const float *gate, float *out, void *out16,
+                                       int n_head, int n_kv, int head_dim, int pos0, int tokens, int dtype,
+                                       int stride, float *part_acc, float *part_ml, int splits);
+
 /* ---- output gate ------------------------------------------------------------ */
 
 /* y[i] = x[i] * sigmoid(gate[i]); y may alias x.  Replaces
@@ -337,6 +349,8 @@ int hipml_gemm_q8_0_f16(hipml_stream_t stream, const void *w, const float *x, fl
  * tokens*k f16 (2 bytes each, 16-byte aligned; the attention's split scratch is free by then): a
  * first kernel gates and rounds the rows to f16 once, the GEMM then reads half the bytes per
  * workgroup.  Same bits as hipml_q_gate_f32 followed by hipml_gemm_q8_0_f16, faster.
+ * attn_out == NULL (then gate must be NULL too): x16 already holds the rows as f16, as
+ * hipml_attn_chunk_q8_split_gate_f16 writes them, and only the GEMM runs.
  * Replaces AttnLayer::apply_output_chunk (q_gate_f32 + the tiled GEMM),
  * crates/hipml-kernels/src/attn_gpu/imp/attn_chunk.rs:343-397. */
 int hipml_attn_output_chunk_q8_0(hipml_stream_t stream, const void *wo, const float *attn_out,

@@ -117,3 +117,10 @@ def test_fused_gate_equals_attention_then_gate(tok, pos0, splits):
     want = orc.q_gate(plain.ravel(), gate.ravel())
     ok, _, _ = report(f"fused gate {tok}@{pos0} splits {splits}", want, host(fused).ravel(), 1e-6, 1e-5)
     assert ok
+    # the same rows delivered as f16 for the output projection: exactly f16 (nearest even) of the above
+    work = torch.full_like(x, float("nan"))
+    out16 = torch.full(x.shape, float("nan"), dtype=torch.float16, device="cuda")
+    attn.chunk_attention_q8_split_gate_f16(dev(q), dev(kb), dev(vb), dev(gate), work, out16, N_HEADS,
+                                           N_KV, HD, pos0, tok, 1, stride, acc, ml, splits)
+    torch.cuda.synchronize()
+    assert np.array_equal(host(out16).view(np.uint16), host(fused).astype(np.float16).view(np.uint16))

@@ -201,6 +201,14 @@ def test_output_chunk_equals_gate_then_gemm():
     attn.gemm_q8_0_f16(wd, ad, ref, m, k, t)
     torch.cuda.synchronize()
     assert torch.equal(plain, ref)
+    # rows that arrive as f16 already (the chunk attention can deliver them so): only the GEMM runs
+    ready = ad.to(torch.float16)
+    direct = torch.full((t, m), float("nan"), dtype=torch.float32, device="cuda")
+    attn.output_chunk_q8_0(wd, None, None, direct, m, k, t, ready)
+    torch.cuda.synchronize()
+    assert torch.equal(direct, ref)
+    with pytest.raises(attn.HipmlError):   # a gate without the f32 rows it applies to
+        attn.output_chunk_q8_0(wd, None, gd, direct, m, k, t, ready)
 
 
 @pytest.mark.parametrize("m,k", [(1024, 5120), (12288, 5120)])
