@@ -4,7 +4,7 @@
 // W is [m][k/32] blocks of 34 bytes (f16 scale d, 32 int8), row-major; y[r][row] = sum_k W[row][k] x[r][k]
 // (crates/hipml-core/src/quant.rs:653-675, crates/hipml-core/src/ops.rs:102-104,136-176).
 //
-// gemv_q8_rows_kernel: up to 4 activation rows per pass, bound by streaming W once from HBM.
+// gemv_q8_rows_kernel: one or two activation rows, bound by streaming W once from HBM.
 //   All MFMAs are v_mfma_f32_16x16x32_f16 with A = x (activation rows), B = W (16 weight rows),
 //   one q8 block = one contraction, so the f16 block scale multiplies an exact integer dot product
 //   in fp32: acc += d * (x . q), as the CPU definition's d*q products summed in fp32.
@@ -18,11 +18,11 @@
 //   tile puts weight row lm back in lane lm (rows of C are activation rows), where its scale is.
 //   int8 -> f16 exactly: byte b^0x80 = b+128 under a high byte 0x64 is the f16 1024 + (b+128);
 //   one packed f16 subtract of 1152 leaves b.  x enters as hi + lo f16 halves (two MFMAs, ~22 bits),
-//   converted once per workgroup into LDS in operand order: that is what limits a pass to 4 rows.
+//   converted once per workgroup into LDS in operand order (whole rows: a pass is a few rows at most).
 //   The waves of a workgroup split k; a wave requests the activations first, then two chunks of
 //   its weight blocks (all of them for k = 6144) before it waits for anything, and the partial sums
 //   meet in LDS in a fixed order (no atomics: the result does not depend on timing).
-// gemv_q8_tile_kernel (further down): the same stream for 5 to 128 rows, activations as full A tiles.
+// gemv_q8_tile_kernel (further down): the same stream for 3 to 128 rows, activations as full A tiles.
 
 #include "common.h"
 
@@ -91,7 +91,7 @@ struct GemvChunk {
     uint2a4 o[CH][TILES];
 };
 
-constexpr int kGemvMaxRows = 4;        // activation rows per pass (their operands live in LDS)
+constexpr int kGemvMaxRows = 2;        // activation rows per pass (their operands live in LDS)
 constexpr int kGemvLdsBudget = 128 << 10;
 
 // Activation rows per pass for a given k: as many (up to kGemvMaxRows) as keep the hi/lo operands of
@@ -317,7 +317,7 @@ __global__ void __launch_bounds__(64 * WAVES, TILES == 1 ? 2 : 1) gemv_q8_rows_k
     }
 }
 
-// ---- gemv_q8_tile_kernel: 5 to 128 activation rows (batched decode, verify groups) --------------
+// ---- gemv_q8_tile_kernel: 3 to 128 activation rows (batched decode, verify groups) --------------
 //
 // The same streaming of W as above, with the activations as full 16-row A tiles: A row = activation
 // row, hi and lo halves as two chained MFMAs, XT tiles (16 or 32 rows) per pass.  The rows' operands
@@ -535,23 +535,19 @@ static int launch_gemv_variant(hipStream_t st, const uint8_t *w, const float *x,
 
 int launch_gemv_q8_rows(hipStream_t st, const uint8_t *w, const float *x, float *y, int m, int k, int rows)
 {
+    // three rows or more: full A tiles of 16 or 32 rows (measured at 5120 x 6144, 4 rows: 14.6 us
+    // against 16.7 us for the row kernel with two weight tiles per workgroup; 1 row: 13.6 against 12.1)
+    if (rows > kGemvMaxRows)
+        return rows > 16 ? launch_gemv_tile<8, 2, 2>(st, w, x, y, m, k, rows)
+                         : launch_gemv_tile<8, 2, 1>(st, w, x, y, m, k, rows);
     int rp = gemv_rows_per_pass(k);
     if (rp < 1)
         return fail(HIPML_ATTN_E_RANGE, "k %d: one activation row does not fit the LDS operand buffer", k);
     rp = rows < rp ? rows : rp;
-    // more than a pass of the row kernel: full A tiles of 16 or 32 rows
-    if (rows > kGemvMaxRows)
-        return rows > 16 ? launch_gemv_tile<8, 2, 2>(st, w, x, y, m, k, rows)
-                         : launch_gemv_tile<8, 2, 1>(st, w, x, y, m, k, rows);
     // One 16-row weight tile per workgroup keeps the kernel inside 128 registers, so two workgroups
     // share a CU and the 320 workgroups of a 5120-row matrix start together (workgroups start in
-    // windows of as many as fit the chip; a second window opens when the first has drained).  With
-    // 3-4 rows per pass the activations' staging needs more registers: two tiles per workgroup,
-    // half as many workgroups, one per CU (measured at 5120 x 6144: 1 row 12.2 vs 15.0 us, 4 rows
-    // 18.5 vs 16.7 us).
-    if (rp <= 2)
-        return launch_gemv_variant<8, 1, 6>(st, w, x, y, m, k, rows, rp);
-    return launch_gemv_variant<8, 2, 6>(st, w, x, y, m, k, rows, rp);
+    // windows of as many as fit the chip; a second window opens when the first has drained).
+    return launch_gemv_variant<8, 1, 6>(st, w, x, y, m, k, rows, rp);
 }
 
 
