@@ -554,8 +554,10 @@ def bench_copycal(torch, steps):
 # CPU baseline (the oracle, timed; never part of the measured GPU path)
 # ---------------------------------------------------------------------------------------
 
-def cpu_prefill(orc, np, tokens, pos0, rows_sample=None):
-    """Scalar single-thread oracle on the headline workload; returns (tok/s, sample text)."""
+def cpu_prefill(orc, np, tokens, pos0, rows_sample=None, n_threads=1, budget=10.0):
+    """The oracle on the headline workload, repeated for about `budget` seconds; the attention runs on
+    `n_threads` threads over query heads (1 = the reference's own single-threaded path); returns
+    (tok/s, seconds, repetitions)."""
     r = orc.Rng(0x5EED0002)
     stride = pos0 + tokens
     q = r.normal_array((tokens, H, HD))
@@ -567,7 +569,7 @@ def cpu_prefill(orc, np, tokens, pos0, rows_sample=None):
     n = tokens if rows is None else len(rows)
     # the whole workload, repeated until about ten seconds of CPU work have been timed
     reps, total = 0, 0.0
-    while total < 10.0 and reps < 50:
+    while total < budget and reps < 50:
         qq, kk = q.copy(), k.copy()
         t0 = time.perf_counter()
         for t in range(tokens):
@@ -576,7 +578,7 @@ def cpu_prefill(orc, np, tokens, pos0, rows_sample=None):
             kk[p] = orc.rope_multi(kk[p], KV, HD, NROT, sec, (p, p, p, p), THETA).reshape(KV, HD)
         kb = orc.quantize(0, kk.transpose(1, 0, 2)).reshape(KV, stride, ROW)
         vb = orc.quantize(0, v.transpose(1, 0, 2)).reshape(KV, stride, ROW)
-        o = orc.attn_chunk_kv(qq, kb, vb, H, KV, HD, pos0, tokens, stride, SCALE, rows=rows, n_threads=1)
+        o = orc.attn_chunk_kv(qq, kb, vb, H, KV, HD, pos0, tokens, stride, SCALE, rows=rows, n_threads=n_threads)
         orc.q_gate(o.ravel(), gate[:n].ravel())
         total += time.perf_counter() - t0
         reps += 1
@@ -636,6 +638,8 @@ def main() -> int:
             "gemv4": lambda: bench_gemv(torch, attn, 4, max(K // 4, 10), LAYERS),
             "gemv16": lambda: bench_gemv(torch, attn, 16, max(K // 4, 10), LAYERS),
             "gemv24": lambda: bench_gemv(torch, attn, 24, max(K // 4, 10), LAYERS),
+            "gemv64": lambda: bench_gemv(torch, attn, 64, max(K // 4, 10), LAYERS),
+            "gemv128": lambda: bench_gemv(torch, attn, 128, max(K // 4, 10), LAYERS),
             "gemm24": lambda: bench_gemm(torch, attn, 24, max(K // 4, 10), LAYERS),
             "gemm128": lambda: bench_gemm(torch, attn, 128, max(K // 4, 10), LAYERS),
             "layer32k": lambda: bench_decode_layer(torch, attn, 32768, max(K // 4, 10), LAYERS),
@@ -706,6 +710,12 @@ def main() -> int:
                       f"1 thread, scalar C restatement of the reference's CPU path",
             "host_cpus": os.cpu_count(),
         }
+        # beside it: the same restatement with its attention spread over the box's CPU share
+        nt = min(16, os.cpu_count() or 1)
+        if nt > 1:
+            mt, msecs, mreps = cpu_prefill(orc, np, 672, 0, n_threads=nt, budget=3.0)
+            line["cpu_baseline"]["threads"] = {"value": mt, "unit": "tok/s", "cores": nt,
+                                               "sample": f"the same workload {mreps} times, {msecs:.1f} s"}
         if not args.main_only:
             line["cpu_baseline"]["decode_us_per_layer"] = {
                 "8192": cpu_decode(orc, 8192), "32768": cpu_decode(orc, 32768)}
