@@ -887,8 +887,6 @@ int proj_init()
                                 hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLds);
     if (e == hipSuccess)
         e = raise_gemv_lds<8, 1, 6>();
-    if (e == hipSuccess)
-        e = raise_gemv_lds<8, 2, 6>();
     if (e != hipSuccess)
         return fail((int)e, "hipFuncSetAttribute(projection LDS) failed: %d (%s)", (int)e, hipGetErrorString(e));
     return 0;
