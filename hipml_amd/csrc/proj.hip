@@ -556,7 +556,7 @@ int launch_gemv_q8_rows(hipStream_t st, const uint8_t *w, const float *x, float 
 // y[t][row] for a 128 (tokens) x 128 (weight rows) tile per workgroup, MFMA-bound:
 // v_mfma_f32_32x32x16_f16 with A = x (f32 -> f16, round to nearest), B = W dequantized to f16 (d*q, one
 // rounding: the precision class of the reference's f16-operand prefill kernels and of this library's
-// chunk attention), fp32 accumulation.  Eight consumer waves, each a 32 x 64 piece (1 x 2 MFMA tiles),
+// chunk attention), fp32 accumulation.  Four consumer waves, each a 64 x 64 piece (2 x 2 MFMA tiles),
 // and eight producer waves that fetch and stage.  A k step is 64 values = one 68-byte pair of blocks per
 // weight row; both operand tiles are staged as [128 rows][64 f16] with a 144-byte row pitch (128-bit
 // reads and writes of 16 consecutive rows then touch every bank once), double buffered, one barrier
@@ -598,7 +598,11 @@ constexpr int kGemmLds = 2 * kGemmBuf;            // double buffered: 73,728 byt
 #ifndef GEMM_WAVES
 #define GEMM_WAVES 8
 #endif
-constexpr int kGemmWaves = GEMM_WAVES;            // waves per role
+#ifndef GEMM_CWAVES
+#define GEMM_CWAVES 4
+#endif
+constexpr int kGemmWaves = GEMM_WAVES;            // producer waves
+constexpr int kGemmCWaves = GEMM_CWAVES;          // consumer waves
 
 // What one producer thread fetches for one step: per unit WN weight (row, quarter) pairs, and XN
 // 16-byte pieces of the activation tile.
@@ -618,19 +622,24 @@ __device__ __forceinline__ half8 dequant8(uint32_t w0, uint32_t w1, _Float16 d)
     return q * dv;
 }
 
-// NW waves per role (consumers first, then producers): 4 + 4 or 8 + 8.  LDS serves a wave at about
-// 34 B/clk for 128-bit reads and 16-20 B/clk for 128-bit writes whatever the others do, up to well
-// over 128 B/clk in all (measured), so eight waves per role move the same tiles in less time.
+// kGemmCWaves consumer waves first, then NW producer waves: 4 + 8.  Consumers own 64 x 64 pieces
+// (2 x 2 MFMA tiles: every operand read feeds two MFMAs, 64 KB of LDS reads per step instead of the
+// 96 KB of eight 32 x 64 pieces), producers one weight (row, quarter) pair and two activation pieces
+// per thread and step.  LDS serves a wave at about 34 B/clk for 128-bit reads and 16-20 B/clk for
+// 128-bit writes whatever the others do, up to well over 128 B/clk in all (measured), so eight
+// producer waves stage a tile in less time than four.  Measured at 5120 x 6144, 672 tokens, gate
+// pass included: 4 + 4 waves 77.3, 8 + 8 waves 76.5, 4 + 8 waves 71.6 us.
 template <bool X16, int NW>
-__global__ void __launch_bounds__(128 * NW) gemm_q8_f16_kernel(const uint8_t *__restrict__ w,
+__global__ void __launch_bounds__(64 * (NW + kGemmCWaves)) gemm_q8_f16_kernel(const uint8_t *__restrict__ w,
                                                               const void *__restrict__ xv,
                                                               float *__restrict__ y, int m, int k, int tokens)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    constexpr int NT = 64 * NW; // threads per role
+    constexpr int NT = 64 * NW; // producer threads
+    constexpr int NC = kGemmCWaves;
     constexpr int KU = kGemmUnits;
-    const bool producer = threadIdx.x >= NT;
-    const int tid = producer ? threadIdx.x - NT : threadIdx.x;
+    const bool producer = threadIdx.x >= 64 * NC;
+    const int tid = producer ? threadIdx.x - 64 * NC : threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63; // within the role
     const int m0 = blockIdx.x * kGemmM, t0 = blockIdx.y * kGemmT;
     const int nunits = k >> 6;
@@ -716,7 +725,7 @@ __global__ void __launch_bounds__(128 * NW) gemm_q8_f16_kernel(const uint8_t *__
 
     // MFMA roles: consumer wave (wt, wm) owns AT 32-token tiles from token wt * 32 AT and weight rows
     // wm*64..: 64 x 64 per wave with four consumers, 32 x 64 with eight
-    constexpr int AT = 8 / NW;
+    constexpr int AT = 8 / NC;
     const int wt_ = wave >> 1, wm_ = wave & 1;
     const int ln = lane & 31, lh = lane >> 5;
     float16v acc[AT][2];
@@ -899,7 +908,7 @@ int launch_gemm_q8_f16(hipStream_t st, const uint8_t *w, const float *x, const f
 {
     const dim3 grid((unsigned)((m + kGemmM - 1) / kGemmM), (unsigned)((tokens + kGemmT - 1) / kGemmT), 1);
     if (x16 == nullptr) {
-        hipLaunchKernelGGL((gemm_q8_f16_kernel<false, kGemmWaves>), grid, dim3(128 * kGemmWaves, 1, 1), kGemmLds,
+        hipLaunchKernelGGL((gemm_q8_f16_kernel<false, kGemmWaves>), grid, dim3(64 * (kGemmWaves + kGemmCWaves), 1, 1), kGemmLds,
                            st, w, x, y, m, k, tokens);
         return launched("gemm_q8_0_f16");
     }
@@ -912,7 +921,7 @@ int launch_gemm_q8_f16(hipStream_t st, const uint8_t *w, const float *x, const f
         if (rc)
             return rc;
     }
-    hipLaunchKernelGGL((gemm_q8_f16_kernel<true, kGemmWaves>), grid, dim3(128 * kGemmWaves, 1, 1), kGemmLds, st, w,
+    hipLaunchKernelGGL((gemm_q8_f16_kernel<true, kGemmWaves>), grid, dim3(64 * (kGemmWaves + kGemmCWaves), 1, 1), kGemmLds, st, w,
                        x16, y, m, k, tokens);
     return launched("gemm_q8_0_f16");
 }
