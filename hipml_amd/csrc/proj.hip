@@ -736,24 +736,39 @@ __global__ void __launch_bounds__(64 * (NW + kGemmCWaves)) gemm_q8_f16_kernel(co
 #pragma unroll
             for (int i = 0; i < 16; i++)
                 acc[a][b][i] = 0.0f;
+    // All operands of a step are named first and the scheduling groups below pin the order: the reads
+    // of the first 16 values of k, then one MFMA and one read in turn, so that a read's LDS latency
+    // is covered by MFMAs (left to itself the compiler read, waited, multiplied: 840 cycles per step
+    // for 512 of MFMA).
     auto multiply = [&](const uint8_t *buf) {
         const uint8_t *xa = buf + (wt_ * 32 * AT + ln) * kGemmPitch + lh * 16;
         const uint8_t *wb = buf + kGemmTile + (wm_ * 64 + ln) * kGemmPitch + lh * 16;
+        half8 A[4 * KU][AT], B[4 * KU][2];
 #pragma unroll
         for (int kk = 0; kk < 4 * KU; kk++) {
-            half8 A[AT], B[2];
 #pragma unroll
             for (int a = 0; a < AT; a++)
-                A[a] = *reinterpret_cast<const half8 *>(xa + a * 32 * kGemmPitch + kk * 32);
+                A[kk][a] = *reinterpret_cast<const half8 *>(xa + a * 32 * kGemmPitch + kk * 32);
 #pragma unroll
             for (int b = 0; b < 2; b++)
-                B[b] = *reinterpret_cast<const half8 *>(wb + b * 32 * kGemmPitch + kk * 32);
+                B[kk][b] = *reinterpret_cast<const half8 *>(wb + b * 32 * kGemmPitch + kk * 32);
+        }
+#pragma unroll
+        for (int kk = 0; kk < 4 * KU; kk++)
 #pragma unroll
             for (int a = 0; a < AT; a++)
 #pragma unroll
                 for (int b = 0; b < 2; b++)
-                    acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[a], B[b], acc[a][b], 0, 0, 0);
+                    acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[kk][a], B[kk][b], acc[a][b], 0, 0, 0);
+        constexpr int per = AT + 2;             // reads per 16 values of k
+        constexpr int reads = 4 * KU * per, mfmas = 4 * KU * AT * 2;
+        __builtin_amdgcn_sched_group_barrier(0x100, per, 0);
+#pragma unroll
+        for (int i = 0; i < reads - per; i++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         }
+        __builtin_amdgcn_sched_group_barrier(0x008, mfmas - (reads - per), 0);
     };
 
     // The second half of the waves produce (fetch, dequantize, write the next step's tiles), the first
