@@ -451,3 +451,59 @@ class DeepKv:
         if pos > 0:
             kv_rows_copy(self.dtype, k, v, self.k, self.v, self.n_kv, self.head_dim, pos, self.seq, pos,
                          stream)
+
+
+class BatchKv:
+    """One layer's quantized caches of `slots` sequences plus the batched decode scratch: the role of
+    the reference's `BatchKv` (crates/hipml-model/src/gpu/batch/kv.rs:11-75).  The caches are
+    contiguous across slots -- slot b starts `b * slot_bytes` into K (and V), each slot laid out
+    [n_kv][stride][row bytes] -- so the batched append and attention address a slot by its index."""
+
+    def __init__(self, slots, n_heads=24, n_kv=4, head_dim=HEAD_DIM, stride=4096, max_rows=None,
+                 device="cuda", dtype=0):
+        assert head_dim == HEAD_DIM
+        assert dtype in (0, 1), "KvDtype id: 0 = q8_0, 1 = q4_0"
+        self.dtype, self.slots = dtype, slots
+        self.row_bytes = ROW_BYTES if dtype == 0 else head_dim // 32 * 18
+        self.n_heads, self.n_kv, self.head_dim, self.seq = n_heads, n_kv, head_dim, stride
+        self.slot_bytes = n_kv * stride * self.row_bytes
+        self.k = torch.zeros((slots, n_kv, stride, self.row_bytes), dtype=torch.uint8, device=device)
+        self.v = torch.zeros_like(self.k)
+        self.splits = batch_splits(stride, n_kv, slots)
+        # one scratch slot per query row: a verify group brings several rows per sequence
+        self.max_rows = max_rows or slots
+        self.acc_slot = n_heads * self.splits * head_dim
+        self.ml_slot = n_heads * self.splits * 2
+        self.part_acc = torch.empty((self.max_rows, self.acc_slot), dtype=torch.float32, device=device)
+        self.part_ml = torch.empty((self.max_rows, self.ml_slot), dtype=torch.float32, device=device)
+
+    def bytes(self) -> int:
+        return 2 * self.slots * self.slot_bytes
+
+    def append(self, k_f32, v_f32, pos, rows, stream=None):
+        """Quantize and append one K/V row per entry of `pos` (device int32 [rows][2] = (position,
+        live length), row i belonging to slot i): `Launcher::kv_encode_rows_ptr`."""
+        kv_encode_rows(self.dtype, k_f32, v_f32, self.k, self.v, self.n_kv, self.head_dim, self.seq, pos,
+                       self.slot_bytes, rows, stream)
+
+    def decode(self, pos, q, out, scale, cols_per_slot=None, gate=None, stream=None):
+        """Batched decode over every slot: one query row per slot (`Launcher::attn_decode_batch`), or
+        `cols_per_slot[b]` rows for slot b -- verify groups beside plain slots in one launch -- with
+        the output gate applied in the merge when `gate` is given.  `pos` is device int32 [rows][2]."""
+        q_slot = self.n_heads * self.head_dim
+        if cols_per_slot is None and gate is None:
+            attn_decode_batch(self.dtype, pos, q, self.k, self.v, self.part_acc, self.part_ml, out,
+                              self.n_heads, self.n_kv, self.head_dim, self.seq, scale, self.splits,
+                              self.slot_bytes, self.acc_slot, self.ml_slot, q_slot, self.slots, 0, stream)
+            return
+        cols = list(cols_per_slot) if cols_per_slot is not None else [1] * self.slots
+        assert len(cols) == self.slots and sum(cols) <= self.max_rows
+        if gate is None:
+            attn_decode_batch_cols(self.dtype, pos, q, self.k, self.v, self.part_acc, self.part_ml, out,
+                                   self.n_heads, self.n_kv, self.head_dim, self.seq, scale, self.splits,
+                                   self.slot_bytes, self.acc_slot, self.ml_slot, q_slot, cols, stream)
+        else:
+            attn_decode_batch_cols_gate(self.dtype, pos, q, self.k, self.v, self.part_acc, self.part_ml,
+                                        out, gate, self.n_heads, self.n_kv, self.head_dim, self.seq, scale,
+                                        self.splits, self.slot_bytes, self.acc_slot, self.ml_slot, q_slot,
+                                        cols, stream)

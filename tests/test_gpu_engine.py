@@ -303,3 +303,48 @@ def test_chunk_layer_with_fused_launches_replays_under_a_captured_graph():
         torch.cuda.synchronize()
         assert torch.equal(y, eager_y) and torch.equal(kc, eager_k), f"replay {i} differs from the eager calls"
         assert bool(torch.isfinite(y).all())
+
+
+def test_batch_kv_owner_appends_and_decodes_every_slot():
+    # the batched engine's cache owner (crates/hipml-model/src/gpu/batch/kv.rs:11-75,
+    # gpu/batch/forward.rs:94-133): contiguous per-slot caches, one appended row and one query row per
+    # slot, depths that differ; every slot against the oracle over its own cache bytes
+    from gpu_util import N_HEADS, N_KV, HD, ROW, SCALE, dev, host
+    slots, stride = 5, 700
+    depths = [0, 1, 63, 300, 699]           # position of the new row = rows already cached
+    r = orc.Rng(0xBA7C)
+    kv = attn.BatchKv(slots, N_HEADS, N_KV, HD, stride)
+    assert kv.slot_bytes == N_KV * stride * ROW and kv.bytes() == 2 * slots * kv.slot_bytes
+    assert kv.splits == attn.batch_splits(stride, N_KV, slots)
+    hk = np.zeros((slots, N_KV, stride, ROW), dtype=np.uint8)
+    hv = np.zeros_like(hk)
+    for b, d in enumerate(depths):
+        if d:
+            kf, vf = r.normal_array((N_KV, d, HD)), r.normal_array((N_KV, d, HD))
+            hk[b, :, :d] = orc.quantize(0, kf).reshape(N_KV, d, ROW)
+            hv[b, :, :d] = orc.quantize(0, vf).reshape(N_KV, d, ROW)
+    kv.k.copy_(dev(hk))
+    kv.v.copy_(dev(hv))
+    k_new, v_new = r.normal_array((slots, N_KV, HD)), r.normal_array((slots, N_KV, HD))
+    q = r.normal_array((slots, N_HEADS, HD))
+    pos = torch.tensor([[d, d + 1] for d in depths], dtype=torch.int32, device="cuda")
+    out = torch.full((slots, N_HEADS, HD), float("nan"), device="cuda")
+    kv.append(dev(k_new), dev(v_new), pos, slots)
+    kv.decode(pos, dev(q), out, SCALE)
+    torch.cuda.synchronize()
+    gk, gv, got = host(kv.k), host(kv.v), host(out)
+    for b, d in enumerate(depths):
+        assert np.array_equal(gk[b, :, d].ravel(), orc.quantize(0, k_new[b]))
+        assert np.array_equal(gv[b, :, d].ravel(), orc.quantize(0, v_new[b]))
+        assert np.array_equal(gk[b, :, :d], hk[b, :, :d]) and not gk[b, :, d + 1:].any()
+        want = orc.attn_decode_kv(q[b], gk[b], gv[b], N_HEADS, N_KV, HD, d + 1, SCALE, stride=stride)
+        ok, ma, _ = orc.compare(want, got[b], 2e-3, 1e-2)
+        assert ok, f"slot {b} depth {d}: max_abs {ma}"
+    # the same rows with the output gate in the merge: the bits of decode followed by the gate kernel
+    gate = dev(r.normal_array((slots, N_HEADS, HD)))
+    gated = torch.empty_like(out)
+    kv.decode(pos, dev(q), gated, SCALE, gate=gate)
+    two = torch.empty_like(out)
+    attn.q_gate(out, gate, two)
+    torch.cuda.synchronize()
+    assert torch.equal(gated, two)
