@@ -39,6 +39,7 @@ EXPORTS = [
     "hipml_kv_rows_copy", "hipml_rope_encode_chunk_f32",
     "hipml_attn_front_encode_f32", "hipml_attn_chunk_front_encode_f32",
     "hipml_attn_chunk_q8_split_gate_f16",
+    "hipml_attn_front_rows_f32", "hipml_attn_front_rows_encode_f32",
 ]
 
 
@@ -104,6 +105,9 @@ def lib() -> C.CDLL:
                                                 i, i, i, i, i, i, i, i, f, f, i]),
             "hipml_attn_chunk_front_encode_f32": (i, [vp, i, vp, vp, vp, vp, vp, vp, vp, vp, vp,
                                                       i, i, i, i, f, f, i, i, i]),
+            "hipml_attn_front_rows_f32": (i, [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, f, f, vp, i]),
+            "hipml_attn_front_rows_encode_f32": (i, [vp, i, vp, vp, vp, vp, vp, vp, vp, vp, vp,
+                                                     i, i, i, i, f, f, i, vp, sz, i]),
             "hipml_kv_rows_copy": (i, [vp, i, vp, vp, vp, vp, i, i, i, i, i]),
             "hipml_rope_encode_chunk_f32": (i, [vp, vp, vp, vp, vp, vp, i, i, i, i, f, i, i, i, i]),
             "hipml_gemv_q8_0_rows": (i, [vp, vp, vp, vp, i, i, i]),
@@ -234,6 +238,24 @@ def chunk_front_encode(dtype, qg, k, v, q, gate, q_norm, k_norm, k_cache, v_cach
                                                    _p(gate), _p(q_norm), _p(k_norm), _p(k_cache),
                                                    _p(v_cache), n_heads, n_kv, head_dim, n_rot, theta,
                                                    eps, pos0, tokens, stride))
+
+
+def front_rows(qg, k, q, gate, q_norm, k_norm, n_heads, n_kv, head_dim, n_rot, theta, eps, pos, rows,
+               stream=None):
+    """`AttnLayer::split_rope_rows`: the front end over one row per sequence, row r at text position
+    pos[r][0] (`pos` = device int32 [rows][2])."""
+    _check(lib().hipml_attn_front_rows_f32(_stream(stream), _p(qg), _p(k), _p(q), _p(gate), _p(q_norm),
+                                           _p(k_norm), n_heads, n_kv, head_dim, n_rot, theta, eps,
+                                           _p(pos), rows))
+
+
+def front_rows_encode(dtype, qg, k, v, q, gate, q_norm, k_norm, k_cache, v_cache, n_heads, n_kv, head_dim,
+                      n_rot, theta, eps, stride, pos, slot_bytes, slots, stream=None):
+    """`front_rows` and `kv_encode_rows` of the same step in one launch (same bits)."""
+    _check(lib().hipml_attn_front_rows_encode_f32(_stream(stream), dtype, _p(qg), _p(k), _p(v), _p(q),
+                                                  _p(gate), _p(q_norm), _p(k_norm), _p(k_cache),
+                                                  _p(v_cache), n_heads, n_kv, head_dim, n_rot, theta, eps,
+                                                  stride, _p(pos), slot_bytes, slots))
 
 
 # ---- KV append ------------------------------------------------------------------------
@@ -485,6 +507,13 @@ class BatchKv:
         live length), row i belonging to slot i): `Launcher::kv_encode_rows_ptr`."""
         kv_encode_rows(self.dtype, k_f32, v_f32, self.k, self.v, self.n_kv, self.head_dim, self.seq, pos,
                        self.slot_bytes, rows, stream)
+
+    def front_append(self, qg, k, v, q, gate, q_norm, k_norm, n_rot, theta, eps, pos, stream=None):
+        """The step in front of `decode`: q|gate split, head norms and RoPE of one row per slot at its
+        own position, and the append of its K/V row, in one launch."""
+        front_rows_encode(self.dtype, qg, k, v, q, gate, q_norm, k_norm, self.k, self.v, self.n_heads,
+                          self.n_kv, self.head_dim, n_rot, theta, eps, self.seq, pos, self.slot_bytes,
+                          self.slots, stream)
 
     def decode(self, pos, q, out, scale, cols_per_slot=None, gate=None, stream=None):
         """Batched decode over every slot: one query row per slot (`Launcher::attn_decode_batch`), or

@@ -497,6 +497,51 @@ int hipml_attn_chunk_front_encode_f32(hipml_stream_t stream, int dtype, const fl
                         stride);
 }
 
+// The batched engine's front end: row r belongs to sequence r and rotates at text position pos[2 r].
+int hipml_attn_front_rows_f32(hipml_stream_t stream, const float *qg, float *k, float *q, float *gate,
+                              const float *q_norm, const float *k_norm, int n_heads, int n_kv,
+                              int head_dim, int n_rot, float theta_base, float eps, const int32_t *pos,
+                              int rows)
+{
+    clear_error();
+    REQUIRE_PTR(pos);
+    int rc = check_front(qg, q, gate, k, q_norm, k_norm, n_heads, n_kv, head_dim, n_rot, theta_base, eps);
+    if (rc)
+        return rc;
+    if (rows < 0)
+        return fail(HIPML_ATTN_E_RANGE, "rows %d is negative", rows);
+    if (rows == 0)
+        return 0;
+    return launch_front(as_stream(stream), qg, q, gate, k, q_norm, k_norm, n_heads, n_kv, n_rot, 0, 0, 0,
+                        0, nullptr, 0, rows, theta_base, eps, g_rope, -1, nullptr, nullptr, nullptr, nullptr,
+                        0, 0, pos, 0);
+}
+
+// The same with the append of every row's K and V into its sequence's cache (slot r starts
+// r * slot_bytes into the caches), at position pos[2 r].
+int hipml_attn_front_rows_encode_f32(hipml_stream_t stream, int dtype, const float *qg, float *k,
+                                     const float *v, float *q, float *gate, const float *q_norm,
+                                     const float *k_norm, void *k_cache, void *v_cache, int n_heads,
+                                     int n_kv, int head_dim, int n_rot, float theta_base, float eps,
+                                     int stride, const int32_t *pos, size_t slot_bytes, int slots)
+{
+    clear_error();
+    REQUIRE_PTR(pos);
+    int rc = check_front(qg, q, gate, k, q_norm, k_norm, n_heads, n_kv, head_dim, n_rot, theta_base, eps);
+    if (rc == 0)
+        rc = check_encode(dtype, k, v, k_cache, v_cache, n_kv, head_dim, stride);
+    if (rc)
+        return rc;
+    if (slots < 0)
+        return fail(HIPML_ATTN_E_RANGE, "slots %d is negative", slots);
+    if (slots == 0)
+        return 0;
+    return launch_front(as_stream(stream), qg, q, gate, k, q_norm, k_norm, n_heads, n_kv, n_rot, 0, 0, 0,
+                        0, nullptr, 0, slots, theta_base, eps, g_rope, dtype, v,
+                        static_cast<uint8_t *>(k_cache), static_cast<uint8_t *>(v_cache), nullptr, 0, stride,
+                        pos, slot_bytes);
+}
+
 int hipml_kv_encode(hipml_stream_t stream, const int32_t *step, int dtype, const float *k_in,
                     const float *v_in, void *k_cache, void *v_cache, int n_kv, int head_dim,
                     int stride)

@@ -68,7 +68,8 @@ int launch_front(hipStream_t st, const float *qg, float *q, float *gate, float *
                  const float *kw, int n_heads, int n_kv, int n_rot, int s0, int s1, int s2, int s3,
                  const int32_t *pos, int pos0, int rows, float theta, float eps, const RopeTable &tab,
                  int enc = -1, const float *v = nullptr, uint8_t *kc = nullptr, uint8_t *vc = nullptr,
-                 const int32_t *step = nullptr, int start = 0, int stride = 0);
+                 const int32_t *step = nullptr, int start = 0, int stride = 0,
+                 const int32_t *rowpos = nullptr, size_t slot_bytes = 0);
 int launch_q_gate(hipStream_t st, const float *x, const float *gate, float *y, size_t n);
 
 struct DecodeLaunch {

@@ -384,11 +384,14 @@ int launch_rope_encode_chunk(hipStream_t st, int q4, float *q, float *k, const f
 // (x * scale) * w; the rotation reads cos/sin as the other RoPE kernels here do.
 // grid: ceil((n_heads + n_kv) * rows / 4) workgroups of 4 waves.  `pos` (device int32[4]) gives
 // the four M-RoPE position ids of a single row; when it is null, row t rotates at pos0 + t.
-// What the append half of a fused launch needs (kv == nullptr: front end only).
+// Per-row positions of a batch of sequences, and what the append half of a fused launch needs.
 struct FrontAppend {
-    const float *v;      // [rows][n_kv][256]
-    uint8_t *kc, *vc;    // caches
-    const int32_t *step; // row 0 goes to position step[0]; null: row r goes to start + r
+    const int32_t *rowpos; // non-null: row r belongs to sequence r and sits at text position
+                           // rowpos[2 r] (device int32 [rows][2] = position, live length)
+    size_t slot_bytes;     // with rowpos: sequence r's cache starts r * slot_bytes into kc / vc
+    const float *v;        // [rows][n_kv][256]
+    uint8_t *kc, *vc;      // caches
+    const int32_t *step;   // row 0 goes to position step[0]; null: row r goes to start + r (or rowpos)
     int start, stride;
 };
 
@@ -415,7 +418,8 @@ __global__ void __launch_bounds__(256) front_kernel(
         // a V row: quantize and append
         const int u = idx - nfront;
         const int row = u / n_kv, h = u - row * n_kv;
-        const int p = ap.step ? ap.step[0] : ap.start + row;
+        const int p = ap.step ? ap.step[0] : ap.rowpos ? ap.rowpos[2 * row] : ap.start + row;
+        uint8_t *vc = ap.vc + (ap.rowpos ? (size_t)row * ap.slot_bytes : 0);
         const float *src = ap.v + (size_t)u * kHeadDim;
         float x[4];
 #pragma unroll
@@ -425,9 +429,9 @@ __global__ void __launch_bounds__(256) front_kernel(
         for (int j = 0; j < 4; j++) {
             const size_t blk = ((size_t)h * ap.stride + p) * (kHeadDim / 32) + 2 * j + (lane >> 5);
             if (ENC == 2)
-                q4_encode_store(x[j], ap.vc + blk * kQ4BlockBytes, lane32);
+                q4_encode_store(x[j], vc + blk * kQ4BlockBytes, lane32);
             else
-                q8_encode_store(x[j], ap.vc + blk * kQ8BlockBytes, lane32);
+                q8_encode_store(x[j], vc + blk * kQ8BlockBytes, lane32);
         }
         return;
     }
@@ -476,7 +480,7 @@ __global__ void __launch_bounds__(256) front_kernel(
         if (e < n_rot) {
             const bool first = e < half;
             const int c = first ? e : e - half;
-            int p = pos ? pos[0] : pos0 + row;
+            int p = pos ? pos[0] : ap.rowpos ? ap.rowpos[2 * row] : pos0 + row;
             if (pos && sect > 0) {
                 const int sc = c % sect;
                 if (sc < s0)
@@ -498,14 +502,15 @@ __global__ void __launch_bounds__(256) front_kernel(
         x[j] = out;
     }
     if (ENC && !is_q) {
-        const int p = ap.step ? ap.step[0] : ap.start + row;
+        const int p = ap.step ? ap.step[0] : ap.rowpos ? ap.rowpos[2 * row] : ap.start + row;
+        uint8_t *kc = ap.kc + (ap.rowpos ? (size_t)row * ap.slot_bytes : 0);
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             const size_t blk = ((size_t)h * ap.stride + p) * (kHeadDim / 32) + 2 * j + (lane >> 5);
             if (ENC == 2)
-                q4_encode_store(x[j], ap.kc + blk * kQ4BlockBytes, lane32);
+                q4_encode_store(x[j], kc + blk * kQ4BlockBytes, lane32);
             else
-                q8_encode_store(x[j], ap.kc + blk * kQ8BlockBytes, lane32);
+                q8_encode_store(x[j], kc + blk * kQ8BlockBytes, lane32);
         }
     }
 }
@@ -515,7 +520,7 @@ int launch_front(hipStream_t st, const float *qg, float *q, float *gate, float *
                  const float *kw, int n_heads, int n_kv, int n_rot, int s0, int s1, int s2, int s3,
                  const int32_t *pos, int pos0, int rows, float theta, float eps, const RopeTable &tab,
                  int enc, const float *v, uint8_t *kc, uint8_t *vc, const int32_t *step, int start,
-                 int stride)
+                 int stride, const int32_t *rowpos, size_t slot_bytes)
 {
     int tab_rows = 0;
     const float *t = table_for(tab, theta, n_rot, &tab_rows);
@@ -524,7 +529,11 @@ int launch_front(hipStream_t st, const float *qg, float *q, float *gate, float *
     for (int r0 = 0; r0 < rows; r0 += max_rows) {
         const int n = rows - r0 < max_rows ? rows - r0 : max_rows;
         const unsigned grid = (unsigned)(((long long)per_row * n + 3) / 4);
-        const FrontAppend ap = {v ? v + (size_t)r0 * n_kv * kHeadDim : nullptr, kc, vc, step, start + r0, stride};
+        const FrontAppend ap = {rowpos ? rowpos + (size_t)r0 * 2 : nullptr, slot_bytes,
+                                v ? v + (size_t)r0 * n_kv * kHeadDim : nullptr,
+                                kc ? kc + (rowpos ? (size_t)r0 * slot_bytes : 0) : nullptr,
+                                vc ? vc + (rowpos ? (size_t)r0 * slot_bytes : 0) : nullptr, step, start + r0,
+                                stride};
         auto kern = enc < 0 ? front_kernel<0> : enc == 0 ? front_kernel<1> : front_kernel<2>;
         hipLaunchKernelGGL(kern, dim3(grid, 1, 1), dim3(256, 1, 1), 0, st,
                            qg + (size_t)r0 * n_heads * 2 * kHeadDim, q + (size_t)r0 * n_heads * kHeadDim,

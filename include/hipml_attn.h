@@ -156,6 +156,26 @@ int hipml_attn_chunk_front_encode_f32(hipml_stream_t stream, int dtype, const fl
                                       int n_kv, int head_dim, int n_rot, float theta_base, float eps,
                                       int pos0, int tokens, int stride);
 
+/* The front end over the rows of a batch of sequences: row r rotates at text position pos[2 r]
+ * (pos is the device int32 [rows][2] = (position, live length) the batched attention reads).  Same
+ * arithmetic as hipml_attn_chunk_front_f32, whose row t sits at pos0 + t.  Replaces
+ * AttnLayer::split_rope_rows -> qg_split_b + head_rmsnorm_b (q, k) + mrope_b (q, k),
+ * crates/hipml-kernels/src/attn_gpu.rs:649-784; call site crates/hipml-model/src/gpu/batch/forward.rs:79-88. */
+int hipml_attn_front_rows_f32(hipml_stream_t stream, const float *qg, float *k, float *q, float *gate,
+                              const float *q_norm, const float *k_norm, int n_heads, int n_kv,
+                              int head_dim, int n_rot, float theta_base, float eps, const int32_t *pos,
+                              int rows);
+
+/* hipml_attn_front_rows_f32 and hipml_kv_encode_rows (below) of the same step in one launch, same
+ * bits: row r's K and V go to position pos[2 r] of sequence r's cache, which starts r * slot_bytes
+ * into k_cache / v_cache.  Replaces split_rope_rows followed by Launcher::kv_encode_batch
+ * (crates/hipml-model/src/gpu/batch/forward.rs:79-106). */
+int hipml_attn_front_rows_encode_f32(hipml_stream_t stream, int dtype, const float *qg, float *k,
+                                     const float *v, float *q, float *gate, const float *q_norm,
+                                     const float *k_norm, void *k_cache, void *v_cache, int n_heads,
+                                     int n_kv, int head_dim, int n_rot, float theta_base, float eps,
+                                     int stride, const int32_t *pos, size_t slot_bytes, int slots);
+
 /* ---- q8_0 / q4_0 KV append ------------------------------------------------------- */
 
 /* One token: quantize k_in/v_in [n_kv][head_dim] into row step[0] of the cache.

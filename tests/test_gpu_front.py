@@ -185,3 +185,48 @@ def test_front_with_append_rejects_bad_arguments():
     with pytest.raises(attn.HipmlError):   # no step buffer
         attn.attn_front_encode(None, 0, t, t, t, t, t, t, t, b, b, N_HEADS, N_KV, HD, N_ROT, SECTIONS,
                                THETA, EPS, 12)
+
+
+@pytest.mark.parametrize("dtype", [0, 1])
+def test_batched_front_uses_each_row_s_own_position_and_cache(dtype):
+    # the batched engine's step (gpu/batch/forward.rs:79-106): one row per sequence, positions that
+    # differ, contiguous per-slot caches.  Against the oracle row by row, and the fused launch against
+    # front_rows followed by kv_encode_rows byte for byte.
+    slots, stride = 6, 96
+    positions = [0, 95, 7, 7, 50, 1]
+    row_bytes = 272 if dtype == 0 else 144
+    slot_bytes = N_KV * stride * row_bytes
+    qg, k, qw, kw = front_inputs(0xF50E + dtype, slots)
+    v = orc.Rng(0xF50F + dtype).normal_array((slots, N_KV, HD))
+    pos = torch.tensor([[p, p + 1] for p in positions], dtype=torch.int32, device="cuda")
+
+    def run(fused):
+        q = torch.full((slots, N_HEADS, HD), float("nan"), device="cuda")
+        gate = torch.full((slots, N_HEADS, HD), float("nan"), device="cuda")
+        kd, vd = dev(k), dev(v)
+        kc = torch.full((slots, N_KV, stride, row_bytes), 0x3C, dtype=torch.uint8, device="cuda")
+        vc = torch.full((slots, N_KV, stride, row_bytes), 0xC3, dtype=torch.uint8, device="cuda")
+        if fused:
+            attn.front_rows_encode(dtype, dev(qg), kd, vd, q, gate, dev(qw), dev(kw), kc, vc, N_HEADS, N_KV,
+                                   HD, N_ROT, THETA, EPS, stride, pos, slot_bytes, slots)
+        else:
+            attn.front_rows(dev(qg), kd, q, gate, dev(qw), dev(kw), N_HEADS, N_KV, HD, N_ROT, THETA, EPS,
+                            pos, slots)
+            attn.kv_encode_rows(dtype, kd, vd, kc, vc, N_KV, HD, stride, pos, slot_bytes, slots)
+        torch.cuda.synchronize()
+        return [host(t) for t in (q, gate, kd, kc, vc)]
+
+    two, one = run(False), run(True)
+    for name, a, b in zip(("q", "gate", "k", "k cache", "v cache"), two, one):
+        assert np.array_equal(a, b), name
+    gq, gg, gk, kc, vc = one
+    for r, p in enumerate(positions):
+        wq, wg, wk = orc.attn_front(qg[r], k[r], qw, kw, N_HEADS, N_KV, HD, N_ROT, (0, 0, 0, 0),
+                                    (p, p, p, p), THETA, EPS, tree=True)
+        assert np.array_equal(gg[r].ravel(), wg) and np.array_equal(gq[r].ravel(), wq), f"row {r}"
+        assert np.array_equal(gk[r].ravel(), wk), f"k row {r}"
+        assert np.array_equal(kc[r, :, p].ravel(), orc.quantize(dtype, wk)), f"slot {r} K row"
+        assert np.array_equal(vc[r, :, p].ravel(), orc.quantize(dtype, v[r].ravel())), f"slot {r} V row"
+        mask = np.ones(stride, dtype=bool)
+        mask[p] = False
+        assert (kc[r][:, mask] == 0x3C).all() and (vc[r][:, mask] == 0xC3).all()
