@@ -309,6 +309,52 @@ def bench_batch(torch, attn, orc, steps, warmup, layers):
     }
 
 
+def bench_batch_layer(torch, attn, orc, steps, layers):
+    """One plain step of the batched engine through the attention block: 16 sequences at the seeded
+    depths of the batched benchmark, one row each -- front end with append (per-row positions,
+    per-slot caches), batched attention with the gate in the merge, W_o over the 16 rows: 4 launches."""
+    r = orc.Rng(0x5EED0005)
+    depths, _ = batch_case(lambda: float(r.uniform()))
+    slots, stride = len(depths), 16448
+    m, k = 5120, H * HD
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(0x5EED000B)
+    kvs, ws = [], []
+    for _ in range(layers):
+        kv = attn.BatchKv(slots, H, KV, HD, stride)
+        for s in range(slots):
+            fill_cache_normal(torch, attn, kv.k[s], kv.v[s], stride, depths[s], gen)
+        kvs.append(kv)
+        ws.append(random_q8_0_weights(torch, m, k, gen))
+    pos = torch.tensor([[d, d + 1] for d in depths], dtype=torch.int32, device="cuda")
+    qg = torch.randn((slots, H, 2 * HD), device="cuda", generator=gen)
+    kx = torch.randn((slots, KV, HD), device="cuda", generator=gen)
+    vx = torch.randn((slots, KV, HD), device="cuda", generator=gen)
+    qw = torch.ones(HD, device="cuda")
+    kw = torch.ones(HD, device="cuda")
+    q = torch.empty((slots, H, HD), device="cuda")
+    gate = torch.empty((slots, H, HD), device="cuda")
+    out = torch.empty((slots, H, HD), device="cuda")
+    y = torch.empty((slots, m), device="cuda")
+    attn.rope_table(THETA, NROT, stride + 64)
+
+    def one_pass():
+        for kv, w in zip(kvs, ws):
+            kv.front_append(qg, kx, vx, q, gate, qw, kw, NROT, THETA, 1e-6, pos)
+            kv.decode(pos, q, out, SCALE, gate=gate)
+            attn.gemv_q8_0_rows(w, out, y, m, k, slots)
+
+    for _ in range(3):
+        one_pass()
+    with Timer(torch) as t:
+        for _ in range(steps):
+            one_pass()
+    return {"workload": f"batched step, {slots} sequences at depths U[512,16384] (seeded), one row each: front "
+                        f"end with append + attention with gate + W_o, {layers} layers per pass (4 launches "
+                        f"per layer)",
+            "us_per_layer": t.ms * 1e3 / (steps * layers), "live_rows": sum(depths) + slots}
+
+
 def bench_front(torch, attn, tokens, steps):
     """Attention front end over a chunk: q|gate split + head RMS norm + RoPE (one launch)."""
     gen = torch.Generator(device="cuda")
@@ -604,7 +650,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--main-only", action="store_true", help="skip the 'also' workloads")
     ap.add_argument("--only", default="", help="run one workload alone (prefill672, decode8k, "
-                    "decode32k, decode128k, chunk100k, batch16, front672, decode32k_q4, gemv1, gemv4, gemv16, gemm672, gemm2048, layer32k, layer672, copycal) for profiling; prints its object")
+                    "decode32k, decode128k, chunk100k, batch16, front672, decode32k_q4, gemv1, gemv4, gemv16, gemm672, gemm2048, layer32k, layer672, blayer16, copycal) for profiling; prints its object")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -643,6 +689,7 @@ def main() -> int:
             "gemm24": lambda: bench_gemm(torch, attn, 24, max(K // 4, 10), LAYERS),
             "gemm128": lambda: bench_gemm(torch, attn, 128, max(K // 4, 10), LAYERS),
             "layer32k": lambda: bench_decode_layer(torch, attn, 32768, max(K // 4, 10), LAYERS),
+            "blayer16": lambda: bench_batch_layer(torch, attn, orc, max(K // 10, 5), 4),
             "layer672": lambda: bench_chunk_layer(torch, attn, 672, 0, max(K // 10, 5), 4),
             "gemm672": lambda: bench_gemm(torch, attn, 672, max(K // 10, 5), 4),
             "gemm2048": lambda: bench_gemm(torch, attn, 2048, max(K // 20, 3), 4),
@@ -697,6 +744,8 @@ def main() -> int:
         also["decode_layer_32768"] = bench_decode_layer(torch, attn, 32768, d_steps, LAYERS)
         torch.cuda.empty_cache()
         also["chunk_layer_672"] = bench_chunk_layer(torch, attn, 672, 0, max(K // 10, 5), 4)
+        torch.cuda.empty_cache()
+        also["batch_layer_16"] = bench_batch_layer(torch, attn, orc, max(K // 10, 5), 4)
         torch.cuda.empty_cache()
         line["also"] = also
 
