@@ -260,9 +260,9 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
     // do still holds its place for as long as the longest one of its window.  A batch has items of
     // very different depth: its launch is therefore exactly one window of workers, and each worker
     // derives its (item, split) from the live lengths in device memory: item i gets
-    // nsp_i = clamp(floor(tiles_i * (workers - items) / sum of tiles), 1, splits) consecutive
-    // workers (their sum cannot exceed `workers`; what the rounding leaves is handed out one by
-    // one), i.e. about equal work per worker.
+    // nsp_i = clamp(ceil(tiles_i / T), 1, splits) consecutive workers, T the smallest number of
+    // tiles per worker for which these add up to no more than `workers` (the launcher keeps
+    // items <= workers), i.e. no worker has more than T tiles.
     int kvh, split, item, nsp;
     if (a.workers > 0) {
         kvh = blockIdx.x / a.workers;
@@ -286,32 +286,48 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
             }
             tiles = (sm + kTileKeys - 1) / kTileKeys;
         }
-        int total = tiles;
+        // the smallest number T of tiles per worker for which the items' shares ceil(tiles / T)
+        // (at least one worker each, at most `splits`) fit the workers there are: no worker then has
+        // more than T tiles, whatever the mix of depths (shares proportional to the tiles and rounded
+        // down left some items with half as many workers again as they needed)
+        int tmax = tiles, total = tiles;
 #pragma unroll
-        for (int off = 32; off > 0; off >>= 1)
+        for (int off = 32; off > 0; off >>= 1) {
+            const int o = __shfl_xor(tmax, off);
+            tmax = o > tmax ? o : tmax;
             total += __shfl_xor(total, off);
-        total = total > 0 ? total : 1;
-        int share = 0;
-        if (lane < a.items) {
-            share = (int)((long long)tiles * (a.workers - a.items) / total);
-            share = share < 1 ? 1 : (share < a.splits ? share : a.splits);
         }
-        // the shares are rounded down: hand the workers left over to the items in turn, one each per
-        // pass, while they are below their cap
-        int used = share;
+        auto share_at = [&](int t) {
+            int sh = 0;
+            if (lane < a.items) {
+                // ceil(tiles / t) through a float quotient (tiles < 2^24: exact or one too many at a
+                // multiple, corrected below); every wave computes the same values
+                sh = (int)((float)tiles / (float)t);
+                sh += sh * t < tiles ? 1 : 0;
+                sh -= (sh - 1) * t >= tiles && sh > 0 ? 1 : 0;
+                sh = sh < 1 ? 1 : (sh < a.splits ? sh : a.splits);
+            }
+            return sh;
+        };
+        // T lies between total / workers and total / (workers - items) (each share is below
+        // tiles / T + 1), so the search is a few steps
+        const int spare = a.workers - a.items;
+        int lo = (total + a.workers - 1) / a.workers;
+        lo = lo < 1 ? 1 : lo;
+        int hi = spare > 0 ? (total + spare - 1) / spare : (tmax > 1 ? tmax : 1);
+        hi = hi < lo ? lo : hi;
+        while (lo < hi) { // uniform over the wave
+            const int mid = (lo + hi) >> 1;
+            int need = share_at(mid);
 #pragma unroll
-        for (int off = 32; off > 0; off >>= 1)
-            used += __shfl_xor(used, off);
-        int left = a.workers - used; // >= 0 by construction
-        for (int pass = 0; pass < 3 && left > 0; pass++) {
-            const bool want = lane < a.items && tiles > share * kWaves && share < a.splits;
-            const unsigned long long m = __ballot(want);
-            const int rank = __builtin_popcountll(m & ((1ull << lane) - 1ull));
-            if (want && rank < left)
-                share++;
-            const int given = __builtin_popcountll(m);
-            left -= given < left ? given : left;
+            for (int off = 32; off > 0; off >>= 1)
+                need += __shfl_xor(need, off);
+            if (need <= a.workers)
+                hi = mid;
+            else
+                lo = mid + 1;
         }
+        const int share = share_at(lo);
         int end = share; // inclusive prefix sum over lanes
 #pragma unroll
         for (int off = 1; off < 64; off <<= 1) {
