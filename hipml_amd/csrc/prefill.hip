@@ -708,32 +708,57 @@ __global__ void __launch_bounds__(256) chunk_combine_kernel(
             return;
         }
     }
-    float m = -INFINITY;
-    for (int s = 0; s < nsp; s++) {
-        const size_t row = ((size_t)s * qslots + tok) * n_head + head;
-        const float2 ml = *reinterpret_cast<const float2 *>(part_ml + row * 2);
-        if (ml.y > 0.0f)
-            m = fmaxf(m, ml.x);
-    }
     float4v num = {0, 0, 0, 0};
     float den = 0.0f;
-    for (int s = 0; s < nsp; s++) {
-        const size_t row = ((size_t)s * qslots + tok) * n_head + head;
-        const float2 ml = *reinterpret_cast<const float2 *>(part_ml + row * 2);
-        const float4v x = *reinterpret_cast<const float4v *>(part_acc + row * kHeadDim + d4);
-        const float w = ml.y > 0.0f ? __builtin_amdgcn_exp2f(ml.x - m) : 0.0f;
-        const float4v z = {0, 0, 0, 0};
-        num += ml.y > 0.0f ? x * w : z;
-        den = fmaf(ml.y > 0.0f ? ml.y : 0.0f, w, den);
+    const float4v z = {0, 0, 0, 0};
+    float4v gt = {0, 0, 0, 0};
+    if (gate)
+        gt = *reinterpret_cast<const float4v *>(gate + o);
+    if (nsp <= 4) {
+        // every slice's (max, sum) and accumulator row asked for before the first is used
+        float2 ml[4];
+        float4v x[4];
+#pragma unroll
+        for (int s = 0; s < 4; s++) {
+            const size_t row = ((size_t)(s < nsp ? s : 0) * qslots + tok) * n_head + head;
+            ml[s] = *reinterpret_cast<const float2 *>(part_ml + row * 2);
+            x[s] = *reinterpret_cast<const float4v *>(part_acc + row * kHeadDim + d4);
+        }
+        float m = -INFINITY;
+#pragma unroll
+        for (int s = 0; s < 4; s++)
+            if (s < nsp && ml[s].y > 0.0f)
+                m = fmaxf(m, ml[s].x);
+#pragma unroll
+        for (int s = 0; s < 4; s++) {
+            const bool on = s < nsp && ml[s].y > 0.0f;
+            const float w = on ? __builtin_amdgcn_exp2f(ml[s].x - m) : 0.0f;
+            num += on ? x[s] * w : z;
+            den = fmaf(on ? ml[s].y : 0.0f, w, den);
+        }
+    } else {
+        float m = -INFINITY;
+        for (int s = 0; s < nsp; s++) {
+            const size_t row = ((size_t)s * qslots + tok) * n_head + head;
+            const float2 ml = *reinterpret_cast<const float2 *>(part_ml + row * 2);
+            if (ml.y > 0.0f)
+                m = fmaxf(m, ml.x);
+        }
+        for (int s = 0; s < nsp; s++) {
+            const size_t row = ((size_t)s * qslots + tok) * n_head + head;
+            const float2 ml = *reinterpret_cast<const float2 *>(part_ml + row * 2);
+            const float4v x = *reinterpret_cast<const float4v *>(part_acc + row * kHeadDim + d4);
+            const float w = ml.y > 0.0f ? __builtin_amdgcn_exp2f(ml.x - m) : 0.0f;
+            num += ml.y > 0.0f ? x * w : z;
+            den = fmaf(ml.y > 0.0f ? ml.y : 0.0f, w, den);
+        }
     }
     const float inv = den > 0.0f ? 1.0f / den : 0.0f;
     float4v r = num * inv;
     if (!(den > 0.0f))
         r = (float4v){0, 0, 0, 0};
-    if (gate) {
-        const float4v gt = *reinterpret_cast<const float4v *>(gate + o);
+    if (gate)
         r = (float4v){gated(r[0], gt[0]), gated(r[1], gt[1]), gated(r[2], gt[2]), gated(r[3], gt[3])};
-    }
     if (out16)
         *reinterpret_cast<half4 *>(out16 + o) = __builtin_convertvector(r, half4);
     else
