@@ -445,41 +445,30 @@ __global__ void __launch_bounds__(256) front_kernel(
                       : k + ((size_t)row * n_kv + h) * kHeadDim;
     const float *w = is_q ? qw : kw;
 
-    float x[4];
+    // everything this wave will need from memory is asked for here: the row, the gate half, the norm
+    // weights and the rotation's cos/sin (the position does not depend on the data)
+    float x[4], wv[4], g[4];
 #pragma unroll
     for (int j = 0; j < 4; j++)
         x[j] = src[lane + 64 * j];
-    if (is_q) {
-        float *gd = gate + ((size_t)row * n_heads + h) * kHeadDim;
-#pragma unroll
-        for (int j = 0; j < 4; j++)
-            gd[lane + 64 * j] = src[kHeadDim + lane + 64 * j];
-    }
-    const float a0 = x[0] * x[0] + x[2] * x[2]; // off = 128
-    const float a1 = x[1] * x[1] + x[3] * x[3];
-    float sum = a0 + a1;                        // off = 64
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1)
-        sum += __shfl_xor(sum, off);
-    const float mean_sq = sum / (float)kHeadDim;
-    const float scale = 1.0f / sqrtf(mean_sq + eps);
 #pragma unroll
     for (int j = 0; j < 4; j++)
-        buf[wave][lane + 64 * j] = x[j] * scale * w[lane + 64 * j];
-    __builtin_amdgcn_wave_barrier();
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-
-    // element e = lane + 64 j: rotated with its partner when e < n_rot (the first half of the pairs
-    // takes x1 c - x2 s, the second x1 s + x2 c), passed through otherwise
+        wv[j] = w[lane + 64 * j];
+    if (is_q) {
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            g[j] = src[kHeadDim + lane + 64 * j];
+    }
     const int half = n_rot >> 1;
     const int sect = s0 + s1 + s2 + s3;
+    float cs[4], sn[4];
 #pragma unroll
     for (int j = 0; j < 4; j++) {
         const int e = lane + 64 * j;
-        float out = buf[wave][e];
+        cs[j] = 1.0f;
+        sn[j] = 0.0f;
         if (e < n_rot) {
-            const bool first = e < half;
-            const int c = first ? e : e - half;
+            const int c = e < half ? e : e - half;
             int p = pos ? pos[0] : ap.rowpos ? ap.rowpos[2 * row] : pos0 + row;
             if (pos && sect > 0) {
                 const int sc = c % sect;
@@ -492,11 +481,41 @@ __global__ void __launch_bounds__(256) front_kernel(
                 else
                     p = pos[3];
             }
-            float cs, sn;
-            rope_cs(tab, tab_rows, half, c, p, n_rot, theta, cs, sn);
+            rope_cs(tab, tab_rows, half, c, p, n_rot, theta, cs[j], sn[j]);
+        }
+    }
+    if (is_q) {
+        float *gd = gate + ((size_t)row * n_heads + h) * kHeadDim;
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            gd[lane + 64 * j] = g[j];
+    }
+    const float a0 = x[0] * x[0] + x[2] * x[2]; // off = 128
+    const float a1 = x[1] * x[1] + x[3] * x[3];
+    float sum = a0 + a1;                        // off = 64
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1)
+        sum += __shfl_xor(sum, off);
+    const float mean_sq = sum / (float)kHeadDim;
+    const float scale = 1.0f / sqrtf(mean_sq + eps);
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+        buf[wave][lane + 64 * j] = x[j] * scale * wv[j];
+    __builtin_amdgcn_wave_barrier();
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+
+    // element e = lane + 64 j: rotated with its partner when e < n_rot (the first half of the pairs
+    // takes x1 c - x2 s, the second x1 s + x2 c), passed through otherwise
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int e = lane + 64 * j;
+        float out = buf[wave][e];
+        if (e < n_rot) {
+            const bool first = e < half;
+            const int c = first ? e : e - half;
             const float x1 = buf[wave][c];
             const float x2 = buf[wave][c + half];
-            out = first ? x1 * cs - x2 * sn : x1 * sn + x2 * cs;
+            out = first ? x1 * cs[j] - x2 * sn[j] : x1 * sn[j] + x2 * cs[j];
         }
         dst[e] = out;
         x[j] = out;
