@@ -627,23 +627,48 @@ __global__ void __launch_bounds__(kPfThreads, 2) chunk_q8_kernel(const ChunkArgs
 
     // ---- epilogue --------------------------------------------------------------------------
     l_run += __shfl_xor(l_run, 32);
-    if (!tok_valid)
-        return;
     if (SPLIT && nsp > 1) {
-        const size_t row = ((size_t)split * a.qslots + tok) * a.n_head + head;
-        float *pa = a.part_acc + row * kHeadDim;
+        // Partials leave through LDS: a lane holds 16-byte pieces of its token's row, 32 rows apart in
+        // memory per store; turned round in this wave's corner of the (now unused) tile buffers, a
+        // store instruction covers two half rows of 512 contiguous bytes.  Two passes of 128 d.
+        lds_barrier(); // every wave has finished with the tiles (nsp is uniform over the workgroup)
+        constexpr int kPitch = 512 + 16;
+        uint8_t *mine = lds + wave * (kQTile * kPitch);
+        const int l32 = lane & 31, rsel = lane >> 5;
 #pragma unroll
-        for (int dt = 0; dt < 8; dt++)
+        for (int hf = 0; hf < 2; hf++) {
 #pragma unroll
-            for (int g = 0; g < 4; g++) {
-                const float4v x = {O[dt][g * 4], O[dt][g * 4 + 1], O[dt][g * 4 + 2], O[dt][g * 4 + 3]};
-                *reinterpret_cast<float4v *>(pa + dt * 32 + g * 8 + lh * 4) = x;
+            for (int dl = 0; dl < 4; dl++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const int dt = hf * 4 + dl;
+                    const float4v x = {O[dt][g * 4], O[dt][g * 4 + 1], O[dt][g * 4 + 2], O[dt][g * 4 + 3]};
+                    *reinterpret_cast<float4v *>(mine + ln * kPitch + (dl * 32 + g * 8 + lh * 4) * 4) = x;
+                }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // this wave's own writes
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int r2 = 0; r2 < 16; r2++) {
+                const int r = r2 * 2 + rsel; // token of the tile
+                const float4v x = *reinterpret_cast<const float4v *>(mine + r * kPitch + l32 * 16);
+                if (task_valid && t0 + r < a.tokens) {
+                    const size_t prow = ((size_t)split * a.qslots + (t0 + r)) * a.n_head + head;
+                    *reinterpret_cast<float4v *>(a.part_acc + prow * kHeadDim + hf * 128 + l32 * 4) = x;
+                }
             }
-        if (lh == 0) {
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // reads done before the next pass overwrites
+            __builtin_amdgcn_wave_barrier();
+        }
+        if (tok_valid && lh == 0) {
+            const size_t row = ((size_t)split * a.qslots + tok) * a.n_head + head;
             a.part_ml[row * 2] = m_run;
             a.part_ml[row * 2 + 1] = l_run;
         }
-    } else {
+        return;
+    }
+    if (!tok_valid)
+        return;
+    {
         const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
         const size_t orow = ((size_t)tok * a.n_head + head) * kHeadDim;
         float *po = a.out + orow;
