@@ -289,58 +289,161 @@ int launch_rope_chunk(hipStream_t st, float *q, float *k, int n_head, int n_kv, 
     return 0;
 }
 
-// RoPE of a chunk and the append of its K/V rows in one launch: the first `q_blocks` workgroups
-// rotate 8 query head rows each (as rope_chunk_kernel does), the others take one (token, kv head)
-// each: thread t holds value t of the K row, pair partners (t, t + 32 for t < 32) meet through a
-// lane exchange inside wave 0, the rotated row is written back and quantized together with the V
-// row (as kv_encode_*_kernel does).  Same expressions, same bits as the two separate launches.
+// A block of 32 values held four per lane by 8 neighbouring lanes (value 4 l8 + j in component j):
+// the same quantizers as above (the maximum is exact whatever the order it is taken in; the q4_0
+// winner is the first of the largest, by index), with 16-bit stores of the packed bytes.
+typedef float float4e __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ void q8_encode_store4(const float4e x, uint8_t *dst_block, int l8)
+{
+    float m = fmaxf(fmaxf(fabsf(x[0]), fabsf(x[1])), fmaxf(fabsf(x[2]), fabsf(x[3])));
+#pragma unroll
+    for (int bit = 4; bit > 0; bit >>= 1)
+        m = fmaxf(m, __shfl_xor(m, bit));
+    const float d = m / 127.0f;
+    const float id = d > 0.0f ? 1.0f / d : 0.0f;
+    uint32_t pk = 0;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const float t = roundf(x[j] * id);
+        const float c = fminf(127.0f, fmaxf(-127.0f, t));
+        const int q = (t != t) ? 0 : (int)c;
+        pk |= (uint32_t)(uint8_t)(int8_t)q << (8 * j);
+    }
+    if (l8 == 0)
+        *reinterpret_cast<__half *>(dst_block) = __float2half_rn(d);
+    uint16_t *p16 = reinterpret_cast<uint16_t *>(dst_block + 2 + 4 * l8);
+    p16[0] = (uint16_t)pk;
+    p16[1] = (uint16_t)(pk >> 16);
+}
+
+__device__ __forceinline__ void q4_encode_store4(const float4e x, uint8_t *dst_block, int l8)
+{
+    // the value of largest magnitude, the first one on a tie; NaN never wins
+    float mag = -2.0f, val = 0.0f;
+    int idx = 0;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        float mj = fabsf(x[j]);
+        if (!(mj == mj))
+            mj = -1.0f;
+        if (mj > mag) {
+            mag = mj;
+            val = x[j];
+            idx = 4 * l8 + j;
+        }
+    }
+#pragma unroll
+    for (int bit = 4; bit > 0; bit >>= 1) {
+        const float om = __shfl_xor(mag, bit);
+        const float ov = __shfl_xor(val, bit);
+        const int oi = __shfl_xor(idx, bit);
+        const bool take = om > mag || (om == mag && oi < idx);
+        mag = take ? om : mag;
+        val = take ? ov : val;
+        idx = take ? oi : idx;
+    }
+    const float vmax = mag > 0.0f ? val : 0.0f;
+    const float d = -vmax / 8.0f;
+    const float id = d != 0.0f ? 1.0f / d : 0.0f;
+    uint32_t pk = 0;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const float t = roundf(x[j] * id) + 8.0f;
+        const float c = fminf(15.0f, fmaxf(0.0f, t));
+        const int q = (t != t) ? 0 : (int)c;
+        const int hi = __shfl_xor(q, 4); // value 16 further on: four lanes up, same component
+        pk |= (uint32_t)(q | (hi << 4)) << (8 * j);
+    }
+    if (l8 == 0)
+        *reinterpret_cast<__half *>(dst_block) = __float2half_rn(d);
+    if (l8 < 4) {
+        uint16_t *p16 = reinterpret_cast<uint16_t *>(dst_block + 2 + 4 * l8);
+        p16[0] = (uint16_t)pk;
+        p16[1] = (uint16_t)(pk >> 16);
+    }
+}
+
+// RoPE of a chunk and the append of its K/V rows in one launch, four values per lane so that the whole
+// chunk is one round of workgroups (with a value per lane the launch was two and a half rounds, each a
+// memory round trip long).  The first `q_blocks` workgroups rotate 32 query head rows each: 8 lanes
+// per row, lane l8 holds x1 = row[4 l8 ..] and x2 = row[32 + 4 l8 ..] of the 32 pairs.  The others
+// take four (token, kv head) units each, one wave per unit: lane l holds values 4 l .. 4 l + 3 of the
+// K row and of the V row; the pair partners of the rotated channels (lanes 0-7 and 8-15) meet through
+// a lane exchange; the rotated row is written back and both rows are quantized, a block of 32 values
+// being 8 neighbouring lanes.  The expressions of rope_chunk_kernel and of the append kernels, so the
+// same bits as the two separate launches.  head_dim 256, n_rot 64 (checked by the caller).
+constexpr int kRecRowsPerBlock = 32; // query rows per workgroup
+constexpr int kRecUnitsPerBlock = 4; // (token, kv head) units per workgroup
 template <bool Q4>
 __global__ void __launch_bounds__(256) rope_encode_chunk_kernel(
     float *__restrict__ q, float *__restrict__ kx, const float *__restrict__ vx, uint8_t *__restrict__ kc,
     uint8_t *__restrict__ vc, int n_head, int n_kv, int n_rot, float theta, int pos0, int tokens,
     int stride, int q_blocks, const float *__restrict__ tab, int tab_rows)
 {
-    const int half = n_rot >> 1;
+    const int half = n_rot >> 1; // 32
+    // cos/sin of pairs 4 g .. 4 g + 3 at position p
+    auto cos_sin = [&](int g, int p, float (&cs)[4], float (&sn)[4]) {
+        if (tab != nullptr && p >= 0 && p < tab_rows) {
+            const float4e *e = reinterpret_cast<const float4e *>(tab + ((size_t)p * half + 4 * g) * 2);
+            const float4e c0 = e[0], c1 = e[1];
+            cs[0] = c0[0], sn[0] = c0[1], cs[1] = c0[2], sn[1] = c0[3];
+            cs[2] = c1[0], sn[2] = c1[1], cs[3] = c1[2], sn[3] = c1[3];
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                rope_cs(tab, tab_rows, half, 4 * g + j, p, n_rot, theta, cs[j], sn[j]);
+        }
+    };
     if ((int)blockIdx.x < q_blocks) {
-        const long long r = (long long)blockIdx.x * 8 + (threadIdx.x >> 5);
+        const long long r = (long long)blockIdx.x * kRecRowsPerBlock + (threadIdx.x >> 3);
         if (r >= (long long)tokens * n_head)
             return;
+        const int l8 = threadIdx.x & 7;
         const int t = (int)(r / n_head);
         float *row = q + (size_t)r * kHeadDim;
-        for (int k = threadIdx.x & 31; k < half; k += 32) {
-            float cs, sn;
-            rope_cs(tab, tab_rows, half, k, pos0 + t, n_rot, theta, cs, sn);
-            const float x1 = row[k];
-            const float x2 = row[half + k];
-            row[k] = x1 * cs - x2 * sn;
-            row[half + k] = x1 * sn + x2 * cs;
+        const float4e x1 = *reinterpret_cast<const float4e *>(row + 4 * l8);
+        const float4e x2 = *reinterpret_cast<const float4e *>(row + half + 4 * l8);
+        float cs[4], sn[4];
+        cos_sin(l8, pos0 + t, cs, sn);
+        float4e y1, y2;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            y1[j] = x1[j] * cs[j] - x2[j] * sn[j];
+            y2[j] = x1[j] * sn[j] + x2[j] * cs[j];
         }
+        *reinterpret_cast<float4e *>(row + 4 * l8) = y1;
+        *reinterpret_cast<float4e *>(row + half + 4 * l8) = y2;
         return;
     }
-    const int u = (int)blockIdx.x - q_blocks; // (token, kv head)
+    const int u = ((int)blockIdx.x - q_blocks) * kRecUnitsPerBlock + (threadIdx.x >> 6); // (token, kv head)
+    if (u >= tokens * n_kv)
+        return; // a whole wave: nothing below crosses waves
     const int tok = u / n_kv, h = u - tok * n_kv;
-    const int t = threadIdx.x;
-    const size_t src = (size_t)u * kHeadDim + t;
-    float xk = kx[src];
-    const float xv = vx[src];
-    if (t < 64) { // wave 0: the rotated channels are 0 .. n_rot-1 <= 64
-        const float other = __shfl_xor(xk, half); // half is 32 here (checked by the launcher)
-        if (t < n_rot) {
-            const int k = t < half ? t : t - half;
-            float cs, sn;
-            rope_cs(tab, tab_rows, half, k, pos0 + tok, n_rot, theta, cs, sn);
-            xk = t < half ? xk * cs - other * sn : other * sn + xk * cs;
-            kx[src] = xk;
-        }
+    const int lane = threadIdx.x & 63, l8 = lane & 7;
+    float *krow = kx + (size_t)u * kHeadDim;
+    float4e xk = *reinterpret_cast<const float4e *>(krow + 4 * lane);
+    const float4e xv = *reinterpret_cast<const float4e *>(vx + (size_t)u * kHeadDim + 4 * lane);
+    float cs[4] = {1, 1, 1, 1}, sn[4] = {0, 0, 0, 0};
+    if (lane < 16)
+        cos_sin(l8, pos0 + tok, cs, sn);
+    float4e other;
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+        other[j] = __shfl_xor(xk[j], 8); // lanes 0-7 hold x1 of the pairs, lanes 8-15 their x2
+    if (lane < 16) {
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            xk[j] = lane < 8 ? xk[j] * cs[j] - other[j] * sn[j] : other[j] * sn[j] + xk[j] * cs[j];
+        *reinterpret_cast<float4e *>(krow + 4 * lane) = xk;
     }
-    const int chunk = t >> 5, lane32 = t & 31;
-    const size_t blk = ((size_t)h * stride + (pos0 + tok)) * (kHeadDim / 32) + chunk;
+    const size_t blk = ((size_t)h * stride + (pos0 + tok)) * (kHeadDim / 32) + (lane >> 3);
     if (Q4) {
-        q4_encode_store(xk, kc + blk * kQ4BlockBytes, lane32);
-        q4_encode_store(xv, vc + blk * kQ4BlockBytes, lane32);
+        q4_encode_store4(xk, kc + blk * kQ4BlockBytes, l8);
+        q4_encode_store4(xv, vc + blk * kQ4BlockBytes, l8);
     } else {
-        q8_encode_store(xk, kc + blk * kQ8BlockBytes, lane32);
-        q8_encode_store(xv, vc + blk * kQ8BlockBytes, lane32);
+        q8_encode_store4(xk, kc + blk * kQ8BlockBytes, l8);
+        q8_encode_store4(xv, vc + blk * kQ8BlockBytes, l8);
     }
 }
 
@@ -353,8 +456,8 @@ int launch_rope_encode_chunk(hipStream_t st, int q4, float *q, float *k, const f
     const int slab = 1 << 18; // tokens per launch: keeps the grid inside 2^31 workgroups
     for (int t0 = 0; t0 < tokens; t0 += slab) {
         const int n = tokens - t0 < slab ? tokens - t0 : slab;
-        const int q_blocks = (int)(((long long)n * n_head + 7) / 8);
-        const dim3 grid((unsigned)(q_blocks + n * n_kv), 1, 1);
+        const int q_blocks = (int)(((long long)n * n_head + kRecRowsPerBlock - 1) / kRecRowsPerBlock);
+        const dim3 grid((unsigned)(q_blocks + (n * n_kv + kRecUnitsPerBlock - 1) / kRecUnitsPerBlock), 1, 1);
         float *qq = q + (size_t)t0 * n_head * kHeadDim;
         float *kk = k + (size_t)t0 * n_kv * kHeadDim;
         const float *vv = v + (size_t)t0 * n_kv * kHeadDim;
