@@ -349,11 +349,16 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
         item = blockIdx.y;
         nsp = a.splits;
     }
-    const int slot = a.kvslot[item];
-    const int row0 = a.row0[item];
-    const int ncols = a.cols[item];
-    const int group = a.nhead[item]; // heads of this item: columns are (row, head) pairs over them
-    const int hbase = kvh * a.group + a.head0[item];
+    // The item tables are byte arrays read with vector loads, and the item is the same for every lane.
+    // Taking the values through readfirstlane puts them in scalar registers and, more to the point,
+    // makes the wave wait for them here, while nothing else is outstanding: the (conditional) Q loads
+    // below come later in the same in-order queue, so a first use behind them would wait for the Q
+    // rows as well, and the first tile could only be requested once those had arrived.
+    const int slot = __builtin_amdgcn_readfirstlane((int)a.kvslot[item]);
+    const int row0 = __builtin_amdgcn_readfirstlane((int)a.row0[item]);
+    const int ncols = __builtin_amdgcn_readfirstlane((int)a.cols[item]);
+    const int group = __builtin_amdgcn_readfirstlane((int)a.nhead[item]); // heads of this item: columns are (row, head) pairs over them
+    const int hbase = kvh * a.group + __builtin_amdgcn_readfirstlane((int)a.head0[item]);
     const int nvalid = ncols * group;
     if (a.workers > 0 && split == 0 && nsp < a.splits) {
         // the splits of this item that no worker takes: empty partials, which the merge skips
@@ -533,6 +538,11 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
         // ---- K tile to LDS, refill the registers ------------------------------------------
         store_unit(Ku[0], tile_lds, sK, ur0, upr, key0 + ur0 < hi);
         store_unit(Ku[1], tile_lds, sK, ur1, upr, key0 + ur1 < hi);
+        // (the refill sits under a branch, so the compiler cannot count the loads in flight and the
+        // next use of an older load waits for all of them; issuing it unconditionally, with idle
+        // addresses for a wave that has no further tile, gives exact waits and measured no faster:
+        // 24.9 against 25.1 us at depth 32,768, 59.0 against 58.1 at 131,072, 80.5 against 78.7 on
+        // the 16-slot batch)
         if (more)
             issue(Ku, kbase, t + DEPTH);
 
@@ -911,6 +921,100 @@ __global__ void __launch_bounds__(256) decode_reduce_kernel(
     }
 }
 
+// The same merge for at most 128 splits, with one barrier instead of three: every wave reads all
+// (m, l) pairs of the (row, head) itself (lane j: splits 2j and 2j+1), so the maximum and the
+// denominator are wave reductions without LDS, a thread takes the weights of its splits
+// (sg + SG k) from the lanes that hold them, and the split groups of a wave meet through row
+// rotations and the row-swap instructions; only the four waves' sums cross LDS.  Measured against
+// the kernel above: 3.3 against 5.2 us for one row of 128 splits.
+// grid (n_heads * 64 / (4 DL), rows), thread = (split group sg, float4 dl of d), as above.
+#ifndef DECODE_REDUCE128_ROWS
+#define DECODE_REDUCE128_ROWS 1
+#endif
+// KN = splits per thread the launch needs (SG KN >= splits): the loops carry no run-time bounds.
+template <int DL, int KN>
+__global__ void __launch_bounds__(256) decode_reduce128_kernel(
+    const float *__restrict__ part_acc, const float *__restrict__ part_ml, float *__restrict__ out,
+    const float *__restrict__ gate, int splits, size_t acc_slot, size_t ml_slot, size_t q_slot)
+{
+    static_assert(DL == 4 || DL == 16, "split groups of a wave are reduced for 4 or 16 lanes of d");
+    constexpr int SG = 256 / DL;   // split groups
+    static_assert(KN >= 1 && SG * KN <= 128, "lane j of a wave holds the weights of splits 2j and 2j+1");
+    constexpr int DQ = 64 / DL;    // workgroups per head
+    __shared__ float4v accs[4][DL];
+    const int head = blockIdx.x / DQ;
+    const int dq = blockIdx.x - head * DQ;
+    const int row = blockIdx.y;
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63;
+    const int sg = tid / DL, dl = tid % DL;
+    const float *ml = part_ml + (size_t)row * ml_slot + (size_t)head * splits * 2;
+    const float *acc = part_acc + (size_t)row * acc_slot + (size_t)head * splits * kHeadDim +
+                       dq * (DL * 4) + dl * 4;
+    const float4v z = {0, 0, 0, 0};
+
+    // the thread's accumulator rows first, then the wave's copy of the (m, l) table
+    float4v x[KN];
+#pragma unroll
+    for (int k = 0; k < KN; k++) {
+        // a split past the end repeats the last one (same cache line); its weight below is zero
+        const int s = sg + SG * k < splits ? sg + SG * k : splits - 1;
+        x[k] = *reinterpret_cast<const float4v *>(acc + (size_t)s * kHeadDim);
+    }
+    float2 v0 = {0.0f, 0.0f}, v1 = {0.0f, 0.0f};
+    if (2 * lane < splits)
+        v0 = *reinterpret_cast<const float2 *>(ml + 4 * lane);
+    if (2 * lane + 1 < splits)
+        v1 = *reinterpret_cast<const float2 *>(ml + 4 * lane + 2);
+    const size_t out_at = (size_t)row * q_slot + (size_t)head * kHeadDim + dq * (DL * 4) + (tid % DL) * 4;
+    float4v gt = z;
+    if (gate != nullptr && tid < DL)
+        gt = *reinterpret_cast<const float4v *>(gate + out_at);
+
+    // weights: 2^(m_s - m) for splits that saw a key, else 0 (`l > 0` is false for NaN as well)
+    const bool live0 = v0.y > 0.0f, live1 = v1.y > 0.0f;
+    float m = fmaxf(live0 ? v0.x : -INFINITY, live1 ? v1.x : -INFINITY);
+    m = wave_reduce<true>(m);
+    const float w0 = live0 ? __builtin_amdgcn_exp2f(v0.x - m) : 0.0f;
+    const float w1 = live1 ? __builtin_amdgcn_exp2f(v1.x - m) : 0.0f;
+    float den = fmaf(live1 ? v1.y : 0.0f, w1, (live0 ? v0.y : 0.0f) * w0);
+    den = wave_reduce<false>(den);
+    // split s lives in lane s / 2, component s % 2 (SG is even: the component is that of sg)
+    float4v num = z;
+#pragma unroll
+    for (int k = 0; k < KN; k++) {
+        const int holder = ((sg >> 1) + (SG / 2) * k) * 4;
+        const float c0 = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(holder, __builtin_bit_cast(int, w0)));
+        const float c1 = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(holder, __builtin_bit_cast(int, w1)));
+        const float w = (sg & 1) ? c1 : c0;
+        // zero-weight slices may hold anything (even NaN from an untouched scratch): select, not multiply
+        num += w > 0.0f ? x[k] * w : z;
+    }
+    // the split groups of the wave: lanes that differ in the bits above those of dl
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        float v = num[j];
+        if (DL == 4) {
+            v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x124, 0xf, 0xf, true)); // row_ror:4
+            v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x128, 0xf, 0xf, true)); // row_ror:8
+        }
+        num[j] = quad_rows<false>(v);
+    }
+    if (lane < DL)
+        accs[wave][lane] = num;
+    __syncthreads();
+    if (tid < DL) {
+        const float4v t = (accs[0][tid] + accs[1][tid]) + (accs[2][tid] + accs[3][tid]);
+        const float inv = den > 0.0f ? 1.0f / den : 0.0f;
+        float4v r = t * inv;
+        if (!(den > 0.0f))
+            r = z;
+        if (gate != nullptr)
+            r = (float4v){gated(r[0], gt[0]), gated(r[1], gt[1]), gated(r[2], gt[2]), gated(r[3], gt[3])};
+        *reinterpret_cast<float4v *>(out + out_at) = r;
+    }
+}
+
 #ifdef DBG_TIMING
 extern "C" int hipml_dbg_read_stamps(unsigned long long *host, size_t n)
 {
@@ -983,10 +1087,33 @@ int launch_decode_q8(hipStream_t st, const DecodeLaunch &L)
     int rc = launched(L.q4 ? "attn_decode_kv_q4" : "attn_decode_kv_q8");
     if (rc)
         return rc;
-    // One row and many splits: 16 d per workgroup (four times the workgroups, a thread's partial rows
-    // all requested at once) is 0.6 us faster at 128 splits and 0.5 us slower at 64 (measured at
-    // depths 32,768 / 131,072 and 8,192).
-    if (L.total_rows == 1 && L.splits >= 128)
+    // Up to 128 splits (every launch the split policies make): the one-barrier merge.  One row: 16 d
+    // per workgroup (four times the workgroups, 64-byte pieces of a partial row per thread group);
+    // several rows: 64 d per workgroup.
+    if (L.splits <= 128 && (L.total_rows == 1 || DECODE_REDUCE128_ROWS == 2)) {
+        const dim3 grid((unsigned)L.n_heads * 16, (unsigned)L.total_rows, 1);
+        if (L.splits <= 64)
+            hipLaunchKernelGGL((decode_reduce128_kernel<4, 1>), grid, dim3(256, 1, 1), 0, st, L.part_acc, L.part_ml,
+                               L.out, L.gate, L.splits, L.acc_slot, L.ml_slot, L.q_slot);
+        else
+            hipLaunchKernelGGL((decode_reduce128_kernel<4, 2>), grid, dim3(256, 1, 1), 0, st, L.part_acc, L.part_ml,
+                               L.out, L.gate, L.splits, L.acc_slot, L.ml_slot, L.q_slot);
+    } else if (L.splits <= 128 && DECODE_REDUCE128_ROWS) {
+        const dim3 grid((unsigned)L.n_heads * 4, (unsigned)L.total_rows, 1);
+        if (L.splits <= 16)
+            hipLaunchKernelGGL((decode_reduce128_kernel<16, 1>), grid, dim3(256, 1, 1), 0, st, L.part_acc, L.part_ml,
+                               L.out, L.gate, L.splits, L.acc_slot, L.ml_slot, L.q_slot);
+        else if (L.splits <= 32)
+            hipLaunchKernelGGL((decode_reduce128_kernel<16, 2>), grid, dim3(256, 1, 1), 0, st, L.part_acc, L.part_ml,
+                               L.out, L.gate, L.splits, L.acc_slot, L.ml_slot, L.q_slot);
+        else if (L.splits <= 64)
+            hipLaunchKernelGGL((decode_reduce128_kernel<16, 4>), grid, dim3(256, 1, 1), 0, st, L.part_acc, L.part_ml,
+                               L.out, L.gate, L.splits, L.acc_slot, L.ml_slot, L.q_slot);
+        else
+            hipLaunchKernelGGL((decode_reduce128_kernel<16, 8>), grid, dim3(256, 1, 1), 0, st, L.part_acc, L.part_ml,
+                               L.out, L.gate, L.splits, L.acc_slot, L.ml_slot, L.q_slot);
+    }
+    else if (L.total_rows == 1)
         hipLaunchKernelGGL(decode_reduce_kernel<4>, dim3((unsigned)L.n_heads * 16, 1, 1), dim3(256, 1, 1), 0,
                            st, L.part_acc, L.part_ml, L.out, L.gate, L.splits, L.acc_slot, L.ml_slot, L.q_slot);
     else
