@@ -104,6 +104,10 @@ struct DecodeArgs {
     const int32_t *pos;
     int n_kv, group, stride, splits;
     int items;     // work items (grid.y of a plain launch)
+    // item 0 once more, as plain scalars: a launch with a single item (one sequence, one query row)
+    // then needs no table lookup, which is a vector load from the kernel-argument segment and a
+    // memory round trip before the first Q and K/V requests can be addressed
+    int i0_row0, i0_cols, i0_slot, i0_head0, i0_nhead;
     int workers;   // > 0: worker launch, workgroups per KV head (see decode_body)
     float scale_log2; // scale * log2(e) * 2^24
     size_t kv_slot_bytes, acc_slot, ml_slot, q_slot;
@@ -264,7 +268,13 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
     // tiles per worker for which these add up to no more than `workers` (the launcher keeps
     // items <= workers), i.e. no worker has more than T tiles.
     int kvh, split, item, nsp;
-    if (a.workers > 0) {
+    // The scalar arguments span two 64-byte lines of the kernel-argument segment, both cold when a
+    // workgroup starts.  Left alone the compiler fetches `workers` (second line) here and the first
+    // line only where the pointers are first used: two memory round trips one after the other.  A
+    // condition over one field of each line asks for both at once (`stride` is positive, checked by
+    // the launcher).
+    const bool worker_launch = (a.workers > 0) & (a.stride > 0);
+    if (worker_launch) {
         kvh = blockIdx.x / a.workers;
         const int w = blockIdx.x - kvh * a.workers;
         // lane i looks at item i (the launcher uses this mode for at most 64 items); item tables
@@ -354,11 +364,21 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
     // makes the wave wait for them here, while nothing else is outstanding: the (conditional) Q loads
     // below come later in the same in-order queue, so a first use behind them would wait for the Q
     // rows as well, and the first tile could only be requested once those had arrived.
-    const int slot = __builtin_amdgcn_readfirstlane((int)a.kvslot[item]);
-    const int row0 = __builtin_amdgcn_readfirstlane((int)a.row0[item]);
-    const int ncols = __builtin_amdgcn_readfirstlane((int)a.cols[item]);
-    const int group = __builtin_amdgcn_readfirstlane((int)a.nhead[item]); // heads of this item: columns are (row, head) pairs over them
-    const int hbase = kvh * a.group + __builtin_amdgcn_readfirstlane((int)a.head0[item]);
+    int slot, row0, ncols, group, head0; // group = heads of this item: columns are (row, head) pairs over them
+    if (a.items == 1) {
+        slot = a.i0_slot;
+        row0 = a.i0_row0;
+        ncols = a.i0_cols;
+        group = a.i0_nhead;
+        head0 = a.i0_head0;
+    } else {
+        slot = __builtin_amdgcn_readfirstlane((int)a.kvslot[item]);
+        row0 = __builtin_amdgcn_readfirstlane((int)a.row0[item]);
+        ncols = __builtin_amdgcn_readfirstlane((int)a.cols[item]);
+        group = __builtin_amdgcn_readfirstlane((int)a.nhead[item]);
+        head0 = __builtin_amdgcn_readfirstlane((int)a.head0[item]);
+    }
+    const int hbase = kvh * a.group + head0;
     const int nvalid = ncols * group;
     if (a.workers > 0 && split == 0 && nsp < a.splits) {
         // the splits of this item that no worker takes: empty partials, which the merge skips
@@ -1074,6 +1094,11 @@ int launch_decode_q8(hipStream_t st, const DecodeLaunch &L)
         }
     }
     a.items = items;
+    a.i0_row0 = a.row0[0];
+    a.i0_cols = a.cols[0];
+    a.i0_slot = a.kvslot[0];
+    a.i0_head0 = a.head0[0];
+    a.i0_nhead = a.nhead[0];
     // batches: one window of workers (two workgroups per CU over 256 CUs), as long as every item can
     // have a worker of its own and lane i of a wave can look at item i
     const int window = 512 / L.n_kv;
