@@ -58,9 +58,12 @@ static int check_kv_dtype(int dtype)
 }
 
 // Decode launchers: the reference's selector also names kernel variants
-// (crates/hipml-kernels/src/launch_kv.rs:146-170,329-334): 0 and 4 are its staged and warp q8_0
-// kernels, 1 and 5 the q4_0 ones.  There is one kernel per format here, so the selector only
-// picks the format; its other values (A/B variants of the reference's kernels) are refused.
+// (crates/hipml-kernels/src/launch_kv.rs:146-170,329-334): 0 and 4 are its q8_0 kernels as shipped,
+// 1 and 5 the q4_0 ones, and 6 keeps its all-f32 staged q8_0 kernel reachable.  Here 0/4 run the
+// q8_0 kernel with f16-class weights, 6 its fp32-class variant (Q and the weights as hi + lo f16
+// pairs: the precision of the reference's f32 arithmetic), 1/5 the q4_0 kernel; the other values
+// (A/B variants of the reference's own kernels) are refused.
+// *kv_dtype: 0 = q8_0, 1 = q4_0, 2 = q8_0 fp32-class.
 static int decode_format(int dtype, int *kv_dtype)
 {
     if (dtype == 0 || dtype == 4) {
@@ -71,8 +74,12 @@ static int decode_format(int dtype, int *kv_dtype)
         *kv_dtype = 1;
         return 0;
     }
+    if (dtype == 6) {
+        *kv_dtype = 2;
+        return 0;
+    }
     return fail(HIPML_ATTN_E_UNSUPPORTED,
-                "KV dtype selector %d: 0/4 (q8_0) and 1/5 (q4_0) are built", dtype);
+                "KV dtype selector %d: 0/4 (q8_0), 6 (q8_0, fp32-class) and 1/5 (q4_0) are built", dtype);
 }
 
 // The MFMA kernels keep more LDS than a launch may use by default; hipml_attn_init raises the limit.
@@ -141,6 +148,7 @@ static int decode_common(hipStream_t st, int dtype, const int32_t *pos, const fl
     L.splits = splits;
     L.slots = slots;
     L.q4 = dtype == 1 ? 1 : 0;
+    L.exact = dtype == 2 ? 1 : 0;
     L.scale = scale;
     L.kv_slot_bytes = kv_slot_bytes;
     L.acc_slot = acc_slot;
@@ -200,12 +208,14 @@ const char *hipml_attn_version(void) { return "hipml-attn-mi355x 0.1 (gfx950)"; 
 
 int hipml_attn_decode_splits(int seq, int n_kv)
 {
-    // One workgroup of four waves walks 32-key tiles; give every workgroup at least one
-    // tile per wave (128 keys) and stop at two workgroups per CU (512) across the KV heads.
+    // One workgroup of four waves walks 32-key tiles; give every workgroup at least one tile per
+    // wave (128 keys) and stop at one workgroup per CU (256) across the KV heads: the merge then
+    // reads half the partials of two workgroups per CU, and the rows stream no slower (measured at
+    // depth 32,768: 19.2 us per layer with 64 splits, 20.4 with 128; at 131,072: 51.9 against 52.5).
     if (seq < 1 || n_kv < 1)
         return 1;
     int by_work = (seq + 127) / 128;
-    int by_cus = 512 / n_kv;
+    int by_cus = 256 / n_kv;
     if (by_cus < 1)
         by_cus = 1;
     int s = by_work < by_cus ? by_work : by_cus;

@@ -83,6 +83,7 @@ struct DecodeLaunch {
     const int32_t *pos; // (pos, seq) pairs, one per row
     int n_heads, n_kv, stride, splits, slots;
     int q4; // cache format: 0 = q8_0, 1 = q4_0
+    int exact; // q8_0 only: the fp32-class variant (Q and the weights as hi + lo f16 pairs)
     float scale;
     size_t kv_slot_bytes, acc_slot, ml_slot, q_slot;
     uint16_t row0[kMaxSlots]; // first row of each slot

@@ -37,6 +37,7 @@
 
 #include <stddef.h>
 #include <string.h>
+#include <type_traits>
 
 namespace hipml {
 
@@ -48,49 +49,18 @@ typedef int int2v __attribute__((ext_vector_type(2)));
 typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
 typedef uint32_t uint4a4 __attribute__((ext_vector_type(4), aligned(4)));
 
-constexpr int kMaxItems = 2 * kMaxSlots;               // work items of one launch (see DecodeArgs)
+constexpr int kMaxItems = 4 * kMaxSlots;               // work items of one launch (see DecodeArgs)
 constexpr int kTileKeys = 32;                         // keys per wave tile
 constexpr int kLdsRow = 288;                          // 256 payload bytes + 32 pad (bank spread)
 constexpr int kTileBytes = kTileKeys * kLdsRow;       // 9216: payload tile (K, then V)
 constexpr int kScaleBytes = 8 * kTileKeys * 2;        // 512: f16 [8 blocks][32 keys]
 constexpr int kWaveLds = kTileBytes + 2 * kScaleBytes; // 10240
-#ifndef DECODE_WAVES
-#define DECODE_WAVES 4
-#endif
-constexpr int kWaves = DECODE_WAVES;   // waves per workgroup
+constexpr int kWaves = 4;            // waves per workgroup
 constexpr int kThreads = 64 * kWaves;
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kTwo24 = 16777216.0f;
-
-#ifndef DECODE_MIN_WAVES
-#define DECODE_MIN_WAVES 2
-#endif
-#ifndef DECODE_DEPTH
-#define DECODE_DEPTH 1
-#endif
-// Optional scheduling fence after each block of the PV loop (off: measured no faster, no leaner).
-#ifdef DECODE_FENCE
-#define SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
-#else
-#define SCHED_FENCE() do { } while (0)
-#endif
-#ifndef DECODE_PLO
-#define DECODE_PLO 0
-#endif
-#ifndef DECODE_QLO
-#define DECODE_QLO 1
-#endif
 // Opaque use-and-redefine of a register: the value must exist here, in a VGPR.
 #define PIN(x) asm volatile("" : "+v"(x))
-constexpr int kDepth = DECODE_DEPTH; // tiles in flight per wave
-
-#ifdef DBG_TIMING
-// debug builds: per-workgroup phase timestamps (100 MHz wall clock), 8 slots per workgroup
-__device__ unsigned long long g_dbg_t[8 * 4096];
-#define STAMP(i) do { if (threadIdx.x == 0 && blockIdx.y == 0 && blockIdx.x < 4096) g_dbg_t[blockIdx.x * 8 + (i)] = wall_clock64(); } while (0)
-#else
-#define STAMP(i) do { } while (0)
-#endif
 
 constexpr int kQLds = 16384 + 2048; // per column tile: Q operands (hi, lo) + bias table
 constexpr int decode_lds_bytes(int nt) { return nt * kQLds + kWaves * kWaveLds; }
@@ -109,12 +79,13 @@ struct DecodeArgs {
     // memory round trip before the first Q and K/V requests can be addressed
     int i0_row0, i0_cols, i0_slot, i0_head0, i0_nhead;
     int workers;   // > 0: worker launch, workgroups per KV head (see decode_body)
+    int stream_once; // the launch has one work item: the cache rows are read once (non-temporal loads)
     float scale_log2; // scale * log2(e) * 2^24
     size_t kv_slot_bytes, acc_slot, ml_slot, q_slot;
-    // Work items (grid.y).  A slot whose rows x heads fit one 16-column MFMA tile is one item; a
-    // wider one (3-4 MTP rows x 6 heads) is cut by heads into items of at most 16 columns that
-    // stream the same cache rows: their workgroups are gridDim.x apart in launch order, a multiple
-    // of the 8 XCDs here, so the second reader finds the rows in the first one's L2.
+    // Work items (grid.y).  A slot whose rows x heads fit the columns of one workgroup (8 in the raw-row
+    // kernel, 16 in the staged one) is one item; a wider one (2-4 MTP rows x 6 heads) is cut by heads
+    // into items that stream the same cache rows: their workgroups are gridDim.x apart in launch
+    // order, a multiple of the 8 XCDs here, so the later readers find the rows in the first one's L2.
     uint16_t row0[kMaxItems];  // first query row of the item's slot
     uint8_t cols[kMaxItems];   // query rows of the slot (1..kMaxCols)
     uint8_t kvslot[kMaxItems]; // slot index, for the cache base
@@ -239,23 +210,16 @@ __device__ __forceinline__ float quad_rows(float v)
     return MAX ? fmaxf(a, b) : a + b;
 }
 
-template <int NT, int DEPTH, bool Q4>
-__device__ __forceinline__ void decode_body(const DecodeArgs &a)
-{
-    typedef typename UnitOf<Q4>::type Unit;
-    constexpr int kRowBytes = Q4 ? hipml::kRowBytesQ4 : hipml::kRowBytes;
-    constexpr int kUnitBytes = Q4 ? 36 : 68;
-    constexpr float kOffset = Q4 ? 8.0f : 128.0f; // what a staged byte carries on top of the value
-    extern __shared__ __attribute__((aligned(16))) uint8_t lds_all[];
-    uint8_t *Qs = lds_all;                       // [NT][hi,lo][8 blocks][64 lanes] half8
-    uint8_t *CBs = lds_all + NT * 16384;         // [NT][8 blocks][16 columns] float4 (one value x4)
-    uint8_t *wave_base = lds_all + NT * kQLds;   // per-wave tile + scale tables
+// The work of one workgroup: which KV head, work item and key split it serves.
+struct Work {
+    int kvh, split, nsp;                    // KV head, split index, splits of this item that have workers
+    int slot, row0, ncols, group, head0;    // the item: cache slot, first query row, rows, heads, first head
+    int hbase, nvalid;                      // first head overall, (row, head) columns of the item
+};
 
-    STAMP(0);
-    const int wave = threadIdx.x >> 6;
-    const int lane = threadIdx.x & 63;
-    const int lm = lane & 15; // MFMA row/col within the 16-tile
-    const int lg = lane >> 4; // k-group
+// Returns false when this workgroup has nothing to do (uniform over the workgroup).
+__device__ __forceinline__ bool find_work(const DecodeArgs &a, int lane, Work &wk)
+{
     // ---- which (kv head, item, split) this workgroup is ---------------------------------------
     // Plain launches: grid (n_kv * splits, items), every split of every item gets tiles.
     // Worker launches (batches, a.workers > 0): grid (n_kv * workers).  The hardware starts the
@@ -346,7 +310,7 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
         }
         const unsigned long long hit = __ballot(lane < a.items && w >= end - share && w < end);
         if (hit == 0)
-            return; // more workers than the shares add up to (uniform over the workgroup)
+            return false; // more workers than the shares add up to (uniform over the workgroup)
         item = __builtin_ctzll(hit);
         nsp = __shfl(share, item);
         split = w - (__shfl(end, item) - nsp);
@@ -383,7 +347,7 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
     if (a.workers > 0 && split == 0 && nsp < a.splits) {
         // the splits of this item that no worker takes: empty partials, which the merge skips
         const int empty = a.splits - nsp;
-        for (int e = threadIdx.x; e < nvalid * empty; e += kThreads) {
+        for (int e = threadIdx.x; e < nvalid * empty; e += (int)blockDim.x) {
             const int n = e / empty, sp = nsp + (e - n * empty);
             const int col = n / group;
             const int head = hbase + (n - col * group);
@@ -392,6 +356,41 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
             pm[1] = 0.0f;
         }
     }
+
+    wk.kvh = kvh;
+    wk.split = split;
+    wk.nsp = nsp;
+    wk.slot = slot;
+    wk.row0 = row0;
+    wk.ncols = ncols;
+    wk.group = group;
+    wk.head0 = head0;
+    wk.hbase = hbase;
+    wk.nvalid = nvalid;
+    return true;
+}
+
+template <int NT, bool Q4, bool PLO>
+__device__ __forceinline__ void decode_body(const DecodeArgs &a)
+{
+    typedef typename UnitOf<Q4>::type Unit;
+    constexpr int kRowBytes = Q4 ? hipml::kRowBytesQ4 : hipml::kRowBytes;
+    constexpr int kUnitBytes = Q4 ? 36 : 68;
+    constexpr float kOffset = Q4 ? 8.0f : 128.0f; // what a staged byte carries on top of the value
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds_all[];
+    uint8_t *Qs = lds_all;                       // [NT][hi,lo][8 blocks][64 lanes] half8
+    uint8_t *CBs = lds_all + NT * 16384;         // [NT][8 blocks][16 columns] float4 (one value x4)
+    uint8_t *wave_base = lds_all + NT * kQLds;   // per-wave tile + scale tables
+
+    const int wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const int lm = lane & 15; // MFMA row/col within the 16-tile
+    const int lg = lane >> 4; // k-group
+    Work wk;
+    if (!find_work(a, lane, wk))
+        return;
+    const int kvh = wk.kvh, split = wk.split, nsp = wk.nsp, slot = wk.slot, row0 = wk.row0, ncols = wk.ncols,
+              group = wk.group, hbase = wk.hbase, nvalid = wk.nvalid;
 
     uint8_t *tile_lds = wave_base + wave * kWaveLds;
     uint8_t *sK = tile_lds + kTileBytes;
@@ -409,8 +408,8 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
     // inside the cache's stride and is masked out), and neighbouring workgroups stream neighbouring rows.
     auto tile_key0 = [&](int t) { return ((t * nsp + split) * kWaves + wave) * kTileKeys; };
 
-    // ---- staging registers: DEPTH tiles in flight, each 2 K units + 2 V units per lane -------
-    Unit Kst[DEPTH][2], Vst[DEPTH][2];
+    // ---- staging registers: one tile in flight, 2 K units + 2 V units per lane -----------------
+    Unit Kst[2], Vst[2];
     // unit j of a tile: u = lane + 64*j -> tile row u/4, block pair u%4
     const int ur0 = lane >> 2, ur1 = 16 + (lane >> 2), upr = lane & 3;
     const int last_row = a.stride - 1;
@@ -446,9 +445,8 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
 
     // ... and right behind them the first tile: loads return in order, so the few Q rows are not
     // queued behind 17 KB of K/V, and the tile is on its way before the live length is known
-    issue(Kst[0], kbase, 0);
-    issue(Vst[0], vbase, 0);
-    STAMP(5); // first tile requested
+    issue(Kst, kbase, 0);
+    issue(Vst, vbase, 0);
 
     // live lengths of this slot's rows
     int seqc[kMaxCols];
@@ -461,7 +459,6 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
         seq_max = s > seq_max ? s : seq_max;
     }
     const int hi = seq_max; // keys at or past it are masked
-    STAMP(6); // live length known
     if (split * kWaves * kTileKeys >= hi) {
         // not one live tile for any wave of this workgroup (a shallow slot of a batch, or more
         // splits than tiles): leave an empty partial and go, the merge skips it
@@ -476,14 +473,7 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
     }
     const int first_key = tile_key0(0), step_keys = nsp * kWaves * kTileKeys;
     const int ntile = first_key < hi ? (hi - first_key + step_keys - 1) / step_keys : 0;
-#pragma unroll
-    for (int st = 1; st < DEPTH; st++)
-        if (ntile > st) {
-            issue(Kst[st], kbase, st);
-            issue(Vst[st], vbase, st);
-        }
 
-    STAMP(1); // ranges known, first K/V loads issued
     // ---- Q operands to LDS as hi + lo f16 ------------------------------------------------------
 #pragma unroll
     for (int k = 0; k < kQEntries; k++) {
@@ -500,7 +490,6 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
         *reinterpret_cast<half8 *>(Qs + (((nt * 2 + 0) * 8 + c) * 64 + l) * 16) = h8;
         *reinterpret_cast<half8 *>(Qs + (((nt * 2 + 1) * 8 + c) * 64 + l) * 16) = l8;
     }
-    STAMP(7); // Q values arrived and written to LDS
     __syncthreads();
     // Bias table: the K bytes enter the MFMA as (b + 128) * 2^-24, so every score of block c
     // carries +128 * 2^-24 * sum_k q[k][n]; its negative is the C operand the block's MFMA starts
@@ -520,7 +509,6 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
         *reinterpret_cast<float4v *>(CBs + ((nt * 8 + c) * 16 + n) * 16) = (float4v){cb, cb, cb, cb};
     }
     __syncthreads();
-    STAMP(2); // Q staged
 
     // per-column causal bound (MTP rows see one more key each)
     int seq_n[NT];
@@ -553,7 +541,7 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
 
     auto process = [&](Unit (&Ku)[2], Unit (&Vu)[2], int t) {
         const int key0 = tile_key0(t);
-        const bool more = t + DEPTH < ntile;
+        const bool more = t + 1 < ntile;
 
         // ---- K tile to LDS, refill the registers ------------------------------------------
         store_unit(Ku[0], tile_lds, sK, ur0, upr, key0 + ur0 < hi);
@@ -564,7 +552,7 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
         // 24.9 against 25.1 us at depth 32,768, 59.0 against 58.1 at 131,072, 80.5 against 78.7 on
         // the 16-slot batch)
         if (more)
-            issue(Ku, kbase, t + DEPTH);
+            issue(Ku, kbase, t + 1);
 
         // ---- scores ------------------------------------------------------------------------
         float S[NT][2][4];
@@ -575,7 +563,6 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
 #pragma unroll
                 for (int i = 0; i < 4; i++)
                     S[nt][ms][i] = 0.0f;
-#ifndef DBG_NO_QK
 #pragma unroll
         for (int c = 0; c < 8; c++) {
             half8 bh[NT], bl[NT];
@@ -596,8 +583,7 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
 #pragma unroll
                 for (int nt = 0; nt < NT; nt++) {
                     float4v part = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, bh[nt], cbias[nt], 0, 0, 0);
-                    if (DECODE_QLO)
-                        part = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, bl[nt], part, 0, 0, 0);
+                    part = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, bl[nt], part, 0, 0, 0);
 #pragma unroll
                     for (int i = 0; i < 4; i++)
                         S[nt][ms][i] = fmaf((float)sk[i], part[i], S[nt][ms][i]);
@@ -613,13 +599,12 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
                     for (int i = 0; i < 4; i++)
                         PIN(S[nt][ms][i]);
         }
-#endif
 
         // ---- V tile over the K tile, refill -----------------------------------------------
         store_unit(Vu[0], tile_lds, sV, ur0, upr, key0 + ur0 < hi);
         store_unit(Vu[1], tile_lds, sV, ur1, upr, key0 + ur1 < hi);
         if (more)
-            issue(Vu, vbase, t + DEPTH);
+            issue(Vu, vbase, t + 1);
 
         // ---- online softmax (log2 units), per column n = lane%16 -----------------------
         // The probabilities are rounded to f16 once, here; the running sum uses the rounded
@@ -651,7 +636,7 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
                     const float e = m_new == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(S[nt][ms][i] - m_new);
-                    if (DECODE_PLO) {
+                    if (PLO) {
                         p[nt][ms][i] = e;
                         ls += e;
                     } else {
@@ -672,7 +657,6 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
         }
 
         // ---- O^T += V^T . P' ---------------------------------------------------------------
-#ifndef DBG_NO_PV
 #pragma unroll
         for (int c = 0; c < 8; c++) {
             // rows past `hi` are duplicates of the last live row: finite scale, p = 0
@@ -681,11 +665,11 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
             for (int ms = 0; ms < 2; ms++)
                 sv[ms] = *reinterpret_cast<const half4 *>(sV + (c * kTileKeys + ms * 16 + lg * 4) * 2);
             // P' = p * block scale.  Default: one packed f16 multiply (f16-class weights);
-            // DECODE_PLO carries hi + lo f16 so the product keeps ~22 bits.
+            // PLO carries hi + lo f16 so the product keeps ~22 bits.
             half8 Ph[NT], Pl[NT];
 #pragma unroll
             for (int nt = 0; nt < NT; nt++) {
-                if (DECODE_PLO) {
+                if (PLO) {
 #pragma unroll
                     for (int ms = 0; ms < 2; ms++)
 #pragma unroll
@@ -711,26 +695,19 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
                     float4v o = O[nt][c * 2 + hf];
                     o = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, Ph[nt], o, 0, 0, 0);
                     o = __builtin_amdgcn_mfma_f32_16x16x32_f16(Abias, Ph[nt], o, 0, 0, 0);
-                    if (DECODE_PLO) {
+                    if (PLO) {
                         o = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, Pl[nt], o, 0, 0, 0);
                         o = __builtin_amdgcn_mfma_f32_16x16x32_f16(Abias, Pl[nt], o, 0, 0, 0);
                     }
                     O[nt][c * 2 + hf] = o;
                 }
             }
-            SCHED_FENCE();
         }
-#endif
     };
 
-    for (int t = 0; t < ntile; t += DEPTH) {
-#pragma unroll
-        for (int st = 0; st < DEPTH; st++)
-            if (t + st < ntile)
-                process(Kst[st], Vst[st], t + st);
-    }
+    for (int t = 0; t < ntile; t++)
+        process(Kst, Vst, t);
 
-    STAMP(3); // wave 0 finished its tiles
     // ---- merge the four waves and write the split's partial -------------------------------
     // O^T C layout: lane holds d = t*16 + lg*4 + i for column n = lane%16.  Rounds of 8 columns:
     // each wave parks 8 columns x 256 d (8 KiB) in its own tile area.
@@ -805,14 +782,538 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
             }
         }
     }
-    STAMP(4);
 }
 
-// One 16-column tile per workgroup (NT = 1): wider slots arrive as several work items.
-template <int DEPTH, bool Q4 = false>
-__global__ void __launch_bounds__(kThreads, DECODE_MIN_WAVES) decode_q8_kernel(const DecodeArgs a)
+// The register-staged kernel: one 16-column tile per workgroup (wider slots arrive as several work
+// items).  It serves q4_0 caches and, with PLO, the fp32-class variant of the q8_0 decode.
+template <bool Q4, bool PLO>
+__global__ void __launch_bounds__(kThreads, 2) decode_staged_kernel(const DecodeArgs a)
 {
-    decode_body<1, DEPTH, Q4>(a);
+    decode_body<1, Q4, PLO>(a);
+}
+
+// ---------------------------------------------------------------------------------------------
+// The q8_0 decode kernel.  Same work split, arithmetic and partial format as the staged kernel
+// above, but the cache rows travel from memory straight into LDS (global_load_lds_dwordx4) and are
+// used as they lie there, 272 bytes per key: no staging registers, no realignment, no LDS writes
+// by the wave, and a refill is one scalar-addressed instruction per KiB.
+//
+//   K operand   lane (key lm, k-group lg) needs the 8 payload bytes of block c at
+//               key*272 + 34c + 2 + 8 lg: two or three aligned dwords (raw_k_operand; the 272-byte
+//               pitch spreads the 16 keys of a read over all banks).
+//   V operand   ds_read_tr8_b64 wants 8-byte aligned addresses, and a block's payload starts
+//               2 (mod 4) bytes into the row.  The rows of O^T may come in any order, though, so
+//               the row is cut into its 17 aligned runs of 16 byte columns instead of 16 runs of
+//               16 values of d: run j is one A operand, its 16 columns are scale bytes (rows that
+//               are never read back) or values of d.  Six runs hold columns of two blocks, whose
+//               weights p * block scale differ: they are multiplied once with each block's
+//               weights, into two accumulators, and each column is taken from the one that
+//               belongs to it at the end.  23 accumulators instead of 16, no data movement.
+//   +128        the bytes enter as (b + 128) * 2^-24.  Scores: the MFMA of block c starts from
+//               -128 * 2^-24 * sum of the block's Q values (a 2 KiB table in LDS).  PV: what has to
+//               come off every row of block c is 128 * 2^-24 * sum_key P'_c[key][n], i.e. the row a
+//               constant A operand of 128 * 2^-24 would produce.  The two scale-byte columns of block
+//               c are such spare rows, and they sit in the first run of the block: their bytes are
+//               replaced by the constant on the way to the MFMA, the row accumulates the correction
+//               next to the data, and the merge subtracts column 34c from the block's columns.
+//               (Block 7 has no scale byte in its own runs: one extra MFMA per tile.)
+//   scales      a wave copies the 256 block scales of a tile into the transposed f16 table
+//               [8 blocks][32 keys] (4 ds_read_u16 + 1 ds_write_b64 per lane) before it uses them.
+//   Q           f16 B operands in registers (8 blocks x 4 registers); each wave fetches and converts
+//               two of the blocks and the four exchange them through LDS.
+//
+// Pipeline of a wave: K rows of tile t+1 are requested as soon as the scores of tile t are done, V
+// rows of tile t+1 after its PV product, so 8.7 to 17.4 KB per wave are in flight at any time.
+// The loads are written as asm: the compiler then neither knows nor waits for them, and the waits
+// are the explicit s_waitcnt below (loads return in order, 9 instructions per tile of rows).
+constexpr int kRawTile = kTileKeys * kRowBytes;              // 8704: 32 key rows as they lie in the cache
+constexpr int kDmaTileLds = 2 * kRawTile;                    // K rows and V rows of one tile
+constexpr int kDmaQLds = 8 * 64 * 16;                        // Q operands on their way to registers: [8 blocks][64 lanes] half8;
+                                                             // afterwards the waves' scale tables (2 x 512 bytes each)
+constexpr int kDmaBiasLds = 8 * 16 * 16;                     // score bias: [8 blocks][16 columns] float4
+// One tile of K and V rows per wave: 79,872 bytes, two workgroups per CU.  (A second tile per wave in
+// LDS, for launches of one workgroup per CU, measured slower: 21.3 against 19.2 us at depth 32,768,
+// as did a streaming probe with 16 instead of 8 KB in flight per wave.)
+constexpr int kDmaLds = kWaves * kDmaTileLds + kDmaQLds + kDmaBiasLds;
+constexpr int kRuns = kRowBytes / 16;                        // 17 runs of 16 byte columns
+constexpr int kAccs = 23;                                    // 3 per block 0..6, 2 for block 7
+
+
+__device__ __forceinline__ uint32_t lds_address(const void *p)
+{
+    return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void *)p;
+}
+
+// 64 lanes x 16 bytes from base + voff (per lane) to LDS address lds_at + 16 * lane.  ONCE: the
+// rows are read by this launch once, so the load is non-temporal (streaming 71 MB that way measured
+// 12.1 against 13.7 us per launch); rows that other work items of the launch read again are left
+// to the L2's ordinary policy.
+template <bool ONCE>
+__device__ __forceinline__ void dma16(uint32_t lds_at, const uint8_t *base, uint32_t voff)
+{
+    if (ONCE)
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt"
+                     :
+                     : "s"(lds_at), "v"(voff), "s"(base)
+                     : "memory");
+    else
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                     :
+                     : "s"(lds_at), "v"(voff), "s"(base)
+                     : "memory");
+}
+
+// A operand of a score MFMA from a raw key row: the 8 payload bytes [8 lg, 8 lg + 8) of block c as
+// f16 (b + 128) * 2^-24; `row_lg` = row + 8 lg.  LDS reads that are not aligned to their size run at a
+// fraction of the rate of aligned ones (measured: 35-64 against 2-3 cycles per ds_read_b64 over the
+// CU), so the bytes are taken from aligned dwords: two for an odd block (its payload starts at a dword),
+// three for an even one (payload 2 bytes into a dword; the byte selects of the conversion do the shift).
+__device__ __forceinline__ half8 raw_k_operand(const uint8_t *row_lg, int c)
+{
+    uint4v r;
+    if (c & 1) {
+        const uint32_t *p = reinterpret_cast<const uint32_t *>(row_lg + c * kQ8BlockBytes + 2);
+        const uint32_t x0 = p[0] ^ 0x80808080u, x1 = p[1] ^ 0x80808080u;
+        r[0] = __builtin_amdgcn_perm(0u, x0, 0x0c010c00u);
+        r[1] = __builtin_amdgcn_perm(0u, x0, 0x0c030c02u);
+        r[2] = __builtin_amdgcn_perm(0u, x1, 0x0c010c00u);
+        r[3] = __builtin_amdgcn_perm(0u, x1, 0x0c030c02u);
+    } else {
+        const uint32_t *p = reinterpret_cast<const uint32_t *>(row_lg + c * kQ8BlockBytes);
+        const uint32_t x0 = p[0] ^ 0x80808080u, x1 = p[1] ^ 0x80808080u, x2 = p[2] ^ 0x80808080u;
+        r[0] = __builtin_amdgcn_perm(0u, x0, 0x0c030c02u);
+        r[1] = __builtin_amdgcn_perm(0u, x1, 0x0c010c00u);
+        r[2] = __builtin_amdgcn_perm(0u, x1, 0x0c030c02u);
+        r[3] = __builtin_amdgcn_perm(0u, x2, 0x0c010c00u);
+    }
+    return __builtin_bit_cast(half8, r);
+}
+
+__device__ __forceinline__ void decode_body_dma(const DecodeArgs &a)
+{
+    static_assert(kWaves * 2 * kScaleBytes <= kDmaQLds, "the scale tables reuse the Q staging area");
+    constexpr int kDmaWaveLds = kDmaTileLds;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds_all[];
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int lane = threadIdx.x & 63;
+    const int lm = lane & 15; // MFMA row/col within the 16-tile
+    const int lg = lane >> 4; // k-group
+    Work wk;
+    if (!find_work(a, lane, wk))
+        return;
+    const int kvh = wk.kvh, split = wk.split, nsp = wk.nsp, slot = wk.slot, row0 = wk.row0, ncols = wk.ncols,
+              group = wk.group, hbase = wk.hbase, nvalid = wk.nvalid;
+
+    uint8_t *wave_lds = lds_all + wave * kDmaWaveLds;
+    uint8_t *Kraw = wave_lds;
+    uint8_t *Vraw = wave_lds + kRawTile;
+    uint8_t *Qst = lds_all + kWaves * kDmaWaveLds;
+    uint8_t *CBs = Qst + kDmaQLds;
+    uint8_t *sK = Qst + wave * 2 * kScaleBytes;
+    uint8_t *sV = sK + kScaleBytes;
+    const uint32_t wave_at = lds_address(wave_lds);
+
+    const uint8_t *kbase = a.k + (size_t)slot * a.kv_slot_bytes + (size_t)kvh * a.stride * kRowBytes;
+    const uint8_t *vbase = a.v + (size_t)slot * a.kv_slot_bytes + (size_t)kvh * a.stride * kRowBytes;
+
+    // tile g of a KV head belongs to split (g / kWaves) % nsp, wave g % kWaves (see the staged kernel)
+    auto tile_key0 = [&](int t) { return ((t * nsp + split) * kWaves + wave) * kTileKeys; };
+
+    // ---- one tile of rows = 8,704 contiguous bytes = 8.5 instructions of 1 KiB ------------------
+    const uint32_t lane16 = lane * 16;
+    const uint32_t region_last = (uint32_t)a.stride * kRowBytes - 16; // last 16 bytes of a KV head's rows
+    auto issue_as = [&](auto once, bool v_rows, int t) {
+        constexpr bool kOnce = decltype(once)::value;
+        const uint32_t lds_at = wave_at + (v_rows ? kRawTile : 0);
+        const uint8_t *region = v_rows ? vbase : kbase;
+        const int key0 = tile_key0(t);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // the wave's own reads of the old rows are done
+        if (key0 + kTileKeys <= a.stride) { // (uniform) the tile lies inside the cache
+            const uint8_t *src = region + (size_t)key0 * kRowBytes;
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+                dma16<kOnce>(lds_at + j * 1024, src + j * 1024, lane16);
+            if (lane < 32)
+                dma16<kOnce>(lds_at + 8192, src + 8192, lane16);
+        } else {
+            // the last rows of the cache: bytes past its end are replaced by its last 16 (rows at or
+            // past the live length are masked whatever they hold)
+            const uint32_t off0 = (uint32_t)key0 * kRowBytes + lane16;
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const uint32_t o = off0 + j * 1024;
+                dma16<kOnce>(lds_at + j * 1024, region, o < region_last ? o : region_last);
+            }
+            if (lane < 32) {
+                const uint32_t o = off0 + 8192;
+                dma16<kOnce>(lds_at + 8192, region, o < region_last ? o : region_last);
+            }
+        }
+    };
+    const bool once = a.stream_once != 0;
+    auto issue = [&](bool v_rows, int t) {
+        if (once)
+            issue_as(std::true_type(), v_rows, t);
+        else
+            issue_as(std::false_type(), v_rows, t);
+    };
+
+    // live lengths of this slot's rows: scalar loads, requested before the first asm statement (the
+    // compiler reads memory it must assume changed with vector loads, and would then wait for all loads)
+    int seqc[kMaxCols];
+    int seq_max = 0;
+#pragma unroll
+    for (int c = 0; c < kMaxCols; c++) {
+        int s = c < ncols ? a.pos[(size_t)(row0 + c) * 2 + 1] : 0;
+        s = s < 0 ? 0 : (s > a.stride ? a.stride : s);
+        seqc[c] = s;
+        seq_max = s > seq_max ? s : seq_max;
+    }
+
+    // ---- the first requests: K rows of tile 0 and the Q rows ------------------------------------
+    // Neither address needs anything from device memory (a tile past the live rows costs one load of
+    // rows inside the cache and is masked out).
+    issue(false, 0);
+    // The item has at most 8 (row, head) columns.  MFMA column lm < 8 carries the f16 value of Q column
+    // lm, MFMA column lm + 8 what that rounding left over (x - f16(x), again as f16): the two halves
+    // of a score are added after the block loop, so Q enters with ~22 bits at the price of one
+    // MFMA.  Wave w fetches two blocks of the Q rows: lane (column n = lm % 8, k-group lg) holds
+    // Q[n][c*32 + lg*8 .. +8]; the waves exchange them through LDS below.  (Every wave fetching all of
+    // it is 16 KB per wave through the CU's L1 in front of the first K/V rows: 1 us later first data.)
+    // These are ordinary loads: the compiler waits for them, and with them for the K rows requested
+    // before them, where the values are first used, which is where both are needed.
+    constexpr int kQB = 8 / kWaves; // Q blocks per wave
+    float4v qf[kQB][2];
+    const int qcol = lm & 7;
+    const bool have_q = qcol < nvalid;
+    {
+        const int col = have_q ? qcol / group : 0;
+        const int head = have_q ? qcol - col * group : 0; // (idle columns fetch column 0 and drop it)
+        const float *qp = a.q + (size_t)(row0 + col) * a.q_slot + (size_t)(hbase + head) * kHeadDim + lg * 8 +
+                          wave * (kQB * 32);
+#pragma unroll
+        for (int cc = 0; cc < kQB; cc++) {
+            qf[cc][0] = *reinterpret_cast<const float4v *>(qp + cc * 32);
+            qf[cc][1] = *reinterpret_cast<const float4v *>(qp + cc * 32 + 4);
+        }
+    }
+
+    const int hi = seq_max; // keys at or past it are masked
+    if (split * kWaves * kTileKeys >= hi) {
+        // not one live tile for any wave of this workgroup: leave an empty partial, which the merge skips
+        if ((int)threadIdx.x < nvalid) {
+            const int col = threadIdx.x / group;
+            const int head = hbase + (threadIdx.x - col * group);
+            float *pm = a.part_ml + (size_t)(row0 + col) * a.ml_slot + ((size_t)head * a.splits + split) * 2;
+            pm[0] = -INFINITY;
+            pm[1] = 0.0f;
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // nothing may land in LDS after the wave has gone
+        return; // uniform over the workgroup
+    }
+    const int first_key = tile_key0(0), step_keys = nsp * kWaves * kTileKeys;
+    const int ntile = first_key < hi ? (hi - first_key + step_keys - 1) / step_keys : 0;
+
+    // ---- Q operands and the score bias of every block ------------------------------------------
+#pragma unroll
+    for (int cc = 0; cc < kQB; cc++) {
+        const int c = kQB * wave + cc;
+        half8 h8;
+        float sum = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const float x = have_q ? (j < 4 ? qf[cc][0][j] : qf[cc][1][j - 4]) : 0.0f;
+            _Float16 h = (_Float16)x;
+            if (lm >= 8)
+                h = (_Float16)(x - (float)h);
+            h8[j] = h;
+            sum += (float)h;
+        }
+        sum = quad_rows<false>(sum); // over the four k-groups: the block's 32 values of MFMA column lm
+        const float cb = -128.0f / kTwo24 * sum;
+        *reinterpret_cast<half8 *>(Qst + (c * 64 + lane) * 16) = h8;
+        if (lg == 0)
+            *reinterpret_cast<float4v *>(CBs + (c * 16 + lm) * 16) = (float4v){cb, cb, cb, cb};
+    }
+    // the K rows are in LDS by now; the V rows of the first tile follow them
+    issue(true, 0);
+    __syncthreads();
+    half8 bh[8];
+#pragma unroll
+    for (int c = 0; c < 8; c++)
+        bh[c] = *reinterpret_cast<const half8 *>(Qst + (c * 64 + lane) * 16);
+    __syncthreads(); // the staging area becomes the waves' scale tables
+
+    // per-column causal bound (MTP rows see one more key each)
+    const int seq_n = qcol < nvalid ? seqc[qcol / group] : 0;
+
+    // ---- running state ----------------------------------------------------------------------
+    float m_run = -INFINITY, l_run = 0.0f;
+    float4v O[kAccs], B7 = {0, 0, 0, 0};
+#pragma unroll
+    for (int i = 0; i < kAccs; i++)
+        O[i] = (float4v){0, 0, 0, 0};
+
+    // V transpose-read address: lane (2r+e) of its 16-lane group supplies key slot r
+    // (slot r<4: key lg*4+r, slot r>=4: key 16+lg*4+(r-4)), bytes [8e, 8e+8) of a 16-column run.
+    const int tr_r = lm >> 1;
+    const int tr_key = (tr_r >> 2) * 16 + lg * 4 + (tr_r & 3);
+    const uint8_t *vtr = Vraw + tr_key * kRowBytes + (lm & 1) * 8;
+    const uint4v bias_bits = {0x00800080u, 0x00800080u, 0x00800080u, 0x00800080u};
+    const half8 Abias = __builtin_bit_cast(half8, bias_bits); // eight times 128 * 2^-24
+    const int lm2 = lm >> 1; // run 2c carries the scale bytes of block c in rows 2c and 2c+1
+
+    // the scales of a tile of raw rows -> f16 table [8 blocks][32 keys]; lane = (block, four keys)
+    const int sc_c = lane >> 3, sc_k = (lane & 7) * 4;
+    auto build_scales = [&](const uint8_t *raw, uint8_t *table, int key0, bool partial) {
+        const uint8_t *p = raw + sc_k * kRowBytes + sc_c * kQ8BlockBytes;
+        uint32_t s0 = *reinterpret_cast<const uint16_t *>(p);
+        uint32_t s1 = *reinterpret_cast<const uint16_t *>(p + kRowBytes);
+        uint32_t s2 = *reinterpret_cast<const uint16_t *>(p + 2 * kRowBytes);
+        uint32_t s3 = *reinterpret_cast<const uint16_t *>(p + 3 * kRowBytes);
+        if (partial) {
+            // a row at or past the live length holds whatever the cache holds there: zero scale, so
+            // that its zero weight cannot meet a non-finite value
+            const int k = key0 + sc_k;
+            s0 = k < hi ? s0 : 0u;
+            s1 = k + 1 < hi ? s1 : 0u;
+            s2 = k + 2 < hi ? s2 : 0u;
+            s3 = k + 3 < hi ? s3 : 0u;
+        }
+        int2v w;
+        w[0] = (int)(s0 | (s1 << 16));
+        w[1] = (int)(s2 | (s3 << 16));
+        *reinterpret_cast<int2v *>(table + (sc_c * kTileKeys + sc_k) * 2) = w;
+    };
+
+    for (int t = 0; t < ntile; t++) {
+        const int key0 = tile_key0(t);
+        const bool more = t + 1 < ntile;
+        const bool partial = key0 + kTileKeys > hi;
+        // Requests complete in the order of issue, 9 per tile of rows: K(0) V(0), then K(t + 1) after the
+        // scores of tile t and V(t + 1) after its PV.
+        // ---- K rows of this tile are in LDS once only the 9 loads of its V rows are outstanding
+        asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
+        build_scales(Kraw, sK, key0, partial);
+
+        // ---- scores ----------------------------------------------------------------------------
+        float S[2][4];
+#pragma unroll
+        for (int ms = 0; ms < 2; ms++)
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                S[ms][i] = 0.0f;
+#pragma unroll
+        for (int c = 0; c < 8; c++) {
+            const float4v cb4 = *reinterpret_cast<const float4v *>(CBs + (c * 16 + lm) * 16);
+#pragma unroll
+            for (int ms = 0; ms < 2; ms++) {
+                const half8 A = raw_k_operand(Kraw + (ms * 16 + lm) * kRowBytes + lg * 8, c);
+                const half4 sk = *reinterpret_cast<const half4 *>(sK + (c * kTileKeys + ms * 16 + lg * 4) * 2);
+                const float4v part = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, bh[c], cb4, 0, 0, 0);
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+                    S[ms][i] = fmaf((float)sk[i], part[i], S[ms][i]);
+            }
+        }
+        // the two halves of every score: MFMA columns n and n + 8 (a rotation by 8 inside the 16-lane row)
+#pragma unroll
+        for (int ms = 0; ms < 2; ms++)
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                S[ms][i] += __builtin_bit_cast(
+                    float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, S[ms][i]), 0x128, 0xf, 0xf, true));
+        // the K rows are used up: request those of the tile that takes their place
+        if (more)
+            issue(false, t + 1);
+
+        // ---- online softmax (log2 units), per column n = lane%16 -----------------------
+        // The probabilities are rounded to f16 once, here; the running sum uses the rounded
+        // values, so numerator and denominator see the same weights.
+        half4 ph[2];
+        float corr;
+        bool grew;
+        {
+            const int lim = hi < seq_n ? hi : seq_n;
+            float mt = -INFINITY;
+#pragma unroll
+            for (int ms = 0; ms < 2; ms++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int key = key0 + ms * 16 + lg * 4 + i;
+                    const float s = key < lim ? S[ms][i] * a.scale_log2 : -INFINITY;
+                    S[ms][i] = s;
+                    mt = fmaxf(mt, s);
+                }
+            mt = quad_rows<true>(mt);
+            // The reference value of the exponentials follows the maximum only when that has grown by
+            // more than 8 (log2 units): weights then stay below 2^8, far inside f16 and f32, and the
+            // 92 accumulator registers are rescaled on a few tiles instead of most.
+            grew = fmaxf(m_run, mt) > m_run + 8.0f;
+            const float m_new = grew ? mt : m_run;
+            corr = m_new == -INFINITY ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_new);
+            float ls = 0.0f;
+#pragma unroll
+            for (int ms = 0; ms < 2; ms++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const float e = m_new == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(S[ms][i] - m_new);
+                    const _Float16 eh = (_Float16)e;
+                    ph[ms][i] = eh;
+                    ls += (float)eh;
+                }
+            l_run = l_run * corr + ls;
+            m_run = m_new;
+        }
+        if (t > 0 && __any(grew)) { // (the accumulators of the first tile are still zero)
+#pragma unroll
+            for (int i = 0; i < kAccs; i++)
+                O[i] *= corr;
+            B7 *= corr;
+        }
+
+        // ---- V rows of this tile: all that may still be outstanding are the next tile's K rows
+        if (more)
+            asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
+        else
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        build_scales(Vraw, sV, key0, partial);
+
+        // ---- O^T += V^T . P' -------------------------------------------------------------------
+        half8 Aprev = Abias; // the run shared with the previous block
+#pragma unroll
+        for (int c = 0; c < 8; c++) {
+            half4 sv[2];
+#pragma unroll
+            for (int ms = 0; ms < 2; ms++)
+                sv[ms] = *reinterpret_cast<const half4 *>(sV + (c * kTileKeys + ms * 16 + lg * 4) * 2);
+            // P' = p * block scale, one packed f16 multiply (f16-class weights)
+            const half4 x0 = ph[0] * sv[0];
+            const half4 x1 = ph[1] * sv[1];
+            const half8 Ph = __builtin_shufflevector(x0, x1, 0, 1, 2, 3, 4, 5, 6, 7);
+            if (c == 7)
+                B7 = __builtin_amdgcn_mfma_f32_16x16x32_f16(Abias, Ph, B7, 0, 0, 0);
+            // the runs that hold columns of block c: 2c .. 2c+2 (15 and 16 for block 7)
+#pragma unroll
+            for (int r = 0; r < (c < 7 ? 3 : 2); r++) {
+                const int j = (c < 7 ? 2 * c : 15) + r;
+                half8 A;
+                if (r == 0 && c > 0 && c < 7) {
+                    A = Aprev;
+                } else {
+                    int2v raw = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+                        (int2v __attribute__((address_space(3))) *)(vtr + j * 16));
+                    if ((j & 1) == 0 && j <= 12) {
+                        // rows j and j+1 of this run are scale bytes: byte 0 enters as 128 * 2^-24
+                        raw[0] = lm2 == j / 2 ? 0 : raw[0];
+                        raw[1] = lm2 == j / 2 ? 0 : raw[1];
+                    }
+                    A = bytes_to_f16_biased<false>(raw);
+                }
+                O[c * 3 + r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, Ph, O[c * 3 + r], 0, 0, 0);
+                if (r == 2)
+                    Aprev = A;
+            }
+        }
+        // the V rows are used up
+        if (more)
+            issue(true, t + 1);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // (a wave without a tile still has its first K rows in flight)
+
+    // ---- merge the four waves and write the split's partial -------------------------------
+    // Run j of O^T: lane holds byte columns 16j + lg*4 + i of the key rows for column n = lane%16.
+    // Rounds of 8 columns n: each wave parks 8 x 272 values, indexed by byte column, in its K rows.
+    l_run = quad_rows<false>(l_run);
+    float *wl = reinterpret_cast<float *>(wave_lds); // per wave: [8][272] acc by byte column
+    float *wml = reinterpret_cast<float *>(sK);  // per wave: [8] m, [8] l
+#pragma unroll
+    for (int half = 0; half < 2; half++) {
+        const int nbase = half * 8;
+        if (nbase >= nvalid)
+            break; // uniform over the workgroup
+        __syncthreads(); // everyone is done with the tile buffers / previous round
+        if ((lm >> 3) == half) {
+            const int n8 = lm & 7;
+#pragma unroll
+            for (int j = 0; j < kRuns; j++) {
+                float4v v;
+                if (j >= 2 && j <= 12 && (j & 1) == 0) {
+                    // columns of blocks j/2 - 1 (below byte 34 * (j/2)) and j/2
+                    const int c1 = j / 2;
+                    const float4v lo = O[3 * c1 - 1];
+                    const float4v up = O[3 * c1];
+#pragma unroll
+                    for (int i = 0; i < 4; i++)
+                        v[i] = 16 * j + lg * 4 + i < kQ8BlockBytes * c1 ? lo[i] : up[i];
+                } else {
+                    const int idx = j == 0 ? 0 : (j >= 14 ? j + 6 : 3 * (j - 1) / 2 + 1);
+                    v = O[idx];
+                    if (j == 14) // byte column 238, the scale of block 7: its correction row
+                        v[2] = lg == 3 ? B7[2] : v[2];
+                }
+                *reinterpret_cast<float4v *>(wl + n8 * kRowBytes + j * 16 + lg * 4) = v;
+            }
+            if (lg == 0) {
+                wml[n8] = m_run;
+                wml[8 + n8] = l_run;
+            }
+        }
+        __syncthreads();
+        // thread -> (column n8, kRun consecutive d of one block): 8 columns x kThreads / 8 runs of d
+        constexpr int kDRuns = kThreads / 8, kRun = kHeadDim / kDRuns;
+        static_assert(kRun == 8 || kRun == 4, "a thread's values of d lie in one block");
+        const int n8 = threadIdx.x / kDRuns;
+        const int d0 = (threadIdx.x % kDRuns) * kRun;
+        const int col0 = d0 + 2 + 2 * (d0 >> 5); // byte column of d0: 34 bytes per 32 values, scale first
+        const int ng = nbase + n8;
+        if (ng < nvalid) {
+            float mw[kWaves], lw[kWaves];
+            float ms = -INFINITY;
+#pragma unroll
+            for (int w = 0; w < kWaves; w++) {
+                const float *o = reinterpret_cast<const float *>(Qst + w * 2 * kScaleBytes);
+                mw[w] = o[n8];
+                lw[w] = o[8 + n8];
+                ms = fmaxf(ms, mw[w]);
+            }
+            float lsum = 0.0f;
+            float wgt[kWaves];
+#pragma unroll
+            for (int w = 0; w < kWaves; w++) {
+                wgt[w] = mw[w] == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(mw[w] - ms);
+                lsum += lw[w] * wgt[w];
+                wgt[w] *= kTwo24;
+            }
+            const int col = ng / group;
+            const int head = hbase + (ng - col * group);
+            const size_t slice = (size_t)head * a.splits + split;
+            float *pa = a.part_acc + (size_t)(row0 + col) * a.acc_slot + slice * kHeadDim + d0;
+#pragma unroll
+            for (int dd = 0; dd < kRun; dd += 4) {
+                float4v acc = {0, 0, 0, 0};
+#pragma unroll
+                for (int w = 0; w < kWaves; w++) {
+                    const float *row = reinterpret_cast<const float *>(lds_all + w * kDmaWaveLds) + n8 * kRowBytes;
+                    const float off = row[(d0 >> 5) * kQ8BlockBytes]; // the block's correction row
+                    const float2 x0 = *reinterpret_cast<const float2 *>(row + col0 + dd);
+                    const float2 x1 = *reinterpret_cast<const float2 *>(row + col0 + dd + 2);
+                    acc += ((float4v){x0.x, x0.y, x1.x, x1.y} - off) * wgt[w];
+                }
+                *reinterpret_cast<float4v *>(pa + dd) = acc;
+            }
+            if (threadIdx.x % kDRuns == 0) {
+                float *pm = a.part_ml + (size_t)(row0 + col) * a.ml_slot + slice * 2;
+                pm[0] = ms;
+                pm[1] = lsum;
+            }
+        }
+    }
+}
+
+__global__ void __launch_bounds__(kThreads, 2) decode_q8_kernel(const DecodeArgs a)
+{
+    decode_body_dma(a);
 }
 
 // Wave-wide reductions without LDS: DPP inside a row of 16 lanes, then the two row-swap
@@ -948,9 +1449,6 @@ __global__ void __launch_bounds__(256) decode_reduce_kernel(
 // rotations and the row-swap instructions; only the four waves' sums cross LDS.  Measured against
 // the kernel above: 3.3 against 5.2 us for one row of 128 splits.
 // grid (n_heads * 64 / (4 DL), rows), thread = (split group sg, float4 dl of d), as above.
-#ifndef DECODE_REDUCE128_ROWS
-#define DECODE_REDUCE128_ROWS 1
-#endif
 // KN = splits per thread the launch needs (SG KN >= splits): the loops carry no run-time bounds.
 template <int DL, int KN>
 __global__ void __launch_bounds__(256) decode_reduce128_kernel(
@@ -1035,24 +1533,19 @@ __global__ void __launch_bounds__(256) decode_reduce128_kernel(
     }
 }
 
-#ifdef DBG_TIMING
-extern "C" int hipml_dbg_read_stamps(unsigned long long *host, size_t n)
-{
-    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_dbg_t), n * 8);
-}
-#endif
 
 int decode_init()
 {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&decode_q8_kernel<kDepth, false>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       decode_lds_bytes(1));
-    if (e == hipSuccess)
-        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&decode_q8_kernel<kDepth, true>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, decode_lds_bytes(1));
-    if (e != hipSuccess)
-        return fail((int)e, "hipFuncSetAttribute(decode LDS) failed: %d (%s)", (int)e,
-                    hipGetErrorString(e));
+    struct { const void *fn; int bytes; } const kernels[] = {
+        {reinterpret_cast<const void *>(&decode_q8_kernel), kDmaLds},
+        {reinterpret_cast<const void *>(&decode_staged_kernel<false, true>), decode_lds_bytes(1)},
+        {reinterpret_cast<const void *>(&decode_staged_kernel<true, false>), decode_lds_bytes(1)},
+    };
+    for (const auto &k : kernels) {
+        const hipError_t e = hipFuncSetAttribute(k.fn, hipFuncAttributeMaxDynamicSharedMemorySize, k.bytes);
+        if (e != hipSuccess)
+            return fail((int)e, "hipFuncSetAttribute(decode LDS) failed: %d (%s)", (int)e, hipGetErrorString(e));
+    }
     return 0;
 }
 
@@ -1079,11 +1572,13 @@ int launch_decode_q8(hipStream_t st, const DecodeLaunch &L)
     memset(a.kvslot, 0, sizeof(a.kvslot));
     memset(a.head0, 0, sizeof(a.head0));
     memset(a.nhead, 0, sizeof(a.nhead));
+    // q8_0: the kernel that streams raw rows into LDS (its tile addressing is 32-bit per KV head);
+    // q4_0, the fp32-class variant and caches of more than 4 GiB per KV head: the staged kernel
+    const bool raw_rows = !L.q4 && !L.exact && (size_t)L.stride * kRowBytes < ((size_t)1 << 32);
+    const int item_cols = raw_rows ? 8 : 16;
     int items = 0;
     for (int s = 0; s < L.slots; s++) {
-        const int columns = L.cols[s] * a.group;
-        const int parts = (columns + 15) / 16;                  // 1 or 2 (cols <= 4, group <= 8)
-        const int per = (a.group + parts - 1) / parts;          // heads per item
+        const int per = item_cols / L.cols[s];                    // heads per item: 2..16 (cols <= 4)
         for (int h0 = 0; h0 < a.group; h0 += per) {
             a.row0[items] = L.row0[s];
             a.cols[items] = L.cols[s];
@@ -1094,6 +1589,7 @@ int launch_decode_q8(hipStream_t st, const DecodeLaunch &L)
         }
     }
     a.items = items;
+    a.stream_once = items == 1;
     a.i0_row0 = a.row0[0];
     a.i0_cols = a.cols[0];
     a.i0_slot = a.kvslot[0];
@@ -1105,17 +1601,19 @@ int launch_decode_q8(hipStream_t st, const DecodeLaunch &L)
     a.workers = items > 1 && items <= 64 && 2 * items <= window ? window : 0;
     const dim3 grid = a.workers > 0 ? dim3((unsigned)(L.n_kv * a.workers), 1, 1)
                                     : dim3((unsigned)(L.n_kv * L.splits), (unsigned)items, 1);
-    if (L.q4)
-        hipLaunchKernelGGL((decode_q8_kernel<kDepth, true>), grid, dim3(kThreads, 1, 1), decode_lds_bytes(1), st, a);
+    if (raw_rows)
+        hipLaunchKernelGGL(decode_q8_kernel, grid, dim3(kThreads, 1, 1), kDmaLds, st, a);
+    else if (L.q4)
+        hipLaunchKernelGGL((decode_staged_kernel<true, false>), grid, dim3(kThreads, 1, 1), decode_lds_bytes(1), st, a);
     else
-        hipLaunchKernelGGL((decode_q8_kernel<kDepth, false>), grid, dim3(kThreads, 1, 1), decode_lds_bytes(1), st, a);
+        hipLaunchKernelGGL((decode_staged_kernel<false, true>), grid, dim3(kThreads, 1, 1), decode_lds_bytes(1), st, a);
     int rc = launched(L.q4 ? "attn_decode_kv_q4" : "attn_decode_kv_q8");
     if (rc)
         return rc;
     // Up to 128 splits (every launch the split policies make): the one-barrier merge.  One row: 16 d
     // per workgroup (four times the workgroups, 64-byte pieces of a partial row per thread group);
     // several rows: 64 d per workgroup.
-    if (L.splits <= 128 && (L.total_rows == 1 || DECODE_REDUCE128_ROWS == 2)) {
+    if (L.splits <= 128 && L.total_rows == 1) {
         const dim3 grid((unsigned)L.n_heads * 16, (unsigned)L.total_rows, 1);
         if (L.splits <= 64)
             hipLaunchKernelGGL((decode_reduce128_kernel<4, 1>), grid, dim3(256, 1, 1), 0, st, L.part_acc, L.part_ml,
@@ -1123,7 +1621,7 @@ int launch_decode_q8(hipStream_t st, const DecodeLaunch &L)
         else
             hipLaunchKernelGGL((decode_reduce128_kernel<4, 2>), grid, dim3(256, 1, 1), 0, st, L.part_acc, L.part_ml,
                                L.out, L.gate, L.splits, L.acc_slot, L.ml_slot, L.q_slot);
-    } else if (L.splits <= 128 && DECODE_REDUCE128_ROWS) {
+    } else if (L.splits <= 128) {
         const dim3 grid((unsigned)L.n_heads * 4, (unsigned)L.total_rows, 1);
         if (L.splits <= 16)
             hipLaunchKernelGGL((decode_reduce128_kernel<16, 1>), grid, dim3(256, 1, 1), 0, st, L.part_acc, L.part_ml,
