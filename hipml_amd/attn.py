@@ -40,6 +40,7 @@ EXPORTS = [
     "hipml_attn_front_encode_f32", "hipml_attn_chunk_front_encode_f32",
     "hipml_attn_chunk_q8_split_gate_f16",
     "hipml_attn_front_rows_f32", "hipml_attn_front_rows_encode_f32",
+    "hipml_attn_decode_kv_noalloc",
 ]
 
 
@@ -93,6 +94,7 @@ def lib() -> C.CDLL:
                                                  i, sz, sz, sz, sz, i, vp]),
             "hipml_attn_decode_kv_gate": (i, [vp, vp, i, vp, vp, vp, vp, vp, vp, vp, i, i, i, i, f, i,
                                               sz, sz]),
+            "hipml_attn_decode_kv_noalloc": (i, [vp, vp, i, vp, vp, vp, vp, i, i, i, i, f, i, sz, sz]),
             "hipml_attn_decode_batch_cols_gate": (i, [vp, i, vp, vp, vp, vp, vp, vp, vp, vp, i, i, i,
                                                       i, f, i, sz, sz, sz, sz, i, vp]),
             "hipml_attn_chunk_q8_split": (i, [vp, vp, vp, vp, vp, i, i, i, i, i, i, i, vp, vp, i]),
@@ -349,6 +351,15 @@ def attn_decode_kv_gate(step, dtype, q, k, v, part_acc, part_ml, out, gate, n_he
     _check(lib().hipml_attn_decode_kv_gate(_stream(stream), _p(step), dtype, _p(q), _p(k), _p(v),
                                            _p(part_acc), _p(part_ml), _p(out), _p(gate), n_heads,
                                            n_kv, head_dim, stride, scale, splits, k_off, v_off))
+
+
+def attn_decode_kv_noalloc(step, dtype, q, k, v, out, n_heads, n_kv, head_dim, stride, scale, splits,
+                           k_off=0, v_off=0, stream=None):
+    """`attn_decode_kv` with the split partials in the library's built-in array: allocates nothing,
+    n_heads * splits <= 4096, calls on one GPU must not overlap."""
+    _check(lib().hipml_attn_decode_kv_noalloc(_stream(stream), _p(step), dtype, _p(q), _p(k), _p(v),
+                                              _p(out), n_heads, n_kv, head_dim, stride, scale, splits,
+                                              k_off, v_off))
 
 
 def attn_decode_batch_cols_gate(dtype, pos, q, k_cache, v_cache, part_acc, part_ml, out, gate,

@@ -13,7 +13,7 @@ namespace hipml {
 
 static thread_local char g_err[512] = "";
 static RopeTable g_rope = {nullptr, 0.0f, 0, 0};
-static bool g_inited = false;
+static bool g_inited[64]; // per device: hipml_attn_init has run with that device current
 
 int fail(int code, const char *fmt, ...)
 {
@@ -24,7 +24,13 @@ int fail(int code, const char *fmt, ...)
     return code;
 }
 
-void clear_error() { g_err[0] = '\0'; }
+// Start of every entry point: no message, and no error left over from an earlier runtime call of
+// the caller's (launched() below reads the runtime's last error after each launch).
+void clear_error()
+{
+    g_err[0] = '\0';
+    (void)hipGetLastError();
+}
 
 int launched(const char *what)
 {
@@ -82,11 +88,15 @@ static int decode_format(int dtype, int *kv_dtype)
                 "KV dtype selector %d: 0/4 (q8_0), 6 (q8_0, fp32-class) and 1/5 (q4_0) are built", dtype);
 }
 
-// The MFMA kernels keep more LDS than a launch may use by default; hipml_attn_init raises the limit.
+// The MFMA kernels keep more LDS than a launch may use by default; hipml_attn_init raises the limit
+// on the device it is called for, so a launch needs that call for the device that is current now.
 static int require_init()
 {
-    if (!g_inited)
-        return fail(HIPML_ATTN_E_STATE, "hipml_attn_init has not been called in this process");
+    int device = -1;
+    const hipError_t e = hipGetDevice(&device);
+    if (e != hipSuccess || device < 0 || device >= 64 || !g_inited[device])
+        return fail(HIPML_ATTN_E_STATE, "hipml_attn_init has not been called for the current device (%d)",
+                    e == hipSuccess ? device : -1);
     return 0;
 }
 
@@ -189,14 +199,28 @@ int hipml_attn_init(int device)
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return fail(HIPML_ATTN_E_DEVICE, "device %d is %s; this library is built for gfx950 only",
                     device, prop.gcnArchName);
+    if (device < 0 || device >= 64)
+        return fail(HIPML_ATTN_E_RANGE, "device %d outside 0..63", device);
+    // the per-kernel limits and the scratch symbol belong to the current device: make `device` current
+    // for the set-up and put the caller's device back afterwards
+    int before = -1;
+    e = hipGetDevice(&before);
+    if (e == hipSuccess && before != device)
+        e = hipSetDevice(device);
+    if (e != hipSuccess)
+        return fail((int)e, "selecting device %d failed: %d (%s)", device, (int)e, hipGetErrorString(e));
     int rc = decode_init();
+    if (rc == 0)
+        rc = decode_static_init(device);
     if (rc == 0)
         rc = prefill_init();
     if (rc == 0)
         rc = proj_init();
+    if (before != device)
+        (void)hipSetDevice(before);
     if (rc)
         return rc;
-    g_inited = true;
+    g_inited[device] = true;
     return 0;
 }
 
@@ -671,6 +695,22 @@ int hipml_attn_decode_kv(hipml_stream_t stream, const int32_t *step, int dtype, 
                          static_cast<const uint8_t *>(v) + v_off, part_acc, part_ml, out, n_heads,
                          n_kv, head_dim, stride, scale, splits, 0, slice * kHeadDim, slice * 2,
                          (size_t)n_heads * kHeadDim, 1, nullptr);
+}
+
+int hipml_attn_decode_kv_noalloc(hipml_stream_t stream, const int32_t *step, int dtype, const float *q,
+                                 const void *k, const void *v, float *out, int n_heads, int n_kv,
+                                 int head_dim, int stride, float scale, int splits, size_t k_off,
+                                 size_t v_off)
+{
+    clear_error();
+    int rc = check_heads(n_heads, n_kv, head_dim);
+    if (rc)
+        return rc;
+    float *part_acc = nullptr, *part_ml = nullptr;
+    if ((rc = decode_static_partials(n_heads, splits, &part_acc, &part_ml)))
+        return rc;
+    return hipml_attn_decode_kv(stream, step, dtype, q, k, v, part_acc, part_ml, out, n_heads, n_kv,
+                                head_dim, stride, scale, splits, k_off, v_off);
 }
 
 int hipml_attn_decode_kv_cols(hipml_stream_t stream, int dtype, const int32_t *pos,

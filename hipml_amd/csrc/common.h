@@ -92,8 +92,12 @@ struct DecodeLaunch {
     int max_cols;
 };
 int launch_decode_q8(hipStream_t st, const DecodeLaunch &a);
-// Raise the decode kernels' dynamic LDS limit (once per process; called by hipml_attn_init).
+// Raise the decode kernels' dynamic LDS limit (once per device; called by hipml_attn_init).
 int decode_init();
+// Look up the current device's copy of the decode kernels' built-in scratch array (called by
+// hipml_attn_init with `device` current), and hand it out as the partial buffers of one call.
+int decode_static_init(int device);
+int decode_static_partials(int n_heads, int splits, float **part_acc, float **part_ml);
 
 // Raise the prefill kernels' dynamic LDS limit (once per process; called by hipml_attn_init).
 int prefill_init();

@@ -1549,6 +1549,50 @@ int decode_init()
     return 0;
 }
 
+// ---- partials without an allocation -------------------------------------------------------------
+// hipml_attn_decode_kv_noalloc keeps the split partials of a call in this array instead of in buffers
+// the caller brings: every GPU the library is initialised on holds one copy (4,227,072 bytes) until
+// the process ends.  In host code the name `scratch` is only a handle for the symbol; the memory is
+// reached through the address hipGetSymbolAddress returns for the current device, kept per device.
+constexpr size_t kStaticSlices = 4096; // (head, split) pairs: n_heads * splits of a call
+static __device__ __align__(256) float scratch[kStaticSlices * (kHeadDim + 2)];
+constexpr int kMaxDevices = 64;
+static float *g_scratch_ptr[kMaxDevices]; // device address of `scratch` on each initialised GPU
+
+// Called by hipml_attn_init with `device` current.
+int decode_static_init(int device)
+{
+    if (device < 0 || device >= kMaxDevices)
+        return fail(HIPML_ATTN_E_RANGE, "device %d outside 0..%d", device, kMaxDevices - 1);
+    float *ptr = nullptr;
+    const hipError_t e = hipGetSymbolAddress(reinterpret_cast<void **>(&ptr), HIP_SYMBOL(scratch));
+    if (e != hipSuccess || ptr == nullptr)
+        return fail(e != hipSuccess ? (int)e : HIPML_ATTN_E_STATE, "hipGetSymbolAddress(scratch) failed: %d (%s)",
+                    (int)e, hipGetErrorString(e));
+    g_scratch_ptr[device] = ptr;
+    return 0;
+}
+
+// The current device's copy of the array, cut into the two partial buffers of a decode call of
+// n_heads x splits slices; nothing is allocated.
+int decode_static_partials(int n_heads, int splits, float **part_acc, float **part_ml)
+{
+    int device = -1;
+    const hipError_t e = hipGetDevice(&device);
+    if (e != hipSuccess)
+        return fail((int)e, "hipGetDevice failed: %d (%s)", (int)e, hipGetErrorString(e));
+    if (device < 0 || device >= kMaxDevices || g_scratch_ptr[device] == nullptr)
+        return fail(HIPML_ATTN_E_STATE, "hipml_attn_init has not been called for device %d", device);
+    if (n_heads < 1 || splits < 1 || (size_t)n_heads * (size_t)splits > kStaticSlices)
+        return fail(HIPML_ATTN_E_RANGE,
+                    "n_heads %d x splits %d: the built-in scratch holds at most %zu (head, split) partials",
+                    n_heads, splits, kStaticSlices);
+    float *ptr = g_scratch_ptr[device];
+    *part_acc = ptr;
+    *part_ml = ptr + (size_t)n_heads * (size_t)splits * kHeadDim;
+    return 0;
+}
+
 int launch_decode_q8(hipStream_t st, const DecodeLaunch &L)
 {
     DecodeArgs a;

@@ -52,9 +52,11 @@ typedef enum hipml_attn_status {
 
 /* ---- library ------------------------------------------------------------ */
 
-/* Bind to `device` (hipSetDevice is NOT called; the caller's current device is
- * used for launches) and check that it is gfx950.  Replaces Launcher::new's
- * module load, crates/hipml-kernels/src/launch.rs:119-141. */
+/* Prepare `device`: check that it is gfx950, raise the kernels' LDS limits and look up the
+ * library's built-in scratch array there.  The caller's current device is left as it was;
+ * launches go to whatever device is current at the call and need this set-up for that device
+ * (HIPML_ATTN_E_STATE otherwise).  Replaces Launcher::new's module load,
+ * crates/hipml-kernels/src/launch.rs:119-141. */
 int hipml_attn_init(int device);
 /* Thread-local text for the last failure on this thread ("" if none). */
 const char *hipml_attn_last_error(void);
@@ -280,6 +282,20 @@ int hipml_attn_decode_batch_cols_gate(hipml_stream_t stream, int dtype, const in
                                       int stride, float scale, int splits, size_t kv_slot_bytes,
                                       size_t acc_slot, size_t ml_slot, size_t q_slot, int slots,
                                       const int32_t *cols_per_slot_host);
+
+/* hipml_attn_decode_kv for callers that cannot allocate or bring scratch: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
+ * reference (whose callers own part_acc / part_ml, crates/hipml-model/src/gpu/deep_kv.rs:80-81).
+ * The split partials live in an array built into the library (one copy of 4,227,072 bytes per GPU
+ * the library has been initialised on, held until the process ends); the call allocates nothing and
+ * frees nothing.  Limit: n_heads * splits <= 4096, else HIPML_ATTN_E_RANGE.  Same kernels, same
+ * bits in `out` as hipml_attn_decode_kv.  All calls on one GPU share the array: calls that overlap
+ * on one GPU (two streams, or a captured graph replayed while another call runs) race; calls on one
+ * stream are ordered and safe.  Nothing in the array has to be cleared between calls. */
+int hipml_attn_decode_kv_noalloc(hipml_stream_t stream, const int32_t *step, int dtype, const float *q,
+                                 const void *k, const void *v, float *out, int n_heads, int n_kv,
+                                 int head_dim, int stride, float scale, int splits, size_t k_off,
+                                 size_t v_off);
 
 /* ---- causal chunk prefill over a q8_0 / q4_0 cache -------------------------------- */
 
