@@ -1146,11 +1146,13 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a)
                     mt = fmaxf(mt, s);
                 }
             mt = quad_rows<true>(mt);
-            // The reference value of the exponentials follows the maximum only when that has grown by
-            // more than 8 (log2 units): weights then stay below 2^8, far inside f16 and f32, and the
-            // 92 accumulator registers are rescaled on a few tiles instead of most.
-            grew = fmaxf(m_run, mt) > m_run + 8.0f;
-            const float m_new = grew ? mt : m_run;
+            // The reference value of the exponentials is not the running maximum: it moves only when
+            // the maximum has passed it by more than 8 (log2 units), and then to 4 below the new
+            // maximum.  Weights stay below 2^8, far inside f16 and f32; the 92 accumulator registers
+            // are rescaled on a few tiles instead of most; and the small weights keep 4 to 8 more
+            // bits above the f16 underflow than they would against the maximum itself.
+            grew = mt > m_run + 8.0f;
+            const float m_new = grew ? mt - 4.0f : m_run;
             corr = m_new == -INFINITY ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_new);
             float ls = 0.0f;
 #pragma unroll

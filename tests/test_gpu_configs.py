@@ -1,0 +1,193 @@
+"""The benchmark configurations at their full sizes, and the launch paths the other test files do
+not reach, each against the CPU oracle:
+  * configuration 1: one token at position 672 through RoPE -> q8_0 append -> decode over 673 rows ->
+    sigmoid gate, beside the reference's f32 golden path (attn_layer_f32's core over an f32 KvState,
+    crates/hipml-core/src/attention.rs:105-163) within its own q8-against-f32 bound of 2e-3
+    (crates/hipml-core/tests/kv_formats.rs:198-227);
+  * configuration 4: the 2,048-token chunk at depth 100,000 with the split count of the policy,
+    sampled rows (the reference's bench fills the prefix with synthetic_blocks as well,
+    crates/hipml-cli/src/attn_chunk_bench.rs:62-71);
+  * batches of more work items than the worker window takes (the plain slot x split grid);
+  * the fp32-class decode variant (selector 6) on the reference's q8 cases at its own Tol::DEFAULT
+    1e-4 / 1e-3 (crates/hipml-core/src/parity_kv.rs:70-117,221-232, parity.rs:34)."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+from oracle import binding as orc  # noqa: E402
+from hipml_amd import attn  # noqa: E402
+from gpu_util import (N_HEADS, N_KV, HD, N_ROT, THETA, SECTIONS, SCALE, ROW, dev, host, quantized_cache,  # noqa: E402
+                      step_buffer, decode_scratch, report)
+
+GATE = (2e-3, 1e-2)
+KERNEL_CLASS = (1e-3, 5e-3)
+TOL_DEFAULT = (1e-4, 1e-3)
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _init():
+    attn.init(0)
+
+
+def test_config1_token_at_672_beside_the_f32_golden_path():
+    n, stride = 673, 680
+    r = orc.Rng(0x5EED_0001)
+    q = r.normal_array((N_HEADS, HD))
+    k = r.normal_array((n, N_KV, HD))
+    v = r.normal_array((n, N_KV, HD))
+    gate = r.normal_array((N_HEADS, HD))
+
+    # ---- the golden path: f32 position-major caches, every position's K rotated at its position
+    kc = np.zeros((stride, N_KV * HD), np.float32)
+    vc = np.zeros((stride, N_KV * HD), np.float32)
+    for t in range(n - 1):
+        kr = orc.rope_multi(k[t], N_KV, HD, N_ROT, SECTIONS, (t, t, t, t), THETA)
+        orc.kv_append(kc, vc, kr, v[t], t, N_KV * HD)
+    want, _, _ = orc.attn_core_token(q, k[n - 1], v[n - 1], gate, kc, vc, N_HEADS, N_KV, HD, N_ROT, SECTIONS,
+                                     n - 1, THETA)
+
+    # ---- the HIP path over a q8_0 cache: chunk RoPE + bulk append of the 672 earlier rows, then the
+    # token at 672: M-RoPE of q and k, append, split-K decode with the gate applied in the merge
+    attn.rope_table(THETA, N_ROT, 1024)
+    cache = attn.DeepKv(N_HEADS, N_KV, HD, stride)
+    qd0 = torch.zeros((n - 1, N_HEADS, HD), dtype=torch.float32, device="cuda")
+    kd0, vd0 = dev(k[:n - 1]), dev(v[:n - 1])
+    attn.rope_chunk(qd0, kd0, N_HEADS, N_KV, HD, N_ROT, THETA, 0, n - 1)
+    attn.kv_encode_bulk(0, kd0, vd0, cache.k, cache.v, N_KV, HD, stride, 0, 0, n - 1)
+    step = step_buffer(n - 1, n)
+    q1, k1, v1 = dev(q), dev(k[n - 1]), dev(v[n - 1])
+    attn.mrope(q1, q1, N_HEADS, HD, N_ROT, SECTIONS, step[4:], THETA)
+    attn.mrope(k1, k1, N_KV, HD, N_ROT, SECTIONS, step[4:], THETA)
+    attn.kv_encode(step, 0, k1, v1, cache.k, cache.v, N_KV, HD, stride)
+    splits = attn.decode_splits(n, N_KV)
+    acc, ml = decode_scratch(N_HEADS, splits)
+    out = torch.full((N_HEADS, HD), float("nan"), dtype=torch.float32, device="cuda")
+    attn.attn_decode_kv_gate(step, 0, q1, cache.k, cache.v, acc, ml, out, dev(gate), N_HEADS, N_KV, HD,
+                             stride, SCALE, splits)
+    torch.cuda.synchronize()
+    ok, ma, _ = report("config 1: token 672, q8_0 HIP path vs f32 golden path", want, host(out).ravel(),
+                       2e-3, 0.0)
+    assert ok and ma <= 2e-3
+
+
+def test_config4_chunk_2048_at_100000_sampled_rows():
+    # seeded N(0,1) rows quantized to q8_0 over the whole cache, as the configuration states.  An
+    # average over 100,000 such keys hides a lost tile or slice, so every sampled row also gets a
+    # needle: one key per KV head that the row's first head of that group matches (k = 0.75 q: about half
+    # of the weight, the other half on the 100,000 ordinary keys), at positions on tile and slice edges,
+    # the last prefix row and the row's own diagonal key.  (A needle that takes all of the weight
+    # early in the key order, k = 1.25 q at position 0, leaves the other keys' weights below the f16
+    # range of P: 3e-3 of a value of 4, the class of any kernel with f16 probabilities.)
+    tok, pos0, pad = 2048, 100_000, 16
+    stride = pos0 + tok + pad
+    r = orc.Rng(0x5EED_0004)
+    q = r.normal_array((tok, N_HEADS, HD))
+    kf = r.normal_array((N_KV, stride, HD))
+    vf = r.normal_array((N_KV, stride, HD))
+    rows = np.array([0, 31, 32, 63, 64, 1000, 1023, 1024, 2016, 2047], dtype=np.int32)
+    needles = [0, 63, 64, 25_599, 25_600, 51_023, 76_543, 99_999, pos0 + 2016, pos0 + 2047]
+    for row, at in zip(rows, needles):
+        assert at <= pos0 + row
+        for g in range(N_KV):
+            kf[g, at] = 0.75 * q[row, g * (N_HEADS // N_KV)]
+    kb = orc.quantize(0, kf).reshape(N_KV, stride, ROW)
+    vb = orc.quantize(0, vf).reshape(N_KV, stride, ROW)
+    del kf, vf
+    splits = attn.chunk_splits(pos0, tok, N_KV)
+    assert splits >= 2
+    want = orc.attn_chunk_kv(q, kb, vb, N_HEADS, N_KV, HD, pos0, tok, stride, SCALE, rows=rows, n_threads=16)
+    assert np.abs(want[:, 0]).max() > 1.0  # the needles carry weight
+    out = torch.full((tok, N_HEADS, HD), float("nan"), dtype=torch.float32, device="cuda")
+    acc, ml = attn.chunk_scratch(tok, N_HEADS, splits)
+    acc.fill_(float("nan"))
+    ml.fill_(float("nan"))
+    attn.chunk_attention_q8_split(dev(q), dev(kb), dev(vb), out, N_HEADS, N_KV, HD, pos0, tok, 1, stride, acc,
+                                  ml, splits)
+    torch.cuda.synchronize()
+    got = host(out)
+    assert np.isfinite(got).all()
+    ok, _, _ = report(f"config 4: chunk 2048@100000 splits {splits}, {len(rows)} rows", want, got[rows], *GATE)
+    assert ok
+    # the heads without a needle average ~100,000 keys: their error is far below the gate
+    plain = [h for h in range(N_HEADS) if h % (N_HEADS // N_KV) != 0]
+    ok, ma, _ = report("config 4: heads without a needle", want[:, plain], got[rows][:, plain], 1e-4, 0.0)
+    assert ok
+
+
+def _batch(depths, cols, stride, seed, splits):
+    r = orc.Rng(seed)
+    slots = len(depths)
+    kc = np.zeros((slots, N_KV, stride, ROW), dtype=np.uint8)
+    vc = np.zeros((slots, N_KV, stride, ROW), dtype=np.uint8)
+    qs, pos = [], []
+    for s, (d, c) in enumerate(zip(depths, cols)):
+        live = d + c
+        kc[s], vc[s] = quantized_cache(r.normal_array((N_KV, live, HD)), r.normal_array((N_KV, live, HD)), stride)
+        for j in range(c):
+            qs.append(r.normal_array((N_HEADS, HD)))
+            pos.append((d + j, d + j + 1))
+    q = np.stack(qs)
+    rows = len(pos)
+    acc, ml = decode_scratch(N_HEADS, splits, rows)
+    out = torch.full((rows, N_HEADS, HD), float("nan"), dtype=torch.float32, device="cuda")
+    attn.attn_decode_batch_cols(0, torch.tensor(pos, dtype=torch.int32, device="cuda"), dev(q), dev(kc), dev(vc),
+                                acc, ml, out, N_HEADS, N_KV, HD, stride, SCALE, splits, N_KV * stride * ROW,
+                                N_HEADS * splits * HD, N_HEADS * splits * 2, N_HEADS * HD, cols)
+    torch.cuda.synchronize()
+    got = host(out)
+    row, worst = 0, 0.0
+    for s, c in enumerate(cols):
+        for j in range(c):
+            want = orc.attn_decode_kv(q[row], kc[s], vc[s], N_HEADS, N_KV, HD, pos[row][1], SCALE, stride=stride)
+            ok, ma, _ = orc.compare(want, got[row], *KERNEL_CLASS)
+            worst = max(worst, ma)
+            assert ok, f"slot {s} row {j} seq {pos[row][1]}: max_abs {ma}"
+            row += 1
+    return worst
+
+
+def test_batch_of_80_single_row_slots_runs_the_plain_grid():
+    # 80 work items: more than the worker window takes (64), so every (item, split) is a workgroup of
+    # its own; ragged depths, several of them shallower than one split or one tile, stride > seq
+    r = orc.Rng(0x80B47C4)
+    depths = [1 + int(float(r.uniform()) * 700) for _ in range(80)]
+    depths[3], depths[17], depths[41], depths[79] = 0, 1, 31, 33
+    worst = _batch(depths, [1] * 80, 768, 0x80B47C5, 5)
+    print(f"[parity] batch of 80 one-row slots (plain grid): worst max_abs {worst:.3e}", flush=True)
+
+
+def test_batch_of_40_verify_slots_runs_the_plain_grid():
+    # 40 slots of 3 MTP rows: 18 columns per slot = 3 work items each = 120 items
+    r = orc.Rng(0x40B47C4)
+    depths = [2 + int(float(r.uniform()) * 500) for _ in range(40)]
+    depths[0], depths[39] = 0, 129
+    worst = _batch(depths, [3] * 40, 640, 0x40B47C5, 4)
+    print(f"[parity] batch of 40 three-row slots (plain grid): worst max_abs {worst:.3e}", flush=True)
+
+
+@pytest.mark.parametrize("name,seed,heads,n_kv,seq,splits", [
+    ("attn_decode_kv_q8_hd256_s1", 0x9E00_0001, 6, 1, 1, 1),
+    ("attn_decode_kv_q8_hd256_s37", 0x9E00_0002, 6, 1, 37, 1),
+    ("attn_decode_kv_q8_hd256_s1000", 0x9E00_0003, 6, 1, 1000, 7),
+    ("attn_decode_kv_q8_hd256_s4096", 0x9E00_0004, 6, 1, 4096, 16),
+    ("attn_decode_kv_q8_hd256_s100000", 0x9E00_1001, 1, 1, 100_000, 256),
+    ("decode 24/4 at 8192", 0x9E00_2001, 24, 4, 8192, 64),
+])
+def test_fp32_class_variant_meets_the_reference_tolerance(name, seed, heads, n_kv, seq, splits):
+    # selector 6: Q and the weights p * V-scale as hi + lo f16 pairs
+    r = orc.Rng(seed)
+    q = r.normal_array((heads, HD))
+    kf = r.normal_array((n_kv, seq, HD), 0.3)
+    vf = r.normal_array((n_kv, seq, HD))
+    kb, vb = quantized_cache(kf, vf)
+    want = orc.attn_decode_kv(q, kb, vb, heads, n_kv, HD, seq, SCALE)
+    acc, ml = decode_scratch(heads, splits)
+    out = torch.full((heads, HD), float("nan"), dtype=torch.float32, device="cuda")
+    attn.attn_decode_kv(step_buffer(seq - 1, seq), 6, dev(q), dev(kb), dev(vb), acc, ml, out, heads, n_kv, HD,
+                        seq, SCALE, splits)
+    torch.cuda.synchronize()
+    ok, ma, mr = report(f"{name} (fp32-class variant)", want, host(out).ravel(), *TOL_DEFAULT)
+    assert ok
+    assert ma <= 1e-4  # the absolute criterion outright
