@@ -111,11 +111,16 @@ def bench_prefill(torch, attn, tokens, pos0, steps, warmup, layers, prefix_fill=
         if pos0 > 0 and prefix_fill:
             fill_cache_normal(torch, attn, k, v, stride, pos0, gen)
         caches.append((k, v))
-    q = torch.randn((tokens, H, HD), device="cuda", generator=gen)
-    kx = torch.randn((tokens, KV, HD), device="cuda", generator=gen)
-    vx = torch.randn((tokens, KV, HD), device="cuda", generator=gen)
-    gate = torch.randn((tokens, H, HD), device="cuda", generator=gen)
-    out = torch.empty((tokens, H, HD), device="cuda")
+    # Every layer has its own activations as well (q, the chunk's K/V rows, gate, out: 75 MB per layer at
+    # 672 tokens), so that a step finds none of its operands in the 256 MiB Infinity Cache from the
+    # step before; the split scratch is one buffer, as it is in an engine.
+    acts = []
+    for _ in range(layers):
+        acts.append((torch.randn((tokens, H, HD), device="cuda", generator=gen),
+                     torch.randn((tokens, KV, HD), device="cuda", generator=gen),
+                     torch.randn((tokens, KV, HD), device="cuda", generator=gen),
+                     torch.randn((tokens, H, HD), device="cuda", generator=gen),
+                     torch.empty((tokens, H, HD), device="cuda")))
     splits = attn.chunk_splits(pos0, tokens, KV)
     acc = ml = None
     if splits >= 2:
@@ -124,6 +129,7 @@ def bench_prefill(torch, attn, tokens, pos0, steps, warmup, layers, prefix_fill=
 
     def attention(i):
         k, v = caches[i % layers]
+        q, kx, vx, gate, out = acts[i % layers]
         attn.chunk_attention_q8_split(q, k, v, out, H, KV, HD, pos0, tokens, 1, stride, acc, ml,
                                       splits)
 
@@ -131,12 +137,14 @@ def bench_prefill(torch, attn, tokens, pos0, steps, warmup, layers, prefix_fill=
         # RoPE and the append share one launch; the gate is applied where the attention result is
         # written (same bits as the separate kernels, two launches and one pass over the rows less)
         k, v = caches[i % layers]
+        q, kx, vx, gate, out = acts[i % layers]
         attn.rope_encode_chunk(q, kx, vx, k, v, H, KV, HD, NROT, THETA, pos0, tokens, 0, stride)
         attn.chunk_attention_q8_split_gate(q, k, v, gate, out, H, KV, HD, pos0, tokens, 1, stride,
                                            acc, ml, splits)
 
     def step_unfused(i):
         k, v = caches[i % layers]
+        q, kx, vx, gate, out = acts[i % layers]
         attn.rope_chunk(q, kx, H, KV, HD, NROT, THETA, pos0, tokens)
         attn.kv_encode_bulk(0, kx, vx, k, v, KV, HD, stride, pos0, 0, tokens)
         attention(i)
@@ -248,15 +256,31 @@ def bench_decode(torch, attn, seq, steps, warmup, layers, dtype=0):
     }
 
 
-def batch_case(orc_rng_uniform, slots=16, verify=4, lo=512, hi=16384):
-    depths = [lo + int(orc_rng_uniform() * (hi - lo + 1)) for _ in range(slots)]
+class Xorshift64Star:
+    """The reference's generator (crates/hipml-core/src/rng.rs:19-38): state = seed | 1, xorshift
+    12/25/27, multiply; uniform() = top 24 bits / 2^24.  Here for the seeded depths of the batch."""
+
+    def __init__(self, seed: int):
+        self.s = (seed | 1) & 0xFFFFFFFFFFFFFFFF
+
+    def uniform(self) -> float:
+        x = self.s
+        x ^= x >> 12
+        x ^= (x << 25) & 0xFFFFFFFFFFFFFFFF
+        x ^= x >> 27
+        self.s = x
+        return (((x * 0x2545F4914F6CDD1D) & 0xFFFFFFFFFFFFFFFF) >> 40) / float(1 << 24)
+
+
+def batch_case(slots=16, verify=4, lo=512, hi=16384):
+    r = Xorshift64Star(0x5EED0005)
+    depths = [lo + int(r.uniform() * (hi - lo + 1)) for _ in range(slots)]
     cols = [3 if s < verify else 1 for s in range(slots)]
     return depths, cols
 
 
-def bench_batch(torch, attn, orc, steps, warmup, layers):
-    r = orc.Rng(0x5EED0005)
-    depths, cols = batch_case(lambda: float(r.uniform()))
+def bench_batch(torch, attn, steps, warmup, layers):
+    depths, cols = batch_case()
     slots = len(depths)
     stride = 16448
     gen = torch.Generator(device="cuda")
@@ -309,12 +333,11 @@ def bench_batch(torch, attn, orc, steps, warmup, layers):
     }
 
 
-def bench_batch_layer(torch, attn, orc, steps, layers):
+def bench_batch_layer(torch, attn, steps, layers):
     """One plain step of the batched engine through the attention block: 16 sequences at the seeded
     depths of the batched benchmark, one row each -- front end with append (per-row positions,
     per-slot caches), batched attention with the gate in the merge, W_o over the 16 rows: 4 launches."""
-    r = orc.Rng(0x5EED0005)
-    depths, _ = batch_case(lambda: float(r.uniform()))
+    depths, _ = batch_case()
     slots, stride = len(depths), 16448
     m, k = 5120, H * HD
     gen = torch.Generator(device="cuda")
@@ -670,14 +693,13 @@ def main() -> int:
     K, W = args.steps, args.warmup
 
     if args.only:
-        from oracle import binding as orc
         fn = {
             "prefill672": lambda: bench_prefill(torch, attn, 672, 0, K, W, LAYERS),
             "decode8k": lambda: bench_decode(torch, attn, 8192, K, W, LAYERS),
             "decode32k": lambda: bench_decode(torch, attn, 32768, K, W, LAYERS),
             "decode128k": lambda: bench_decode(torch, attn, 131072, K, W, LAYERS),
-            "chunk100k": lambda: bench_prefill(torch, attn, 2048, 100_000, K, W, 2),
-            "batch16": lambda: bench_batch(torch, attn, orc, K, W, 4),
+            "chunk100k": lambda: bench_prefill(torch, attn, 2048, 100_000, max(K, 10), W, 2),
+            "batch16": lambda: bench_batch(torch, attn, K, W, 4),
             "copycal": lambda: bench_copycal(torch, K),
             "front672": lambda: bench_front(torch, attn, 672, max(K, 20)),
             "decode32k_q4": lambda: bench_decode(torch, attn, 32768, max(K, 20), 3, LAYERS, 1),
@@ -690,10 +712,10 @@ def main() -> int:
             "gemm24": lambda: bench_gemm(torch, attn, 24, max(K // 4, 10), LAYERS),
             "gemm128": lambda: bench_gemm(torch, attn, 128, max(K // 4, 10), LAYERS),
             "layer32k": lambda: bench_decode_layer(torch, attn, 32768, max(K // 4, 10), LAYERS),
-            "blayer16": lambda: bench_batch_layer(torch, attn, orc, max(K // 10, 5), 4),
-            "layer672": lambda: bench_chunk_layer(torch, attn, 672, 0, max(K // 10, 5), 4),
-            "gemm672": lambda: bench_gemm(torch, attn, 672, max(K // 10, 5), 4),
-            "gemm2048": lambda: bench_gemm(torch, attn, 2048, max(K // 20, 3), 4),
+            "blayer16": lambda: bench_batch_layer(torch, attn, max(K // 10, 10), 4),
+            "layer672": lambda: bench_chunk_layer(torch, attn, 672, 0, max(K // 10, 10), 4),
+            "gemm672": lambda: bench_gemm(torch, attn, 672, max(K // 10, 10), 4),
+            "gemm2048": lambda: bench_gemm(torch, attn, 2048, max(K // 20, 10), 4),
         }[args.only]
         print(json.dumps(fn()))
         return 0
@@ -726,28 +748,27 @@ def main() -> int:
         torch.cuda.empty_cache()
         # beyond the two benchmark depths: shows what the same kernel does once launch and ramp-up
         # stop dominating (285 MB per layer)
-        also["decode_131072"] = bench_decode(torch, attn, 131072, max(d_steps // 4, 5), 2, LAYERS)
+        also["decode_131072"] = bench_decode(torch, attn, 131072, max(d_steps // 4, 10), 2, LAYERS)
         torch.cuda.empty_cache()
         also["chunk_2048_at_100000"] = bench_prefill(torch, attn, 2048, 100_000,
-                                                     max(K // 20, 3), 1, 2)
+                                                     max(K // 20, 10), 2, 2)
         torch.cuda.empty_cache()
         also["front_672"] = bench_front(torch, attn, 672, d_steps)
         also["decode_32768_q4_0"] = bench_decode(torch, attn, 32768, d_steps, max(W // 4, 2), LAYERS, 1)
-        from oracle import binding as orc  # only for the seeded depth recipe and the CPU leg
-        also["batch16_mtp"] = bench_batch(torch, attn, orc, d_steps, max(W // 4, 2), 4)
+        also["batch16_mtp"] = bench_batch(torch, attn, d_steps, max(W // 4, 2), 4)
         torch.cuda.empty_cache()
         # the step after the path: output projection over Q8_0 weights (decode rows, then a chunk)
         also["wo_rows_1"] = bench_gemv(torch, attn, 1, d_steps, LAYERS)
         also["wo_rows_4"] = bench_gemv(torch, attn, 4, d_steps, LAYERS)
         also["wo_rows_24"] = bench_gemv(torch, attn, 24, d_steps, LAYERS)  # the batch of 16 slots with 4 verify groups
         torch.cuda.empty_cache()
-        also["wo_chunk_672"] = bench_gemm(torch, attn, 672, max(K // 20, 5), 4)
+        also["wo_chunk_672"] = bench_gemm(torch, attn, 672, max(K // 20, 10), 4)
         torch.cuda.empty_cache()
         also["decode_layer_32768"] = bench_decode_layer(torch, attn, 32768, d_steps, LAYERS)
         torch.cuda.empty_cache()
-        also["chunk_layer_672"] = bench_chunk_layer(torch, attn, 672, 0, max(K // 10, 5), 4)
+        also["chunk_layer_672"] = bench_chunk_layer(torch, attn, 672, 0, max(K // 10, 10), 4)
         torch.cuda.empty_cache()
-        also["batch_layer_16"] = bench_batch_layer(torch, attn, orc, max(K // 10, 5), 4)
+        also["batch_layer_16"] = bench_batch_layer(torch, attn, max(K // 10, 10), 4)
         torch.cuda.empty_cache()
         line["also"] = also
 

@@ -40,7 +40,7 @@ EXPORTS = [
     "hipml_attn_front_encode_f32", "hipml_attn_chunk_front_encode_f32",
     "hipml_attn_chunk_q8_split_gate_f16",
     "hipml_attn_front_rows_f32", "hipml_attn_front_rows_encode_f32",
-    "hipml_attn_decode_kv_noalloc",
+    "hipml_attn_decode_kv_noalloc", "hipml_rope_allow_device_angles",
 ]
 
 
@@ -95,6 +95,7 @@ def lib() -> C.CDLL:
             "hipml_attn_decode_kv_gate": (i, [vp, vp, i, vp, vp, vp, vp, vp, vp, vp, i, i, i, i, f, i,
                                               sz, sz]),
             "hipml_attn_decode_kv_noalloc": (i, [vp, vp, i, vp, vp, vp, vp, i, i, i, i, f, i, sz, sz]),
+            "hipml_rope_allow_device_angles": (i, [i]),
             "hipml_attn_decode_batch_cols_gate": (i, [vp, i, vp, vp, vp, vp, vp, vp, vp, vp, i, i, i,
                                                       i, f, i, sz, sz, sz, sz, i, vp]),
             "hipml_attn_chunk_q8_split": (i, [vp, vp, vp, vp, vp, i, i, i, i, i, i, i, vp, vp, i]),
@@ -181,6 +182,11 @@ def rope_table(theta: float, n_rot: int, max_pos: int, device="cuda") -> torch.T
 
 def rope_clear_table() -> None:
     _check(lib().hipml_rope_set_table(0, 0.0, 0, 0))
+
+
+def rope_allow_device_angles(allow: bool) -> None:
+    """Opt in to (or out of) device-computed angles for positions outside the registered table."""
+    _check(lib().hipml_rope_allow_device_angles(1 if allow else 0))
 
 
 def mrope(x, y, n_heads, head_dim, n_rot, sections, pos, theta, stream=None):

@@ -12,7 +12,7 @@
 namespace hipml {
 
 static thread_local char g_err[512] = "";
-static RopeTable g_rope = {nullptr, 0.0f, 0, 0};
+static RopeTable g_rope = {nullptr, 0.0f, 0, 0, 0};
 static bool g_inited[64]; // per device: hipml_attn_init has run with that device current
 
 int fail(int code, const char *fmt, ...)
@@ -341,6 +341,25 @@ int hipml_rope_set_table(const float *dev_table, float theta_base, int n_rot, in
     return 0;
 }
 
+int hipml_rope_allow_device_angles(int allow)
+{
+    clear_error();
+    g_rope.device_angles = allow ? 1 : 0;
+    return 0;
+}
+
+// Positions pos0 .. pos0 + tokens - 1 known to the host: all inside the table, unless the caller has
+// opted in to device angles.
+static int check_rope_range(int pos0, int tokens)
+{
+    if (!g_rope.device_angles && tokens > 0 && (long long)pos0 + tokens > g_rope.max_pos)
+        return fail(HIPML_ATTN_E_RANGE,
+                    "positions %d..%lld lie outside the RoPE table of %d rows (register n_ctx rows with "
+                    "hipml_rope_set_table, or opt in with hipml_rope_allow_device_angles)",
+                    pos0, (long long)pos0 + tokens - 1, g_rope.max_pos);
+    return 0;
+}
+
 static int check_rope(int n_heads, int head_dim, int n_rot, float theta)
 {
     if (n_heads <= 0 || head_dim <= 0)
@@ -404,6 +423,8 @@ int hipml_rope_chunk_f32(hipml_stream_t stream, float *q, float *k, int n_head, 
         return fail(HIPML_ATTN_E_SHAPE, "n_kv %d must be positive", n_kv);
     if (pos0 < 0 || tokens < 0)
         return fail(HIPML_ATTN_E_RANGE, "pos0 %d / tokens %d must be non-negative", pos0, tokens);
+    if ((rc = check_rope_range(pos0, tokens)))
+        return rc;
     if (tokens == 0)
         return 0;
     return launch_rope_chunk(as_stream(stream), q, k, n_head, n_kv, head_dim, n_rot, theta_base,
@@ -460,6 +481,8 @@ int hipml_attn_chunk_front_f32(hipml_stream_t stream, const float *qg, float *k,
         return rc;
     if (pos0 < 0 || tokens < 0)
         return fail(HIPML_ATTN_E_RANGE, "pos0 %d / tokens %d must be non-negative", pos0, tokens);
+    if ((rc = check_rope_range(pos0, tokens)))
+        return rc;
     if (tokens == 0)
         return 0;
     return launch_front(as_stream(stream), qg, q, gate, k, q_norm, k_norm, n_heads, n_kv, n_rot, 0, 0, 0,
@@ -520,6 +543,8 @@ int hipml_attn_chunk_front_encode_f32(hipml_stream_t stream, int dtype, const fl
         return rc;
     if (pos0 < 0 || tokens < 0)
         return fail(HIPML_ATTN_E_RANGE, "pos0 %d / tokens %d must be non-negative", pos0, tokens);
+    if ((rc = check_rope_range(pos0, tokens)))
+        return rc;
     if ((long long)pos0 + tokens > stride)
         return fail(HIPML_ATTN_E_RANGE, "rows [%d, %d) do not fit a cache of %d rows per head", pos0,
                     pos0 + tokens, stride);
@@ -625,6 +650,8 @@ int hipml_rope_encode_chunk_f32(hipml_stream_t stream, float *q, float *k, const
                     head_dim, n_rot, kHeadDim);
     if (pos0 < 0 || tokens < 0)
         return fail(HIPML_ATTN_E_RANGE, "pos0 %d / tokens %d must be non-negative", pos0, tokens);
+    if ((rc = check_rope_range(pos0, tokens)))
+        return rc;
     if ((long long)pos0 + tokens > stride)
         return fail(HIPML_ATTN_E_RANGE, "rows [%d, %d) do not fit a cache of %d rows per head", pos0,
                     pos0 + tokens, stride);

@@ -48,6 +48,7 @@ struct RopeTable {
     float theta;
     int n_rot;
     int max_pos;
+    int device_angles; // opt-in: positions outside the table may use f64 pow/sincos on the device
 };
 
 int launch_mrope(hipStream_t st, const float *x, float *y, int n_heads, int head_dim, int n_rot,

@@ -154,16 +154,24 @@ int launch_kv_encode(hipStream_t st, int q4, const float *k, const float *v, uin
 // ---- RoPE ----------------------------------------------------------------------
 //
 // NeoX pair k is (k, k + n_rot/2); the angle of pair k at position p is
-// p * theta^(-2k/n_rot).  cos/sin come from the host-built f32 table when the
-// position is inside it; otherwise from f64 pow/sincos on the device.
+// p * theta^(-2k/n_rot).  cos/sin come from the host-built f32 table.  A position outside the
+// table is an error: the entry points refuse it where the host knows the positions, and where they
+// live in device memory the rotated values come out as NaN.  Only when the caller has opted in
+// (hipml_rope_allow_device_angles) such a position is served by f64 pow/sincos on the device, within
+// one f32 ulp of the table but not bit-identical to it.  The kernels take the table's row count with
+// a sign: tab_rows >= 0 allows the device angles, -(rows) - 1 does not.
+
+__device__ __forceinline__ int rope_rows(int tab_rows) { return tab_rows >= 0 ? tab_rows : -(tab_rows + 1); }
 
 __device__ __forceinline__ void rope_cs(const float *__restrict__ tab, int tab_rows, int half,
                                         int k, int p, int n_rot, float theta, float &cs, float &sn)
 {
-    if (tab != nullptr && p >= 0 && p < tab_rows) {
+    if (tab != nullptr && p >= 0 && p < rope_rows(tab_rows)) {
         const float2 e = reinterpret_cast<const float2 *>(tab)[(size_t)p * half + k];
         cs = e.x;
         sn = e.y;
+    } else if (tab_rows < 0) {
+        cs = sn = __builtin_nanf("");
     } else {
         const double freq = pow((double)theta, -2.0 * (double)k / (double)n_rot);
         double s, c;
@@ -243,7 +251,7 @@ __global__ void __launch_bounds__(256) rope_chunk_kernel(
 static const float *table_for(const RopeTable &tab, float theta, int n_rot, int *rows)
 {
     if (tab.dev != nullptr && tab.theta == theta && tab.n_rot == n_rot) {
-        *rows = tab.max_pos;
+        *rows = tab.device_angles ? tab.max_pos : -tab.max_pos - 1;
         return tab.dev;
     }
     *rows = 0;
@@ -384,7 +392,7 @@ __global__ void __launch_bounds__(256) rope_encode_chunk_kernel(
     const int half = n_rot >> 1; // 32
     // cos/sin of pairs 4 g .. 4 g + 3 at position p
     auto cos_sin = [&](int g, int p, float (&cs)[4], float (&sn)[4]) {
-        if (tab != nullptr && p >= 0 && p < tab_rows) {
+        if (tab != nullptr && p >= 0 && p < rope_rows(tab_rows)) {
             const float4e *e = reinterpret_cast<const float4e *>(tab + ((size_t)p * half + 4 * g) * 2);
             const float4e c0 = e[0], c1 = e[1];
             cs[0] = c0[0], sn[0] = c0[1], cs[1] = c0[2], sn[1] = c0[3];

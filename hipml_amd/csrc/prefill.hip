@@ -49,9 +49,6 @@ constexpr int kQLdsSteps = 3;                          // d-steps of the Q opera
 constexpr int kQLdsOff = 2 * kBufBytes;                // after the two tile buffers (137,216)
 constexpr int kPfLds = kQLdsOff + kTasks * kQLdsSteps * 1024; // 161,792 of 163,840
 constexpr float kLog2e = 1.4426950408889634f;
-#ifndef PF_SKEW
-#define PF_SKEW 1
-#endif
 
 struct ChunkArgs {
     const float *q;
@@ -226,23 +223,6 @@ __device__ __host__ __forceinline__ int block_slices(int tb, int ntask, int grou
     const int n = (tiles + slice_tiles - 1) / slice_tiles;
     return n < 1 ? 1 : (n < splits ? n : splits);
 }
-
-#ifdef PF_TIMING
-// debug builds: per-wave accumulated cycles of each slot of the tile loop, for one workgroup:
-// [wave][16] = 10 phases, total cycles, total time in 100 MHz ticks
-__device__ unsigned long long g_pf_t[8 * 16];
-#define TSTART() unsigned long long t_w0 = wall_clock64(); unsigned long long t_prev = clock64(), t_now; unsigned long long t_acc[16] = {0,0,0,0,0,0,0,0,0,0,0,0,0,0,0,0}; const unsigned long long t_c0 = t_prev
-#if PF_TIMING >= 2
-#define TMARK(i) do { t_now = clock64(); t_acc[i] += t_now - t_prev; t_prev = t_now; } while (0)
-#else
-#define TMARK(i) do { (void)t_now; (void)t_prev; } while (0)
-#endif
-#define TDUMP() do { t_acc[10] = clock64() - t_c0; t_acc[11] = wall_clock64() - t_w0; if (blockIdx.x == 8 && (threadIdx.x & 63) == 0) for (int i = 0; i < 16; i++) g_pf_t[(threadIdx.x >> 6) * 16 + i] = t_acc[i]; } while (0)
-#else
-#define TSTART() do { } while (0)
-#define TMARK(i) do { } while (0)
-#define TDUMP() do { } while (0)
-#endif
 
 // max(x[lane], x[lane ^ 32]) without going through LDS: swapping the upper half of one copy
 // with the lower half of another leaves {lo, lo} and {hi, hi}.  (Written as asm: the
@@ -582,48 +562,32 @@ __global__ void __launch_bounds__(kPfThreads, 2) chunk_q8_kernel(const ChunkArgs
         issue0(1);
     }
     lds_barrier();
-    if (PF_SKEW && set == 1)
+    if (set == 1)
         lds_barrier();
     if (ntile > 0)
         scores(0, 0);
     lds_barrier();
-    TSTART();
     for (int t = 0; t < ntile; t++) {
         if (t + 1 < ntile)
             stage0(t + 1);
-        TMARK(12);
         issue1(t + 1);
-        TMARK(13);
         softmax(t, 0);
-        TMARK(0);
         lds_barrier();
-        TMARK(1);
         pv(t, 0);
-        TMARK(2);
         scores(t, 1);
-        TMARK(3);
         lds_barrier();
-        TMARK(4);
         if (t + 1 < ntile)
             stage1(t + 1);
-        TMARK(14);
         issue0(t + 2);
-        TMARK(15);
         softmax(t, 1);
-        TMARK(5);
         lds_barrier();
-        TMARK(6);
         pv(t, 1);
-        TMARK(7);
         if (t + 1 < ntile)
             scores(t + 1, 0);
-        TMARK(8);
         lds_barrier();
-        TMARK(9);
     }
-    if (PF_SKEW && set == 0)
+    if (set == 0)
         lds_barrier();
-    TDUMP();
 
     // ---- epilogue --------------------------------------------------------------------------
     l_run += __shfl_xor(l_run, 32);
@@ -797,13 +761,6 @@ __global__ void __launch_bounds__(256) rows_f16_kernel(const float4v *__restrict
     if (i < n4)
         y[i] = __builtin_convertvector(x[i], half4);
 }
-
-#ifdef PF_TIMING
-extern "C" int hipml_dbg_read_pf(unsigned long long *host, size_t n)
-{
-    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_pf_t), (n < 128 ? n : 128) * 8);
-}
-#endif
 
 int prefill_init()
 {

@@ -37,17 +37,6 @@ typedef uint32_t uint3a4 __attribute__((ext_vector_type(3), aligned(4)));
 
 constexpr int kQ8Block = 34;
 
-#ifdef GEMV_TIMING
-// debug builds: per-workgroup phase timestamps (100 MHz wall clock), 8 slots per workgroup
-__device__ unsigned long long g_gemv_t[8 * 1024];
-#define GSTAMP(i) do { if ((threadIdx.x & 63) == 0 && blockIdx.y == 0 && blockIdx.x < 1024 && (threadIdx.x >> 6) == ((i) >> 3)) g_gemv_t[blockIdx.x * 8 + ((i) & 7)] = wall_clock64(); } while (0)
-extern "C" int hipml_dbg_read_gemv(unsigned long long *host, size_t n)
-{
-    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_gemv_t), n * 8);
-}
-#else
-#define GSTAMP(i) do { } while (0)
-#endif
 
 // 8 int8 (two dwords) -> 8 f16 holding the same integers, exactly.
 __device__ __forceinline__ half8 int8x8_to_f16(uint32_t w0, uint32_t w1)
@@ -159,7 +148,6 @@ __global__ void __launch_bounds__(64 * WAVES, TILES == 1 ? 2 : 1) gemv_q8_rows_k
             }
         }
     };
-    GSTAMP(0);
     x_issue(threadIdx.x);
     // every wave's activation requests enter the CU's memory pipeline before any wave's weight
     // requests: the pipeline serves them in order, and the first barrier below waits for the last
@@ -196,11 +184,8 @@ __global__ void __launch_bounds__(64 * WAVES, TILES == 1 ? 2 : 1) gemv_q8_rows_k
     __builtin_amdgcn_sched_barrier(0);
 
     // ---- 3. activations to LDS as MFMA operands -----------------------------------------------
-    GSTAMP(1);
     x_store(threadIdx.x); // XG covers every group: the launcher sizes the pass for that
-    GSTAMP(2);
     __syncthreads();
-    GSTAMP(3);
 
     // ---- 4. the block steps --------------------------------------------------------------------
     float4v acc[TILES];
@@ -278,9 +263,7 @@ __global__ void __launch_bounds__(64 * WAVES, TILES == 1 ? 2 : 1) gemv_q8_rows_k
     // the loop head, behind a wait for every outstanding load).
     if (u_hi > u_lo) {
         compute(A, u_lo);
-        GSTAMP(4);
         compute(B, u_lo + CH);
-        GSTAMP(5);
         for (int u = u_lo + 2 * CH; u < u_hi; u += 2 * CH) {
             fetch(A, u);
             fetch(B, u + CH);
@@ -297,7 +280,6 @@ __global__ void __launch_bounds__(64 * WAVES, TILES == 1 ? 2 : 1) gemv_q8_rows_k
             red[(wave * TILES + t) * 32 + lane] = acc[t];
     }
     __syncthreads();
-    GSTAMP(6);
     if (threadIdx.x < 16 * TILES) {
         const int t = threadIdx.x >> 4, l = threadIdx.x & 15;
         float4v hi = red[t * 32 + l], lo = red[t * 32 + 16 + l];
@@ -571,19 +553,6 @@ int launch_gemv_q8_rows(hipStream_t st, const uint8_t *w, const float *x, float 
 // every one of the m/128 workgroups of a token tile repeats that; f16 halves it and drops the
 // conversion.
 
-#ifdef GEMM_TIMING
-// debug builds: cycles spent between marks, summed over the steps, per wave of the first workgroups
-__device__ unsigned long long g_gemm_t[16 * 16 * 8];
-#define GT(i) do { __builtin_amdgcn_sched_barrier(0); const unsigned long long now_ = __builtin_readcyclecounter(); if ((i) > 0) gt_sum[(i)] += now_ - gt_last; gt_last = now_; __builtin_amdgcn_sched_barrier(0); } while (0)
-#define GTDUMP() do { if ((threadIdx.x & 63) == 0 && blockIdx.x < 4 && blockIdx.y < 4) for (int i_ = 0; i_ < 8; i_++) g_gemm_t[((blockIdx.y * 4 + blockIdx.x) * 16 + (threadIdx.x >> 6)) * 8 + i_] = gt_sum[i_]; } while (0)
-extern "C" int hipml_dbg_read_gemm(unsigned long long *host, size_t n)
-{
-    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_gemm_t), n * 8);
-}
-#else
-#define GT(i) do { } while (0)
-#define GTDUMP() do { } while (0)
-#endif
 
 typedef float float16v __attribute__((ext_vector_type(16)));
 typedef _Float16 half4v __attribute__((ext_vector_type(4)));
@@ -595,14 +564,8 @@ constexpr int kGemmPitch = kGemmK * 2 + 16;       // 144: an odd number of 16-by
 constexpr int kGemmTile = 128 * kGemmPitch;       // one operand tile
 constexpr int kGemmBuf = 2 * kGemmTile;           // x tile + w tile
 constexpr int kGemmLds = 2 * kGemmBuf;            // double buffered: 73,728 bytes
-#ifndef GEMM_WAVES
-#define GEMM_WAVES 8
-#endif
-#ifndef GEMM_CWAVES
-#define GEMM_CWAVES 4
-#endif
-constexpr int kGemmWaves = GEMM_WAVES;            // producer waves
-constexpr int kGemmCWaves = GEMM_CWAVES;          // consumer waves
+constexpr int kGemmWaves = 8;                     // producer waves
+constexpr int kGemmCWaves = 4;                    // consumer waves
 
 // What one producer thread fetches for one step: per unit WN weight (row, quarter) pairs, and XN
 // 16-byte pieces of the activation tile.
@@ -776,9 +739,6 @@ __global__ void __launch_bounds__(64 * (NW + kGemmCWaves)) gemm_q8_f16_kernel(co
     // over.  A SIMD holds waves of both kinds, and a VALU wave and an MFMA wave of one SIMD issue side
     // by side.  (Two units per step, half as many barriers, measured slower: 76.5 against 72.8 us at
     // 672 tokens.)
-#ifdef GEMM_TIMING
-    unsigned long long gt_sum[8] = {0, 0, 0, 0, 0, 0, 0, 0}, gt_last = 0;
-#endif
     if (producer) {
         // Four fetch records in rotation: a record is refilled as soon as it has been staged and is
         // staged again four steps later, so its loads have three steps to arrive (with two records the
@@ -794,13 +754,9 @@ __global__ void __launch_bounds__(64 * (NW + kGemmCWaves)) gemm_q8_f16_kernel(co
         __syncthreads();
         int s = 0;
         for (; s + 4 <= nsteps; s += 4) {
-            GT(0);
             stage(r1, lds + kGemmBuf, s + 1); // step s + 1, while step s is multiplied
-            GT(1);
             fetch(r1, s + 5);
-            GT(2);
             __syncthreads();
-            GT(3);
             stage(r2, lds, s + 2);
             fetch(r2, s + 6);
             __syncthreads();
@@ -811,7 +767,6 @@ __global__ void __launch_bounds__(64 * (NW + kGemmCWaves)) gemm_q8_f16_kernel(co
             fetch(r0, s + 8);
             __syncthreads();
         }
-        GTDUMP();
         // the last one to three steps: their records are already on the way
         const int rest = nsteps - s;
         if (rest >= 1) {
@@ -830,15 +785,11 @@ __global__ void __launch_bounds__(64 * (NW + kGemmCWaves)) gemm_q8_f16_kernel(co
     }
     __syncthreads();
     for (int s = 0; s + 2 <= nsteps; s += 2) {
-        GT(0);
         multiply(lds);
-        GT(1);
         __syncthreads();
-        GT(3);
         multiply(lds + kGemmBuf);
         __syncthreads();
     }
-    GTDUMP();
     if (nsteps & 1) {
         multiply(lds);
         __syncthreads();

@@ -83,10 +83,16 @@ int hipml_attn_chunk_splits(int pos0, int tokens, int n_kv);
  * f32 [max_pos][n_rot/2][2]. */
 size_t hipml_rope_table_bytes(int n_rot, int max_pos);
 int hipml_rope_table_fill_host(float *host_table, float theta_base, int n_rot, int max_pos);
-/* Register a device copy of the table (caller owns the memory).  Positions at
- * or beyond max_pos fall back to f64 pow/sincos on the device, which is within
- * one f32 ulp of the table but not guaranteed identical. */
+/* Register a device copy of the table (caller owns the memory; the engine registers n_ctx rows).
+ * The table and the switch below are one per process: set them up before launches start, from one
+ * thread.  Without a table for (theta_base, n_rot) the RoPE entry points return
+ * HIPML_ATTN_E_STATE.  A position at or beyond max_pos is an error: HIPML_ATTN_E_RANGE where the
+ * host knows the positions (the chunk entry points), and NaN in the rotated channels where they
+ * live in device memory (the step buffer, the pos arrays). */
 int hipml_rope_set_table(const float *dev_table, float theta_base, int n_rot, int max_pos);
+/* Opt in (allow != 0) to f64 pow/sincos on the device for positions outside the table: within one
+ * f32 ulp of the host's values, not guaranteed identical to them.  Off by default. */
+int hipml_rope_allow_device_angles(int allow);
 
 /* M-RoPE over [n_heads][head_dim] at the four position ids in device memory
  * pos[0..3] (the step buffer's words 4..7).  x and y may alias.

@@ -202,21 +202,36 @@ def test_fused_rope_and_append_has_the_bits_of_the_two_launches(pos0, tokens, dt
     assert bool((kc2[:, :pos0] == 0x5A).all()) and bool((kc2[:, pos0 + tokens:] == 0x5A).all())
 
 
-def test_rope_beyond_table_falls_back_to_device_math():
-    # positions past the table are computed on the device: within one f32 ulp of the
-    # host definition (not guaranteed identical), so this is a tolerance check.
+def test_rope_beyond_table_is_an_error_unless_device_angles_are_allowed():
+    # bit-exactness is the contract: a position outside the registered table is refused where the host
+    # knows it, gives NaN where it lives in device memory, and is computed on the device (within one
+    # f32 ulp of the host definition, a tolerance check) only after the explicit opt-in.
     attn.rope_table(THETA, N_ROT, 64)
     try:
         r = orc.Rng(3)
         x = r.normal_array((N_KV, HD))
-        y = torch.empty((N_KV, HD), dtype=torch.float32, device="cuda")
-        attn.mrope(dev(x), y, N_KV, HD, N_ROT, SECTIONS,
-                   torch.tensor([70_000] * 4, dtype=torch.int32, device="cuda"), THETA)
+        far = torch.tensor([70_000] * 4, dtype=torch.int32, device="cuda")
+        y = torch.zeros((N_KV, HD), dtype=torch.float32, device="cuda")
+        attn.mrope(dev(x), y, N_KV, HD, N_ROT, SECTIONS, far, THETA)
+        torch.cuda.synchronize()
+        got = host(y)
+        assert np.isnan(got[:, :N_ROT]).all()                  # the rotated channels
+        assert np.array_equal(got[:, N_ROT:], x[:, N_ROT:])    # the others pass through
+        q = torch.zeros((8, N_HEADS, HD), dtype=torch.float32, device="cuda")
+        k = torch.zeros((8, N_KV, HD), dtype=torch.float32, device="cuda")
+        with pytest.raises(attn.HipmlError) as e:
+            attn.rope_chunk(q, k, N_HEADS, N_KV, HD, N_ROT, THETA, 60, 8)  # positions 60..67, table of 64
+        assert e.value.code == -4
+        attn.rope_chunk(q, k, N_HEADS, N_KV, HD, N_ROT, THETA, 56, 8)      # 56..63: inside
+        attn.rope_allow_device_angles(True)
+        attn.mrope(dev(x), y, N_KV, HD, N_ROT, SECTIONS, far, THETA)
+        attn.rope_chunk(q, k, N_HEADS, N_KV, HD, N_ROT, THETA, 60, 8)
         torch.cuda.synchronize()
         want = orc.rope_multi(x, N_KV, HD, N_ROT, SECTIONS, [70_000] * 4, THETA)
-        ok, _, _ = report("mrope device fallback", want, host(y), 1e-6, 1e-5)
+        ok, _, _ = report("mrope device angles (opt-in)", want, host(y), 1e-6, 1e-5)
         assert ok
     finally:
+        attn.rope_allow_device_angles(False)
         attn.rope_table(THETA, N_ROT, 131072)
 
 
