@@ -1225,17 +1225,15 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a)
 
     // ---- merge the four waves and write the split's partial -------------------------------
     // Run j of O^T: lane holds byte columns 16j + lg*4 + i of the key rows for column n = lane%16.
-    // Rounds of 8 columns n: each wave parks 8 x 272 values, indexed by byte column, in its K rows.
+    // The item's (at most 8) columns n: each wave parks 8 x 272 values, indexed by byte column, in its
+    // own K rows and its (m, l) pairs in its own scale table, so nothing has to be waited for before
+    // the writes; the other waves read them after the barrier.
     l_run = quad_rows<false>(l_run);
     float *wl = reinterpret_cast<float *>(wave_lds); // per wave: [8][272] acc by byte column
     float *wml = reinterpret_cast<float *>(sK);  // per wave: [8] m, [8] l
-#pragma unroll
-    for (int half = 0; half < 2; half++) {
-        const int nbase = half * 8;
-        if (nbase >= nvalid)
-            break; // uniform over the workgroup
-        __syncthreads(); // everyone is done with the tile buffers / previous round
-        if ((lm >> 3) == half) {
+    {
+        constexpr int nbase = 0;
+        if (lm < 8) {
             const int n8 = lm & 7;
 #pragma unroll
             for (int j = 0; j < kRuns; j++) {
