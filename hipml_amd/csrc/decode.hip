@@ -970,33 +970,38 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a)
         seq_max = s > seq_max ? s : seq_max;
     }
 
-    // ---- the first requests: K rows of tile 0 and the Q rows ------------------------------------
-    // Neither address needs anything from device memory (a tile past the live rows costs one load of
-    // rows inside the cache and is masked out).
-    issue(false, 0);
+    // ---- the first requests: the Q rows, then K and V rows of tile 0 ---------------------------
+    // No address here needs anything from device memory (a tile past the live rows costs one load of
+    // rows inside the cache and is masked out), so all 20 requests leave before the first wait.
     // The item has at most 8 (row, head) columns.  MFMA column lm < 8 carries the f16 value of Q column
     // lm, MFMA column lm + 8 what that rounding left over (x - f16(x), again as f16): the two halves
     // of a score are added after the block loop, so Q enters with ~22 bits at the price of one
-    // MFMA.  Wave w fetches two blocks of the Q rows: lane (column n = lm % 8, k-group lg) holds
-    // Q[n][c*32 + lg*8 .. +8]; the waves exchange them through LDS below.  (Every wave fetching all of
-    // it is 16 KB per wave through the CU's L1 in front of the first K/V rows: 1 us later first data.)
-    // These are ordinary loads: the compiler waits for them, and with them for the K rows requested
-    // before them, where the values are first used, which is where both are needed.
+    // MFMA.  Wave w fetches two blocks of the Q rows, 2 KB, and the four exchange the operands made
+    // of them through LDS below.  (Every wave fetching all of it is 16 KB per wave through the CU's L1
+    // in front of the first K/V rows: 1 us later first data.)  The Q rows take the same road as the
+    // K/V rows, global memory -> LDS, into the quarter of the staging area that the wave's operands
+    // go to afterwards: written as ordinary loads they would be waited for by the compiler with
+    // vmcnt(0), that is together with the K and V rows of tile 0 behind them.
+    // Request i of lane l brings 16 bytes: column l % 8, block 2w + i, k-group (l / 8) % 4, half l / 32.
     constexpr int kQB = 8 / kWaves; // Q blocks per wave
-    float4v qf[kQB][2];
+    static_assert(kQB == 2, "two requests of 64 x 16 bytes fetch a wave's share of the Q rows");
     const int qcol = lm & 7;
     const bool have_q = qcol < nvalid;
+    uint8_t *Qraw = Qst + wave * (kQB * 1024);
     {
-        const int col = have_q ? qcol / group : 0;
-        const int head = have_q ? qcol - col * group : 0; // (idle columns fetch column 0 and drop it)
-        const float *qp = a.q + (size_t)(row0 + col) * a.q_slot + (size_t)(hbase + head) * kHeadDim + lg * 8 +
-                          wave * (kQB * 32);
-#pragma unroll
-        for (int cc = 0; cc < kQB; cc++) {
-            qf[cc][0] = *reinterpret_cast<const float4v *>(qp + cc * 32);
-            qf[cc][1] = *reinterpret_cast<const float4v *>(qp + cc * 32 + 4);
-        }
+        const int fcol = (lane & 7) < nvalid ? (lane & 7) : 0; // (idle columns fetch column 0 and drop it)
+        const int col = fcol / group;
+        const int head = fcol - col * group;
+        // (per-lane byte offsets from the uniform base: the Q rows of a launch are far below 4 GB)
+        const uint32_t qoff = (uint32_t)(((size_t)(row0 + col) * a.q_slot + (size_t)(hbase + head) * kHeadDim +
+                                          wave * (kQB * 32) + ((lane >> 3) & 3) * 8 + (lane >> 5) * 4) *
+                                         sizeof(float));
+        const uint32_t at = lds_address(Qraw);
+        dma16<false>(at, reinterpret_cast<const uint8_t *>(a.q), qoff);
+        dma16<false>(at + 1024, reinterpret_cast<const uint8_t *>(a.q), qoff + 32 * sizeof(float));
     }
+    issue(false, 0);
+    issue(true, 0);
 
     const int hi = seq_max; // keys at or past it are masked
     if (split * kWaves * kTileKeys >= hi) {
@@ -1015,6 +1020,13 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a)
     const int ntile = first_key < hi ? (hi - first_key + step_keys - 1) / step_keys : 0;
 
     // ---- Q operands and the score bias of every block ------------------------------------------
+    asm volatile("s_waitcnt vmcnt(18)" ::: "memory"); // the Q rows are in LDS: 9 + 9 requests follow them
+    float4v qf[kQB][2];
+#pragma unroll
+    for (int cc = 0; cc < kQB; cc++)
+#pragma unroll
+        for (int h = 0; h < 2; h++)
+            qf[cc][h] = *reinterpret_cast<const float4v *>(Qraw + cc * 1024 + ((h << 5) | (lg << 3) | qcol) * 16);
 #pragma unroll
     for (int cc = 0; cc < kQB; cc++) {
         const int c = kQB * wave + cc;
@@ -1031,12 +1043,11 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a)
         }
         sum = quad_rows<false>(sum); // over the four k-groups: the block's 32 values of MFMA column lm
         const float cb = -128.0f / kTwo24 * sum;
+        // (the wave's own quarter: every lane has read its raw values, LDS works in program order)
         *reinterpret_cast<half8 *>(Qst + (c * 64 + lane) * 16) = h8;
         if (lg == 0)
             *reinterpret_cast<float4v *>(CBs + (c * 16 + lm) * 16) = (float4v){cb, cb, cb, cb};
     }
-    // the K rows are in LDS by now; the V rows of the first tile follow them
-    issue(true, 0);
     __syncthreads();
     half8 bh[8];
 #pragma unroll
@@ -1618,7 +1629,10 @@ int launch_decode_q8(hipStream_t st, const DecodeLaunch &L)
     memset(a.nhead, 0, sizeof(a.nhead));
     // q8_0: the kernel that streams raw rows into LDS (its tile addressing is 32-bit per KV head);
     // q4_0, the fp32-class variant and caches of more than 4 GiB per KV head: the staged kernel
-    const bool raw_rows = !L.q4 && !L.exact && (size_t)L.stride * kRowBytes < ((size_t)1 << 32);
+    // the kernel that moves raw rows addresses a KV head's rows and the Q rows with 32-bit byte offsets
+    const bool raw_rows = !L.q4 && !L.exact && (size_t)L.stride * kRowBytes < ((size_t)1 << 32) &&
+                          ((size_t)L.total_rows * L.q_slot + (size_t)L.n_heads * kHeadDim) * sizeof(float) <
+                              ((size_t)1 << 32);
     const int item_cols = raw_rows ? 8 : 16;
     int items = 0;
     for (int s = 0; s < L.slots; s++) {
