@@ -24,8 +24,12 @@
  *     high nibbles are elements j / j+16; value = (nibble - 8) * scale, kv.rs:201-218).
  *   - `dtype` of the append entry points is the reference's KvDtype id: 0 = q8_0, 1 = q4_0.
  *     The decode entry points take the reference's kernel selector: 0 or 4 = q8_0, 1 or 5 =
- *     q4_0 (crates/hipml-kernels/src/launch_kv.rs:146-170,329-334; its other values pick
- *     variants of the reference's own kernels and are rejected).  The chunk entry points
+ *     q4_0, 6 = q8_0 through the fp32-class kernel (in the reference 6 keeps its staged q8_0
+ *     kernel reachable next to the shipped one; here it selects the variant that carries the
+ *     softmax weights as hi + lo f16 pairs and meets the reference's 1e-4 / 1e-3 parity
+ *     tolerance, at a lower speed) (crates/hipml-kernels/src/launch_kv.rs:146-170,329-334;
+ *     its other values pick variants of the reference's own kernels and are rejected).  The
+ *     chunk entry points
  *     take 1 = q8_0, 2 = q4_0 (attn_gpu/imp/attn_chunk_kv.rs:41-60).
  */
 #ifndef HIPML_ATTN_H
