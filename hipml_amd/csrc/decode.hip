@@ -79,7 +79,8 @@ struct DecodeArgs {
     // memory round trip before the first Q and K/V requests can be addressed
     int i0_row0, i0_cols, i0_slot, i0_head0, i0_nhead;
     int workers;   // > 0: worker launch, workgroups per KV head (see decode_body)
-    int stream_once; // the launch has one work item: the cache rows are read once (non-temporal loads)
+    int stream_once; // the launch has one work item, so the cache rows are read once (non-temporal loads);
+                     // the kernel decides the same per item for launches with several
     float scale_log2; // scale * log2(e) * 2^24
     size_t kv_slot_bytes, acc_slot, ml_slot, q_slot;
     // Work items (grid.y).  A slot whose rows x heads fit the columns of one workgroup (8 in the raw-row
@@ -950,7 +951,8 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a)
             }
         }
     };
-    const bool once = a.stream_once != 0;
+    // (an item that carries every head of its KV head is its slot's only reader of these rows)
+    const bool once = a.stream_once != 0 || group == a.group;
     auto issue = [&](bool v_rows, int t) {
         if (once)
             issue_as(std::true_type(), v_rows, t);
