@@ -83,10 +83,11 @@ struct DecodeArgs {
                      // the kernel decides the same per item for launches with several
     float scale_log2; // scale * log2(e) * 2^24
     size_t kv_slot_bytes, acc_slot, ml_slot, q_slot;
-    // Work items (grid.y).  A slot whose rows x heads fit the columns of one workgroup (8 in the raw-row
-    // kernel, 16 in the staged one) is one item; a wider one (2-4 MTP rows x 6 heads) is cut by heads
-    // into items that stream the same cache rows: their workgroups are gridDim.x apart in launch
-    // order, a multiple of the 8 XCDs here, so the later readers find the rows in the first one's L2.
+    // Work items (grid.y).  A slot whose rows x heads fit the columns of one workgroup (16; the raw-row
+    // kernel runs items of up to 8 columns through its narrow body and wider ones through its wide
+    // one) is one item; a wider one (2-4 MTP rows x 6 heads) is cut by heads into
+    // items that stream the same cache rows: their workgroups are gridDim.x apart in launch order, a
+    // multiple of the 8 XCDs here, so the later readers find the rows in the first one's L2.
     uint16_t row0[kMaxItems];  // first query row of the item's slot
     uint8_t cols[kMaxItems];   // query rows of the slot (1..kMaxCols)
     uint8_t kvslot[kMaxItems]; // slot index, for the cache base
@@ -890,18 +891,20 @@ __device__ __forceinline__ half8 raw_k_operand(const uint8_t *row_lg, int c)
     return __builtin_bit_cast(half8, r);
 }
 
-__device__ __forceinline__ void decode_body_dma(const DecodeArgs &a)
+// WIDE: the item has 9 to 16 (row, head) columns (rows of an MTP-verify slot).  Then every MFMA column
+// is a real one, the two f16 halves of Q are two B operands and two MFMAs per block, and the raw Q rows
+// (16 KB) pass through the waves' V rows before the first V rows are requested.
+template <bool WIDE>
+__device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Work &wk)
 {
     static_assert(kWaves * 2 * kScaleBytes <= kDmaQLds, "the scale tables reuse the Q staging area");
+    constexpr int kCols = WIDE ? 16 : 8; // columns of an item
     constexpr int kDmaWaveLds = kDmaTileLds;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds_all[];
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int lane = threadIdx.x & 63;
     const int lm = lane & 15; // MFMA row/col within the 16-tile
     const int lg = lane >> 4; // k-group
-    Work wk;
-    if (!find_work(a, lane, wk))
-        return;
     const int kvh = wk.kvh, split = wk.split, nsp = wk.nsp, slot = wk.slot, row0 = wk.row0, ncols = wk.ncols,
               group = wk.group, hbase = wk.hbase, nvalid = wk.nvalid;
 
@@ -986,24 +989,37 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a)
     // vmcnt(0), that is together with the K and V rows of tile 0 behind them.
     // Request i of lane l brings 16 bytes: column l % 8, block 2w + i, k-group (l / 8) % 4, half l / 32.
     constexpr int kQB = 8 / kWaves; // Q blocks per wave
-    static_assert(kQB == 2, "two requests of 64 x 16 bytes fetch a wave's share of the Q rows");
-    const int qcol = lm & 7;
+    static_assert(kQB == 2, "two requests of 64 x 16 bytes fetch a wave's share of the Q rows of 8 columns");
+    const int qcol = WIDE ? lm : lm & 7;
     const bool have_q = qcol < nvalid;
-    uint8_t *Qraw = Qst + wave * (kQB * 1024);
+    // WIDE: four requests per wave (16 columns) into the wave's V rows, whose first tile is requested
+    // once the values are in registers; request i of lane l: column l % 16, block 2w + i / 2,
+    // k-group l / 16, half i % 2, so every lane finds its own values in its own slots.
+    uint8_t *Qraw = WIDE ? Vraw : Qst + wave * (kQB * 1024);
     {
-        const int fcol = (lane & 7) < nvalid ? (lane & 7) : 0; // (idle columns fetch column 0 and drop it)
+        const int lcol = WIDE ? (lane & 15) : (lane & 7);
+        const int fcol = lcol < nvalid ? lcol : 0; // (idle columns fetch column 0 and drop it)
         const int col = fcol / group;
         const int head = fcol - col * group;
+        const int kg = WIDE ? (lane >> 4) : ((lane >> 3) & 3);
         // (per-lane byte offsets from the uniform base: the Q rows of a launch are far below 4 GB)
         const uint32_t qoff = (uint32_t)(((size_t)(row0 + col) * a.q_slot + (size_t)(hbase + head) * kHeadDim +
-                                          wave * (kQB * 32) + ((lane >> 3) & 3) * 8 + (lane >> 5) * 4) *
+                                          wave * (kQB * 32) + kg * 8 + (WIDE ? 0 : (lane >> 5) * 4)) *
                                          sizeof(float));
         const uint32_t at = lds_address(Qraw);
-        dma16<false>(at, reinterpret_cast<const uint8_t *>(a.q), qoff);
-        dma16<false>(at + 1024, reinterpret_cast<const uint8_t *>(a.q), qoff + 32 * sizeof(float));
+        const uint8_t *qb = reinterpret_cast<const uint8_t *>(a.q);
+        if (WIDE) {
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                dma16<false>(at + i * 1024, qb, qoff + ((i >> 1) * 32 + (i & 1) * 4) * sizeof(float));
+        } else {
+            dma16<false>(at, qb, qoff);
+            dma16<false>(at + 1024, qb, qoff + 32 * sizeof(float));
+        }
     }
     issue(false, 0);
-    issue(true, 0);
+    if (!WIDE)
+        issue(true, 0);
 
     const int hi = seq_max; // keys at or past it are masked
     if (split * kWaves * kTileKeys >= hi) {
@@ -1022,40 +1038,72 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a)
     const int ntile = first_key < hi ? (hi - first_key + step_keys - 1) / step_keys : 0;
 
     // ---- Q operands and the score bias of every block ------------------------------------------
-    asm volatile("s_waitcnt vmcnt(18)" ::: "memory"); // the Q rows are in LDS: 9 + 9 requests follow them
+    // the Q rows are in LDS once only the requests behind them are outstanding: K(0) [and V(0)]
+    if (WIDE)
+        asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
+    else
+        asm volatile("s_waitcnt vmcnt(18)" ::: "memory");
     float4v qf[kQB][2];
 #pragma unroll
     for (int cc = 0; cc < kQB; cc++)
 #pragma unroll
         for (int h = 0; h < 2; h++)
-            qf[cc][h] = *reinterpret_cast<const float4v *>(Qraw + cc * 1024 + ((h << 5) | (lg << 3) | qcol) * 16);
+            qf[cc][h] = WIDE ? *reinterpret_cast<const float4v *>(Qraw + (cc * 2 + h) * 1024 + lane * 16)
+                             : *reinterpret_cast<const float4v *>(Qraw + cc * 1024 + ((h << 5) | (lg << 3) | qcol) * 16);
+    half8 qlo[kQB]; // WIDE: what the rounding to f16 left over, the second B operand
 #pragma unroll
     for (int cc = 0; cc < kQB; cc++) {
         const int c = kQB * wave + cc;
         half8 h8;
-        float sum = 0.0f;
+        float sum = 0.0f, sum_lo = 0.0f;
 #pragma unroll
         for (int j = 0; j < 8; j++) {
             const float x = have_q ? (j < 4 ? qf[cc][0][j] : qf[cc][1][j - 4]) : 0.0f;
             _Float16 h = (_Float16)x;
-            if (lm >= 8)
-                h = (_Float16)(x - (float)h);
-            h8[j] = h;
+            const _Float16 l = (_Float16)(x - (float)h);
+            if (WIDE) {
+                qlo[cc][j] = l;
+                sum_lo += (float)l;
+            } else if (lm >= 8) {
+                h = l;
+            }
             sum += (float)h;
+            h8[j] = h;
         }
         sum = quad_rows<false>(sum); // over the four k-groups: the block's 32 values of MFMA column lm
         const float cb = -128.0f / kTwo24 * sum;
-        // (the wave's own quarter: every lane has read its raw values, LDS works in program order)
+        // (narrow: the wave's own quarter: every lane has read its raw values, LDS works in program order)
         *reinterpret_cast<half8 *>(Qst + (c * 64 + lane) * 16) = h8;
-        if (lg == 0)
+        if (WIDE) {
+            // both halves' biases side by side: every sum is formed as the narrow variant forms it in
+            // its two column halves, so a column's result does not depend on the width of its item
+            sum_lo = quad_rows<false>(sum_lo);
+            const float cbl = -128.0f / kTwo24 * sum_lo;
+            if (lg == 0)
+                *reinterpret_cast<float4v *>(CBs + (c * 16 + lm) * 16) = (float4v){cb, cbl, 0.0f, 0.0f};
+        } else if (lg == 0) {
             *reinterpret_cast<float4v *>(CBs + (c * 16 + lm) * 16) = (float4v){cb, cb, cb, cb};
+        }
     }
+    if (WIDE)
+        issue(true, 0); // the raw Q values have left the V rows
     __syncthreads();
-    half8 bh[8];
+    half8 bh[8], bl[WIDE ? 8 : 1];
 #pragma unroll
     for (int c = 0; c < 8; c++)
         bh[c] = *reinterpret_cast<const half8 *>(Qst + (c * 64 + lane) * 16);
-    __syncthreads(); // the staging area becomes the waves' scale tables
+    __syncthreads();
+    if (WIDE) {
+#pragma unroll
+        for (int cc = 0; cc < kQB; cc++)
+            *reinterpret_cast<half8 *>(Qst + ((kQB * wave + cc) * 64 + lane) * 16) = qlo[cc];
+        __syncthreads();
+#pragma unroll
+        for (int c = 0; c < 8; c++)
+            bl[WIDE ? c : 0] = *reinterpret_cast<const half8 *>(Qst + (c * 64 + lane) * 16);
+        __syncthreads();
+    }
+    // (the staging area is the waves' scale tables from here on)
 
     // per-column causal bound (MTP rows see one more key each)
     const int seq_n = qcol < nvalid ? seqc[qcol / group] : 0;
@@ -1110,12 +1158,12 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a)
         build_scales(Kraw, sK, key0, partial);
 
         // ---- scores ----------------------------------------------------------------------------
-        float S[2][4];
+        float S[2][4], Sl[WIDE ? 2 : 1][4]; // (Sl: the scores' lower halves where they have no columns of their own)
 #pragma unroll
         for (int ms = 0; ms < 2; ms++)
 #pragma unroll
             for (int i = 0; i < 4; i++)
-                S[ms][i] = 0.0f;
+                S[ms][i] = Sl[WIDE ? ms : 0][i] = 0.0f;
 #pragma unroll
         for (int c = 0; c < 8; c++) {
             const float4v cb4 = *reinterpret_cast<const float4v *>(CBs + (c * 16 + lm) * 16);
@@ -1123,19 +1171,41 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a)
             for (int ms = 0; ms < 2; ms++) {
                 const half8 A = raw_k_operand(Kraw + (ms * 16 + lm) * kRowBytes + lg * 8, c);
                 const half4 sk = *reinterpret_cast<const half4 *>(sK + (c * kTileKeys + ms * 16 + lg * 4) * 2);
-                const float4v part = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, bh[c], cb4, 0, 0, 0);
+                if (WIDE) {
+                    const float4v ch = {cb4[0], cb4[0], cb4[0], cb4[0]}, cl = {cb4[1], cb4[1], cb4[1], cb4[1]};
+                    const float4v part = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, bh[c], ch, 0, 0, 0);
+                    const float4v parl = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, bl[WIDE ? c : 0], cl, 0, 0, 0);
 #pragma unroll
-                for (int i = 0; i < 4; i++)
-                    S[ms][i] = fmaf((float)sk[i], part[i], S[ms][i]);
+                    for (int i = 0; i < 4; i++) {
+                        S[ms][i] = fmaf((float)sk[i], part[i], S[ms][i]);
+                        Sl[WIDE ? ms : 0][i] = fmaf((float)sk[i], parl[i], Sl[WIDE ? ms : 0][i]);
+                    }
+                } else {
+                    const float4v part = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, bh[c], cb4, 0, 0, 0);
+#pragma unroll
+                    for (int i = 0; i < 4; i++)
+                        S[ms][i] = fmaf((float)sk[i], part[i], S[ms][i]);
+                }
             }
         }
-        // the two halves of every score: MFMA columns n and n + 8 (a rotation by 8 inside the 16-lane row)
+        // the two halves of every score: MFMA columns n and n + 8 (a rotation by 8 inside the 16-lane
+        // row), or the second set of sums
 #pragma unroll
         for (int ms = 0; ms < 2; ms++)
 #pragma unroll
-            for (int i = 0; i < 4; i++)
-                S[ms][i] += __builtin_bit_cast(
-                    float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, S[ms][i]), 0x128, 0xf, 0xf, true));
+            for (int i = 0; i < 4; i++) {
+                if (WIDE)
+                    S[ms][i] += Sl[WIDE ? ms : 0][i];
+                else
+                    S[ms][i] += __builtin_bit_cast(
+                        float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, S[ms][i]), 0x128, 0xf, 0xf, true));
+            }
+        if (WIDE) {
+            // (a fixed point for the instruction scheduler where the other variant has its lane moves:
+            // without one it spreads the block loop over the softmax and runs out of registers)
+            asm volatile("" : "+v"(S[0][0]), "+v"(S[0][1]), "+v"(S[0][2]), "+v"(S[0][3]), "+v"(S[1][0]), "+v"(S[1][1]),
+                         "+v"(S[1][2]), "+v"(S[1][3]));
+        }
         // the K rows are used up: request those of the tile that takes their place
         if (more)
             issue(false, t + 1);
@@ -1238,16 +1308,16 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a)
 
     // ---- merge the four waves and write the split's partial -------------------------------
     // Run j of O^T: lane holds byte columns 16j + lg*4 + i of the key rows for column n = lane%16.
-    // The item's (at most 8) columns n: each wave parks 8 x 272 values, indexed by byte column, in its
-    // own K rows and its (m, l) pairs in its own scale table, so nothing has to be waited for before
-    // the writes; the other waves read them after the barrier.
+    // Each wave parks the item's columns as kCols x 272 values, indexed by byte column, in its own
+    // rows (8 columns fill the K rows, 16 the K and V rows) and its (m, l) pairs in its own scale
+    // table, so nothing has to be waited for before the writes; the other waves read them after the
+    // barrier.
     l_run = quad_rows<false>(l_run);
-    float *wl = reinterpret_cast<float *>(wave_lds); // per wave: [8][272] acc by byte column
-    float *wml = reinterpret_cast<float *>(sK);  // per wave: [8] m, [8] l
+    float *wl = reinterpret_cast<float *>(wave_lds); // per wave: [kCols][272] acc by byte column
+    float *wml = reinterpret_cast<float *>(sK);  // per wave: [kCols] m, [kCols] l
     {
-        constexpr int nbase = 0;
-        if (lm < 8) {
-            const int n8 = lm & 7;
+        if (WIDE || lm < 8) {
+            const int nc = lm & (kCols - 1);
 #pragma unroll
             for (int j = 0; j < kRuns; j++) {
                 float4v v;
@@ -1265,29 +1335,28 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a)
                     if (j == 14) // byte column 238, the scale of block 7: its correction row
                         v[2] = lg == 3 ? B7[2] : v[2];
                 }
-                *reinterpret_cast<float4v *>(wl + n8 * kRowBytes + j * 16 + lg * 4) = v;
+                *reinterpret_cast<float4v *>(wl + nc * kRowBytes + j * 16 + lg * 4) = v;
             }
             if (lg == 0) {
-                wml[n8] = m_run;
-                wml[8 + n8] = l_run;
+                wml[nc] = m_run;
+                wml[kCols + nc] = l_run;
             }
         }
         __syncthreads();
-        // thread -> (column n8, kRun consecutive d of one block): 8 columns x kThreads / 8 runs of d
-        constexpr int kDRuns = kThreads / 8, kRun = kHeadDim / kDRuns;
-        static_assert(kRun == 8 || kRun == 4, "a thread's values of d lie in one block");
-        const int n8 = threadIdx.x / kDRuns;
+        // thread -> (column nc, kRun consecutive d of one block): kCols columns x kThreads / kCols runs of d
+        constexpr int kDRuns = kThreads / kCols, kRun = kHeadDim / kDRuns;
+        static_assert(kRun == 16 || kRun == 8, "a thread's values of d lie in one block");
+        const int nc = threadIdx.x / kDRuns;
         const int d0 = (threadIdx.x % kDRuns) * kRun;
         const int col0 = d0 + 2 + 2 * (d0 >> 5); // byte column of d0: 34 bytes per 32 values, scale first
-        const int ng = nbase + n8;
-        if (ng < nvalid) {
+        if (nc < nvalid) {
             float mw[kWaves], lw[kWaves];
             float ms = -INFINITY;
 #pragma unroll
             for (int w = 0; w < kWaves; w++) {
                 const float *o = reinterpret_cast<const float *>(Qst + w * 2 * kScaleBytes);
-                mw[w] = o[n8];
-                lw[w] = o[8 + n8];
+                mw[w] = o[nc];
+                lw[w] = o[kCols + nc];
                 ms = fmaxf(ms, mw[w]);
             }
             float lsum = 0.0f;
@@ -1298,8 +1367,8 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a)
                 lsum += lw[w] * wgt[w];
                 wgt[w] *= kTwo24;
             }
-            const int col = ng / group;
-            const int head = hbase + (ng - col * group);
+            const int col = nc / group;
+            const int head = hbase + (nc - col * group);
             const size_t slice = (size_t)head * a.splits + split;
             float *pa = a.part_acc + (size_t)(row0 + col) * a.acc_slot + slice * kHeadDim + d0;
 #pragma unroll
@@ -1307,7 +1376,7 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a)
                 float4v acc = {0, 0, 0, 0};
 #pragma unroll
                 for (int w = 0; w < kWaves; w++) {
-                    const float *row = reinterpret_cast<const float *>(lds_all + w * kDmaWaveLds) + n8 * kRowBytes;
+                    const float *row = reinterpret_cast<const float *>(lds_all + w * kDmaWaveLds) + nc * kRowBytes;
                     const float off = row[(d0 >> 5) * kQ8BlockBytes]; // the block's correction row
                     const float2 x0 = *reinterpret_cast<const float2 *>(row + col0 + dd);
                     const float2 x1 = *reinterpret_cast<const float2 *>(row + col0 + dd + 2);
@@ -1324,9 +1393,16 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a)
     }
 }
 
+// One workgroup = one (KV head, key split, work item); the item's width picks the body.
 __global__ void __launch_bounds__(kThreads, 2) decode_q8_kernel(const DecodeArgs a)
 {
-    decode_body_dma(a);
+    Work wk;
+    if (!find_work(a, threadIdx.x & 63, wk))
+        return;
+    if (wk.nvalid > 8) // uniform over the workgroup
+        decode_body_dma<true>(a, wk);
+    else
+        decode_body_dma<false>(a, wk);
 }
 
 // Wave-wide reductions without LDS: DPP inside a row of 16 lanes, then the two row-swap
@@ -1635,16 +1711,24 @@ int launch_decode_q8(hipStream_t st, const DecodeLaunch &L)
     const bool raw_rows = !L.q4 && !L.exact && (size_t)L.stride * kRowBytes < ((size_t)1 << 32) &&
                           ((size_t)L.total_rows * L.q_slot + (size_t)L.n_heads * kHeadDim) * sizeof(float) <
                               ((size_t)1 << 32);
-    const int item_cols = raw_rows ? 8 : 16;
+    // Work items: a slot whose rows x heads fit 8 columns is one item; a wider one (rows of an
+    // MTP-verify slot) is cut by heads into as few items of at most 16 columns as will do, of equal
+    // width where the heads divide that way (3 rows x 6 heads: two items of 9 columns).
     int items = 0;
     for (int s = 0; s < L.slots; s++) {
-        const int per = item_cols / L.cols[s];                    // heads per item: 2..16 (cols <= 4)
-        for (int h0 = 0; h0 < a.group; h0 += per) {
+        const int cols = L.cols[s];
+        const int cap = !raw_rows || cols * a.group > 8 ? 16 : 8;
+        const int per_max = cap / cols;                           // heads per item: 2..16 (cols <= 4)
+        const int n_items = (a.group + per_max - 1) / per_max;
+        const int base = a.group / n_items, extra = a.group % n_items;
+        for (int i = 0, h0 = 0; i < n_items; i++) {
+            const int nh = base + (i < extra ? 1 : 0);
             a.row0[items] = L.row0[s];
-            a.cols[items] = L.cols[s];
+            a.cols[items] = (uint8_t)cols;
             a.kvslot[items] = (uint8_t)s;
             a.head0[items] = (uint8_t)h0;
-            a.nhead[items] = (uint8_t)(a.group - h0 < per ? a.group - h0 : per);
+            a.nhead[items] = (uint8_t)nh;
+            h0 += nh;
             items++;
         }
     }
@@ -1657,8 +1741,10 @@ int launch_decode_q8(hipStream_t st, const DecodeLaunch &L)
     a.i0_nhead = a.nhead[0];
     // batches: one window of workers (two workgroups per CU over 256 CUs), as long as every item can
     // have a worker of its own and lane i of a wave can look at item i
+    // (the items of one sequence, a verify group, share their depth: the plain grid gives every row
+    // the tile-to-split partition its plain decode has, so that its result is the same bit for bit)
     const int window = 512 / L.n_kv;
-    a.workers = items > 1 && items <= 64 && 2 * items <= window ? window : 0;
+    a.workers = L.slots > 1 && items > 1 && items <= 64 && 2 * items <= window ? window : 0;
     const dim3 grid = a.workers > 0 ? dim3((unsigned)(L.n_kv * a.workers), 1, 1)
                                     : dim3((unsigned)(L.n_kv * L.splits), (unsigned)items, 1);
     if (raw_rows)
@@ -1670,10 +1756,12 @@ int launch_decode_q8(hipStream_t st, const DecodeLaunch &L)
     int rc = launched(L.q4 ? "attn_decode_kv_q4" : "attn_decode_kv_q8");
     if (rc)
         return rc;
-    // Up to 128 splits (every launch the split policies make): the one-barrier merge.  One row: 16 d
-    // per workgroup (four times the workgroups, 64-byte pieces of a partial row per thread group);
-    // several rows: 64 d per workgroup.
-    if (L.splits <= 128 && L.total_rows == 1) {
+    // Up to 128 splits (every launch the split policies make): the one-barrier merge.  One sequence
+    // (a query row, or the rows of a verify group: the same merge, so that a column of a group is
+    // bit for bit the plain decode of its row, as the reference's column check demands): 16 d per
+    // workgroup (four times the workgroups, 64-byte pieces of a partial row per thread group);
+    // a batch: 64 d per workgroup.
+    if (L.splits <= 128 && L.slots == 1) {
         const dim3 grid((unsigned)L.n_heads * 16, (unsigned)L.total_rows, 1);
         if (L.splits <= 64)
             hipLaunchKernelGGL((decode_reduce128_kernel<4, 1>), grid, dim3(256, 1, 1), 0, st, L.part_acc, L.part_ml,
@@ -1696,8 +1784,8 @@ int launch_decode_q8(hipStream_t st, const DecodeLaunch &L)
             hipLaunchKernelGGL((decode_reduce128_kernel<16, 8>), grid, dim3(256, 1, 1), 0, st, L.part_acc, L.part_ml,
                                L.out, L.gate, L.splits, L.acc_slot, L.ml_slot, L.q_slot);
     }
-    else if (L.total_rows == 1)
-        hipLaunchKernelGGL(decode_reduce_kernel<4>, dim3((unsigned)L.n_heads * 16, 1, 1), dim3(256, 1, 1), 0,
+    else if (L.slots == 1)
+        hipLaunchKernelGGL(decode_reduce_kernel<4>, dim3((unsigned)L.n_heads * 16, (unsigned)L.total_rows, 1), dim3(256, 1, 1), 0,
                            st, L.part_acc, L.part_ml, L.out, L.gate, L.splits, L.acc_slot, L.ml_slot, L.q_slot);
     else
         hipLaunchKernelGGL(decode_reduce_kernel<16>,
