@@ -126,12 +126,38 @@ def bench_prefill(torch, attn, tokens, pos0, steps, warmup, layers, prefix_fill=
     if splits >= 2:
         acc, ml = attn.chunk_scratch(tokens, H, splits)
     attn.rope_table(THETA, NROT, max(pos0 + tokens, 1024))
+    # the f16 copy of every layer cache, current up to the prefix (as earlier chunks would have left it)
+    copies = []
+    for k, v in caches:
+        c = attn.kv_f16_alloc(stride, KV)
+        if pos0 > 0:
+            attn.kv_f16_rows(0, k, v, c, KV, HD, stride, 0, pos0)
+        copies.append(c)
 
     def attention(i):
         k, v = caches[i % layers]
         q, kx, vx, gate, out = acts[i % layers]
         attn.chunk_attention_q8_split(q, k, v, out, H, KV, HD, pos0, tokens, 1, stride, acc, ml,
                                       splits)
+
+    def attention_copy(i):
+        q, kx, vx, gate, out = acts[i % layers]
+        attn.chunk_attention_kv_f16(q, copies[i % layers], None, out, None, H, KV, HD, pos0, tokens, stride,
+                                    acc, ml, splits)
+
+    def step_copy(i, rebuild=False):
+        # the same step with the attention reading the f16 copy of the cache: the chunk's rows are added
+        # to the copy after the append (rebuild: the whole copy is made again from row 0, what a caller
+        # does who keeps one copy for all layers)
+        k, v = caches[i % layers]
+        q, kx, vx, gate, out = acts[i % layers]
+        attn.rope_encode_chunk(q, kx, vx, k, v, H, KV, HD, NROT, THETA, pos0, tokens, 0, stride)
+        if rebuild:
+            attn.kv_f16_rows(0, k, v, copies[i % layers], KV, HD, stride, 0, pos0 + tokens)
+        else:
+            attn.kv_f16_rows(0, k, v, copies[i % layers], KV, HD, stride, pos0, tokens)
+        attn.chunk_attention_kv_f16(q, copies[i % layers], gate, out, None, H, KV, HD, pos0, tokens, stride,
+                                    acc, ml, splits)
 
     def step(i):
         # RoPE and the append share one launch; the gate is applied where the attention result is
@@ -162,14 +188,20 @@ def bench_prefill(torch, attn, tokens, pos0, steps, warmup, layers, prefix_fill=
 
     unfused_ms = wall(step_unfused)
     wall_ms = wall(step)
+    copy_ms = wall(step_copy)
+    copy_rebuilt_ms = wall(lambda i: step_copy(i, True))
 
     # the attention launch alone, HIP events on the launch stream
-    for i in range(min(warmup, 3)):
-        attention(i)
-    with Timer(torch) as t:
-        for i in range(steps):
-            attention(i)
-    attn_ms = t.ms / steps
+    def events(fn):
+        for i in range(min(warmup, 3)):
+            fn(i)
+        with Timer(torch) as t:
+            for i in range(steps):
+                fn(i)
+        return t.ms / steps
+
+    attn_ms = events(attention)
+    attn_copy_ms = events(attention_copy)
     flop = prefill_flop(pos0, tokens)
     tf = flop / (attn_ms * 1e-3) / 1e12
     wl = {(672, 0): "prefill672", (2048, 100_000): "chunk100k"}.get((tokens, pos0), "")
@@ -183,6 +215,14 @@ def bench_prefill(torch, attn, tokens, pos0, steps, warmup, layers, prefix_fill=
         "ms_per_step_separate_launches": unfused_ms,
         "attn_ms": attn_ms,
         "attn_tok_per_s": tokens / (attn_ms * 1e-3),
+        "over_f16_copy": {
+            "note": "the same step with the attention reading an f16 copy of the cache that the step keeps "
+                    "current (hipml_kv_f16_rows for the chunk's rows after the append, then "
+                    "hipml_attn_chunk_kv_f16); rebuilt = the whole copy made again from row 0 in every step",
+            "ms_per_step": copy_ms, "tok_per_s": tokens / (copy_ms * 1e-3),
+            "ms_per_step_copy_rebuilt": copy_rebuilt_ms,
+            "attn_ms": attn_copy_ms, "attn_frac": flop / (attn_copy_ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TF,
+            "copy_bytes_per_layer": attn.kv_f16_bytes(stride, KV)},
         "roofline": {"bound": "mfma", "achieved": tf, "peak": MFMA_F16_PEAK_TF, "unit": "TFLOP/s",
                      "frac": tf / MFMA_F16_PEAK_TF, "traffic": traffic,
                      "kernel": "chunk_q8_kernel" + (" + chunk_combine_kernel" if splits >= 2 else ""),

@@ -39,6 +39,9 @@ EXPORTS = [
     "hipml_kv_rows_copy", "hipml_rope_encode_chunk_f32",
     "hipml_attn_front_encode_f32", "hipml_attn_chunk_front_encode_f32",
     "hipml_attn_chunk_q8_split_gate_f16",
+    "hipml_kv_f16_bytes",
+    "hipml_kv_f16_rows",
+    "hipml_attn_chunk_kv_f16",
     "hipml_attn_front_rows_f32", "hipml_attn_front_rows_encode_f32",
     "hipml_attn_decode_kv_noalloc", "hipml_rope_allow_device_angles",
 ]
@@ -101,6 +104,9 @@ def lib() -> C.CDLL:
             "hipml_attn_chunk_q8_split": (i, [vp, vp, vp, vp, vp, i, i, i, i, i, i, i, vp, vp, i]),
             "hipml_attn_chunk_q8_split_gate": (i, [vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, i, vp, vp, i]),
             "hipml_attn_chunk_q8_split_gate_f16": (i, [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, i, vp, vp, i]),
+            "hipml_kv_f16_bytes": (sz, [i, i]),
+            "hipml_kv_f16_rows": (i, [vp, i, vp, vp, vp, i, i, i, i, i]),
+            "hipml_attn_chunk_kv_f16": (i, [vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, vp, vp, i]),
             "hipml_q_gate_f32": (i, [vp, vp, vp, vp, sz]),
             "hipml_attn_front_f32": (i, [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, i, i, vp, f, f]),
             "hipml_attn_chunk_front_f32": (i, [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, f, f, i, i]),
@@ -405,6 +411,29 @@ def chunk_attention_q8_split_gate_f16(q, kc, vc, gate, out, out16, n_head, n_kv,
                                                     _p(out), _p(out16), n_head, n_kv, head_dim, pos0,
                                                     tokens, dtype, stride, _p(part_acc), _p(part_ml),
                                                     splits))
+
+
+def kv_f16_bytes(stride: int, n_kv: int) -> int:
+    """Bytes of the f16 copy of a layer cache of `stride` rows per KV head."""
+    return int(lib().hipml_kv_f16_bytes(stride, n_kv))
+
+
+def kv_f16_alloc(stride: int, n_kv: int, device="cuda"):
+    return torch.empty(kv_f16_bytes(stride, n_kv), dtype=torch.uint8, device=device)
+
+
+def kv_f16_rows(dtype, k_cache, v_cache, kv_f16, n_kv, head_dim, stride, start, rows, stream=None):
+    """Bring the tiles of the f16 copy that hold cache rows [start, start + rows) up to date."""
+    _check(lib().hipml_kv_f16_rows(_stream(stream), dtype, _p(k_cache), _p(v_cache), _p(kv_f16), n_kv,
+                                   head_dim, stride, start, rows))
+
+
+def chunk_attention_kv_f16(q, kv_f16, gate, out, out16, n_head, n_kv, head_dim, pos0, tokens, stride,
+                           part_acc, part_ml, splits, stream=None):
+    """Chunk attention over the f16 copy of the cache; gate and out16 may be None."""
+    _check(lib().hipml_attn_chunk_kv_f16(_stream(stream), _p(q), _p(kv_f16), _p(gate), _p(out), _p(out16),
+                                         n_head, n_kv, head_dim, pos0, tokens, stride, _p(part_acc),
+                                         _p(part_ml), splits))
 
 
 def chunk_scratch(tokens: int, n_head: int, splits: int, device="cuda"):

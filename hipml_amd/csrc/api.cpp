@@ -862,7 +862,8 @@ int hipml_attn_decode_batch_cols_gate(hipml_stream_t stream, int dtype, const in
 static int chunk_q8_common(hipml_stream_t stream, const float *q, const void *kc, const void *vc,
                            float *out, const float *gate, bool want_gate, int n_head, int n_kv,
                            int head_dim, int pos0, int tokens, int dtype, int stride, float *part_acc,
-                           float *part_ml, int splits, void *out16 = nullptr, bool want_f16 = false)
+                           float *part_ml, int splits, void *out16 = nullptr, bool want_f16 = false,
+                           const void *kv_f16 = nullptr)
 {
     clear_error();
     REQUIRE_PTR(q);
@@ -907,7 +908,7 @@ static int chunk_q8_common(hipml_stream_t stream, const float *q, const void *kc
     return launch_chunk_q8(as_stream(stream), q, static_cast<const uint8_t *>(kc),
                            static_cast<const uint8_t *>(vc), out, n_head, n_kv, pos0, tokens,
                            stride, part_acc, part_ml, splits, want_gate ? gate : nullptr, dtype == 2 ? 1 : 0,
-                           want_f16 ? out16 : nullptr);
+                           want_f16 ? out16 : nullptr, kv_f16);
 }
 
 int hipml_attn_chunk_q8_split(hipml_stream_t stream, const float *q, const void *kc,
@@ -935,6 +936,53 @@ int hipml_attn_chunk_q8_split_gate_f16(hipml_stream_t stream, const float *q, co
 {
     return chunk_q8_common(stream, q, kc, vc, out, gate, true, n_head, n_kv, head_dim, pos0, tokens,
                            dtype, stride, part_acc, part_ml, splits, out16, true);
+}
+
+// ---- chunk prefill over the f16 copy of a cache ----------------------------------------------------
+
+size_t hipml_kv_f16_bytes(int stride, int n_kv)
+{
+    if (stride < 1 || n_kv < 1)
+        return 0;
+    return kv_f16_bytes(stride, n_kv);
+}
+
+int hipml_kv_f16_rows(hipml_stream_t stream, int dtype, const void *k_cache, const void *v_cache,
+                      void *kv_f16, int n_kv, int head_dim, int stride, int start, int rows)
+{
+    clear_error();
+    REQUIRE_PTR(k_cache);
+    REQUIRE_PTR(v_cache);
+    REQUIRE_PTR(kv_f16);
+    if (dtype != 0 && dtype != 1)
+        return fail(HIPML_ATTN_E_UNSUPPORTED, "KV dtype %d: 0 (q8_0) and 1 (q4_0) are built", dtype);
+    if (head_dim != kHeadDim)
+        return fail(HIPML_ATTN_E_UNSUPPORTED, "head_dim %d: the kernels are built for %d", head_dim, kHeadDim);
+    if (n_kv < 1 || stride < 1)
+        return fail(HIPML_ATTN_E_RANGE, "n_kv %d / stride %d must be positive", n_kv, stride);
+    if (start < 0 || rows < 0 || (long long)start + rows > stride)
+        return fail(HIPML_ATTN_E_RANGE, "rows [%d, %d + %d) do not fit a cache of %d rows per head", start,
+                    start, rows, stride);
+    int rc;
+    if ((rc = check_aligned16(k_cache, "k cache")) || (rc = check_aligned16(v_cache, "v cache")) ||
+        (rc = check_aligned16(kv_f16, "kv_f16")))
+        return rc;
+    if (rows == 0)
+        return 0;
+    if ((rc = require_init()))
+        return rc;
+    return launch_kv_f16_rows(as_stream(stream), static_cast<const uint8_t *>(k_cache),
+                              static_cast<const uint8_t *>(v_cache), kv_f16, n_kv, stride, start, rows, dtype);
+}
+
+int hipml_attn_chunk_kv_f16(hipml_stream_t stream, const float *q, const void *kv_f16, const float *gate,
+                            float *out, void *out16, int n_head, int n_kv, int head_dim, int pos0, int tokens,
+                            int stride, float *part_acc, float *part_ml, int splits)
+{
+    clear_error();
+    REQUIRE_PTR(kv_f16);
+    return chunk_q8_common(stream, q, kv_f16, kv_f16, out, gate, gate != nullptr, n_head, n_kv, head_dim, pos0,
+                           tokens, 1, stride, part_acc, part_ml, splits, out16, out16 != nullptr, kv_f16);
 }
 
 // ---- gate ---------------------------------------------------------------------------------------------

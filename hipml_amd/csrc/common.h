@@ -104,7 +104,13 @@ int decode_static_partials(int n_heads, int splits, float **part_acc, float **pa
 int prefill_init();
 int launch_chunk_q8(hipStream_t st, const float *q, const uint8_t *kc, const uint8_t *vc,
                     float *out, int n_head, int n_kv, int pos0, int tokens, int stride,
-                    float *part_acc, float *part_ml, int splits, const float *gate, int q4, void *out16 = nullptr);
+                    float *part_acc, float *part_ml, int splits, const float *gate, int q4, void *out16 = nullptr,
+                    const void *kv_f16 = nullptr);
+// The f16 copy of a cache that launch_chunk_q8 can read instead of the cache (kv_f16): its size for
+// `stride` rows per KV head, and the conversion of the 64-key tiles that hold rows [start, start + rows).
+size_t kv_f16_bytes(int stride, int n_kv);
+int launch_kv_f16_rows(hipStream_t st, const uint8_t *kc, const uint8_t *vc, void *copy, int n_kv, int stride,
+                       int start, int rows, int q4);
 
 // y[r][row] = W[row][:] . x[r][:] over a Q8_0 weight matrix, rows <= 128 activation rows (proj.hip).
 int launch_gemv_q8_rows(hipStream_t st, const uint8_t *w, const float *x, float *y, int m, int k, int rows);

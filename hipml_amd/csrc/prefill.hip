@@ -48,12 +48,24 @@ constexpr int kBufBytes = kKTile * (kKRow + kVRow);    // 68,608
 constexpr int kQLdsSteps = 3;                          // d-steps of the Q operand parked in LDS
 constexpr int kQLdsOff = 2 * kBufBytes;                // after the two tile buffers (137,216)
 constexpr int kPfLds = kQLdsOff + kTasks * kQLdsSteps * 1024; // 161,792 of 163,840
+// The f16 copy of a cache (hipml_kv_f16_rows): per KV head and 64-key tile, the K rows as they lie in
+// LDS (pitch kKRow) and the V rows transposed, [256 d][64 keys in operand order] with a pitch of 144
+// bytes (128-bit reads of 32 consecutive rows fall into distinct banks).  A tile is then one
+// contiguous piece of memory that global_load_lds copies to LDS as it is.
+constexpr int kVtRow = 144;
+constexpr int kKTileBytes = kKTile * kKRow;              // 33,792
+constexpr int kVtTileBytes = kHeadDim * kVtRow;          // 36,864
+constexpr int kBufBytesF = kKTileBytes + kVtTileBytes;   // 70,656
+constexpr int kPfLdsF = 2 * kBufBytesF;                  // 141,312: no Q steps parked, the staging registers are free
 constexpr float kLog2e = 1.4426950408889634f;
 
 struct ChunkArgs {
     const float *q;
     const uint8_t *kc;
     const uint8_t *vc;
+    const uint8_t *k16; // f16 copy of the cache (F16 kernels): K tiles, [n_kv][tile_stride][kKTileBytes]
+    const uint8_t *vt;  //                                      V^T tiles, [n_kv][tile_stride][kVtTileBytes]
+    int tile_stride;    // tiles per KV head in the copy
     float *out;
     const float *gate; // optional [tokens][n_head][256]: out = attention * sigmoid(gate)
     float *part_acc;
@@ -246,9 +258,36 @@ __device__ __forceinline__ void lds_barrier()
     __builtin_amdgcn_sched_barrier(0);
 }
 
-template <bool SPLIT, bool Q4 = false>
+__device__ __forceinline__ uint32_t lds_address(const void *p)
+{
+    return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void *)p;
+}
+
+// 64 lanes x 16 bytes from base + voff (per lane) to LDS address lds_at + 16 * lane, not through
+// registers.  The compiler neither knows nor waits for these loads: s_waitcnt vmcnt(n) by hand.
+__device__ __forceinline__ void dma16(uint32_t lds_at, const uint8_t *base, uint32_t voff)
+{
+    // (both are the same in every lane; taking them from the first one tells the compiler so)
+    const uint32_t at = __builtin_amdgcn_readfirstlane(lds_at);
+    const uint64_t b = (uint64_t)(uintptr_t)base;
+    // (the builtin returns an int: without the casts its low half would be sign-extended over the high one)
+    const uint64_t bu = (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)b) |
+                        ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(b >> 32)) << 32);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(at), "v"(voff), "s"(bu)
+                 : "memory");
+}
+
+// F16: K and V come from the f16 copy of the cache (a.k16, a.vt), tile by tile through
+// global_load_lds, instead of being dequantized by this workgroup.
+template <bool SPLIT, bool Q4 = false, bool F16 = false>
 __global__ void __launch_bounds__(kPfThreads, 2) chunk_q8_kernel(const ChunkArgs a)
 {
+    static_assert(!(F16 && Q4), "the f16 copy has one format");
+    constexpr int kBuf = F16 ? kBufBytesF : kBufBytes;  // one tile buffer
+    constexpr int kVAt = F16 ? kKTileBytes : kVOff;     // V tile inside it
+    constexpr int kQSteps = F16 ? 0 : kQLdsSteps;       // Q steps parked in LDS
     typedef typename HalfOf<Q4>::type Half;
     constexpr int kRowBytes = Q4 ? hipml::kRowBytesQ4 : hipml::kRowBytes;
     constexpr int kUnitBytes = Q4 ? 36 : 68;
@@ -322,7 +361,13 @@ __global__ void __launch_bounds__(kPfThreads, 2) chunk_q8_kernel(const ChunkArgs
     const int last_tok = ((tt_last + 1) * kQTile < a.tokens ? (tt_last + 1) * kQTile : a.tokens) - 1;
     const int seq_block = a.pos0 + last_tok + 1;
     int klo = 0, khi = seq_block;
-    if (SPLIT) {
+    if (SPLIT && F16) {
+        // whole tiles: the transposed V tiles of the copy start at multiples of kKTile
+        const int tiles_block = (seq_block + kKTile - 1) / kKTile;
+        klo = (int)((long long)tiles_block * split / nsp) * kKTile;
+        khi = (int)((long long)tiles_block * (split + 1) / nsp) * kKTile;
+        khi = khi < seq_block ? khi : seq_block;
+    } else if (SPLIT) {
         klo = (int)((long long)seq_block * split / nsp);
         khi = (int)((long long)seq_block * (split + 1) / nsp);
     }
@@ -352,15 +397,54 @@ __global__ void __launch_bounds__(kPfThreads, 2) chunk_q8_kernel(const ChunkArgs
         key = key < khi ? key : khi - 1;
         return sbase + (size_t)key * kRowBytes;
     };
-    auto issue0 = [&](int t) { load_half0(half, unit_ptr(t)); };
-    auto issue1 = [&](int t) { load_half1(half, unit_ptr(t)); };
-    auto stage0 = [&](int t) { stage_block0(half, lds + (t & 1) * kBufBytes + sdst); };
-    auto stage1 = [&](int t) { stage_block1(half, lds + (t & 1) * kBufBytes + sdst); };
+    auto issue0 = [&](int t) {
+        if constexpr (!F16)
+            load_half0(half, unit_ptr(t));
+    };
+    auto issue1 = [&](int t) {
+        if constexpr (!F16)
+            load_half1(half, unit_ptr(t));
+    };
+    auto stage0 = [&](int t) {
+        if constexpr (!F16)
+            stage_block0(half, lds + (t & 1) * kBuf + sdst);
+    };
+    auto stage1 = [&](int t) {
+        if constexpr (!F16)
+            stage_block1(half, lds + (t & 1) * kBuf + sdst);
+    };
     Half first1; // block 1 of the first tile: fetched together with block 0, ahead of the Q loads
-    if (ntile > 0) {
+    if (!F16 && ntile > 0) {
         issue0(0);
         load_half1(first1, unit_ptr(0));
     }
+    // F16: tile t of the slice is tile klo / kKTile + t of the copy, one contiguous piece per K and per
+    // V^T tile; the 33 (K) and 36 (V^T) KiB go as 1-KiB requests i = wave, wave + 8, ..., five per wave
+    // and tile (the last ones repeat the tile's last KiB, so that every wave's count is the same and
+    // the waits below are constants).  A tile past the slice's last repeats that one: it lands in the
+    // buffer nobody reads any more.
+    constexpr int kDmaPerTile = 5;
+    const uint32_t lds_at = lds_address(lds); // (lane l's 16 bytes land at the request's address + 16 l)
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    auto dma_tile = [&](int t, bool v_tile) {
+        if constexpr (F16) {
+            const int tc = t < ntile ? t : ntile - 1;
+            const size_t tile = (size_t)kvh * a.tile_stride + (klo / kKTile + tc);
+            const uint8_t *src = v_tile ? a.vt + tile * kVtTileBytes : a.k16 + tile * kKTileBytes;
+            const int last = (v_tile ? kVtTileBytes : kKTileBytes) / 1024 - 1;
+            const uint32_t dst = lds_at + (t & 1) * kBuf + (v_tile ? kVAt : 0);
+#pragma unroll
+            for (int j = 0; j < kDmaPerTile; j++) {
+                int i = wave_u + 8 * j;
+                i = i < last ? i : last;
+                dma16(dst + i * 1024, src + i * 1024, lane * 16);
+            }
+        }
+    };
+    auto dma_wait_oldest = [&]() { // all but the newest tile's requests have landed
+        if constexpr (F16)
+            asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
+    };
 
     // ---- Q^T operand: 16 k-steps of 8 f16 (d = ks*16 + lh*8 + j) ---------------------------
     // Steps 0..kQLdsSteps-1 are parked in this wave's corner of LDS and re-read per use: 256
@@ -372,7 +456,7 @@ __global__ void __launch_bounds__(kPfThreads, 2) chunk_q8_kernel(const ChunkArgs
     // which are still unused: a lane-per-token fetch of 16-byte pieces from rows 24 KB apart took
     // several times longer to arrive.  The operand is then read back with the K tile's pattern.
     half8 qf[16];
-    uint8_t *qlds = lds + kQLdsOff + wave * kQLdsSteps * 1024 + lane * 16;
+    uint8_t *qlds = lds + kQLdsOff + wave * kQLdsSteps * 1024 + lane * 16; // (unused when no step is parked)
     {
         uint8_t *qt = lds + wave * (kQTile * kKRow);
         const float *qh = a.q + (size_t)head * kHeadDim + lane * 4;
@@ -399,7 +483,7 @@ __global__ void __launch_bounds__(kPfThreads, 2) chunk_q8_kernel(const ChunkArgs
 #pragma unroll
         for (int ks = 0; ks < 16; ks++) {
             const half8 h = *reinterpret_cast<const half8 *>(qt + ln * kKRow + ks * 32 + lh * 16);
-            if (ks < kQLdsSteps)
+            if (ks < kQSteps)
                 *reinterpret_cast<half8 *>(qlds + ks * 1024) = h;
             else
                 qf[ks] = h;
@@ -420,7 +504,7 @@ __global__ void __launch_bounds__(kPfThreads, 2) chunk_q8_kernel(const ChunkArgs
     // V transpose-read geometry: 16-lane group G = lane/16 covers d rows (G&1)*16.. of the
     // 32-row tile and k half-group lh = G>>1; lane L of the group supplies key (L/4), d run (L%4)*4.
     const int gl = lane & 15;
-    const int vtr_off = kVOff + (gl >> 2) * kVRow + (((lane >> 4) & 1) * 16 + (gl & 3) * 4) * 2;
+    const int vtr_off = kVAt + (gl >> 2) * kVRow + (((lane >> 4) & 1) * 16 + (gl & 3) * 4) * 2;
 
     // a 32-key half of tile t that this task can see at all (wave-uniform)
     auto live = [&](int t, int hk) {
@@ -435,24 +519,24 @@ __global__ void __launch_bounds__(kPfThreads, 2) chunk_q8_kernel(const ChunkArgs
     auto scores = [&](int t, int hk) {
         if (!live(t, hk))
             return;
-        const uint8_t *Kh = lds + (t & 1) * kBufBytes + hk * 32 * kKRow + ln * kKRow + lh * 16;
+        const uint8_t *Kh = lds + (t & 1) * kBuf + hk * 32 * kKRow + ln * kKRow + lh * 16;
         float16v acc;
 #pragma unroll
         for (int i = 0; i < 16; i++)
             acc[i] = 0.0f;
-        half8 A[16], B[kQLdsSteps];
+        half8 A[16], B[kQSteps > 0 ? kQSteps : 1];
 #pragma unroll
-        for (int ks = 0; ks < kQLdsSteps; ks++)
+        for (int ks = 0; ks < kQSteps; ks++)
             B[ks] = *reinterpret_cast<const half8 *>(qlds + ks * 1024);
 #pragma unroll
         for (int ks = 0; ks < 16; ks++)
             A[ks] = *reinterpret_cast<const half8 *>(Kh + ks * 32);
 #pragma unroll
         for (int ks = 0; ks < 16; ks++)
-            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[ks], ks < kQLdsSteps ? B[ks] : qf[ks], acc,
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[ks], ks < kQSteps ? B[ks] : qf[ks], acc,
                                                          0, 0, 0);
         S = acc;
-        __builtin_amdgcn_sched_group_barrier(0x100, 2 + kQLdsSteps, 0); // operands of the first steps
+        __builtin_amdgcn_sched_group_barrier(0x100, 2 + kQSteps, 0); // operands of the first steps
 #pragma unroll
         for (int ks = 0; ks < 14; ks++) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // 1 MFMA
@@ -506,24 +590,34 @@ __global__ void __launch_bounds__(kPfThreads, 2) chunk_q8_kernel(const ChunkArgs
     auto pv = [&](int t, int hk) {
         if (!live(t, hk))
             return;
-        const uint8_t *Vh = lds + (t & 1) * kBufBytes + vtr_off + hk * 32 * kVRow;
         half8 A[16];
+        if constexpr (F16) {
+            // row d of the transposed tile holds the keys in operand order: one 128-bit read per operand
+            const uint8_t *Vt = lds + (t & 1) * kBuf + kVAt + ln * kVtRow + (hk * 32 + lh * 8) * 2;
 #pragma unroll
-        for (int u = 0; u < 2; u++) {
+            for (int u = 0; u < 2; u++)
 #pragma unroll
-            for (int dt = 0; dt < 8; dt++) {
-                // keys of read q: (2u+q)*8 + lh*4 + {0..3}
-                const uint8_t *vp = Vh + dt * 64;
-                const short4v r0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                    (short4v __attribute__((address_space(3))) *)(vp + ((2 * u) * 8 + lh * 4) * kVRow));
-                const short4v r1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                    (short4v __attribute__((address_space(3))) *)(vp + ((2 * u + 1) * 8 + lh * 4) * kVRow));
-                const half4 h0 = __builtin_bit_cast(half4, r0);
-                const half4 h1 = __builtin_bit_cast(half4, r1);
+                for (int dt = 0; dt < 8; dt++)
+                    A[u * 8 + dt] = *reinterpret_cast<const half8 *>(Vt + dt * 32 * kVtRow + u * 32);
+        } else {
+            const uint8_t *Vh = lds + (t & 1) * kBuf + vtr_off + hk * 32 * kVRow;
 #pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    A[u * 8 + dt][j] = h0[j];
-                    A[u * 8 + dt][4 + j] = h1[j];
+            for (int u = 0; u < 2; u++) {
+#pragma unroll
+                for (int dt = 0; dt < 8; dt++) {
+                    // keys of read q: (2u+q)*8 + lh*4 + {0..3}
+                    const uint8_t *vp = Vh + dt * 64;
+                    const short4v r0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                        (short4v __attribute__((address_space(3))) *)(vp + ((2 * u) * 8 + lh * 4) * kVRow));
+                    const short4v r1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                        (short4v __attribute__((address_space(3))) *)(vp + ((2 * u + 1) * 8 + lh * 4) * kVRow));
+                    const half4 h0 = __builtin_bit_cast(half4, r0);
+                    const half4 h1 = __builtin_bit_cast(half4, r1);
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        A[u * 8 + dt][j] = h0[j];
+                        A[u * 8 + dt][4 + j] = h1[j];
+                    }
                 }
             }
         }
@@ -532,11 +626,12 @@ __global__ void __launch_bounds__(kPfThreads, 2) chunk_q8_kernel(const ChunkArgs
 #pragma unroll
             for (int dt = 0; dt < 8; dt++)
                 O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[u * 8 + dt], P[u], O[dt], 0, 0, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 4, 0); // 2 operands up front
+        constexpr int kReads = F16 ? 1 : 2; // LDS reads per operand
+        __builtin_amdgcn_sched_group_barrier(0x100, 2 * kReads, 0); // 2 operands up front
 #pragma unroll
         for (int k = 0; k < 14; k++) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, kReads, 0);
         }
         __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
     };
@@ -556,7 +651,15 @@ __global__ void __launch_bounds__(kPfThreads, 2) chunk_q8_kernel(const ChunkArgs
     // M1(t-1), which set 1 finished one slot before V1(t), and K(t+1) is first read in M2(t).  Set 1
     // writes V(t+1) in its V1(t) and V2(t), which are set 0's M1(t) and M2(t); the V(t-1) it replaces
     // was last read in M2(t-1), finished by both sets before that, and V(t+1) is first read in M1(t+1).
-    if (ntile > 0) {
+    if constexpr (F16) {
+        // K(t + 1) is requested at the head of the slot M2(t - 1) and waited for at the end of M1(t), V(t + 1)
+        // at the head of M1(t) and the end of M2(t): each has three slots to arrive in, and the buffer it
+        // lands in was last read one slot before the request, by either set.
+        dma_tile(0, false);
+        dma_tile(0, true);
+        dma_tile(1, false);
+        dma_wait_oldest();
+    } else if (ntile > 0) {
         stage0(0);
         stage_block1(first1, lds + sdst);
         issue0(1);
@@ -573,21 +676,27 @@ __global__ void __launch_bounds__(kPfThreads, 2) chunk_q8_kernel(const ChunkArgs
         issue1(t + 1);
         softmax(t, 0);
         lds_barrier();
+        dma_tile(t + 1, true);
         pv(t, 0);
         scores(t, 1);
+        dma_wait_oldest();
         lds_barrier();
         if (t + 1 < ntile)
             stage1(t + 1);
         issue0(t + 2);
         softmax(t, 1);
         lds_barrier();
+        dma_tile(t + 2, false);
         pv(t, 1);
         if (t + 1 < ntile)
             scores(t + 1, 0);
+        dma_wait_oldest();
         lds_barrier();
     }
     if (set == 0)
         lds_barrier();
+    if constexpr (F16)
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // the tile buffers are about to be reused
 
     // ---- epilogue --------------------------------------------------------------------------
     l_run += __shfl_xor(l_run, 32);
@@ -762,6 +871,96 @@ __global__ void __launch_bounds__(256) rows_f16_kernel(const float4v *__restrict
         y[i] = __builtin_convertvector(x[i], half4);
 }
 
+// The f16 copy of 64-key tiles of a cache: what a chunk workgroup would stage for itself, made once.
+// grid (tiles, n_kv); tile = tile0 + blockIdx.x; rows at or past seq_end repeat row seq_end - 1 (the
+// attention kernels mask them; a later call that brings the rows overwrites the tile).
+// The K rows leave as they lie in LDS; the V tile leaves through the transposing reads of the PV
+// product, so row d of the copy holds, for every 16 keys, the eight values of k-group 0 and the eight
+// of k-group 1 in operand order (key (j/4)*8 + g*4 + j%4 of the sixteen at position g*8 + j).
+template <bool Q4>
+__global__ void __launch_bounds__(256) kv_f16_tiles_kernel(const uint8_t *__restrict__ kc,
+                                                           const uint8_t *__restrict__ vc, uint8_t *__restrict__ k16,
+                                                           uint8_t *__restrict__ vt, int stride, int tile0,
+                                                           int seq_end, int tile_stride)
+{
+    typedef typename HalfOf<Q4>::type Half;
+    constexpr int kRowBytes = Q4 ? hipml::kRowBytesQ4 : hipml::kRowBytes;
+    constexpr int kUnitBytes = Q4 ? 36 : 68;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const int tile = tile0 + blockIdx.x;
+    const int kvh = blockIdx.y;
+    const int su = threadIdx.x;
+    const int lane = su & 63, wave = su >> 6;
+    // thread -> (row, unit) as in the chunk kernel's staging: conflict-free 128-bit LDS writes
+    const int srow = (su >> 6) * 16 + ((su >> 1) & 7) + ((su >> 5) & 1) * 8;
+    const int spr = (su & 1) | ((su >> 3) & 2);
+    int key = tile * kKTile + srow;
+    key = key < seq_end ? key : seq_end - 1;
+    const size_t src = ((size_t)kvh * stride + key) * kRowBytes + spr * kUnitBytes;
+    Half hk0, hk1, hv0, hv1;
+    load_half0(hk0, kc + src);
+    load_half1(hk1, kc + src);
+    load_half0(hv0, vc + src);
+    load_half1(hv1, vc + src);
+    uint8_t *kd = lds + srow * kKRow + spr * 128;
+    uint8_t *vd = lds + kVOff + srow * kVRow + spr * 128;
+    stage_block0(hk0, kd);
+    stage_block1(hk1, kd);
+    stage_block0(hv0, vd);
+    stage_block1(hv1, vd);
+    __syncthreads();
+    const size_t at = (size_t)kvh * tile_stride + tile;
+    {
+        const uint4v *from = reinterpret_cast<const uint4v *>(lds);
+        uint4v *to = reinterpret_cast<uint4v *>(k16 + at * kKTileBytes);
+        for (int i = su; i < kKTileBytes / 16; i += 256)
+            to[i] = from[i];
+    }
+    {
+        const int ln = lane & 31, lh = lane >> 5, gl = lane & 15;
+        const int vtr_off = kVOff + (gl >> 2) * kVRow + (((lane >> 4) & 1) * 16 + (gl & 3) * 4) * 2;
+        uint8_t *to = vt + at * kVtTileBytes;
+#pragma unroll
+        for (int o8 = 0; o8 < 8; o8++) {
+            const int o = wave * 8 + o8; // operand (half hk, step u, d tile dt) of the tile's 32
+            const int hk = o >> 4, u = (o >> 3) & 1, dt = o & 7;
+            const uint8_t *vp = lds + vtr_off + hk * 32 * kVRow + dt * 64;
+            const short4v r0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                (short4v __attribute__((address_space(3))) *)(vp + ((2 * u) * 8 + lh * 4) * kVRow));
+            const short4v r1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                (short4v __attribute__((address_space(3))) *)(vp + ((2 * u + 1) * 8 + lh * 4) * kVRow));
+            const uint32_t *w0 = reinterpret_cast<const uint32_t *>(&r0), *w1 = reinterpret_cast<const uint32_t *>(&r1);
+            const uint4v piece = {w0[0], w0[1], w1[0], w1[1]};
+            *reinterpret_cast<uint4v *>(to + (dt * 32 + ln) * kVtRow + (hk * 32 + u * 16 + lh * 8) * 2) = piece;
+        }
+    }
+}
+
+size_t kv_f16_bytes(int stride, int n_kv)
+{
+    const size_t tiles = ((size_t)stride + kKTile - 1) / kKTile;
+    return (size_t)n_kv * tiles * kBufBytesF;
+}
+
+int launch_kv_f16_rows(hipStream_t st, const uint8_t *kc, const uint8_t *vc, void *copy, int n_kv, int stride,
+                       int start, int rows, int q4)
+{
+    if (rows < 1)
+        return 0;
+    const int tile_stride = (stride + kKTile - 1) / kKTile;
+    uint8_t *k16 = static_cast<uint8_t *>(copy);
+    uint8_t *vt = k16 + (size_t)n_kv * tile_stride * kKTileBytes;
+    const int tile0 = start / kKTile, tile1 = (start + rows + kKTile - 1) / kKTile;
+    const dim3 grid((unsigned)(tile1 - tile0), (unsigned)n_kv, 1);
+    if (q4)
+        hipLaunchKernelGGL(kv_f16_tiles_kernel<true>, grid, dim3(256, 1, 1), kBufBytes, st, kc, vc, k16, vt, stride,
+                           tile0, start + rows, tile_stride);
+    else
+        hipLaunchKernelGGL(kv_f16_tiles_kernel<false>, grid, dim3(256, 1, 1), kBufBytes, st, kc, vc, k16, vt, stride,
+                           tile0, start + rows, tile_stride);
+    return launched("kv_f16_rows");
+}
+
 int prefill_init()
 {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&chunk_q8_kernel<false>),
@@ -775,6 +974,18 @@ int prefill_init()
     if (e == hipSuccess)
         e = hipFuncSetAttribute(reinterpret_cast<const void *>(&chunk_q8_kernel<true, true>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, kPfLds);
+    if (e == hipSuccess)
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&chunk_q8_kernel<false, false, true>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, kPfLdsF);
+    if (e == hipSuccess)
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&chunk_q8_kernel<true, false, true>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, kPfLdsF);
+    if (e == hipSuccess)
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&kv_f16_tiles_kernel<false>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, kBufBytes);
+    if (e == hipSuccess)
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&kv_f16_tiles_kernel<true>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, kBufBytes);
     if (e != hipSuccess)
         return fail((int)e, "hipFuncSetAttribute(prefill LDS) failed: %d (%s)", (int)e,
                     hipGetErrorString(e));
@@ -783,9 +994,14 @@ int prefill_init()
 
 int launch_chunk_q8(hipStream_t st, const float *q, const uint8_t *kc, const uint8_t *vc,
                     float *out, int n_head, int n_kv, int pos0, int tokens, int stride,
-                    float *part_acc, float *part_ml, int splits, const float *gate, int q4, void *out16)
+                    float *part_acc, float *part_ml, int splits, const float *gate, int q4, void *out16,
+                    const void *kv_f16)
 {
     ChunkArgs a;
+    // kv_f16 != nullptr: K and V are read from the f16 copy of the cache (kc, vc unused)
+    a.tile_stride = (stride + kKTile - 1) / kKTile;
+    a.k16 = static_cast<const uint8_t *>(kv_f16);
+    a.vt = a.k16 + (size_t)n_kv * a.tile_stride * kKTileBytes;
     a.gate = gate;
     a.q = q;
     a.kc = kc;
@@ -829,11 +1045,13 @@ int launch_chunk_q8(hipStream_t st, const float *q, const uint8_t *kc, const uin
             grid = (unsigned)(combos * a.nblock);
     }
     if (splits < 2) {
-        if (q4)
+        if (kv_f16)
+            hipLaunchKernelGGL((chunk_q8_kernel<false, false, true>), dim3(grid, 1, 1), block, kPfLdsF, st, a);
+        else if (q4)
             hipLaunchKernelGGL((chunk_q8_kernel<false, true>), dim3(grid, 1, 1), block, kPfLds, st, a);
         else
             hipLaunchKernelGGL(chunk_q8_kernel<false>, dim3(grid, 1, 1), block, kPfLds, st, a);
-        int rc = launched(q4 ? "attn_chunk_q4" : "attn_chunk_q8");
+        int rc = launched(kv_f16 ? "attn_chunk_f16" : q4 ? "attn_chunk_q4" : "attn_chunk_q8");
         if (rc || out16 == nullptr)
             return rc;
         const size_t n4 = (size_t)tokens * n_head * kHeadDim / 4;
@@ -841,11 +1059,13 @@ int launch_chunk_q8(hipStream_t st, const float *q, const uint8_t *kc, const uin
                            reinterpret_cast<const float4v *>(out), static_cast<half4 *>(out16), n4);
         return launched("attn_chunk_rows_f16");
     }
-    if (q4)
+    if (kv_f16)
+        hipLaunchKernelGGL((chunk_q8_kernel<true, false, true>), dim3(grid, 1, 1), block, kPfLdsF, st, a);
+    else if (q4)
         hipLaunchKernelGGL((chunk_q8_kernel<true, true>), dim3(grid, 1, 1), block, kPfLds, st, a);
     else
         hipLaunchKernelGGL(chunk_q8_kernel<true>, dim3(grid, 1, 1), block, kPfLds, st, a);
-    int rc = launched(q4 ? "attn_chunk_q4_split" : "attn_chunk_q8_split");
+    int rc = launched(kv_f16 ? "attn_chunk_f16_split" : q4 ? "attn_chunk_q4_split" : "attn_chunk_q8_split");
     if (rc)
         return rc;
     hipLaunchKernelGGL(chunk_combine_kernel, dim3((unsigned)tokens, (unsigned)((n_head + 3) / 4), 1),

@@ -346,6 +346,37 @@ int hipml_attn_chunk_q8_split_gate_f16(hipml_stream_t stream, const float *q, co
                                        int n_head, int n_kv, int head_dim, int pos0, int tokens, int dtype,
                                        int stride, float *part_acc, float *part_ml, int splits);
 
+/* ---- chunk prefill over an f16 copy of the cache -------------------------------------------------
+ * The reference's chunk kernel dequantizes the cache rows it attends over inside every workgroup
+ * (crates/hipml-kernels/kernels/attn_chunk_wmma.hip:187-399), and so do the entry points above: at a
+ * long prefix that is 40 % of the kernel's vector instructions, done once per 256 (token, head)
+ * pairs.  These three have no counterpart in the reference.  They keep a second form of a layer's
+ * cache, f16(d * q) of every K and V value (exactly the operands the kernels above compute), laid
+ * out in 64-key tiles the way the attention kernel wants them in LDS, K rows as they are and V
+ * transposed; the attention kernel then copies whole tiles and spends its vector instructions on
+ * the softmax alone.  The copy costs hipml_kv_f16_bytes(stride, n_kv) = n_kv * ceil(stride / 64) *
+ * 70,656 bytes per layer cache (450 MB for 102,048 rows) and is kept up to date by the caller: after
+ * appending rows [start, start + rows) to the cache, call hipml_kv_f16_rows for the same rows.  It
+ * rewrites every 64-key tile that holds one of them from the tile's first row on, so a partly
+ * filled tile is completed by the next call; rows of a tile at or past start + rows hold copies
+ * of row start + rows - 1.  One copy can also be shared by all layers and rebuilt from row 0
+ * before each layer's attention (start = 0, rows = pos0 + tokens: one pass over the cache).
+ * dtype is the KvDtype id of the cache, as for the append entry points (0 = q8_0, 1 = q4_0).
+ * kv_f16 is 16-byte aligned device memory of at least hipml_kv_f16_bytes(stride, n_kv). */
+size_t hipml_kv_f16_bytes(int stride, int n_kv);
+int hipml_kv_f16_rows(hipml_stream_t stream, int dtype, const void *k_cache, const void *v_cache,
+                      void *kv_f16, int n_kv, int head_dim, int stride, int start, int rows);
+
+/* hipml_attn_chunk_q8_split (splits >= 2, with scratch) or hipml_attn_chunk_q8 (splits <= 1) over the
+ * copy: rows [0, pos0 + tokens) of kv_f16 must be current.  gate (may be NULL) and out16 (may be NULL)
+ * as in hipml_attn_chunk_q8_split_gate / _gate_f16.  The operands are the same values, so results
+ * differ from those entry points only through the key slices, which here end at multiples of 64
+ * keys.  Same scratch sizes, same split policy (hipml_attn_chunk_splits). */
+int hipml_attn_chunk_kv_f16(hipml_stream_t stream, const float *q, const void *kv_f16,
+                            const float *gate, float *out, void *out16, int n_head, int n_kv,
+                            int head_dim, int pos0, int tokens, int stride, float *part_acc,
+                            float *part_ml, int splits);
+
 /* ---- output gate ------------------------------------------------------------ */
 
 /* y[i] = x[i] * sigmoid(gate[i]); y may alias x.  Replaces
