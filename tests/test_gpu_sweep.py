@@ -109,6 +109,20 @@ def test_chunk_sweep(i, n_kv, group, tok, pos0, pad, splits, q4):
     ok, ma, mr = orc.compare(want, host(out), *CHUNK_GATE)
     assert ok, f"case {i}: kv {n_kv} group {group} tok {tok} pos0 {pos0} pad {pad} splits {splits} q4 {q4}: " \
                f"max_abs {ma:.3e} max_rel {mr:.3e}"
+    # the same chunk over the f16 copy of the cache, brought up to date in two calls
+    copy = attn.kv_f16_alloc(stride, n_kv)
+    copy.fill_(0xFF)
+    first = (pos0 + tok) // 2
+    attn.kv_f16_rows(dtype, dev(kb), dev(vb), copy, n_kv, HD, stride, 0, first)
+    attn.kv_f16_rows(dtype, dev(kb), dev(vb), copy, n_kv, HD, stride, first, pos0 + tok - first)
+    out.fill_(float("nan"))
+    if splits >= 2:
+        acc.fill_(float("nan"))
+        ml.fill_(float("nan"))
+    attn.chunk_attention_kv_f16(dev(q), copy, None, out, None, n_heads, n_kv, HD, pos0, tok, stride, acc, ml, splits)
+    torch.cuda.synchronize()
+    ok, ma, mr = orc.compare(want, host(out), *CHUNK_GATE)
+    assert ok, f"case {i} over the f16 copy: max_abs {ma:.3e} max_rel {mr:.3e}"
 
 
 def proj_cases(n):
