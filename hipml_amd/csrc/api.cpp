@@ -226,7 +226,7 @@ int hipml_attn_init(int device)
 
 const char *hipml_attn_last_error(void) { return g_err; }
 
-const char *hipml_attn_version(void) { return "hipml-attn-mi355x 0.1 (gfx950)"; }
+const char *hipml_attn_version(void) { return "hipml-attn-mi355x 0.2 (gfx950)"; }
 
 // ---- split policies -------------------------------------------------------------------
 
