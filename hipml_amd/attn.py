@@ -494,6 +494,20 @@ class DeepKv:
                                     dtype=torch.float32, device=device)
         self.part_ml = torch.empty((max_cols, n_heads, self.max_splits, 2), dtype=torch.float32,
                                    device=device)
+        self.f16 = None  # the optional f16 copy of the rows (enable_f16_copy)
+
+    def enable_f16_copy(self, live: int = 0, stream=None):
+        """Keep an f16 copy of this cache for chunk prefill over long prefixes (chunk_attention_kv_f16
+        reads it); `live` rows are converted now, later appends are followed by sync_f16."""
+        if self.f16 is None:
+            self.f16 = kv_f16_alloc(self.seq, self.n_kv, self.k.device)
+        self.sync_f16(0, live, stream)
+
+    def sync_f16(self, start: int, rows: int, stream=None):
+        """After rows [start, start + rows) were appended (or restored): bring the copy up to date."""
+        if self.f16 is not None and rows > 0:
+            kv_f16_rows(self.dtype, self.k, self.v, self.f16, self.n_kv, self.head_dim, self.seq, start, rows,
+                        stream)
 
     def splits(self, seq: int) -> int:
         return min(decode_splits(seq, self.n_kv), self.max_splits)
@@ -519,6 +533,7 @@ class DeepKv:
         if pos > 0:
             kv_rows_copy(self.dtype, k, v, self.k, self.v, self.n_kv, self.head_dim, pos, self.seq, pos,
                          stream)
+            self.sync_f16(0, pos, stream)
 
 
 class BatchKv:

@@ -154,3 +154,21 @@ def test_argument_errors_are_reported():
     with pytest.raises(attn.HipmlError):
         attn.kv_f16_rows(3, kb, kb, copy, N_KV, HD, 128, 0, 10)  # unknown format
     assert attn.kv_f16_bytes(0, 4) == 0
+
+
+def test_cache_owner_keeps_its_copy_current_through_append_and_restore():
+    # DeepKv with a copy: a prefix restored into it and a chunk appended after it give the attention over the
+    # copy the same rows as the attention over the cache
+    tok, pos0, pad = 48, 200, 8
+    q, kb, vb, stride = chunk_inputs(0xF16_0002, tok, pos0, pad)
+    kv = attn.DeepKv(N_HEADS, N_KV, HD, stride)
+    kv.enable_f16_copy()
+    kv.restore(dev(kb[:, :pos0].copy()), dev(vb[:, :pos0].copy()))  # the prefix, as a snapshot would bring it
+    kv.k[:, pos0:pos0 + tok] = dev(kb[:, pos0:pos0 + tok].copy())  # the chunk's rows, as an append leaves them
+    kv.v[:, pos0:pos0 + tok] = dev(vb[:, pos0:pos0 + tok].copy())
+    kv.sync_f16(pos0, tok)
+    out = torch.full((tok, N_HEADS, HD), float("nan"), dtype=torch.float32, device="cuda")
+    attn.chunk_attention_kv_f16(dev(q), kv.f16, None, out, None, N_HEADS, N_KV, HD, pos0, tok, stride, None, None, 1)
+    torch.cuda.synchronize()
+    want = run_chunk(q, kb, vb, pos0, tok, stride, 1)
+    assert np.array_equal(host(out).view(np.uint32), want.view(np.uint32))
