@@ -263,7 +263,10 @@ int hipml_attn_decode_batch(hipml_stream_t stream, int dtype, const int32_t *pos
  * rows that share slot s's cache (plain slots and MTP-verify slots mixed in ONE
  * launch).  Rows are numbered slot-major: row r has (pos,seq) = pos[r*2..],
  * q + r*q_slot, scratch r*acc_slot / r*ml_slot; slot s's cache is base +
- * s*kv_slot_bytes.  cols_per_slot is a HOST array read during the call.
+ * s*kv_slot_bytes.  cols_per_slot is a HOST array read during the call: the rows per slot
+ * become part of the launch (its grid and item tables), so a graph captured around this
+ * call replays that layout; positions and live lengths stay device data and may change
+ * between replays.
  * The reference has no single-launch form of this: it issues one launch pair
  * per verify slot (crates/hipml-model/src/gpu/batch/verify.rs:321-366). */
 int hipml_attn_decode_batch_cols(hipml_stream_t stream, int dtype, const int32_t *pos,
