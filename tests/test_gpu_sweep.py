@@ -125,6 +125,32 @@ def test_chunk_sweep(i, n_kv, group, tok, pos0, pad, splits, q4):
     assert ok, f"case {i} over the f16 copy: max_abs {ma:.3e} max_rel {mr:.3e}"
 
 
+def batch_cases(n):
+    r = orc.Rng(0x5EE9_0004)
+    cases = []
+    for i in range(n):
+        slots = (1, 2, 3, 5, 8, 16, 24, 40)[draw(r, 0, 7)]
+        cols = [(1, 1, 1, 2, 3, 4)[draw(r, 0, 5)] for _ in range(slots)]
+        deep = draw(r, 0, 3) == 0
+        depths = [draw(r, 0, 2500 if deep else 300) for _ in range(slots)]
+        if slots > 1:
+            depths[draw(r, 0, slots - 1)] = 0  # a slot whose only keys are its own rows
+        stride = max(d + c for d, c in zip(depths, cols)) + draw(r, 0, 100)
+        splits = (1, 2, 5, 8, 32)[draw(r, 0, 4)]
+        cases.append((i, depths, cols, stride, splits))
+    return cases
+
+
+@pytest.mark.parametrize("i,depths,cols,stride,splits", batch_cases(16))
+def test_batch_sweep(i, depths, cols, stride, splits):
+    # plain and verify slots mixed in one launch: work items of 6 to 16 columns, worker launches (few
+    # items) and plain grids (many), slots at depth 0, depths around tile and split edges
+    from test_gpu_configs import _batch
+    worst = _batch(depths, cols, stride, 0xBA7C_0000 + i, splits)
+    print(f"[parity] batch sweep {i}: {len(depths)} slots, {sum(cols)} rows, stride {stride}, splits {splits}: "
+          f"worst max_abs {worst:.3e}", flush=True)
+
+
 def proj_cases(n):
     r = orc.Rng(0x5EE9_0003)
     return [(i, draw(r, 1, 300), 64 * draw(r, 1, 40), draw(r, 1, 9)) for i in range(n)]
