@@ -114,6 +114,23 @@ def test_config4_chunk_2048_at_100000_sampled_rows():
     plain = [h for h in range(N_HEADS) if h % (N_HEADS // N_KV) != 0]
     ok, ma, _ = report("config 4: heads without a needle", want[:, plain], got[rows][:, plain], 1e-4, 0.0)
     assert ok
+    # the same chunk over the f16 copy of the cache: the prefix converted first, the chunk's rows after it
+    kd, vd = dev(kb), dev(vb)
+    copy = attn.kv_f16_alloc(stride, N_KV)
+    attn.kv_f16_rows(0, kd, vd, copy, N_KV, HD, stride, 0, pos0)
+    attn.kv_f16_rows(0, kd, vd, copy, N_KV, HD, stride, pos0, tok)
+    out.fill_(float("nan"))
+    acc.fill_(float("nan"))
+    ml.fill_(float("nan"))
+    attn.chunk_attention_kv_f16(dev(q), copy, None, out, None, N_HEADS, N_KV, HD, pos0, tok, stride, acc, ml, splits)
+    torch.cuda.synchronize()
+    got = host(out)
+    assert np.isfinite(got).all()
+    ok, _, _ = report(f"config 4 over the f16 copy: splits {splits}, {len(rows)} rows", want, got[rows], *GATE)
+    assert ok
+    ok, ma, _ = report("config 4 over the f16 copy: heads without a needle", want[:, plain], got[rows][:, plain],
+                       1e-4, 0.0)
+    assert ok
 
 
 def _batch(depths, cols, stride, seed, splits):
