@@ -1313,34 +1313,58 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Work 
     // table, so nothing has to be waited for before the writes; the other waves read them after the
     // barrier.
     l_run = quad_rows<false>(l_run);
-    float *wl = reinterpret_cast<float *>(wave_lds); // per wave: [kCols][272] acc by byte column
+    // 8 columns: the rows are 276 floats apart and the lanes of MFMA columns 8..15, which hold the same
+    // values as columns 0..7, write the run ten further on, so that the sixteen lanes of a k-group cover
+    // all 64 banks once per 128-bit write (measured for four waves parking at once: 470 cycles against
+    // 1,360 with rows of 272 floats written by half the lanes).  16 columns keep rows of 272 floats: 276
+    // would reach into the next wave's rows.
+    constexpr int kParkPitch = WIDE ? kRowBytes : kRowBytes + 4;
+    float *wl = reinterpret_cast<float *>(wave_lds); // per wave: [kCols][kParkPitch] acc by byte column
     float *wml = reinterpret_cast<float *>(sK);  // per wave: [kCols] m, [kCols] l
     {
-        if (WIDE || lm < 8) {
-            const int nc = lm & (kCols - 1);
+        auto run_values = [&](int j) {
+            float4v v;
+            if (j >= 2 && j <= 12 && (j & 1) == 0) {
+                // columns of blocks j/2 - 1 (below byte 34 * (j/2)) and j/2
+                const int c1 = j / 2;
+                const float4v lo = O[3 * c1 - 1];
+                const float4v up = O[3 * c1];
 #pragma unroll
-            for (int j = 0; j < kRuns; j++) {
-                float4v v;
-                if (j >= 2 && j <= 12 && (j & 1) == 0) {
-                    // columns of blocks j/2 - 1 (below byte 34 * (j/2)) and j/2
-                    const int c1 = j / 2;
-                    const float4v lo = O[3 * c1 - 1];
-                    const float4v up = O[3 * c1];
+                for (int i = 0; i < 4; i++)
+                    v[i] = 16 * j + lg * 4 + i < kQ8BlockBytes * c1 ? lo[i] : up[i];
+            } else {
+                const int idx = j == 0 ? 0 : (j >= 14 ? j + 6 : 3 * (j - 1) / 2 + 1);
+                v = O[idx];
+                if (j == 14) // byte column 238, the scale of block 7: its correction row
+                    v[2] = lg == 3 ? B7[2] : v[2];
+            }
+            return v;
+        };
+        const int pc = lm & (kCols - 1); // the column this lane parks
+        if (WIDE) {
 #pragma unroll
-                    for (int i = 0; i < 4; i++)
-                        v[i] = 16 * j + lg * 4 + i < kQ8BlockBytes * c1 ? lo[i] : up[i];
-                } else {
-                    const int idx = j == 0 ? 0 : (j >= 14 ? j + 6 : 3 * (j - 1) / 2 + 1);
-                    v = O[idx];
-                    if (j == 14) // byte column 238, the scale of block 7: its correction row
-                        v[2] = lg == 3 ? B7[2] : v[2];
+            for (int j = 0; j < kRuns; j++)
+                *reinterpret_cast<float4v *>(wl + pc * kParkPitch + j * 16 + lg * 4) = run_values(j);
+        } else {
+            static_assert(kRuns == 17, "runs j and j + 10 for j < 7, 7 and 9, and 8 alone");
+            const bool first = lm < 8;
+#pragma unroll
+            for (int j = 0; j < 9; j++) {
+                const int jp = j < 7 ? j + 10 : 9;
+                const float4v a4 = run_values(j);
+                if (j < 8) {
+                    const float4v b4 = run_values(jp);
+                    const float4v v = {first ? a4[0] : b4[0], first ? a4[1] : b4[1], first ? a4[2] : b4[2],
+                                       first ? a4[3] : b4[3]};
+                    *reinterpret_cast<float4v *>(wl + pc * kParkPitch + (first ? j : jp) * 16 + lg * 4) = v;
+                } else if (first) {
+                    *reinterpret_cast<float4v *>(wl + pc * kParkPitch + j * 16 + lg * 4) = a4;
                 }
-                *reinterpret_cast<float4v *>(wl + nc * kRowBytes + j * 16 + lg * 4) = v;
             }
-            if (lg == 0) {
-                wml[nc] = m_run;
-                wml[kCols + nc] = l_run;
-            }
+        }
+        if ((WIDE || lm < 8) && lg == 0) {
+            wml[pc] = m_run;
+            wml[kCols + pc] = l_run;
         }
         __syncthreads();
         // thread -> (column nc, kRun consecutive d of one block): kCols columns x kThreads / kCols runs of d
@@ -1376,7 +1400,7 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Work 
                 float4v acc = {0, 0, 0, 0};
 #pragma unroll
                 for (int w = 0; w < kWaves; w++) {
-                    const float *row = reinterpret_cast<const float *>(lds_all + w * kDmaWaveLds) + nc * kRowBytes;
+                    const float *row = reinterpret_cast<const float *>(lds_all + w * kDmaWaveLds) + nc * kParkPitch;
                     const float off = row[(d0 >> 5) * kQ8BlockBytes]; // the block's correction row
                     const float2 x0 = *reinterpret_cast<const float2 *>(row + col0 + dd);
                     const float2 x1 = *reinterpret_cast<const float2 *>(row + col0 + dd + 2);
