@@ -1,12 +1,18 @@
-// Split-K decode attention over a q8_0 KV cache for gfx950 (wave64, MFMA).
+// Split-K decode attention over a quantized KV cache for gfx950 (wave64, MFMA).
 //
-// One workgroup (4 waves) owns one (kv head, key split, work item = slot or half of its heads).  Each wave walks
-// its own 32-key tiles of the split with a private online softmax and no
-// workgroup barrier in the loop; the four waves merge in LDS at the end and
-// write one unnormalised partial per (row, head, split).  A second kernel
-// merges the splits.
+// One workgroup (4 waves) owns one (kv head, key split, work item = the (row, head) columns of a slot
+// or a part of them).  Each wave walks its own 32-key tiles of the split with a private online softmax
+// and no workgroup barrier in the loop; the four waves merge in LDS at the end and write one
+// unnormalised partial per (row, head, split).  A second kernel merges the splits.
 //
-// Memory pipeline.  A tile's K (or V) rows are 32 x 272 contiguous bytes.  A
+// Two split kernels live here.
+//
+// decode_q8_kernel (q8_0, the shipped path; described where it is defined): the rows of a tile go
+// from the cache to LDS as they lie (global_load_lds), and the MFMA operands are made where they are
+// read.  Work items carry up to 8 columns (the two f16 halves of Q share one MFMA) or 9 to 16 (two MFMAs).
+//
+// decode_staged_kernel (q4_0, and q8_0 with fp32-class weights): the first kernel of this build.
+// Memory pipeline: a tile's K (or V) rows are 32 x 272 contiguous bytes.  A
 // lane fetches "units" of 68 bytes = two whole 34-byte blocks of one key, with
 // dword-aligned 128-bit loads; a wave's load instruction covers a
 // contiguous 4,352-byte span.  Two tiles (K and V each) are kept in flight per
@@ -15,23 +21,23 @@
 // [32 keys][288 B]; block scales go to a transposed f16 table [8 blocks][32 keys].
 // K and V of a tile use the same LDS tile one after the other.
 //
-// Arithmetic (all MFMAs are v_mfma_f32_16x16x32_f16):
-//   S^T[key][n]  = K[key][:] . Q^T[:][n]      A = K bytes as f16, B = Q (hi + lo f16, from LDS)
+// Arithmetic of both (all MFMAs are v_mfma_f32_16x16x32_f16):
+//   S^T[key][n]  = K[key][:] . Q^T[:][n]      A = K bytes as f16, B = Q (hi + lo f16)
 //   O^T[d][n]   += V^T[d][key] . P'[key][n]   A = V bytes as f16 (LDS transpose read),
-//                                              B = P' = p * scale_of_block(key, d/32), hi + lo f16
+//                                              B = P' = p * scale_of_block(key, d/32)
 // n runs over (query row, head) pairs, at most 16 per workgroup: a slot with more (3-4 MTP
-// rows x 6-8 heads) is cut by heads into two work items.  The C layout of S^T (row = 4*(lane/16)+i, col = lane%16)
+// rows x 6-8 heads) is cut by heads into work items.  The C layout of S^T (row = 4*(lane/16)+i, col = lane%16)
 // is exactly the B layout the PV product needs, so probabilities never leave
 // their lane, and every per-column scalar (max, sum, rescale) lives in lane%16.
 //
 // Exactness:
 //   - int8 -> f16 without rounding: byte b^0x80 = b+128 placed in the low byte of
-//     an f16 is the subnormal (b+128)*2^-24; one packed f16 subtract of 128*2^-24
-//     gives b*2^-24 exactly, and MFMA multiplies subnormals exactly.
+//     an f16 is the subnormal (b+128)*2^-24; the offset of 128 is removed exactly (a packed f16
+//     subtract in the staged kernel, a bias term in the other), and MFMA multiplies subnormals exactly.
 //   - one q8 block (32 values) is one MFMA contraction, so the f16 block scale
 //     multiplies an exact integer dot product in fp32 (as the CPU definition's
 //     d * q does, crates/hipml-core/src/ops.rs:486-515 of the reference).
-//   - Q and P' are split into hi + lo f16 halves: two MFMAs, ~22 bits each.
+//   - Q is split into hi + lo f16 halves (~22 bits); the fp32-class variant splits P' as well.
 
 #include "common.h"
 
