@@ -20,6 +20,10 @@
 // Numerics follow the reference's chunk kernel: Q, dequantized K/V (f16 scale x
 // int8, one rounding) and P are f16 operands; scores, softmax and accumulation
 // are fp32; softmax runs in log2 units.
+//
+// The same kernel also runs over an f16 copy of the cache (template parameter F16): then nothing is
+// dequantized or staged by the waves, whole tiles come in through global_load_lds, and the V tile is
+// stored transposed so that the PV operands are plain 128-bit reads.  kv_f16_tiles_kernel makes that copy.
 
 #include "common.h"
 
