@@ -269,33 +269,57 @@ int hipml_attn_batch_splits(int stride, int n_kv, int slots)
 
 int hipml_attn_chunk_splits(int pos0, int tokens, int n_kv)
 {
-    // A prefill workgroup is 8 tasks of (32 tokens x 1 head) and owns a whole CU (two 66 KiB
-    // LDS buffers), so the launch wants a few hundred workgroups: split the keys until there
-    // are about two rounds of 256, keep at least 128 keys per slice, and prefer a slice count
-    // that makes n_kv * splits a multiple of the 8 XCDs (the kernel then keeps each slice's
-    // K/V stream inside one XCD's L2).  Heads per KV head are taken as 6, the geometry built.
+    // A prefill workgroup is 8 tasks of (32 tokens x 1 head) and owns a whole CU (two 66 KiB LDS
+    // buffers), and the hardware starts workgroups in rounds of as many as fit the chip (256).  A
+    // launch of `splits` key slices is therefore priced as
+    //     rounds x (key tiles of the longest slice + 4),   rounds = ceil(workgroups / 256),
+    // the 4 tiles standing for what a workgroup costs whatever its slice (fetching and transposing its
+    // Q rows, writing its partial rows), with the workgroups counted as the kernel cuts them (a task
+    // block whose last token sees few key tiles gets fewer slices), and the cheapest slice count wins:
+    // it is the one that fills its last round (672 tokens at depth 32,768: 4 slices = one full round,
+    // 584 us, against 610 for the two rounds of 8; 256 tokens there: 10 slices = 240 workgroups, where
+    // 12 would leave a second round of 32).  Slices keep at least 128 keys, and n_kv * splits is a
+    // multiple of the 8 XCDs where that is possible (the kernel then keeps each slice's K/V stream
+    // inside one XCD's L2).  Heads per KV head are taken as 6, the geometry built.
     if (tokens < 1 || n_kv < 1)
         return 1;
-    const int ntask = (tokens + 31) / 32 * 6;
-    const int wgs = n_kv * ((ntask + 7) / 8);
-    if (wgs >= 512)
+    const int group = 6, tasks_per_wg = 8, q_tile = 32, k_tile = 64;
+    const int ntask = (tokens + q_tile - 1) / q_tile * group;
+    const int nblock = (ntask + tasks_per_wg - 1) / tasks_per_wg;
+    if (n_kv * nblock >= 512)
         return 1;
-    int s = (512 + wgs - 1) / wgs;
     const int keys = pos0 + tokens;
     const int by_work = keys / 128;
-    if (s > by_work)
-        s = by_work;
-    if (s > 16)
-        s = 16;
-    int up = s;
-    while (up <= 16 && up <= by_work && (n_kv * up) % 8 != 0)
-        up++;
-    if (up <= 16 && up <= by_work)
-        s = up;
-    else
-        while (s > 1 && (n_kv * s) % 8 != 0)
-            s--;
-    return s < 1 ? 1 : s;
+    const int tiles_last = (keys + k_tile - 1) / k_tile;
+    int best = 1;
+    double best_cost = 0.0;
+    for (int pass = 0; pass < 2; pass++) { // first the slice counts that suit the XCDs, then any
+        for (int s = 1; s <= 16 && s <= (by_work > 1 ? by_work : 1); s++) {
+            if (pass == 0 && s > 1 && (n_kv * s) % 8 != 0)
+                continue;
+            const int slice_tiles = (tiles_last + s - 1) / s;
+            long wg = 0;
+            for (int tb = 0; tb < nblock; tb++) {
+                const int last_task = tb * tasks_per_wg + tasks_per_wg - 1 < ntask ? tb * tasks_per_wg + tasks_per_wg - 1
+                                                                                 : ntask - 1;
+                const int tt_last = last_task / group;
+                const int last_tok = ((tt_last + 1) * q_tile < tokens ? (tt_last + 1) * q_tile : tokens) - 1;
+                const int tiles_b = (pos0 + last_tok + 1 + k_tile - 1) / k_tile;
+                const int n = (tiles_b + slice_tiles - 1) / slice_tiles;
+                wg += n < 1 ? 1 : (n < s ? n : s);
+            }
+            wg *= n_kv;
+            const long rounds = (wg + 255) / 256;
+            const double cost = (double)rounds * (slice_tiles + 4.0);
+            if (best_cost == 0.0 || cost < best_cost) {
+                best = s;
+                best_cost = cost;
+            }
+        }
+        if (best > 1)
+            break;
+    }
+    return best;
 }
 
 // ---- RoPE ----------------------------------------------------------------------------------

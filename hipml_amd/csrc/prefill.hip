@@ -838,6 +838,40 @@ __global__ void __launch_bounds__(256) chunk_combine_kernel(
             num += on ? x[s] * w : z;
             den = fmaf(on ? ml[s].y : 0.0f, w, den);
         }
+    } else if (nsp <= 16) {
+        // up to 16 slices: every (max, sum) pair first, then the accumulator rows four at a time, each
+        // group asked for before its first row is used
+        float2 ml[16];
+#pragma unroll
+        for (int s = 0; s < 16; s++) {
+            const size_t row = ((size_t)(s < nsp ? s : 0) * qslots + tok) * n_head + head;
+            ml[s] = *reinterpret_cast<const float2 *>(part_ml + row * 2);
+        }
+        float m = -INFINITY;
+#pragma unroll
+        for (int s = 0; s < 16; s++)
+            if (s < nsp && ml[s].y > 0.0f)
+                m = fmaxf(m, ml[s].x);
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            if (g * 4 < nsp) { // uniform over the workgroup's threads of this head
+                float4v x[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int sl = g * 4 + i;
+                    const size_t row = ((size_t)(sl < nsp ? sl : 0) * qslots + tok) * n_head + head;
+                    x[i] = *reinterpret_cast<const float4v *>(part_acc + row * kHeadDim + d4);
+                }
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int sl = g * 4 + i;
+                    const bool on = sl < nsp && ml[sl].y > 0.0f;
+                    const float w = on ? __builtin_amdgcn_exp2f(ml[sl].x - m) : 0.0f;
+                    num += on ? x[i] * w : z;
+                    den = fmaf(on ? ml[sl].y : 0.0f, w, den);
+                }
+            }
+        }
     } else {
         float m = -INFINITY;
         for (int s = 0; s < nsp; s++) {
