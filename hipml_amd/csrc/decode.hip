@@ -835,11 +835,14 @@ __global__ void __launch_bounds__(kThreads, 2) decode_staged_kernel(const Decode
 // The loads are written as asm: the compiler then neither knows nor waits for them, and the waits
 // are the explicit s_waitcnt below (loads return in order, 9 instructions per tile of rows).
 constexpr int kRawTile = kTileKeys * kRowBytes;              // 8704: 32 key rows as they lie in the cache
-constexpr int kDmaTileLds = 2 * kRawTile;                    // K rows and V rows of one tile
+constexpr int kParkPitch = kRowBytes + 4;                    // floats between parked accumulator rows (see the merge of the waves)
+constexpr int kDmaTileLds = 16 * kParkPitch * 4;             // K rows and V rows of one tile (17,408 bytes), and room for a
+                                                             // wave to park 16 columns of accumulators at the end (17,664)
+static_assert(kDmaTileLds >= 2 * kRawTile, "a wave's K and V rows");
 constexpr int kDmaQLds = 8 * 64 * 16;                        // Q operands on their way to registers: [8 blocks][64 lanes] half8;
                                                              // afterwards the waves' scale tables (2 x 512 bytes each)
 constexpr int kDmaBiasLds = 8 * 16 * 16;                     // score bias: [8 blocks][16 columns] float4
-// One tile of K and V rows per wave: 79,872 bytes, two workgroups per CU.  (A second tile per wave in
+// One tile of K and V rows per wave: 80,896 bytes, two workgroups per CU.  (A second tile per wave in
 // LDS, for launches of one workgroup per CU, measured slower: 21.3 against 19.2 us at depth 32,768,
 // as did a streaming probe with 16 instead of 8 KB in flight per wave.)
 constexpr int kDmaLds = kWaves * kDmaTileLds + kDmaQLds + kDmaBiasLds;
@@ -1319,12 +1322,11 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Work 
     // table, so nothing has to be waited for before the writes; the other waves read them after the
     // barrier.
     l_run = quad_rows<false>(l_run);
-    // 8 columns: the rows are 276 floats apart and the lanes of MFMA columns 8..15, which hold the same
-    // values as columns 0..7, write the run ten further on, so that the sixteen lanes of a k-group cover
-    // all 64 banks once per 128-bit write (measured for four waves parking at once: 470 cycles against
-    // 1,360 with rows of 272 floats written by half the lanes).  16 columns keep rows of 272 floats: 276
-    // would reach into the next wave's rows.
-    constexpr int kParkPitch = WIDE ? kRowBytes : kRowBytes + 4;
+    // The parked rows are 276 floats apart, so that the sixteen lanes of a k-group cover all 64 banks once
+    // per 128-bit write (20 n mod 64 is a different multiple of 4 for each of 16 columns n).  With 8
+    // columns the lanes of MFMA columns 8..15, which hold the same values as columns 0..7, write the run
+    // ten further on, which lands in the other half of the banks (measured for four waves parking at
+    // once: 470 cycles against 1,360 with rows of 272 floats written by half the lanes).
     float *wl = reinterpret_cast<float *>(wave_lds); // per wave: [kCols][kParkPitch] acc by byte column
     float *wml = reinterpret_cast<float *>(sK);  // per wave: [kCols] m, [kCols] l
     {
