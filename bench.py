@@ -121,10 +121,11 @@ def bench_prefill(torch, attn, tokens, pos0, steps, warmup, layers, prefix_fill=
                      torch.randn((tokens, KV, HD), device="cuda", generator=gen),
                      torch.randn((tokens, H, HD), device="cuda", generator=gen),
                      torch.empty((tokens, H, HD), device="cuda")))
-    splits = attn.chunk_splits(pos0, tokens, KV)
+    splits = attn.chunk_splits(pos0, tokens, KV)  # 0: the keys are cut inside the workgroups, no scratch
+    slices = attn.chunk_slices(pos0, tokens, KV)  # the attention over the f16 copy is always the sliced kernel
     acc = ml = None
-    if splits >= 2:
-        acc, ml = attn.chunk_scratch(tokens, H, splits)
+    if max(splits, slices) >= 2:
+        acc, ml = attn.chunk_scratch(tokens, H, max(splits, slices))
     attn.rope_table(THETA, NROT, max(pos0 + tokens, 1024))
     # the f16 copy of every layer cache, current up to the prefix (as earlier chunks would have left it)
     copies = []
@@ -143,7 +144,7 @@ def bench_prefill(torch, attn, tokens, pos0, steps, warmup, layers, prefix_fill=
     def attention_copy(i):
         q, kx, vx, gate, out = acts[i % layers]
         attn.chunk_attention_kv_f16(q, copies[i % layers], None, out, None, H, KV, HD, pos0, tokens, stride,
-                                    acc, ml, splits)
+                                    acc, ml, slices)
 
     def step_copy(i, rebuild=False):
         # the same step with the attention reading the f16 copy of the cache: the chunk's rows are added
@@ -157,7 +158,7 @@ def bench_prefill(torch, attn, tokens, pos0, steps, warmup, layers, prefix_fill=
         else:
             attn.kv_f16_rows(0, k, v, copies[i % layers], KV, HD, stride, pos0, tokens)
         attn.chunk_attention_kv_f16(q, copies[i % layers], gate, out, None, H, KV, HD, pos0, tokens, stride,
-                                    acc, ml, splits)
+                                    acc, ml, slices)
 
     def step(i):
         # RoPE and the append share one launch; the gate is applied where the attention result is
@@ -207,11 +208,11 @@ def bench_prefill(torch, attn, tokens, pos0, steps, warmup, layers, prefix_fill=
     wl = {(672, 0): "prefill672", (2048, 100_000): "chunk100k"}.get((tokens, pos0), "")
     # (the instantiation that reads the cache: <SPLIT, q4_0, over the f16 copy>)
     traffic = measured_traffic(wl, ["chunk_q8_kernel<true, false, false>", "chunk_q8_kernel<false, false, false>",
-                                    "chunk_combine_kernel"])
+                                    "chunk_combine_kernel", "chunk_wg_kernel<false>"])
     return {
         "workload": f"prefill {tokens}@{pos0}: rope + q8_0 append + causal GQA attention + gate, "
                     f"1 layer, {H}q/{KV}kv heads, head_dim {HD}",
-        "tokens": tokens, "pos0": pos0, "splits": splits, "layers_rotated": layers,
+        "tokens": tokens, "pos0": pos0, "splits": splits, "slices_over_f16_copy": slices, "layers_rotated": layers,
         "ms_per_step": wall_ms,
         "tok_per_s": tokens / (wall_ms * 1e-3),
         "ms_per_step_separate_launches": unfused_ms,
@@ -227,7 +228,8 @@ def bench_prefill(torch, attn, tokens, pos0, steps, warmup, layers, prefix_fill=
             "copy_bytes_per_layer": attn.kv_f16_bytes(stride, KV)},
         "roofline": {"bound": "mfma", "achieved": tf, "peak": MFMA_F16_PEAK_TF, "unit": "TFLOP/s",
                      "frac": tf / MFMA_F16_PEAK_TF, "traffic": traffic,
-                     "kernel": "chunk_q8_kernel" + (" + chunk_combine_kernel" if splits >= 2 else ""),
+                     "kernel": "chunk_wg_kernel" if splits == 0 else
+                     "chunk_q8_kernel" + (" + chunk_combine_kernel" if splits >= 2 else ""),
                      "flop_per_launch": flop, "launch_ms": attn_ms},
     }
 

@@ -27,6 +27,7 @@ HEAD_DIM = 256
 EXPORTS = [
     "hipml_attn_init", "hipml_attn_last_error", "hipml_attn_version",
     "hipml_attn_decode_splits", "hipml_attn_batch_splits", "hipml_attn_chunk_splits",
+    "hipml_attn_chunk_slices",
     "hipml_rope_table_bytes", "hipml_rope_table_fill_host", "hipml_rope_set_table",
     "hipml_mrope_f32", "hipml_mrope_rows_f32", "hipml_rope_chunk_f32",
     "hipml_kv_encode", "hipml_kv_encode_bulk", "hipml_kv_encode_rows",
@@ -76,6 +77,7 @@ def lib() -> C.CDLL:
             "hipml_attn_decode_splits": (i, [i, i]),
             "hipml_attn_batch_splits": (i, [i, i, i]),
             "hipml_attn_chunk_splits": (i, [i, i, i]),
+            "hipml_attn_chunk_slices": (i, [i, i, i]),
             "hipml_rope_table_bytes": (sz, [i, i]),
             "hipml_rope_table_fill_host": (i, [vp, f, i, i]),
             "hipml_rope_set_table": (i, [vp, f, i, i]),
@@ -165,7 +167,13 @@ def batch_splits(stride: int, n_kv: int, slots: int) -> int:
 
 
 def chunk_splits(pos0: int, tokens: int, n_kv: int = 4) -> int:
+    """0 = keys cut inside the workgroups (no scratch), 1 = single pass, n >= 2 = n key slices with scratch."""
     return lib().hipml_attn_chunk_splits(pos0, tokens, n_kv)
+
+
+def chunk_slices(pos0: int, tokens: int, n_kv: int = 4) -> int:
+    """The slice count (>= 1) of the sliced kernel, also where `chunk_splits` prefers the other one."""
+    return lib().hipml_attn_chunk_slices(pos0, tokens, n_kv)
 
 
 # ---- RoPE ----------------------------------------------------------------------------

@@ -267,7 +267,7 @@ int hipml_attn_batch_splits(int stride, int n_kv, int slots)
     return s < 1 ? 1 : s;
 }
 
-int hipml_attn_chunk_splits(int pos0, int tokens, int n_kv)
+int hipml_attn_chunk_slices(int pos0, int tokens, int n_kv)
 {
     // A prefill workgroup is 8 tasks of (32 tokens x 1 head) and owns a whole CU (two 66 KiB LDS
     // buffers), and the hardware starts workgroups in rounds of as many as fit the chip (256).  A
@@ -320,6 +320,21 @@ int hipml_attn_chunk_splits(int pos0, int tokens, int n_kv)
             break;
     }
     return best;
+}
+
+int hipml_attn_chunk_splits(int pos0, int tokens, int n_kv)
+{
+    // 0 = the kernel that keeps the key slices inside the workgroup (no partial rows in memory, no merge
+    // launch).  Its workgroups share the dequantized K/V among two heads instead of eight tasks, so it
+    // pays where the rows (Q, gate, output, partial rows) outweigh the keys: chunks near position 0.
+    // Measured against the best slice count of the other kernel, whole step in us (this one first):
+    // 32 @ 0 16.7 / 20.6, 128 @ 0 18.5 / 26.4, 256 @ 0 24.8 / 35.1, 672 @ 0 41.7 / 52.1, 1,024 @ 0 61.6 / 66.8,
+    // 1,536 @ 0 101 / 113, 2,048 @ 0 150 / 149, 4,096 @ 0 428 / 416; 128 @ 256 27.2 / 31.4, 256 @ 512 38.0 /
+    // 37.8, 672 @ 512 54.1 / 58.2, 1,024 @ 512 84.3 / 103, 672 @ 1,024 68.7 / 68.0, 256 @ 1,024 48.9 / 43.6,
+    // 64 @ 1,000 45.4 / 34.5, 672 @ 8,192 293 / 200.
+    if (tokens >= 1 && n_kv >= 1 && pos0 >= 0 && (long long)pos0 + tokens <= 1792 && pos0 <= 2 * tokens)
+        return 0;
+    return hipml_attn_chunk_slices(pos0, tokens, n_kv);
 }
 
 // ---- RoPE ----------------------------------------------------------------------------------

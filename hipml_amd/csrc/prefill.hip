@@ -71,6 +71,7 @@ struct ChunkArgs {
     const uint8_t *vt;  //                                      V^T tiles, [n_kv][tile_stride][kVtTileBytes]
     int tile_stride;    // tiles per KV head in the copy
     float *out;
+    _Float16 *out16;   // chunk_wg_kernel only: if set, the finished rows go here as f16 instead of to `out`
     const float *gate; // optional [tokens][n_head][256]: out = attention * sigmoid(gate)
     float *part_acc;
     float *part_ml;
@@ -449,6 +450,10 @@ __global__ void __launch_bounds__(kPfThreads, 2) chunk_q8_kernel(const ChunkArgs
         if constexpr (F16)
             asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
     };
+    auto dma_wait_all = [&]() {
+        if constexpr (F16)
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    };
 
     // ---- Q^T operand: 16 k-steps of 8 f16 (d = ks*16 + lh*8 + j) ---------------------------
     // Steps 0..kQLdsSteps-1 are parked in this wave's corner of LDS and re-read per use: 256
@@ -671,9 +676,11 @@ __global__ void __launch_bounds__(kPfThreads, 2) chunk_q8_kernel(const ChunkArgs
     // writes V(t+1) in its V1(t) and V2(t), which are set 0's M1(t) and M2(t); the V(t-1) it replaces
     // was last read in M2(t-1), finished by both sets before that, and V(t+1) is first read in M1(t+1).
     if constexpr (F16) {
-        // K(t + 1) is requested at the head of the slot M2(t - 1) and waited for at the end of M1(t), V(t + 1)
-        // at the head of M1(t) and the end of M2(t): each has three slots to arrive in, and the buffer it
-        // lands in was last read one slot before the request, by either set.
+        // K(t + 1) is requested at the head of the slot M2(t - 1) and waited for at the end of M1(t) (three
+        // slots to arrive in), V(t + 1) at the head of M1(t) and the end of V2(t) (two slots: the set that
+        // runs ahead reads its first V operands in V1(t + 1), which is the other set's M2(t), so every wave's
+        // share must have landed one barrier before that); the buffer a tile lands in was last read one
+        // slot before the request, by either set.
         dma_tile(0, false);
         dma_tile(0, true);
         dma_tile(1, false);
@@ -706,12 +713,12 @@ __global__ void __launch_bounds__(kPfThreads, 2) chunk_q8_kernel(const ChunkArgs
         issue0(t + 2);
         softmax(t, 1);
         pre_pv(t, 1);
+        dma_wait_all(); // V(t + 1), before the barrier after which the other set reads it ahead of its M1(t + 1)
         lds_barrier();
         dma_tile(t + 2, false);
         pv(t, 1);
         if (t + 1 < ntile)
             scores(t + 1, 0);
-        dma_wait_oldest();
         lds_barrier();
     }
     if (set == 0)
@@ -790,6 +797,439 @@ __global__ void __launch_bounds__(kPfThreads, 2) chunk_q8_kernel(const ChunkArgs
                                    O[dt][g * 4 + 3] * inv};
                 *reinterpret_cast<float4v *>(po + dt * 32 + g * 8 + lh * 4) = x;
             }
+    }
+}
+
+// ---- chunk prefill with the key split inside the workgroup -----------------------------------------
+// Near position 0 a chunk has few keys per token and little to do in total (672 tokens at depth 0:
+// 5.6 GFLOP, 1.5 MB of cache), but as many Q and output rows as at any depth.  The kernel above then
+// has too few workgroups for the chip unless the keys are cut into slices, and slices cost partial
+// rows in memory and a second launch that is longer than the attention itself.  Here the slices stay
+// inside the workgroup: it takes one tile of 32 tokens and two heads of one KV head, and cuts their
+// keys into four slices, one wave per (slice, head).  The two waves of a slice share its K/V tiles
+// (32 keys per step, dequantized by those two waves, single-buffered: 4 x 34 KB of LDS); the four
+// partial results of a head meet in LDS at the end, each wave finishing 64 of the 256 output
+// columns, gate included.  672 tokens x 24 heads are 252 such workgroups, one round of the chip.
+//
+// A step takes four slots, each closed by a workgroup barrier:
+//   A: dequantize K(s+1) into the K tile, request V(s+1), softmax of step s      (VALU)
+//   B: PV of step s                                                              (MFMA)
+//   C: dequantize V(s+1) into the V tile, request K(s+2)                         (VALU)
+//   D: scores of step s+1                                                        (MFMA)
+// Slices 0 and 1 (waves 0..3) run one slot ahead of slices 2 and 3 (waves 4..7), so each SIMD has one
+// wave in a VALU slot and one in an MFMA slot.  The two waves of a slice are always in the same slot:
+// K(s) is last read in D(s-1) and overwritten in A(s), V(s) last read in B(s) and overwritten in C(s).
+// Operand layouts, MFMA shapes and numerics are those of chunk_q8_kernel.
+constexpr int kWgSlices = 4;                   // key slices of a task, one wave each
+constexpr int kWgStep = 32;                    // keys per step
+constexpr int kWgK = kWgStep * kKRow;          // 16,896: K tile of a slice
+constexpr int kWgV = kWgStep * kVRow;          // 17,408: its V tile
+constexpr int kWgSlice = kWgK + kWgV;          // 34,304
+constexpr int kWgQPark = 2;                   // d-steps of the Q operand read from LDS at every use: 256 registers do not hold the rest
+constexpr int kWgQAt = kWgSlices * kWgSlice;   // 137,216: [head 2][step][lane] x 16 bytes
+constexpr int kWgLds = kWgQAt + 2 * kWgQPark * 1024;
+constexpr int kWgXAt = 4096;                   // merge: (max, sum) table below, accumulator exchange from here
+constexpr int kWgXArea = 8192;                 // two 32-column tiles of one wave
+constexpr int kWgOutPitch = 272;               // a token's 64 finished columns + pad
+constexpr float kWgLazy = 8.0f;                // growth of a maximum (log2 units) that moves the reference exponent
+
+template <bool Q4>
+__global__ void __launch_bounds__(kPfThreads, 1) chunk_wg_kernel(const ChunkArgs a)
+{
+    typedef typename HalfOf<Q4>::type Half;
+    constexpr int kRowBytes = Q4 ? hipml::kRowBytesQ4 : hipml::kRowBytes;
+    constexpr int kUnitBytes = Q4 ? 36 : 68;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    static_assert(kWgLds <= 160 * 1024 && kWgXAt + 12 * kWgXArea <= kWgLds && kWgXAt + 8 * kQTile * kWgOutPitch <= kWgLds, "merge areas");
+
+    // (the same in every lane: taking it from the first one lets everything derived from it live in scalar registers)
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    const int ln = lane & 31;
+    const int lh = lane >> 5;
+    const int set = wave >> 2;                    // waves w and w + 4 share a SIMD
+    const int sl = set * 2 + ((wave >> 1) & 1);   // key slice
+    const int hp = wave & 1;                      // head of the pair
+
+    // blockIdx.x -> (token tile, kv head, head pair), the token tiles with the most keys first
+    const int pairs = (a.group + 1) >> 1;
+    const int per_tt = a.n_kv * pairs;
+    const int ntt = (a.tokens + kQTile - 1) / kQTile;
+    const int tt = ntt - 1 - (int)blockIdx.x / per_tt;
+    const int rem = (int)blockIdx.x % per_tt;
+    const int kvh = rem % a.n_kv;
+    const int hq = (rem / a.n_kv) * 2 + hp;
+    const bool task_valid = hq < a.group;        // (an odd group leaves the last pair one head)
+    const int head = kvh * a.group + (task_valid ? hq : a.group - 1);
+    const int t0 = tt * kQTile;
+    const int last_tok = ((tt + 1) * kQTile < a.tokens ? (tt + 1) * kQTile : a.tokens) - 1;
+    const int khi = a.pos0 + last_tok + 1;                          // keys the tile's last token sees
+    const int nstep = ((khi + kWgStep - 1) / kWgStep + kWgSlices - 1) / kWgSlices; // per slice, same for all
+    const int kbeg = sl * nstep * kWgStep;                          // this slice's first key
+    const int tok = t0 + ln;
+    const int my_last_key = a.pos0 + tok;
+    const bool tok_valid = task_valid && tok < a.tokens;
+
+    uint8_t *Kt = lds + sl * kWgSlice;
+    uint8_t *Vt = Kt + kWgK;
+
+    // ---- staging role: lane -> one unit (two blocks) of the slice's K tile and one of its V tile ----
+    // (the (row, unit) pattern of chunk_q8_kernel over the slice's 128 lanes: conflict-free 128-bit writes)
+    const int su = hp * 64 + lane;
+    const int srow = (su >> 6) * 16 + ((su >> 1) & 7) + ((su >> 5) & 1) * 8;
+    const int spr = (su & 1) | ((su >> 3) & 2);
+    // (uniform base + 32-bit lane offset: a KV head's rows span less than 4 GB)
+    const uint8_t *kbase = a.kc + (size_t)kvh * a.stride * kRowBytes;
+    const uint8_t *vbase = a.vc + (size_t)kvh * a.stride * kRowBytes;
+    // (a row past the visible keys repeats the last one: unconditional loads keep their registers out of
+    // branches; such keys are masked)
+    auto unit_at = [&](int s) {
+        int key = kbeg + s * kWgStep + srow;
+        key = key < khi ? key : khi - 1;
+        return (uint32_t)key * (uint32_t)kRowBytes + (uint32_t)(spr * kUnitBytes);
+    };
+    // One unit is in flight at a time, alternately the K and the V unit: a unit is requested when the
+    // one before it has been dequantized and travels through the MFMA slot that follows.
+    Half r0, r1;
+    auto issue_k = [&](int s) {
+        const uint8_t *u = kbase + unit_at(s);
+        load_half0(r0, u);
+        load_half1(r1, u);
+    };
+    auto issue_v = [&](int s) {
+        const uint8_t *u = vbase + unit_at(s);
+        load_half0(r0, u);
+        load_half1(r1, u);
+    };
+    auto stage_k = [&]() {
+        uint8_t *d = Kt + srow * kKRow + spr * 128;
+        stage_block0(r0, d);
+        stage_block1(r1, d);
+    };
+    auto stage_v = [&]() {
+        uint8_t *d = Vt + srow * kVRow + spr * 128;
+        stage_block0(r0, d);
+        stage_block1(r1, d);
+    };
+    issue_k(0);
+    Half v0a, v0b; // V(0): requested now, in registers of its own (the accumulators are not live yet)
+    {
+        const uint8_t *u = vbase + unit_at(0);
+        load_half0(v0a, u);
+        load_half1(v0b, u);
+    }
+
+    // ---- Q^T operand of this wave's head: the head's four waves fetch eight token rows each (one
+    // instruction = one token's 256 floats), convert them and write them as f16 rows into the V tile of
+    // slice `hp`, which is unused until the first V tile is staged; every wave then reads all 16 steps.
+    half8 qf[16];
+    uint8_t *qpark = lds + kWgQAt + hp * kWgQPark * 1024 + lane * 16;
+    {
+        uint8_t *qa = lds + hp * kWgSlice + kWgK;
+        const float *qh = a.q + (size_t)head * kHeadDim + lane * 4;
+        const size_t tok_stride = (size_t)a.n_head * kHeadDim;
+        float4v f[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const int tr = t0 + sl * 8 + i;
+            f[i] = *reinterpret_cast<const float4v *>(qh + (size_t)(tr < a.tokens ? tr : a.tokens - 1) * tok_stride);
+        }
+        stage_k();
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            half4 h;
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                h[j] = (_Float16)f[i][j];
+            *reinterpret_cast<half4 *>(qa + (sl * 8 + i) * kKRow + lane * 8) = h;
+        }
+        lds_barrier(); // Q rows and K(0) are in LDS
+#pragma unroll
+        for (int ks = 0; ks < 16; ks++) {
+            const half8 h = *reinterpret_cast<const half8 *>(qa + ln * kKRow + ks * 32 + lh * 16);
+            if (ks >= kWgQPark)
+                qf[ks] = h;
+            else if ((ks & 3) == sl) // the head's four waves read the same values: each parks its share
+                *reinterpret_cast<half8 *>(qpark + ks * 1024) = h;
+        }
+        lds_barrier(); // every wave has its Q: the V tiles may be written
+        {
+            uint8_t *d = Vt + srow * kVRow + spr * 128;
+            stage_block0(v0a, d);
+            stage_block1(v0b, d);
+        }
+        issue_k(1);
+    }
+
+    float16v O[8];
+#pragma unroll
+    for (int t = 0; t < 8; t++)
+#pragma unroll
+        for (int i = 0; i < 16; i++)
+            O[t][i] = 0.0f;
+    float m_run = -INFINITY, l_run = 0.0f;
+    float16v S;
+    half8 P[2];
+
+    const int gl = lane & 15;
+    const int vtr_off = (gl >> 2) * kVRow + (((lane >> 4) & 1) * 16 + (gl & 3) * 4) * 2;
+
+    auto live = [&](int s) { return task_valid && kbeg + s * kWgStep < khi; }; // wave-uniform
+
+    auto scores = [&](int s) {
+        if (!live(s))
+            return;
+        const uint8_t *Kh = Kt + ln * kKRow + lh * 16;
+        float16v acc;
+#pragma unroll
+        for (int i = 0; i < 16; i++)
+            acc[i] = 0.0f;
+        half8 A[16], B[kWgQPark > 0 ? kWgQPark : 1];
+#pragma unroll
+        for (int ks = 0; ks < kWgQPark; ks++)
+            B[ks] = *reinterpret_cast<const half8 *>(qpark + ks * 1024);
+#pragma unroll
+        for (int ks = 0; ks < 16; ks++)
+            A[ks] = *reinterpret_cast<const half8 *>(Kh + ks * 32);
+#pragma unroll
+        for (int ks = 0; ks < 16; ks++)
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[ks], ks < kWgQPark ? B[ks] : qf[ks], acc, 0, 0, 0);
+        S = acc;
+        // operands two MFMAs ahead; the parked Q steps come first in the chain, two reads per MFMA
+        constexpr int kTwo = kWgQPark > 2 ? kWgQPark - 2 : 0; // MFMAs whose look-ahead is a (K, Q) pair
+        __builtin_amdgcn_sched_group_barrier(0x100, kWgQPark >= 2 ? 4 : 2 + kWgQPark, 0);
+#pragma unroll
+        for (int ks = 0; ks < kTwo; ks++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        }
+#pragma unroll
+        for (int ks = kTwo; ks < 14; ks++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+    };
+
+    // lane holds keys (i/4)*8 + lh*4 + i%4 of the step for token ln
+    auto softmax = [&](int s) {
+        if (!live(s))
+            return;
+        const int k0 = kbeg + s * kWgStep;
+        const bool need_mask = (k0 + 31 > a.pos0 + t0) || (k0 + 32 > khi);
+        if (need_mask) {
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const int kg = k0 + (i >> 2) * 8 + lh * 4 + (i & 3);
+                S[i] = (kg <= my_last_key && kg < khi) ? S[i] : -INFINITY;
+            }
+        }
+        float mt = S[0];
+#pragma unroll
+        for (int i = 1; i < 16; i++)
+            mt = fmaxf(mt, S[i]);
+        mt = xor32_max(mt) * a.scale_log2;
+        // m_run is the exponent the sums are held against, not the running maximum: it follows the
+        // maximum only when some token's maximum has grown by more than kWgLazy since it was set, so
+        // the 128 accumulator registers are rescaled on few steps.  Until then probabilities may be as
+        // large as 2^kWgLazy, which f16 holds with the same relative precision.
+        if (__any(mt > m_run + kWgLazy)) {
+            const float m_new = fmaxf(m_run, mt);
+            const float corr = m_new == -INFINITY ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_new);
+            l_run *= corr;
+#pragma unroll
+            for (int dt = 0; dt < 8; dt++)
+                O[dt] *= corr;
+            m_run = m_new;
+        }
+        const float mneg = m_run == -INFINITY ? 0.0f : -m_run;
+        float ls = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const float e = __builtin_amdgcn_exp2f(fmaf(S[i], a.scale_log2, mneg));
+            ls += e;
+            P[i >> 3][i & 7] = (_Float16)e;
+        }
+        l_run += ls;
+        asm volatile("" : "+v"(P[0]), "+v"(P[1]), "+v"(l_run), "+v"(m_run));
+    };
+
+    auto pv = [&](int s) {
+        if (!live(s))
+            return;
+        half8 A[16];
+        const uint8_t *Vh = Vt + vtr_off;
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+#pragma unroll
+            for (int dt = 0; dt < 8; dt++) {
+                const uint8_t *vp = Vh + dt * 64;
+                const short4v r0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (short4v __attribute__((address_space(3))) *)(vp + ((2 * u) * 8 + lh * 4) * kVRow));
+                const short4v r1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (short4v __attribute__((address_space(3))) *)(vp + ((2 * u + 1) * 8 + lh * 4) * kVRow));
+                const half4 h0 = __builtin_bit_cast(half4, r0);
+                const half4 h1 = __builtin_bit_cast(half4, r1);
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    A[u * 8 + dt][j] = h0[j];
+                    A[u * 8 + dt][4 + j] = h1[j];
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 2; u++)
+#pragma unroll
+            for (int dt = 0; dt < 8; dt++)
+                O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[u * 8 + dt], P[u], O[dt], 0, 0, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+        for (int k = 0; k < 14; k++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+    };
+
+    lds_barrier(); // V(0) is in LDS
+    if (set == 1)
+        lds_barrier();
+    scores(0);
+    lds_barrier();
+    for (int s = 0; s < nstep; s++) {
+        const bool more = s + 1 < nstep;
+        if (more)
+            stage_k();      // K(s + 1)
+        issue_v(s + 1);
+        softmax(s);
+        lds_barrier();
+        pv(s);
+        lds_barrier();
+        if (more)
+            stage_v();      // V(s + 1)
+        issue_k(s + 2);
+        lds_barrier();
+        if (more)
+            scores(s + 1);
+        lds_barrier();
+    }
+    if (set == 0)
+        lds_barrier();
+
+    // ---- the four slices of a head meet -------------------------------------------------------------
+    // Wave `sl` finishes columns 64 sl .. 64 sl + 63 (accumulators 2 sl and 2 sl + 1) of its head.  The
+    // gate values of the rows it will write are requested first.
+    const int orow = lane >> 4, opiece = lane & 15; // output pass r2: token r2 * 4 + orow, 16-byte piece
+    float4v gt[8];
+    if (a.gate) {
+#pragma unroll
+        for (int r2 = 0; r2 < 8; r2++) {
+            const int tr = t0 + r2 * 4 + orow;
+            gt[r2] = *reinterpret_cast<const float4v *>(
+                a.gate + ((size_t)(tr < a.tokens ? tr : a.tokens - 1) * a.n_head + head) * kHeadDim + sl * 64 + opiece * 4);
+        }
+    }
+    l_run += __shfl_xor(l_run, 32);
+    float2 *mlx = reinterpret_cast<float2 *>(lds); // [head 2][slice 4][token 32]
+    if (lh == 0)
+        mlx[(hp * kWgSlices + sl) * kQTile + ln] = make_float2(m_run, l_run);
+    lds_barrier();
+    float m = -INFINITY, den = 0.0f, w_mine = 0.0f;
+    {
+        float2 v[kWgSlices];
+#pragma unroll
+        for (int j = 0; j < kWgSlices; j++) {
+            v[j] = mlx[(hp * kWgSlices + j) * kQTile + ln];
+            if (v[j].y > 0.0f)
+                m = fmaxf(m, v[j].x);
+        }
+#pragma unroll
+        for (int j = 0; j < kWgSlices; j++) {
+            const bool on = v[j].y > 0.0f;
+            const float w = on ? __builtin_amdgcn_exp2f(v[j].x - m) : 0.0f;
+            den = fmaf(on ? v[j].y : 0.0f, w, den);
+            w_mine = j == sl ? w : w_mine;
+        }
+    }
+    const float inv = den > 0.0f ? 1.0f / den : 0.0f;
+#pragma unroll
+    for (int dt = 0; dt < 8; dt++)
+        O[dt] *= w_mine;
+    // Two passes, columns 0..127 and 128..255: every wave hands the accumulators it does not finish to
+    // the wave that does (the layout is the same in every wave, so lane l writes and reads slot l).
+    uint8_t *xbase = lds + kWgXAt;
+#pragma unroll
+    for (int p = 0; p < 2; p++) {
+#pragma unroll
+        for (int q2 = 0; q2 < 2; q2++) {
+            const int qd = 2 * p + q2;
+            if (sl != qd) {
+                const int from = sl < qd ? sl : sl - 1;
+                float4v *dst = reinterpret_cast<float4v *>(xbase + ((hp * 2 + q2) * 3 + from) * kWgXArea) + lane;
+#pragma unroll
+                for (int dtl = 0; dtl < 2; dtl++)
+#pragma unroll
+                    for (int g = 0; g < 4; g++)
+                        dst[(dtl * 4 + g) * 64] = (float4v){O[2 * qd + dtl][g * 4], O[2 * qd + dtl][g * 4 + 1],
+                                                            O[2 * qd + dtl][g * 4 + 2], O[2 * qd + dtl][g * 4 + 3]};
+            }
+        }
+        lds_barrier();
+#pragma unroll
+        for (int q2 = 0; q2 < 2; q2++) {
+            const int qd = 2 * p + q2;
+            if (sl == qd) {
+#pragma unroll
+                for (int from = 0; from < 3; from++) {
+                    const float4v *src =
+                        reinterpret_cast<const float4v *>(xbase + ((hp * 2 + q2) * 3 + from) * kWgXArea) + lane;
+#pragma unroll
+                    for (int dtl = 0; dtl < 2; dtl++)
+#pragma unroll
+                        for (int g = 0; g < 4; g++) {
+                            const float4v x = src[(dtl * 4 + g) * 64];
+#pragma unroll
+                            for (int j = 0; j < 4; j++)
+                                O[2 * qd + dtl][g * 4 + j] += x[j];
+                        }
+                }
+            }
+        }
+        lds_barrier();
+    }
+    float16v R[2];
+#pragma unroll
+    for (int qd = 0; qd < 4; qd++)
+        if (sl == qd) {
+            R[0] = O[2 * qd];
+            R[1] = O[2 * qd + 1];
+        }
+    // Turned round in this wave's corner of LDS, a store instruction covers four tokens' 256 contiguous bytes.
+    uint8_t *mine = xbase + wave * (kQTile * kWgOutPitch);
+#pragma unroll
+    for (int dtl = 0; dtl < 2; dtl++)
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            const float4v x = {R[dtl][g * 4] * inv, R[dtl][g * 4 + 1] * inv, R[dtl][g * 4 + 2] * inv,
+                               R[dtl][g * 4 + 3] * inv};
+            *reinterpret_cast<float4v *>(mine + ln * kWgOutPitch + (dtl * 32 + g * 8 + lh * 4) * 4) = x;
+        }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // this wave's own writes
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int r2 = 0; r2 < 8; r2++) {
+        const int r = r2 * 4 + orow;
+        float4v x = *reinterpret_cast<const float4v *>(mine + r * kWgOutPitch + opiece * 16);
+        if (task_valid && t0 + r < a.tokens) {
+            const size_t o = ((size_t)(t0 + r) * a.n_head + head) * kHeadDim + sl * 64 + opiece * 4;
+            if (a.gate)
+                x = (float4v){gated(x[0], gt[r2][0]), gated(x[1], gt[r2][1]), gated(x[2], gt[r2][2]),
+                              gated(x[3], gt[r2][3])};
+            if (a.out16)
+                *reinterpret_cast<half4 *>(a.out16 + o) = __builtin_convertvector(x, half4);
+            else
+                *reinterpret_cast<float4v *>(a.out + o) = x;
+        }
     }
 }
 
@@ -1041,6 +1481,12 @@ int prefill_init()
     if (e == hipSuccess)
         e = hipFuncSetAttribute(reinterpret_cast<const void *>(&kv_f16_tiles_kernel<true>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, kBufBytes);
+    if (e == hipSuccess)
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&chunk_wg_kernel<false>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, kWgLds);
+    if (e == hipSuccess)
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&chunk_wg_kernel<true>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, kWgLds);
     if (e != hipSuccess)
         return fail((int)e, "hipFuncSetAttribute(prefill LDS) failed: %d (%s)", (int)e,
                     hipGetErrorString(e));
@@ -1075,6 +1521,17 @@ int launch_chunk_q8(hipStream_t st, const float *q, const uint8_t *kc, const uin
     a.ntask = (tokens + kQTile - 1) / kQTile * a.group;
     a.nblock = (a.ntask + kTasks - 1) / kTasks;
     a.scale_log2 = kLog2e / 16.0f; // 1/sqrt(256), as the reference's chunk launcher fixes it
+    a.out16 = nullptr;
+    if (splits == 0 && kv_f16 == nullptr) {
+        // the key slices stay inside the workgroup: no partial rows, gate and f16 rows in the same launch
+        a.out16 = static_cast<_Float16 *>(out16);
+        const unsigned wgs = (unsigned)((tokens + kQTile - 1) / kQTile * n_kv * ((a.group + 1) / 2));
+        if (q4)
+            hipLaunchKernelGGL(chunk_wg_kernel<true>, dim3(wgs, 1, 1), dim3(kPfThreads, 1, 1), kWgLds, st, a);
+        else
+            hipLaunchKernelGGL(chunk_wg_kernel<false>, dim3(wgs, 1, 1), dim3(kPfThreads, 1, 1), kWgLds, st, a);
+        return launched(q4 ? "attn_chunk_q4_wg" : "attn_chunk_q8_wg");
+    }
     // slices per block: the last block (most keys) gets `splits`, a block with fewer key tiles gets
     // proportionally fewer, so a chunk near position 0 does not write and re-read `splits` partial
     // copies of rows that see only a few tiles

@@ -76,8 +76,15 @@ int hipml_attn_decode_splits(int seq, int n_kv);
  * crates/hipml-model/src/gpu/batch/kv.rs:39-42. */
 int hipml_attn_batch_splits(int stride, int n_kv, int slots);
 /* Key splits for a prefill chunk starting at pos0.  Same role as split_count,
- * crates/hipml-model/src/gpu/attn_tile.rs:138-151. */
+ * crates/hipml-model/src/gpu/attn_tile.rs:138-151.  0 (chunks near position 0: pos0 + tokens <=
+ * 1,792 and pos0 <= 2 * tokens) selects the kernel that cuts the keys inside its workgroups and
+ * needs no scratch; 1 the single-pass kernel; n >= 2 that kernel over n key slices with scratch
+ * and a merge launch. */
 int hipml_attn_chunk_splits(int pos0, int tokens, int n_kv);
+/* The slice count (>= 1) for callers that want the sliced kernel whatever the shape, and for
+ * hipml_attn_chunk_kv_f16, which has no in-workgroup variant: what hipml_attn_chunk_splits
+ * returns where it does not return 0. */
+int hipml_attn_chunk_slices(int pos0, int tokens, int n_kv);
 
 /* ---- RoPE ----------------------------------------------------------------
  * The reference's CPU definition builds the angle in f64 with the host libm
@@ -314,8 +321,10 @@ int hipml_attn_decode_kv_noalloc(hipml_stream_t stream, const int32_t *step, int
 
 /* tokens query rows at positions pos0..pos0+tokens-1 attend keys [0, pos0+t]
  * of a cache that already holds the chunk's own rows.  `dtype` follows the
- * reference's chunk launcher: 1 = q8_0, 2 = q4_0.  splits < 2 runs the single-pass kernel
- * and ignores the scratch; otherwise part_acc is f32
+ * reference's chunk launcher: 1 = q8_0, 2 = q4_0.  splits == 1 runs the single-pass kernel
+ * and splits == 0 the kernel that cuts the keys into four slices inside each workgroup (one
+ * workgroup per 32 tokens x 2 heads; made for chunks near position 0, correct at any depth);
+ * both ignore the scratch.  Otherwise part_acc is f32
  * [splits][ceil32(tokens)][n_head][head_dim] and part_ml [..][2].
  * Replaces AttnLayer::chunk_attention_q8_split -> attn_chunk_wmma_f16 /
  * attn_chunk_full_f16 + attn_chunk_combine_f32,
@@ -374,7 +383,8 @@ int hipml_kv_f16_rows(hipml_stream_t stream, int dtype, const void *k_cache, con
  * copy: rows [0, pos0 + tokens) of kv_f16 must be current.  gate (may be NULL) and out16 (may be NULL)
  * as in hipml_attn_chunk_q8_split_gate / _gate_f16.  The operands are the same values, so results
  * differ from those entry points only through the key slices, which here end at multiples of 64
- * keys.  Same scratch sizes, same split policy (hipml_attn_chunk_splits). */
+ * keys.  Same scratch sizes; slice counts from hipml_attn_chunk_slices (splits == 0 is taken as 1:
+ * there is no in-workgroup variant over the copy). */
 int hipml_attn_chunk_kv_f16(hipml_stream_t stream, const float *q, const void *kv_f16,
                             const float *gate, float *out, void *out16, int n_head, int n_kv,
                             int head_dim, int pos0, int tokens, int stride, float *part_acc,

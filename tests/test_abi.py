@@ -50,7 +50,13 @@ def test_split_policies(lib):
     assert attn.chunk_splits(0, 8192, 4) == 1
     s = attn.chunk_splits(100_000, 2048, 4)
     assert s > 1 and (4 * s) % 8 == 0
-    assert attn.chunk_splits(0, 1, 4) >= 1
+    assert attn.chunk_slices(0, 1, 4) >= 1
+    # near position 0 the keys are cut inside the workgroups (0); deep chunks and long ones are not
+    assert attn.chunk_splits(0, 672, 4) == 0 and attn.chunk_splits(0, 1, 4) == 0
+    assert attn.chunk_splits(512, 672, 4) == 0
+    assert attn.chunk_splits(0, 2048, 4) == attn.chunk_slices(0, 2048, 4) >= 1
+    assert attn.chunk_splits(1000, 64, 4) == attn.chunk_slices(1000, 64, 4) >= 2
+    assert attn.chunk_slices(0, 672, 4) >= 2
 
 
 def test_rope_table_on_the_host_is_the_f64_definition(lib):

@@ -1,0 +1,102 @@
+"""Chunk prefill with the key slices inside the workgroups (splits = 0 of the chunk entry points): the
+kernel for chunks near position 0.  Same oracle and same gate (2e-3 / 1e-2) as the sliced kernel; its
+sums are held against a reference exponent that lags the running maximum by up to 2^8, which the gate
+covers (f16 keeps its relative precision over that range)."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+from oracle import binding as orc  # noqa: E402
+from hipml_amd import attn  # noqa: E402
+from gpu_util import N_HEADS, N_KV, HD, SCALE, dev, host, report  # noqa: E402
+from test_gpu_prefill import chunk_inputs, run_chunk, GATE  # noqa: E402
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _init():
+    attn.init(0)
+
+
+@pytest.mark.parametrize("tok,pos0,pad", [(1, 0, 0), (33, 0, 3), (37, 29, 0), (37, 29, 8), (96, 64, 0), (130, 63, 1),
+                                          (64, 1000, 24), (300, 0, 5), (31, 1, 0), (128, 127, 2)])
+def test_reference_chunk_cases(tok, pos0, pad):
+    q, kb, vb, stride = chunk_inputs(0xC4A0_9876_5432, tok, pos0, pad)
+    want = orc.attn_chunk_kv(q, kb, vb, N_HEADS, N_KV, HD, pos0, tok, stride, SCALE, n_threads=8)
+    got = run_chunk(q, kb, vb, pos0, tok, stride, 0)
+    ok, _, _ = report(f"chunk {tok}@{pos0} pad {pad}, slices inside the workgroups", want, got, *GATE)
+    assert ok
+    assert np.isfinite(got).all()
+
+
+def test_prefill_672_at_0_plain_gated_and_as_f16_rows():
+    # the headline shape; the policy picks this kernel for it
+    tok, pos0 = 672, 0
+    assert attn.chunk_splits(pos0, tok, N_KV) == 0
+    q, kb, vb, stride = chunk_inputs(0x5EED_0002, tok, pos0, 8)
+    gate = orc.Rng(0x6A7E).normal_array((tok, N_HEADS, HD))
+    plain = run_chunk(q, kb, vb, pos0, tok, stride, 0)
+    want = orc.attn_chunk_kv(q, kb, vb, N_HEADS, N_KV, HD, pos0, tok, stride, SCALE, n_threads=16)
+    ok, _, _ = report("prefill 672@0, slices inside the workgroups", want, plain, *GATE)
+    assert ok
+    # the fused gate gives the bits of the attention followed by the gate kernel
+    x = dev(plain)
+    two = torch.empty_like(x)
+    attn.q_gate(x, dev(gate), two)
+    fused = torch.full_like(x, float("nan"))
+    attn.chunk_attention_q8_split_gate(dev(q), dev(kb), dev(vb), dev(gate), fused, N_HEADS, N_KV, HD, pos0, tok, 1,
+                                       stride, None, None, 0)
+    torch.cuda.synchronize()
+    assert np.array_equal(host(two).view(np.uint32), host(fused).view(np.uint32))
+    # and the f16 rows are f16 (nearest even) of those
+    out16 = torch.full((tok, N_HEADS, HD), float("nan"), dtype=torch.float16, device="cuda")
+    work = torch.empty_like(x)
+    attn.chunk_attention_q8_split_gate_f16(dev(q), dev(kb), dev(vb), dev(gate), work, out16, N_HEADS, N_KV, HD, pos0,
+                                           tok, 1, stride, None, None, 0)
+    torch.cuda.synchronize()
+    assert np.array_equal(host(out16).view(np.uint16), host(fused).astype(np.float16).view(np.uint16))
+
+
+def test_agrees_with_the_sliced_kernel_and_is_repeatable():
+    tok, pos0 = 200, 90
+    q, kb, vb, stride = chunk_inputs(0x77AA, tok, pos0, 6)
+    a = run_chunk(q, kb, vb, pos0, tok, stride, 0)
+    b = run_chunk(q, kb, vb, pos0, tok, stride, 0)
+    assert np.array_equal(a.view(np.uint32), b.view(np.uint32))  # fixed order of every sum
+    c = run_chunk(q, kb, vb, pos0, tok, stride, 3)
+    ok, _, _ = report("in-workgroup slices vs 3 key slices", c, a, 1e-3, 1e-2)
+    assert ok
+
+
+def test_large_scores_move_the_reference_exponent():
+    # Q scaled so that scores spread over hundreds of log2 units and the running maximum keeps jumping
+    # by more than the lag the kernel allows itself: the rescaling path.  At this scale the f16 rounding of
+    # Q alone moves every kernel 1.5e-2 from the f32 oracle, so the check is against the single-pass kernel,
+    # which has the same operands and rescales at every step.
+    tok, pos0 = 96, 40
+    q, kb, vb, stride = chunk_inputs(0xB16_5C0E, tok, pos0, 0)
+    q = (q * 12.0).astype(np.float32)
+    mono = run_chunk(q, kb, vb, pos0, tok, stride, 1)
+    got = run_chunk(q, kb, vb, pos0, tok, stride, 0)
+    ok, _, _ = report("large scores, in-workgroup slices vs single pass", mono, got, 1e-3, 1e-2)
+    assert ok
+    assert np.isfinite(got).all()
+    want = orc.attn_chunk_kv(q, kb, vb, N_HEADS, N_KV, HD, pos0, tok, stride, SCALE, n_threads=8)
+    ok, _, _ = report("large scores vs the oracle (f16 Q operands)", want, got, 3e-2, 1e-2)
+    assert ok
+
+
+def test_q4_cache():
+    tok, pos0, pad = 150, 20, 3
+    stride = pos0 + tok + pad
+    r = orc.Rng(0x0404)
+    q = r.normal_array((tok, N_HEADS, HD))
+    kb = orc.quantize(1, r.normal_array((N_KV, stride, HD))).reshape(N_KV, stride, -1)
+    vb = orc.quantize(1, r.normal_array((N_KV, stride, HD))).reshape(N_KV, stride, -1)
+    want = orc.attn_chunk_kv(q, kb, vb, N_HEADS, N_KV, HD, pos0, tok, stride, SCALE, dtype=1, n_threads=8)
+    out = torch.full((tok, N_HEADS, HD), float("nan"), dtype=torch.float32, device="cuda")
+    attn.chunk_attention_q8_split(dev(q), dev(kb), dev(vb), out, N_HEADS, N_KV, HD, pos0, tok, 2, stride, None, None, 0)
+    torch.cuda.synchronize()
+    ok, _, _ = report("q4_0 cache, slices inside the workgroups", want, host(out), *GATE)
+    assert ok

@@ -123,6 +123,13 @@ def test_chunk_sweep(i, n_kv, group, tok, pos0, pad, splits, q4):
     torch.cuda.synchronize()
     ok, ma, mr = orc.compare(want, host(out), *CHUNK_GATE)
     assert ok, f"case {i} over the f16 copy: max_abs {ma:.3e} max_rel {mr:.3e}"
+    # and with the keys cut inside the workgroups (splits = 0: no scratch)
+    out.fill_(float("nan"))
+    attn.chunk_attention_q8_split(dev(q), dev(kb), dev(vb), out, n_heads, n_kv, HD, pos0, tok, 1 + dtype,
+                                  stride, None, None, 0)
+    torch.cuda.synchronize()
+    ok, ma, mr = orc.compare(want, host(out), *CHUNK_GATE)
+    assert ok, f"case {i} with in-workgroup slices: max_abs {ma:.3e} max_rel {mr:.3e}"
 
 
 def batch_cases(n):
