@@ -207,8 +207,9 @@ def bench_prefill(torch, attn, tokens, pos0, steps, warmup, layers, prefix_fill=
     tf = flop / (attn_ms * 1e-3) / 1e12
     wl = {(672, 0): "prefill672", (2048, 100_000): "chunk100k"}.get((tokens, pos0), "")
     # (the instantiation that reads the cache: <SPLIT, q4_0, over the f16 copy>)
-    traffic = measured_traffic(wl, ["chunk_q8_kernel<true, false, false>", "chunk_q8_kernel<false, false, false>",
-                                    "chunk_combine_kernel", "chunk_wg_kernel<false>"])
+    traffic = measured_traffic(wl, ["chunk_wg_kernel<false>"] if splits == 0 else
+                               ["chunk_q8_kernel<true, false, false>", "chunk_q8_kernel<false, false, false>",
+                                "chunk_combine_kernel"])
     return {
         "workload": f"prefill {tokens}@{pos0}: rope + q8_0 append + causal GQA attention + gate, "
                     f"1 layer, {H}q/{KV}kv heads, head_dim {HD}",

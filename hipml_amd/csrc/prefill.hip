@@ -811,15 +811,10 @@ __global__ void __launch_bounds__(kPfThreads, 2) chunk_q8_kernel(const ChunkArgs
 // partial results of a head meet in LDS at the end, each wave finishing 64 of the 256 output
 // columns, gate included.  672 tokens x 24 heads are 252 such workgroups, one round of the chip.
 //
-// A step takes four slots, each closed by a workgroup barrier:
-//   A: dequantize K(s+1) into the K tile, request V(s+1), softmax of step s      (VALU)
-//   B: PV of step s                                                              (MFMA)
-//   C: dequantize V(s+1) into the V tile, request K(s+2)                         (VALU)
-//   D: scores of step s+1                                                        (MFMA)
-// Slices 0 and 1 (waves 0..3) run one slot ahead of slices 2 and 3 (waves 4..7), so each SIMD has one
-// wave in a VALU slot and one in an MFMA slot.  The two waves of a slice are always in the same slot:
-// K(s) is last read in D(s-1) and overwritten in A(s), V(s) last read in B(s) and overwritten in C(s).
-// Operand layouts, MFMA shapes and numerics are those of chunk_q8_kernel.
+// A step is a VALU slot (dequantize the next K tile and this step's V tile, softmax) and an MFMA slot (PV
+// of this step, scores of the next), each closed by a workgroup barrier; see the loop.
+// Operand layouts, MFMA shapes and numerics are those of chunk_q8_kernel, except that the running sums
+// are held against a reference exponent that follows the running maximum lazily (see softmax below).
 constexpr int kWgSlices = 4;                   // key slices of a task, one wave each
 constexpr int kWgStep = 32;                    // keys per step
 constexpr int kWgK = kWgStep * kKRow;          // 16,896: K tile of a slice
@@ -831,6 +826,8 @@ constexpr int kWgLds = kWgQAt + 2 * kWgQPark * 1024;
 constexpr int kWgXAt = 4096;                   // merge: (max, sum) table below, accumulator exchange from here
 constexpr int kWgXArea = 8192;                 // two 32-column tiles of one wave
 constexpr int kWgOutPitch = 272;               // a token's 64 finished columns + pad
+constexpr int kWgAhead = 2;     // K operands read this many MFMAs ahead of their use
+constexpr int kWgAheadPv = 2; // V operands
 constexpr float kWgLazy = 8.0f;                // growth of a maximum (log2 units) that moves the reference exponent
 
 template <bool Q4>
@@ -847,8 +844,7 @@ __global__ void __launch_bounds__(kPfThreads, 1) chunk_wg_kernel(const ChunkArgs
     const int lane = threadIdx.x & 63;
     const int ln = lane & 31;
     const int lh = lane >> 5;
-    const int set = wave >> 2;                    // waves w and w + 4 share a SIMD
-    const int sl = set * 2 + ((wave >> 1) & 1);   // key slice
+    const int sl = wave >> 1;                     // key slice
     const int hp = wave & 1;                      // head of the pair
 
     // blockIdx.x -> (token tile, kv head, head pair), the token tiles with the most keys first
@@ -912,12 +908,6 @@ __global__ void __launch_bounds__(kPfThreads, 1) chunk_wg_kernel(const ChunkArgs
         stage_block1(r1, d);
     };
     issue_k(0);
-    Half v0a, v0b; // V(0): requested now, in registers of its own (the accumulators are not live yet)
-    {
-        const uint8_t *u = vbase + unit_at(0);
-        load_half0(v0a, u);
-        load_half1(v0b, u);
-    }
 
     // ---- Q^T operand of this wave's head: the head's four waves fetch eight token rows each (one
     // instruction = one token's 256 floats), convert them and write them as f16 rows into the V tile of
@@ -935,6 +925,7 @@ __global__ void __launch_bounds__(kPfThreads, 1) chunk_wg_kernel(const ChunkArgs
             f[i] = *reinterpret_cast<const float4v *>(qh + (size_t)(tr < a.tokens ? tr : a.tokens - 1) * tok_stride);
         }
         stage_k();
+        issue_k(1);
 #pragma unroll
         for (int i = 0; i < 8; i++) {
             half4 h;
@@ -953,12 +944,6 @@ __global__ void __launch_bounds__(kPfThreads, 1) chunk_wg_kernel(const ChunkArgs
                 *reinterpret_cast<half8 *>(qpark + ks * 1024) = h;
         }
         lds_barrier(); // every wave has its Q: the V tiles may be written
-        {
-            uint8_t *d = Vt + srow * kVRow + spr * 128;
-            stage_block0(v0a, d);
-            stage_block1(v0b, d);
-        }
-        issue_k(1);
     }
 
     float16v O[8];
@@ -995,20 +980,16 @@ __global__ void __launch_bounds__(kPfThreads, 1) chunk_wg_kernel(const ChunkArgs
         for (int ks = 0; ks < 16; ks++)
             acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[ks], ks < kWgQPark ? B[ks] : qf[ks], acc, 0, 0, 0);
         S = acc;
-        // operands two MFMAs ahead; the parked Q steps come first in the chain, two reads per MFMA
-        constexpr int kTwo = kWgQPark > 2 ? kWgQPark - 2 : 0; // MFMAs whose look-ahead is a (K, Q) pair
-        __builtin_amdgcn_sched_group_barrier(0x100, kWgQPark >= 2 ? 4 : 2 + kWgQPark, 0);
+        // K operands are read kWgAhead MFMAs ahead (an LDS read under the load of eight waves takes longer
+        // than two MFMAs); the parked Q steps head the chain and are all read up front
+        static_assert(kWgQPark <= kWgAhead, "the parked steps are read with the first K operands");
+        __builtin_amdgcn_sched_group_barrier(0x100, kWgAhead + kWgQPark, 0);
 #pragma unroll
-        for (int ks = 0; ks < kTwo; ks++) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-        }
-#pragma unroll
-        for (int ks = kTwo; ks < 14; ks++) {
+        for (int ks = 0; ks < 16 - kWgAhead; ks++) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
             __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         }
-        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, kWgAhead, 0);
     };
 
     // lane holds keys (i/4)*8 + lh*4 + i%4 of the step for token ln
@@ -1082,39 +1063,40 @@ __global__ void __launch_bounds__(kPfThreads, 1) chunk_wg_kernel(const ChunkArgs
 #pragma unroll
             for (int dt = 0; dt < 8; dt++)
                 O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[u * 8 + dt], P[u], O[dt], 0, 0, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2 * kWgAheadPv, 0);
 #pragma unroll
-        for (int k = 0; k < 14; k++) {
+        for (int k = 0; k < 16 - kWgAheadPv; k++) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
             __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
         }
-        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, kWgAheadPv, 0);
     };
 
-    lds_barrier(); // V(0) is in LDS
-    if (set == 1)
-        lds_barrier();
+    // Two slots per step, each closed by a barrier, every wave in the same slot:
+    //   V: dequantize K(s+1) into the K tile, request V(s), softmax of step s, dequantize V(s) into the
+    //      V tile, request K(s+2)                                                             (VALU)
+    //   M: PV of step s, scores of step s+1                                                   (MFMA)
+    // K(s) is last read in M(s-1) and V(s-1) as well, so both tiles are free in V(s).  One K or V unit is
+    // in flight per lane: K travels through an M slot, V through the softmax.  (Running waves 4..7 half a
+    // step behind waves 0..3, one set in its VALU slot while the other issues MFMAs as chunk_q8_kernel
+    // does, needs four barriers per step here, because a slice's tiles are single-buffered: 32.7 us
+    // against 31.9 at 672 @ 0.)
     scores(0);
     lds_barrier();
     for (int s = 0; s < nstep; s++) {
         const bool more = s + 1 < nstep;
         if (more)
             stage_k();      // K(s + 1)
-        issue_v(s + 1);
+        issue_v(s);
         softmax(s);
-        lds_barrier();
-        pv(s);
-        lds_barrier();
-        if (more)
-            stage_v();      // V(s + 1)
+        stage_v();          // V(s)
         issue_k(s + 2);
         lds_barrier();
+        pv(s);
         if (more)
             scores(s + 1);
         lds_barrier();
     }
-    if (set == 0)
-        lds_barrier();
 
     // ---- the four slices of a head meet -------------------------------------------------------------
     // Wave `sl` finishes columns 64 sl .. 64 sl + 63 (accumulators 2 sl and 2 sl + 1) of its head.  The
@@ -1135,6 +1117,7 @@ __global__ void __launch_bounds__(kPfThreads, 1) chunk_wg_kernel(const ChunkArgs
         mlx[(hp * kWgSlices + sl) * kQTile + ln] = make_float2(m_run, l_run);
     lds_barrier();
     float m = -INFINITY, den = 0.0f, w_mine = 0.0f;
+    float wj[kWgSlices]; // weight of each slice's sums for this lane's token
     {
         float2 v[kWgSlices];
 #pragma unroll
@@ -1149,12 +1132,10 @@ __global__ void __launch_bounds__(kPfThreads, 1) chunk_wg_kernel(const ChunkArgs
             const float w = on ? __builtin_amdgcn_exp2f(v[j].x - m) : 0.0f;
             den = fmaf(on ? v[j].y : 0.0f, w, den);
             w_mine = j == sl ? w : w_mine;
+            wj[j] = w;
         }
     }
     const float inv = den > 0.0f ? 1.0f / den : 0.0f;
-#pragma unroll
-    for (int dt = 0; dt < 8; dt++)
-        O[dt] *= w_mine;
     // Two passes, columns 0..127 and 128..255: every wave hands the accumulators it does not finish to
     // the wave that does (the layout is the same in every wave, so lane l writes and reads slot l).
     uint8_t *xbase = lds + kWgXAt;
@@ -1179,10 +1160,15 @@ __global__ void __launch_bounds__(kPfThreads, 1) chunk_wg_kernel(const ChunkArgs
         for (int q2 = 0; q2 < 2; q2++) {
             const int qd = 2 * p + q2;
             if (sl == qd) {
+                // (the accumulators arrive as they are; each is weighted here, where it is added)
+#pragma unroll
+                for (int dtl = 0; dtl < 2; dtl++)
+                    O[2 * qd + dtl] *= w_mine;
 #pragma unroll
                 for (int from = 0; from < 3; from++) {
                     const float4v *src =
                         reinterpret_cast<const float4v *>(xbase + ((hp * 2 + q2) * 3 + from) * kWgXArea) + lane;
+                    const float w = wj[from < qd ? from : from + 1];
 #pragma unroll
                     for (int dtl = 0; dtl < 2; dtl++)
 #pragma unroll
@@ -1190,7 +1176,7 @@ __global__ void __launch_bounds__(kPfThreads, 1) chunk_wg_kernel(const ChunkArgs
                             const float4v x = src[(dtl * 4 + g) * 64];
 #pragma unroll
                             for (int j = 0; j < 4; j++)
-                                O[2 * qd + dtl][g * 4 + j] += x[j];
+                                O[2 * qd + dtl][g * 4 + j] = fmaf(x[j], w, O[2 * qd + dtl][g * 4 + j]);
                         }
                 }
             }
