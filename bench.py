@@ -165,6 +165,13 @@ def bench_prefill(torch, attn, tokens, pos0, steps, warmup, layers, prefix_fill=
         # written (same bits as the separate kernels, two launches and one pass over the rows less)
         k, v = caches[i % layers]
         q, kx, vx, gate, out = acts[i % layers]
+        if splits == 0:
+            # the in-workgroup kernel rotates the query rows where it loads them: the first launch rotates and
+            # appends the K/V rows only, and q is never rewritten (same bits in `out`)
+            attn.rope_encode_chunk(None, kx, vx, k, v, H, KV, HD, NROT, THETA, pos0, tokens, 0, stride)
+            attn.chunk_attention_rope_q8(q, k, v, gate, out, None, H, KV, HD, NROT, THETA, pos0, tokens, 1, stride,
+                                         acc, ml, splits)
+            return
         attn.rope_encode_chunk(q, kx, vx, k, v, H, KV, HD, NROT, THETA, pos0, tokens, 0, stride)
         attn.chunk_attention_q8_split_gate(q, k, v, gate, out, H, KV, HD, pos0, tokens, 1, stride,
                                            acc, ml, splits)
@@ -207,7 +214,7 @@ def bench_prefill(torch, attn, tokens, pos0, steps, warmup, layers, prefix_fill=
     tf = flop / (attn_ms * 1e-3) / 1e12
     wl = {(672, 0): "prefill672", (2048, 100_000): "chunk100k"}.get((tokens, pos0), "")
     # (the instantiation that reads the cache: <SPLIT, q4_0, over the f16 copy>)
-    traffic = measured_traffic(wl, ["chunk_wg_kernel<false>"] if splits == 0 else
+    traffic = measured_traffic(wl, ["chunk_wg_kernel<false, true>"] if splits == 0 else
                                ["chunk_q8_kernel<true, false, false>", "chunk_q8_kernel<false, false, false>",
                                 "chunk_combine_kernel"])
     return {

@@ -39,7 +39,7 @@ EXPORTS = [
     "hipml_gemv_q8_0_rows", "hipml_gemm_q8_0_f16", "hipml_attn_output_chunk_q8_0",
     "hipml_kv_rows_copy", "hipml_rope_encode_chunk_f32",
     "hipml_attn_front_encode_f32", "hipml_attn_chunk_front_encode_f32",
-    "hipml_attn_chunk_q8_split_gate_f16",
+    "hipml_attn_chunk_q8_split_gate_f16", "hipml_attn_chunk_rope_q8",
     "hipml_kv_f16_bytes",
     "hipml_kv_f16_rows",
     "hipml_attn_chunk_kv_f16",
@@ -106,6 +106,8 @@ def lib() -> C.CDLL:
             "hipml_attn_chunk_q8_split": (i, [vp, vp, vp, vp, vp, i, i, i, i, i, i, i, vp, vp, i]),
             "hipml_attn_chunk_q8_split_gate": (i, [vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, i, vp, vp, i]),
             "hipml_attn_chunk_q8_split_gate_f16": (i, [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, i, vp, vp, i]),
+            # stream, q, kc, vc, gate, out, out16, n_head, n_kv, head_dim, n_rot, theta, pos0, tokens, dtype, stride, acc, ml, splits
+            "hipml_attn_chunk_rope_q8": (i, [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, f, i, i, i, i, vp, vp, i]),
             "hipml_kv_f16_bytes": (sz, [i, i]),
             "hipml_kv_f16_rows": (i, [vp, i, vp, vp, vp, i, i, i, i, i]),
             "hipml_attn_chunk_kv_f16": (i, [vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, vp, vp, i]),
@@ -419,6 +421,15 @@ def chunk_attention_q8_split_gate_f16(q, kc, vc, gate, out, out16, n_head, n_kv,
                                                     _p(out), _p(out16), n_head, n_kv, head_dim, pos0,
                                                     tokens, dtype, stride, _p(part_acc), _p(part_ml),
                                                     splits))
+
+
+def chunk_attention_rope_q8(q, kc, vc, gate, out, out16, n_head, n_kv, head_dim, n_rot, theta, pos0, tokens,
+                            dtype, stride, part_acc, part_ml, splits, stream=None):
+    """RoPE of the (unrotated) query rows and the chunk attention in one call; gate and out16 may be None.
+    splits == 0: rotated inside the attention kernel, q untouched; otherwise q is rotated in place first."""
+    _check(lib().hipml_attn_chunk_rope_q8(_stream(stream), _p(q), _p(kc), _p(vc), _p(gate), _p(out), _p(out16),
+                                          n_head, n_kv, head_dim, n_rot, theta, pos0, tokens, dtype, stride,
+                                          _p(part_acc), _p(part_ml), splits))
 
 
 def kv_f16_bytes(stride: int, n_kv: int) -> int:

@@ -678,7 +678,7 @@ int hipml_rope_encode_chunk_f32(hipml_stream_t stream, float *q, float *k, const
                                 float theta_base, int pos0, int tokens, int dtype, int stride)
 {
     clear_error();
-    REQUIRE_PTR(q);
+    // (q may be NULL: only the K rows are rotated, for a caller whose attention call rotates the query rows)
     int rc = check_rope(n_head, head_dim, n_rot, theta_base);
     if (rc == 0)
         rc = check_encode(dtype, k, v, k_cache, v_cache, n_kv, head_dim, stride);
@@ -902,7 +902,7 @@ static int chunk_q8_common(hipml_stream_t stream, const float *q, const void *kc
                            float *out, const float *gate, bool want_gate, int n_head, int n_kv,
                            int head_dim, int pos0, int tokens, int dtype, int stride, float *part_acc,
                            float *part_ml, int splits, void *out16 = nullptr, bool want_f16 = false,
-                           const void *kv_f16 = nullptr)
+                           const void *kv_f16 = nullptr, const float *rope_tab = nullptr)
 {
     clear_error();
     REQUIRE_PTR(q);
@@ -947,7 +947,7 @@ static int chunk_q8_common(hipml_stream_t stream, const float *q, const void *kc
     return launch_chunk_q8(as_stream(stream), q, static_cast<const uint8_t *>(kc),
                            static_cast<const uint8_t *>(vc), out, n_head, n_kv, pos0, tokens,
                            stride, part_acc, part_ml, splits, want_gate ? gate : nullptr, dtype == 2 ? 1 : 0,
-                           want_f16 ? out16 : nullptr, kv_f16);
+                           want_f16 ? out16 : nullptr, kv_f16, rope_tab);
 }
 
 int hipml_attn_chunk_q8_split(hipml_stream_t stream, const float *q, const void *kc,
@@ -975,6 +975,38 @@ int hipml_attn_chunk_q8_split_gate_f16(hipml_stream_t stream, const float *q, co
 {
     return chunk_q8_common(stream, q, kc, vc, out, gate, true, n_head, n_kv, head_dim, pos0, tokens,
                            dtype, stride, part_acc, part_ml, splits, out16, true);
+}
+
+int hipml_attn_chunk_rope_q8(hipml_stream_t stream, float *q, const void *kc, const void *vc, const float *gate,
+                             float *out, void *out16, int n_head, int n_kv, int head_dim, int n_rot,
+                             float theta_base, int pos0, int tokens, int dtype, int stride, float *part_acc,
+                             float *part_ml, int splits)
+{
+    clear_error();
+    REQUIRE_PTR(q);
+    int rc = check_rope(n_head, head_dim, n_rot, theta_base);
+    if (rc)
+        return rc;
+    if (pos0 < 0 || tokens < 0)
+        return fail(HIPML_ATTN_E_RANGE, "pos0 %d / tokens %d must be non-negative", pos0, tokens);
+    if ((rc = check_rope_range(pos0, tokens)))
+        return rc;
+    // The in-workgroup kernel rotates the rows where it loads them (table positions only); any other
+    // kernel gets them rotated in place first.
+    const bool in_kernel = splits == 0 && n_rot == 64 && head_dim == kHeadDim &&
+                           (long long)pos0 + tokens <= g_rope.max_pos;
+    if (!in_kernel && tokens > 0) {
+        if ((rc = check_aligned16(q, "q")))
+            return rc;
+        if ((rc = require_init()))
+            return rc;
+        if ((rc = launch_rope_chunk(as_stream(stream), q, q, n_head, 0, head_dim, n_rot, theta_base, pos0, tokens,
+                                    g_rope)))
+            return rc;
+    }
+    return chunk_q8_common(stream, q, kc, vc, out, gate, gate != nullptr, n_head, n_kv, head_dim, pos0, tokens,
+                           dtype, stride, part_acc, part_ml, splits, out16, out16 != nullptr, nullptr,
+                           in_kernel ? g_rope.dev : nullptr);
 }
 
 // ---- chunk prefill over the f16 copy of a cache ----------------------------------------------------

@@ -105,7 +105,7 @@ int prefill_init();
 int launch_chunk_q8(hipStream_t st, const float *q, const uint8_t *kc, const uint8_t *vc,
                     float *out, int n_head, int n_kv, int pos0, int tokens, int stride,
                     float *part_acc, float *part_ml, int splits, const float *gate, int q4, void *out16 = nullptr,
-                    const void *kv_f16 = nullptr);
+                    const void *kv_f16 = nullptr, const float *rope_tab = nullptr);
 // The f16 copy of a cache that launch_chunk_q8 can read instead of the cache (kv_f16): its size for
 // `stride` rows per KV head, and the conversion of the 64-key tiles that hold rows [start, start + rows).
 size_t kv_f16_bytes(int stride, int n_kv);

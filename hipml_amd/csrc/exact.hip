@@ -464,9 +464,10 @@ int launch_rope_encode_chunk(hipStream_t st, int q4, float *q, float *k, const f
     const int slab = 1 << 18; // tokens per launch: keeps the grid inside 2^31 workgroups
     for (int t0 = 0; t0 < tokens; t0 += slab) {
         const int n = tokens - t0 < slab ? tokens - t0 : slab;
-        const int q_blocks = (int)(((long long)n * n_head + kRecRowsPerBlock - 1) / kRecRowsPerBlock);
+        // (q == nullptr: the query rows are rotated elsewhere, e.g. where the attention kernel loads them)
+        const int q_blocks = q == nullptr ? 0 : (int)(((long long)n * n_head + kRecRowsPerBlock - 1) / kRecRowsPerBlock);
         const dim3 grid((unsigned)(q_blocks + (n * n_kv + kRecUnitsPerBlock - 1) / kRecUnitsPerBlock), 1, 1);
-        float *qq = q + (size_t)t0 * n_head * kHeadDim;
+        float *qq = q == nullptr ? nullptr : q + (size_t)t0 * n_head * kHeadDim;
         float *kk = k + (size_t)t0 * n_kv * kHeadDim;
         const float *vv = v + (size_t)t0 * n_kv * kHeadDim;
         if (q4)

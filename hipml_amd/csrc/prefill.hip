@@ -72,6 +72,7 @@ struct ChunkArgs {
     int tile_stride;    // tiles per KV head in the copy
     float *out;
     _Float16 *out16;   // chunk_wg_kernel only: if set, the finished rows go here as f16 instead of to `out`
+    const float *rope_tab; // chunk_wg_kernel<., true> only: cos/sin table [position][32][2]; q holds unrotated rows
     const float *gate; // optional [tokens][n_head][256]: out = attention * sigmoid(gate)
     float *part_acc;
     float *part_ml;
@@ -820,7 +821,7 @@ constexpr int kWgStep = 32;                    // keys per step
 constexpr int kWgK = kWgStep * kKRow;          // 16,896: K tile of a slice
 constexpr int kWgV = kWgStep * kVRow;          // 17,408: its V tile
 constexpr int kWgSlice = kWgK + kWgV;          // 34,304
-constexpr int kWgQPark = 2;                   // d-steps of the Q operand read from LDS at every use: 256 registers do not hold the rest
+constexpr int kWgQPark = 3;                   // d-steps of the Q operand read from LDS at every use: 256 registers do not hold the rest
 constexpr int kWgQAt = kWgSlices * kWgSlice;   // 137,216: [head 2][step][lane] x 16 bytes
 constexpr int kWgLds = kWgQAt + 2 * kWgQPark * 1024;
 constexpr int kWgXAt = 4096;                   // merge: (max, sum) table below, accumulator exchange from here
@@ -830,7 +831,10 @@ constexpr int kWgAhead = 2;     // K operands read this many MFMAs ahead of thei
 constexpr int kWgAheadPv = 2; // V operands
 constexpr float kWgLazy = 8.0f;                // growth of a maximum (log2 units) that moves the reference exponent
 
-template <bool Q4>
+// ROPE: the query rows are rotated (NeoX pairs (k, k + 32) of the first 64 columns, position pos0 + token)
+// between their load and their conversion to f16, with the expressions of the RoPE kernels and
+// without contraction, so the operands are the bits those kernels would have left in memory.
+template <bool Q4, bool ROPE>
 __global__ void __launch_bounds__(kPfThreads, 1) chunk_wg_kernel(const ChunkArgs a)
 {
     typedef typename HalfOf<Q4>::type Half;
@@ -924,8 +928,41 @@ __global__ void __launch_bounds__(kPfThreads, 1) chunk_wg_kernel(const ChunkArgs
             const int tr = t0 + sl * 8 + i;
             f[i] = *reinterpret_cast<const float4v *>(qh + (size_t)(tr < a.tokens ? tr : a.tokens - 1) * tok_stride);
         }
+        // (cos, sin) of pairs 4 l8 .. 4 l8 + 3; lanes 0..15 hold columns 0..63, the others load a row they do not use
+        float4v cs0[ROPE ? 8 : 1], cs1[ROPE ? 8 : 1];
+        if constexpr (ROPE) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const int tr = t0 + sl * 8 + i;
+                const float4v *e = reinterpret_cast<const float4v *>(
+                    a.rope_tab + ((size_t)(a.pos0 + (tr < a.tokens ? tr : a.tokens - 1)) * 32 + 4 * (lane & 7)) * 2);
+                cs0[i] = e[0];
+                cs1[i] = e[1];
+            }
+        }
         stage_k();
         issue_k(1);
+        if constexpr (ROPE) {
+            // y1 = x1 cos - x2 sin (lanes 0..7 hold x1), y2 = x1 sin + x2 cos (lanes 8..15 hold x2): each
+            // product rounded by itself, then one addition, as the RoPE kernels compute them
+#pragma clang fp contract(off)
+            const bool lo = lane < 8, rot = lane < 16;
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const float c[4] = {cs0[i][0], cs0[i][2], cs1[i][0], cs1[i][2]};
+                const float sn[4] = {cs0[i][1], cs0[i][3], cs1[i][1], cs1[i][3]};
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const float x = f[i][j];
+                    // lane l ^ 8 of the same 16 lanes: a rotation of the row by 8
+                    const float other = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x128, 0xf, 0xf, false));
+                    const float own = x * c[j];
+                    const float cross = other * sn[j];
+                    const float y = own + (lo ? -cross : cross);
+                    f[i][j] = rot ? y : x;
+                }
+            }
+        }
 #pragma unroll
         for (int i = 0; i < 8; i++) {
             half4 h;
@@ -982,7 +1019,6 @@ __global__ void __launch_bounds__(kPfThreads, 1) chunk_wg_kernel(const ChunkArgs
         S = acc;
         // K operands are read kWgAhead MFMAs ahead (an LDS read under the load of eight waves takes longer
         // than two MFMAs); the parked Q steps head the chain and are all read up front
-        static_assert(kWgQPark <= kWgAhead, "the parked steps are read with the first K operands");
         __builtin_amdgcn_sched_group_barrier(0x100, kWgAhead + kWgQPark, 0);
 #pragma unroll
         for (int ks = 0; ks < 16 - kWgAhead; ks++) {
@@ -1468,10 +1504,16 @@ int prefill_init()
         e = hipFuncSetAttribute(reinterpret_cast<const void *>(&kv_f16_tiles_kernel<true>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, kBufBytes);
     if (e == hipSuccess)
-        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&chunk_wg_kernel<false>),
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&chunk_wg_kernel<false, false>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, kWgLds);
     if (e == hipSuccess)
-        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&chunk_wg_kernel<true>),
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&chunk_wg_kernel<true, false>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, kWgLds);
+    if (e == hipSuccess)
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&chunk_wg_kernel<false, true>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, kWgLds);
+    if (e == hipSuccess)
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&chunk_wg_kernel<true, true>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, kWgLds);
     if (e != hipSuccess)
         return fail((int)e, "hipFuncSetAttribute(prefill LDS) failed: %d (%s)", (int)e,
@@ -1482,8 +1524,9 @@ int prefill_init()
 int launch_chunk_q8(hipStream_t st, const float *q, const uint8_t *kc, const uint8_t *vc,
                     float *out, int n_head, int n_kv, int pos0, int tokens, int stride,
                     float *part_acc, float *part_ml, int splits, const float *gate, int q4, void *out16,
-                    const void *kv_f16)
+                    const void *kv_f16, const float *rope_tab)
 {
+    // rope_tab != nullptr (splits == 0 only): q holds unrotated rows, the kernel rotates them as it loads them
     ChunkArgs a;
     // kv_f16 != nullptr: K and V are read from the f16 copy of the cache (kc, vc unused)
     a.tile_stride = (stride + kKTile - 1) / kKTile;
@@ -1512,10 +1555,15 @@ int launch_chunk_q8(hipStream_t st, const float *q, const uint8_t *kc, const uin
         // the key slices stay inside the workgroup: no partial rows, gate and f16 rows in the same launch
         a.out16 = static_cast<_Float16 *>(out16);
         const unsigned wgs = (unsigned)((tokens + kQTile - 1) / kQTile * n_kv * ((a.group + 1) / 2));
-        if (q4)
-            hipLaunchKernelGGL(chunk_wg_kernel<true>, dim3(wgs, 1, 1), dim3(kPfThreads, 1, 1), kWgLds, st, a);
+        a.rope_tab = rope_tab;
+        if (q4 && rope_tab)
+            hipLaunchKernelGGL((chunk_wg_kernel<true, true>), dim3(wgs, 1, 1), dim3(kPfThreads, 1, 1), kWgLds, st, a);
+        else if (q4)
+            hipLaunchKernelGGL((chunk_wg_kernel<true, false>), dim3(wgs, 1, 1), dim3(kPfThreads, 1, 1), kWgLds, st, a);
+        else if (rope_tab)
+            hipLaunchKernelGGL((chunk_wg_kernel<false, true>), dim3(wgs, 1, 1), dim3(kPfThreads, 1, 1), kWgLds, st, a);
         else
-            hipLaunchKernelGGL(chunk_wg_kernel<false>, dim3(wgs, 1, 1), dim3(kPfThreads, 1, 1), kWgLds, st, a);
+            hipLaunchKernelGGL((chunk_wg_kernel<false, false>), dim3(wgs, 1, 1), dim3(kPfThreads, 1, 1), kWgLds, st, a);
         return launched(q4 ? "attn_chunk_q4_wg" : "attn_chunk_q8_wg");
     }
     // slices per block: the last block (most keys) gets `splits`, a block with fewer key tiles gets

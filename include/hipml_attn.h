@@ -212,6 +212,8 @@ int hipml_kv_encode_bulk(hipml_stream_t stream, int dtype, const float *k_f32, c
 /* RoPE of a chunk and the append of its K/V rows in one launch: hipml_rope_chunk_f32(q, k, ...)
  * followed by hipml_kv_encode_bulk(dtype, k, v, ..., start = pos0, src0 = 0, rows = tokens), with the
  * same bits in q, k and both caches.  v is f32 [tokens][n_kv][head_dim].  head_dim 256, n_rot 64.
+ * q may be NULL: then only the K rows are rotated (for hipml_attn_chunk_rope_q8, which rotates the
+ * query rows itself).
  * Replaces the RoPE half of AttnLayer::chunk_front + Launcher::kv_encode_bulk as issued per chunk,
  * crates/hipml-model/src/gpu/attn_tile.rs:53-68. */
 int hipml_rope_encode_chunk_f32(hipml_stream_t stream, float *q, float *k, const float *v, void *k_cache,
@@ -357,6 +359,23 @@ int hipml_attn_chunk_q8_split_gate_f16(hipml_stream_t stream, const float *q, co
                                        const void *vc, const float *gate, float *out, void *out16,
                                        int n_head, int n_kv, int head_dim, int pos0, int tokens, int dtype,
                                        int stride, float *part_acc, float *part_ml, int splits);
+
+/* hipml_rope_chunk_f32 of the query rows and the chunk attention in one call: q holds the
+ * UNROTATED query rows.  With splits == 0 (and n_rot 64, positions inside the registered table) the
+ * attention kernel rotates each row between its load and its use, with the expressions of the RoPE
+ * kernels, and q is left as it was: the pass that rotates the query rows in memory (33 MB of traffic
+ * for 672 tokens) goes away; pair it with hipml_rope_encode_chunk_f32(q = NULL), which rotates and
+ * appends the K rows only.  With any other `splits` the rows are first rotated in place
+ * (hipml_rope_chunk_f32 on q alone) and the call continues as hipml_attn_chunk_q8_split_gate /
+ * _gate_f16; q then holds the rotated rows.  Either way the results are the bits of the separate
+ * calls.  gate and out16 may be NULL (no gate / f32 rows in `out`); with out16 the rows are
+ * delivered as f16 there and `out` is working memory.  Replaces the query half of the RoPE in
+ * norm_rope_chunk_f32 (AttnLayer::chunk_front, crates/hipml-kernels/src/attn_gpu/imp/attn_chunk.rs:167-199)
+ * followed by chunk_attention_q8_split (attn_chunk_kv.rs:72-107). */
+int hipml_attn_chunk_rope_q8(hipml_stream_t stream, float *q, const void *kc, const void *vc,
+                             const float *gate, float *out, void *out16, int n_head, int n_kv,
+                             int head_dim, int n_rot, float theta_base, int pos0, int tokens, int dtype,
+                             int stride, float *part_acc, float *part_ml, int splits);
 
 /* ---- chunk prefill over an f16 copy of the cache -------------------------------------------------
  * The reference's chunk kernel dequantizes the cache rows it attends over inside every workgroup

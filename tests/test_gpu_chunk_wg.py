@@ -100,3 +100,66 @@ def test_q4_cache():
     torch.cuda.synchronize()
     ok, _, _ = report("q4_0 cache, slices inside the workgroups", want, host(out), *GATE)
     assert ok
+
+
+@pytest.mark.parametrize("tok,pos0,splits", [(672, 0, 0), (70, 33, 0), (100, 40, 3), (64, 5, 1)])
+def test_query_rows_rotated_inside_the_attention_call(tok, pos0, splits):
+    # hipml_attn_chunk_rope_q8 on unrotated query rows = hipml_rope_chunk_f32 on them, then the attention:
+    # the same bits, with the rows rotated in the kernel (splits 0, q untouched) or in place first
+    n_rot, theta = 64, 1e7
+    attn.rope_table(theta, n_rot, 2048)
+    q, kb, vb, stride = chunk_inputs(0x120E + tok, tok, pos0, 4)
+    gate = orc.Rng(0x6A7F + tok).normal_array((tok, N_HEADS, HD))
+    kd, vd, gd = dev(kb), dev(vb), dev(gate)
+    acc = ml = None
+    if splits >= 2:
+        acc, ml = attn.chunk_scratch(tok, N_HEADS, splits)
+    # separate calls (k rows are not involved: a dummy stands in)
+    q_rot = dev(q)
+    k_dummy = torch.zeros((tok, N_KV, HD), dtype=torch.float32, device="cuda")
+    attn.rope_chunk(q_rot, k_dummy, N_HEADS, N_KV, HD, n_rot, theta, pos0, tok)
+    want = torch.full((tok, N_HEADS, HD), float("nan"), dtype=torch.float32, device="cuda")
+    attn.chunk_attention_q8_split_gate(q_rot, kd, vd, gd, want, N_HEADS, N_KV, HD, pos0, tok, 1, stride, acc, ml,
+                                       splits)
+    # one call
+    q_in = dev(q)
+    got = torch.full((tok, N_HEADS, HD), float("nan"), dtype=torch.float32, device="cuda")
+    attn.chunk_attention_rope_q8(q_in, kd, vd, gd, got, None, N_HEADS, N_KV, HD, n_rot, theta, pos0, tok, 1,
+                                 stride, acc, ml, splits)
+    torch.cuda.synchronize()
+    assert np.array_equal(host(got).view(np.uint32), host(want).view(np.uint32))
+    if splits == 0:
+        assert np.array_equal(host(q_in).view(np.uint32), q.view(np.uint32))  # left as it was
+    else:
+        assert np.array_equal(host(q_in).view(np.uint32), host(q_rot).view(np.uint32))  # rotated in place
+    # f16 rows, no gate
+    out16 = torch.full((tok, N_HEADS, HD), float("nan"), dtype=torch.float16, device="cuda")
+    work = torch.empty_like(got)
+    plain = torch.empty_like(got)
+    attn.chunk_attention_q8_split(q_rot, kd, vd, plain, N_HEADS, N_KV, HD, pos0, tok, 1, stride, acc, ml, splits)
+    attn.chunk_attention_rope_q8(dev(q), kd, vd, None, work, out16, N_HEADS, N_KV, HD, n_rot, theta, pos0, tok, 1,
+                                 stride, acc, ml, splits)
+    torch.cuda.synchronize()
+    assert np.array_equal(host(out16).view(np.uint16), host(plain).astype(np.float16).view(np.uint16))
+
+
+def test_fused_append_may_leave_the_query_rows_alone():
+    # hipml_rope_encode_chunk_f32 with q = NULL: K rotated, K/V appended, same bits as with q given
+    tok, pos0, n_rot, theta = 50, 7, 64, 1e7
+    attn.rope_table(theta, n_rot, 2048)
+    stride = 64
+    r = orc.Rng(0xA99E)
+    q = r.normal_array((tok, N_HEADS, HD))
+    k = r.normal_array((tok, N_KV, HD))
+    v = r.normal_array((tok, N_KV, HD))
+    res = []
+    for with_q in (True, False):
+        kc = torch.zeros((N_KV, stride, 272), dtype=torch.uint8, device="cuda")
+        vc = torch.zeros_like(kc)
+        kd = dev(k)
+        attn.rope_encode_chunk(dev(q) if with_q else None, kd, dev(v), kc, vc, N_HEADS, N_KV, HD, n_rot, theta, pos0,
+                               tok, 0, stride)
+        torch.cuda.synchronize()
+        res.append((host(kc), host(vc), host(kd)))
+    for a, b in zip(*res):
+        assert np.array_equal(a.view(np.uint8), b.view(np.uint8))
