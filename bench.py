@@ -129,7 +129,7 @@ def bench_prefill(torch, attn, tokens, pos0, steps, warmup, layers, prefix_fill=
     attn.rope_table(THETA, NROT, max(pos0 + tokens, 1024))
     # the f16 copy of every layer cache, current up to the prefix (as earlier chunks would have left it)
     copies = []
-    for k, v in caches:
+    for k, v in caches if splits != 0 else []:
         c = attn.kv_f16_alloc(stride, KV)
         if pos0 > 0:
             attn.kv_f16_rows(0, k, v, c, KV, HD, stride, 0, pos0)
@@ -196,8 +196,11 @@ def bench_prefill(torch, attn, tokens, pos0, steps, warmup, layers, prefix_fill=
 
     unfused_ms = wall(step_unfused)
     wall_ms = wall(step)
-    copy_ms = wall(step_copy)
-    copy_rebuilt_ms = wall(lambda i: step_copy(i, True))
+    # the f16 copy of the cache serves long prefixes: the sliced kernel over it is not what a chunk near
+    # position 0 would run (splits == 0), so that leg is left out there
+    with_copy = splits != 0
+    copy_ms = wall(step_copy) if with_copy else None
+    copy_rebuilt_ms = wall(lambda i: step_copy(i, True)) if with_copy else None
 
     # the attention launch alone, HIP events on the launch stream
     def events(fn):
@@ -209,7 +212,7 @@ def bench_prefill(torch, attn, tokens, pos0, steps, warmup, layers, prefix_fill=
         return t.ms / steps
 
     attn_ms = events(attention)
-    attn_copy_ms = events(attention_copy)
+    attn_copy_ms = events(attention_copy) if with_copy else None
     flop = prefill_flop(pos0, tokens)
     tf = flop / (attn_ms * 1e-3) / 1e12
     wl = {(672, 0): "prefill672", (2048, 100_000): "chunk100k"}.get((tokens, pos0), "")
@@ -226,7 +229,7 @@ def bench_prefill(torch, attn, tokens, pos0, steps, warmup, layers, prefix_fill=
         "ms_per_step_separate_launches": unfused_ms,
         "attn_ms": attn_ms,
         "attn_tok_per_s": tokens / (attn_ms * 1e-3),
-        "over_f16_copy": {
+        "over_f16_copy": None if not with_copy else {
             "note": "the same step with the attention reading an f16 copy of the cache that the step keeps "
                     "current (hipml_kv_f16_rows for the chunk's rows after the append, then "
                     "hipml_attn_chunk_kv_f16); rebuilt = the whole copy made again from row 0 in every step",
