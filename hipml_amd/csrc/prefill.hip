@@ -911,7 +911,6 @@ __global__ void __launch_bounds__(kPfThreads, 1) chunk_wg_kernel(const ChunkArgs
         stage_block0(r0, d);
         stage_block1(r1, d);
     };
-    issue_k(0);
 
     // ---- Q^T operand of this wave's head: the head's four waves fetch eight token rows each (one
     // instruction = one token's 256 floats), convert them and write them as f16 rows into the V tile of
@@ -928,6 +927,7 @@ __global__ void __launch_bounds__(kPfThreads, 1) chunk_wg_kernel(const ChunkArgs
             const int tr = t0 + sl * 8 + i;
             f[i] = *reinterpret_cast<const float4v *>(qh + (size_t)(tr < a.tokens ? tr : a.tokens - 1) * tok_stride);
         }
+        issue_k(0); // (behind the query rows: they come from further away)
         // (cos, sin) of pairs 4 l8 .. 4 l8 + 3; lanes 0..15 hold columns 0..63, the others load a row they do not use
         float4v cs0[ROPE ? 8 : 1], cs1[ROPE ? 8 : 1];
         if constexpr (ROPE) {
@@ -974,13 +974,12 @@ __global__ void __launch_bounds__(kPfThreads, 1) chunk_wg_kernel(const ChunkArgs
         lds_barrier(); // Q rows and K(0) are in LDS
 #pragma unroll
         for (int ks = 0; ks < 16; ks++) {
-            const half8 h = *reinterpret_cast<const half8 *>(qa + ln * kKRow + ks * 32 + lh * 16);
-            if (ks >= kWgQPark)
-                qf[ks] = h;
-            else if ((ks & 3) == sl) // the head's four waves read the same values: each parks its share
-                *reinterpret_cast<half8 *>(qpark + ks * 1024) = h;
+            // (steps below kWgQPark stay in registers for the first scores only; their parked copies are
+            // read from the second scores on, two barriers after they are written)
+            qf[ks] = *reinterpret_cast<const half8 *>(qa + ln * kKRow + ks * 32 + lh * 16);
+            if (ks < kWgQPark && (ks & 3) == sl) // the head's four waves read the same values: each parks its share
+                *reinterpret_cast<half8 *>(qpark + ks * 1024) = qf[ks];
         }
-        lds_barrier(); // every wave has its Q: the V tiles may be written
     }
 
     float16v O[8];
@@ -998,7 +997,8 @@ __global__ void __launch_bounds__(kPfThreads, 1) chunk_wg_kernel(const ChunkArgs
 
     auto live = [&](int s) { return task_valid && kbeg + s * kWgStep < khi; }; // wave-uniform
 
-    auto scores = [&](int s) {
+    auto scores = [&](int s, auto first) { // first: the scores of step 0, every Q step still in registers
+        constexpr bool kFirst = decltype(first)::value;
         if (!live(s))
             return;
         const uint8_t *Kh = Kt + ln * kKRow + lh * 16;
@@ -1007,19 +1007,21 @@ __global__ void __launch_bounds__(kPfThreads, 1) chunk_wg_kernel(const ChunkArgs
         for (int i = 0; i < 16; i++)
             acc[i] = 0.0f;
         half8 A[16], B[kWgQPark > 0 ? kWgQPark : 1];
+        if constexpr (!kFirst) {
 #pragma unroll
-        for (int ks = 0; ks < kWgQPark; ks++)
-            B[ks] = *reinterpret_cast<const half8 *>(qpark + ks * 1024);
+            for (int ks = 0; ks < kWgQPark; ks++)
+                B[ks] = *reinterpret_cast<const half8 *>(qpark + ks * 1024);
+        }
 #pragma unroll
         for (int ks = 0; ks < 16; ks++)
             A[ks] = *reinterpret_cast<const half8 *>(Kh + ks * 32);
 #pragma unroll
         for (int ks = 0; ks < 16; ks++)
-            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[ks], ks < kWgQPark ? B[ks] : qf[ks], acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[ks], !kFirst && ks < kWgQPark ? B[ks] : qf[ks], acc, 0, 0, 0);
         S = acc;
         // K operands are read kWgAhead MFMAs ahead (an LDS read under the load of eight waves takes longer
         // than two MFMAs); the parked Q steps head the chain and are all read up front
-        __builtin_amdgcn_sched_group_barrier(0x100, kWgAhead + kWgQPark, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, kWgAhead + (kFirst ? 0 : kWgQPark), 0);
 #pragma unroll
         for (int ks = 0; ks < 16 - kWgAhead; ks++) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
@@ -1117,8 +1119,8 @@ __global__ void __launch_bounds__(kPfThreads, 1) chunk_wg_kernel(const ChunkArgs
     // step behind waves 0..3, one set in its VALU slot while the other issues MFMAs as chunk_q8_kernel
     // does, needs four barriers per step here, because a slice's tiles are single-buffered: 32.7 us
     // against 31.9 at 672 @ 0.)
-    scores(0);
-    lds_barrier();
+    scores(0, std::true_type());
+    lds_barrier(); // K(0) may be replaced, and every wave has read its Q: the V tiles may be written
     for (int s = 0; s < nstep; s++) {
         const bool more = s + 1 < nstep;
         if (more)
@@ -1130,7 +1132,7 @@ __global__ void __launch_bounds__(kPfThreads, 1) chunk_wg_kernel(const ChunkArgs
         lds_barrier();
         pv(s);
         if (more)
-            scores(s + 1);
+            scores(s + 1, std::false_type());
         lds_barrier();
     }
 
@@ -1151,10 +1153,10 @@ __global__ void __launch_bounds__(kPfThreads, 1) chunk_wg_kernel(const ChunkArgs
     float2 *mlx = reinterpret_cast<float2 *>(lds); // [head 2][slice 4][token 32]
     if (lh == 0)
         mlx[(hp * kWgSlices + sl) * kQTile + ln] = make_float2(m_run, l_run);
-    lds_barrier();
-    float m = -INFINITY, den = 0.0f, w_mine = 0.0f;
+    float den = 0.0f, w_mine = 0.0f;
     float wj[kWgSlices]; // weight of each slice's sums for this lane's token
-    {
+    auto weights = [&]() { // (after the first barrier below: the table travels with the first accumulators)
+        float m = -INFINITY;
         float2 v[kWgSlices];
 #pragma unroll
         for (int j = 0; j < kWgSlices; j++) {
@@ -1170,8 +1172,7 @@ __global__ void __launch_bounds__(kPfThreads, 1) chunk_wg_kernel(const ChunkArgs
             w_mine = j == sl ? w : w_mine;
             wj[j] = w;
         }
-    }
-    const float inv = den > 0.0f ? 1.0f / den : 0.0f;
+    };
     // Two passes, columns 0..127 and 128..255: every wave hands the accumulators it does not finish to
     // the wave that does (the layout is the same in every wave, so lane l writes and reads slot l).
     uint8_t *xbase = lds + kWgXAt;
@@ -1192,6 +1193,8 @@ __global__ void __launch_bounds__(kPfThreads, 1) chunk_wg_kernel(const ChunkArgs
             }
         }
         lds_barrier();
+        if (p == 0)
+            weights();
 #pragma unroll
         for (int q2 = 0; q2 < 2; q2++) {
             const int qd = 2 * p + q2;
@@ -1219,6 +1222,7 @@ __global__ void __launch_bounds__(kPfThreads, 1) chunk_wg_kernel(const ChunkArgs
         }
         lds_barrier();
     }
+    const float inv = den > 0.0f ? 1.0f / den : 0.0f;
     float16v R[2];
 #pragma unroll
     for (int qd = 0; qd < 4; qd++)
