@@ -235,6 +235,25 @@ def test_rope_beyond_table_is_an_error_unless_device_angles_are_allowed():
         attn.rope_table(THETA, N_ROT, 131072)
 
 
+def test_q_gate_over_the_whole_range_of_gates():
+    # the kernels take the exponential and the quotient from the hardware's 1-ulp instructions: held to the
+    # same 1e-6 / 1e-5 over gates from where the sigmoid underflows to where it is 1, and exact at the ends
+    g = np.concatenate([np.linspace(-104.0, 104.0, 8321), [0.0, -0.0, 88.7, -88.7, 1e-30, -1e-30]]).astype(np.float32)
+    q = (np.arange(g.size) % 7 - 3).astype(np.float32) * 0.37 + 0.11
+    out = dev(q)
+    attn.q_gate(out, dev(g), out)
+    torch.cuda.synchronize()
+    got = host(out)
+    ok, _, _ = report("q_gate, gates -104 .. 104", orc.q_gate(q, g), got, 1e-6, 1e-5)
+    assert ok
+    ends = np.array([-np.inf, np.inf, -1e4, 1e4], np.float32)
+    x = np.array([2.5, 2.5, -3.0, -3.0], np.float32)
+    o = dev(x)
+    attn.q_gate(o, dev(ends), o)
+    torch.cuda.synchronize()
+    assert np.array_equal(host(o), np.array([0.0, 2.5, -0.0, -3.0], np.float32))
+
+
 def test_q_gate_within_tight_tolerance():
     # attn_parity.rs:66-78 (n = 384) and the chunk shape 672 x 24 x 256
     r = orc.Rng(0x5555_6666_7777_8888)
