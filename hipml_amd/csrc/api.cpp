@@ -41,7 +41,7 @@ int launched(const char *what)
     return (int)e;
 }
 
-int check_heads(int n_heads, int n_kv, int head_dim)
+int check_heads(int n_heads, int n_kv, int head_dim, bool narrow)
 {
     if (n_kv <= 0 || n_heads <= 0 || n_heads % n_kv != 0)
         return fail(HIPML_ATTN_E_SHAPE, "n_heads %d is not a multiple of n_kv %d", n_heads, n_kv);
@@ -49,9 +49,11 @@ int check_heads(int n_heads, int n_kv, int head_dim)
     if (group > kMaxGroup)
         return fail(HIPML_ATTN_E_SHAPE, "GQA group %d > %d: one workgroup covers at most %d heads",
                     group, kMaxGroup, kMaxGroup);
+    if (narrow && head_dim == 64)
+        return 0;
     if (head_dim != kHeadDim)
-        return fail(HIPML_ATTN_E_SHAPE, "head_dim %d: the gfx950 attention kernels are head_dim %d only",
-                    head_dim, kHeadDim);
+        return fail(HIPML_ATTN_E_SHAPE, "head_dim %d: the gfx950 attention kernels are head_dim %d%s",
+                    head_dim, kHeadDim, narrow ? " (decode also 64)" : " only");
     return 0;
 }
 
@@ -126,7 +128,7 @@ static int decode_common(hipStream_t st, int dtype, const int32_t *pos, const fl
     REQUIRE_PTR(part_acc);
     REQUIRE_PTR(part_ml);
     REQUIRE_PTR(out);
-    int rc = check_heads(n_heads, n_kv, head_dim);
+    int rc = check_heads(n_heads, n_kv, head_dim, true);
     if (rc)
         return rc;
     if (stride <= 0)
@@ -154,6 +156,7 @@ static int decode_common(hipStream_t st, int dtype, const int32_t *pos, const fl
     L.pos = pos;
     L.n_heads = n_heads;
     L.n_kv = n_kv;
+    L.head_dim = head_dim;
     L.stride = stride;
     L.splits = splits;
     L.slots = slots;
@@ -759,8 +762,8 @@ int hipml_attn_decode_kv(hipml_stream_t stream, const int32_t *step, int dtype, 
     const size_t slice = (size_t)(n_heads > 0 ? n_heads : 0) * (size_t)(splits > 0 ? splits : 0);
     return decode_common(as_stream(stream), fmt, step, q, static_cast<const uint8_t *>(k) + k_off,
                          static_cast<const uint8_t *>(v) + v_off, part_acc, part_ml, out, n_heads,
-                         n_kv, head_dim, stride, scale, splits, 0, slice * kHeadDim, slice * 2,
-                         (size_t)n_heads * kHeadDim, 1, nullptr);
+                         n_kv, head_dim, stride, scale, splits, 0, slice * (size_t)(head_dim > 0 ? head_dim : 0), slice * 2,
+                         (size_t)n_heads * (size_t)(head_dim > 0 ? head_dim : 0), 1, nullptr);
 }
 
 int hipml_attn_decode_kv_noalloc(hipml_stream_t stream, const int32_t *step, int dtype, const float *q,
@@ -872,8 +875,8 @@ int hipml_attn_decode_kv_gate(hipml_stream_t stream, const int32_t *step, int dt
     const size_t slice = (size_t)(n_heads > 0 ? n_heads : 0) * (size_t)(splits > 0 ? splits : 0);
     return decode_common(as_stream(stream), fmt, step, q, static_cast<const uint8_t *>(k) + k_off,
                          static_cast<const uint8_t *>(v) + v_off, part_acc, part_ml, out, n_heads,
-                         n_kv, head_dim, stride, scale, splits, 0, slice * kHeadDim, slice * 2,
-                         (size_t)n_heads * kHeadDim, 1, nullptr, gate);
+                         n_kv, head_dim, stride, scale, splits, 0, slice * (size_t)(head_dim > 0 ? head_dim : 0), slice * 2,
+                         (size_t)n_heads * (size_t)(head_dim > 0 ? head_dim : 0), 1, nullptr, gate);
 }
 
 int hipml_attn_decode_batch_cols_gate(hipml_stream_t stream, int dtype, const int32_t *pos,

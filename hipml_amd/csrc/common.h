@@ -43,7 +43,8 @@ inline hipStream_t as_stream(hipml_stream_t s) { return reinterpret_cast<hipStre
 
 // n_heads / n_kv / head_dim rules shared by the attention launchers
 // (crates/hipml-kernels/src/launch_kv.rs:130-148 in the reference).
-int check_heads(int n_heads, int n_kv, int head_dim);
+// (narrow: the decode launchers also take head_dim 64)
+int check_heads(int n_heads, int n_kv, int head_dim, bool narrow = false);
 
 // Kernel launchers implemented in the .hip translation units -------------------
 
@@ -87,6 +88,7 @@ struct DecodeLaunch {
     const float *gate;  // rows laid out like `out`, or nullptr: out *= sigmoid(gate) in the merge
     const int32_t *pos; // (pos, seq) pairs, one per row
     int n_heads, n_kv, stride, splits, slots;
+    int head_dim; // 256: the MFMA kernels; 64: the plain fp32 kernels
     int q4; // cache format: 0 = q8_0, 1 = q4_0
     int exact; // q8_0 only: the fp32-class variant (Q and the weights as hi + lo f16 pairs)
     float scale;

@@ -1714,8 +1714,201 @@ int decode_static_partials(int n_heads, int splits, float **part_acc, float **pa
     return 0;
 }
 
+// ---- head widths other than 256 ------------------------------------------------------------------------
+// The reference's decode launchers take any head_dim that is a multiple of the block size, and its
+// parity table runs head_dim 64 (crates/hipml-core/src/parity_kv.rs:166-213).  The model this library
+// is built for has head_dim 256 and every kernel above is laid out for that; the two kernels below serve
+// head_dim 64 with the same arguments, partial format and merge rule, in plain fp32 arithmetic: one wave
+// per (query row, head, key split), one key per lane and turn, the lane's running maximum, sum and
+// head_dim accumulators in registers, the lanes' states merged with lane exchanges at the end.  They are
+// there for completeness of the interface, not tuned.
+struct DecodeHdArgs {
+    const float *q;
+    const uint8_t *k;
+    const uint8_t *v;
+    float *part_acc;
+    float *part_ml;
+    float *out;
+    const float *gate;
+    const int32_t *pos;
+    int n_heads, n_kv, group, stride, splits;
+    float scale_log2; // scale * log2(e)
+    size_t kv_slot_bytes, acc_slot, ml_slot, q_slot;
+    uint8_t slot_of_row[kMaxSlots * kMaxCols];
+};
+
+// block b of a cached row as 32 floats (f16 scale x integer)
+template <bool Q4>
+__device__ __forceinline__ void hd_block(const uint8_t *row, int b, float (&x)[32])
+{
+    constexpr int kBlockBytes = Q4 ? kQ4BlockBytes : kQ8BlockBytes;
+    const uint16_t *w = reinterpret_cast<const uint16_t *>(row + b * kBlockBytes); // blocks are 2-byte aligned
+    const float d = (float)__builtin_bit_cast(_Float16, w[0]);
+    if (Q4) {
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const uint32_t two = w[1 + j]; // bytes 2j, 2j + 1: elements 2j, 2j + 1 in the low nibbles, + 16 in the high ones
+            x[2 * j] = d * (float)((int)(two & 15) - 8);
+            x[2 * j + 16] = d * (float)((int)((two >> 4) & 15) - 8);
+            x[2 * j + 1] = d * (float)((int)((two >> 8) & 15) - 8);
+            x[2 * j + 17] = d * (float)((int)((two >> 12) & 15) - 8);
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < 16; j++) {
+            const uint32_t two = w[1 + j];
+            x[2 * j] = d * (float)(int8_t)(two & 0xff);
+            x[2 * j + 1] = d * (float)(int8_t)(two >> 8);
+        }
+    }
+}
+
+template <int HD, bool Q4>
+__global__ void __launch_bounds__(64 * kMaxGroup, 1) decode_hd_kernel(const DecodeHdArgs a)
+{
+    constexpr int kRow = HD / 32 * (Q4 ? kQ4BlockBytes : kQ8BlockBytes);
+    __shared__ float qs[kMaxGroup][HD];
+    const int lane = threadIdx.x & 63, hq = threadIdx.x >> 6;
+    const int kvh = blockIdx.x / a.splits, split = blockIdx.x - kvh * a.splits;
+    const int r = blockIdx.y;
+    const int head = kvh * a.group + hq;
+    for (int d = lane; d < HD; d += 64)
+        qs[hq][d] = a.q[(size_t)r * a.q_slot + (size_t)head * HD + d];
+    __syncthreads();
+    int seq = a.pos[2 * r + 1];
+    seq = seq < 0 ? 0 : (seq > a.stride ? a.stride : seq);
+    const int per = (seq + a.splits - 1) / a.splits; // the reference's partition (attn_decode_kv_w.hip:124-126)
+    const int lo = split * per;
+    const int hi = lo + per < seq ? lo + per : seq;
+    const size_t base = (size_t)a.slot_of_row[r] * a.kv_slot_bytes + (size_t)kvh * a.stride * kRow;
+    float m = -INFINITY, l = 0.0f, acc[HD];
+#pragma unroll
+    for (int d = 0; d < HD; d++)
+        acc[d] = 0.0f;
+    for (int key = lo + lane; key < hi; key += 64) {
+        float x[32];
+        float dot = 0.0f;
+#pragma unroll
+        for (int b = 0; b < HD / 32; b++) {
+            hd_block<Q4>(a.k + base + (size_t)key * kRow, b, x);
+#pragma unroll
+            for (int d = 0; d < 32; d++)
+                dot = fmaf(qs[hq][b * 32 + d], x[d], dot);
+        }
+        const float sc = dot * a.scale_log2;
+        const float mn = fmaxf(m, sc);
+        const float corr = __builtin_amdgcn_exp2f(m - mn); // (m = -inf the first time: 0)
+        const float pr = __builtin_amdgcn_exp2f(sc - mn);
+        l = l * corr + pr;
+#pragma unroll
+        for (int b = 0; b < HD / 32; b++) {
+            hd_block<Q4>(a.v + base + (size_t)key * kRow, b, x);
+#pragma unroll
+            for (int d = 0; d < 32; d++)
+                acc[b * 32 + d] = fmaf(pr, x[d], acc[b * 32 + d] * corr);
+        }
+        m = mn;
+    }
+    // the lanes' states against the wave's maximum
+    float mw = m;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1)
+        mw = fmaxf(mw, __shfl_xor(mw, o));
+    const float w = m == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(m - mw);
+    float lw = l * w;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1)
+        lw += __shfl_xor(lw, o);
+    const size_t part = (size_t)head * a.splits + split;
+    float *pa = a.part_acc + (size_t)r * a.acc_slot + part * HD;
+#pragma unroll
+    for (int d = 0; d < HD; d++) {
+        float t = acc[d] * w;
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1)
+            t += __shfl_xor(t, o);
+        if (lane == (d & 63))
+            pa[d] = t;
+    }
+    if (lane == 0) {
+        float *pm = a.part_ml + (size_t)r * a.ml_slot + part * 2;
+        pm[0] = lw > 0.0f ? mw : 0.0f;
+        pm[1] = lw;
+    }
+}
+
+// out[row][head][d] = sum_s acc_s[d] 2^(m_s - m) / sum_s l_s 2^(m_s - m), 0 when no split saw a key
+// (crates/hipml-kernels/kernels/attn_decode_kv.hip:491-532); grid (n_heads, rows), one thread per d.
+template <int HD>
+__global__ void __launch_bounds__(HD) decode_hd_reduce_kernel(const DecodeHdArgs a)
+{
+    const int head = blockIdx.x, r = blockIdx.y, d = threadIdx.x;
+    const float *pm = a.part_ml + (size_t)r * a.ml_slot + (size_t)head * a.splits * 2;
+    const float *pa = a.part_acc + (size_t)r * a.acc_slot + (size_t)head * a.splits * HD;
+    float m = -INFINITY;
+    for (int s = 0; s < a.splits; s++)
+        if (pm[2 * s + 1] > 0.0f)
+            m = fmaxf(m, pm[2 * s]);
+    float num = 0.0f, den = 0.0f;
+    for (int s = 0; s < a.splits; s++) {
+        const float ls = pm[2 * s + 1];
+        if (ls > 0.0f) {
+            const float w = __builtin_amdgcn_exp2f(pm[2 * s] - m);
+            num = fmaf(pa[(size_t)s * HD + d], w, num);
+            den = fmaf(ls, w, den);
+        }
+    }
+    float y = den > 0.0f ? num / den : 0.0f;
+    const size_t at = (size_t)r * a.q_slot + (size_t)head * HD + d;
+    if (a.gate)
+        y = gated(y, a.gate[at]);
+    a.out[at] = y;
+}
+
+static int launch_decode_hd(hipStream_t st, const DecodeLaunch &L)
+{
+    DecodeHdArgs a;
+    a.q = L.q;
+    a.k = L.k;
+    a.v = L.v;
+    a.part_acc = L.part_acc;
+    a.part_ml = L.part_ml;
+    a.out = L.out;
+    a.gate = L.gate;
+    a.pos = L.pos;
+    a.n_heads = L.n_heads;
+    a.n_kv = L.n_kv;
+    a.group = L.n_heads / L.n_kv;
+    a.stride = L.stride;
+    a.splits = L.splits;
+    a.scale_log2 = L.scale * kLog2e;
+    a.kv_slot_bytes = L.kv_slot_bytes;
+    a.acc_slot = L.acc_slot;
+    a.ml_slot = L.ml_slot;
+    a.q_slot = L.q_slot;
+    memset(a.slot_of_row, 0, sizeof(a.slot_of_row));
+    for (int s = 0; s < L.slots; s++)
+        for (int c = 0; c < L.cols[s]; c++)
+            a.slot_of_row[L.row0[s] + c] = (uint8_t)s;
+    const dim3 grid((unsigned)(L.n_kv * L.splits), (unsigned)L.total_rows, 1), block((unsigned)(64 * a.group), 1, 1);
+    const dim3 rgrid((unsigned)L.n_heads, (unsigned)L.total_rows, 1);
+    if (L.head_dim != 64)
+        return fail(HIPML_ATTN_E_SHAPE, "head_dim %d: 256 and 64 are built", L.head_dim);
+    if (L.q4)
+        hipLaunchKernelGGL((decode_hd_kernel<64, true>), grid, block, 0, st, a);
+    else
+        hipLaunchKernelGGL((decode_hd_kernel<64, false>), grid, block, 0, st, a);
+    int rc = launched("attn_decode_kv_hd");
+    if (rc)
+        return rc;
+    hipLaunchKernelGGL(decode_hd_reduce_kernel<64>, rgrid, dim3(64, 1, 1), 0, st, a);
+    return launched("attn_decode_kv_hd_reduce");
+}
+
 int launch_decode_q8(hipStream_t st, const DecodeLaunch &L)
 {
+    if (L.head_dim != kHeadDim)
+        return launch_decode_hd(st, L);
     DecodeArgs a;
     a.q = L.q;
     a.k = L.k;

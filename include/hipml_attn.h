@@ -227,7 +227,11 @@ int hipml_kv_encode_rows(hipml_stream_t stream, int dtype, const float *k_f32, c
                          void *k_cache, void *v_cache, int n_kv, int head_dim, int stride,
                          const int32_t *pos, size_t slot_bytes, int slots);
 
-/* ---- decode attention over a q8_0 / q4_0 cache ----------------------------------- */
+/* ---- decode attention over a q8_0 / q4_0 cache -----------------------------------
+ * head_dim is 256 (the MFMA kernels) or 64: the reference's launchers take any multiple of the block
+ * size and its parity table runs 64 (crates/hipml-core/src/parity_kv.rs:166-213); that width is
+ * served by plain fp32 kernels behind the same arguments, untuned (hipml_attn_decode_kv_noalloc: 256
+ * only).  Other widths are HIPML_ATTN_E_SHAPE. */
 
 /* One query row, live length step[1].  Split pass + merge.
  * part_acc: f32 [n_heads][splits][head_dim]; part_ml: f32 [n_heads][splits][2].
