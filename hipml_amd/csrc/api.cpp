@@ -5,6 +5,7 @@
 #include "common.h"
 
 #include <math.h>
+#include <mutex>
 #include <stdarg.h>
 #include <stdio.h>
 #include <string.h>
@@ -12,8 +13,21 @@
 namespace hipml {
 
 static thread_local char g_err[512] = "";
-static RopeTable g_rope = {nullptr, 0.0f, 0, 0, 0};
+// The registered RoPE table is a device pointer, so there is one registration per device: the entry
+// points work on a snapshot of the current device's, taken under the lock when they start
+// (clear_error), and the two calls that change it write under the same lock.
+static RopeTable g_rope_dev[64];
+static std::mutex g_rope_mu;
+static thread_local RopeTable g_rope = {nullptr, 0.0f, 0, 0, 0};
 static bool g_inited[64]; // per device: hipml_attn_init has run with that device current
+
+static int rope_device()
+{
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64)
+        device = 0;
+    return device;
+}
 
 int fail(int code, const char *fmt, ...)
 {
@@ -30,6 +44,9 @@ void clear_error()
 {
     g_err[0] = '\0';
     (void)hipGetLastError();
+    const int device = rope_device();
+    std::lock_guard<std::mutex> lock(g_rope_mu);
+    g_rope = g_rope_dev[device];
 }
 
 int launched(const char *what)
@@ -376,17 +393,22 @@ int hipml_rope_set_table(const float *dev_table, float theta_base, int n_rot, in
     if (dev_table != nullptr && (n_rot <= 0 || (n_rot & 1) || max_pos <= 0))
         return fail(HIPML_ATTN_E_RANGE, "n_rot %d must be even and positive, max_pos %d positive",
                     n_rot, max_pos);
-    g_rope.dev = dev_table;
-    g_rope.theta = theta_base;
-    g_rope.n_rot = n_rot;
-    g_rope.max_pos = dev_table ? max_pos : 0;
+    const int device = rope_device();
+    std::lock_guard<std::mutex> lock(g_rope_mu);
+    RopeTable &t = g_rope_dev[device];
+    t.dev = dev_table;
+    t.theta = theta_base;
+    t.n_rot = n_rot;
+    t.max_pos = dev_table ? max_pos : 0;
     return 0;
 }
 
 int hipml_rope_allow_device_angles(int allow)
 {
     clear_error();
-    g_rope.device_angles = allow ? 1 : 0;
+    const int device = rope_device();
+    std::lock_guard<std::mutex> lock(g_rope_mu);
+    g_rope_dev[device].device_angles = allow ? 1 : 0;
     return 0;
 }
 

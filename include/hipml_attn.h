@@ -95,8 +95,10 @@ int hipml_attn_chunk_slices(int pos0, int tokens, int n_kv);
 size_t hipml_rope_table_bytes(int n_rot, int max_pos);
 int hipml_rope_table_fill_host(float *host_table, float theta_base, int n_rot, int max_pos);
 /* Register a device copy of the table (caller owns the memory; the engine registers n_ctx rows).
- * The table and the switch below are one per process: set them up before launches start, from one
- * thread.  Without a table for (theta_base, n_rot) the RoPE entry points return
+ * The table and the switch below belong to the device that is current when they are set (the pointer is
+ * that device's memory), one registration per device; they may be set from any thread, and a call that
+ * is already running keeps the registration it started with.  Without a table for (theta_base, n_rot) on
+ * the current device the RoPE entry points return
  * HIPML_ATTN_E_STATE.  A position at or beyond max_pos is an error: HIPML_ATTN_E_RANGE where the
  * host knows the positions (the chunk entry points), and NaN in the rotated channels where they
  * live in device memory (the step buffer, the pos arrays). */
