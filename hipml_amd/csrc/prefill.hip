@@ -62,6 +62,7 @@ constexpr int kVtTileBytes = kHeadDim * kVtRow;          // 36,864
 constexpr int kBufBytesF = kKTileBytes + kVtTileBytes;   // 70,656
 constexpr int kPfLdsF = 2 * kBufBytesF;                  // 141,312: no Q steps parked, the staging registers are free
 constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kPfLazy = 8.0f; // growth of a maximum (log2 units) that moves the reference exponent of chunk_q8_kernel
 
 struct ChunkArgs {
     const float *q;
@@ -572,11 +573,22 @@ __global__ void __launch_bounds__(kPfThreads, 2) chunk_q8_kernel(const ChunkArgs
 #pragma unroll
         for (int i = 1; i < 16; i++)
             mt = fmaxf(mt, S[i]);
-        mt = xor32_max(mt);
-        const float m_new = fmaxf(m_run, mt * a.scale_log2);
-        const bool dead = m_new == -INFINITY;
-        const float corr = dead ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_new);
-        const float mneg = dead ? 0.0f : -m_new;
+        mt = xor32_max(mt) * a.scale_log2;
+        // m_run is the exponent the sums are held against, not the running maximum: it follows the maximum
+        // only when some token's maximum has grown by more than kPfLazy since it was set.  Deep in a long
+        // prefix a token of the 32 still finds a new maximum in every third tile, and each time the 128
+        // accumulator registers would be rescaled; until the exponent moves, probabilities may be as
+        // large as 2^kPfLazy, which f16 holds with the same relative precision.
+        if (__any(mt > m_run + kPfLazy)) {
+            const float m_new = fmaxf(m_run, mt);
+            const float corr = m_new == -INFINITY ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_new);
+            l_run *= corr;
+#pragma unroll
+            for (int dt = 0; dt < 8; dt++)
+                O[dt] *= corr;
+            m_run = m_new;
+        }
+        const float mneg = m_run == -INFINITY ? 0.0f : -m_run;
         float ls = 0.0f;
 #pragma unroll
         for (int i = 0; i < 16; i++) {
@@ -584,13 +596,7 @@ __global__ void __launch_bounds__(kPfThreads, 2) chunk_q8_kernel(const ChunkArgs
             ls += e;
             P[i >> 3][i & 7] = (_Float16)e;
         }
-        l_run = l_run * corr + ls;
-        if (__any(m_new > m_run)) {
-#pragma unroll
-            for (int dt = 0; dt < 8; dt++)
-                O[dt] *= corr;
-        }
-        m_run = m_new;
+        l_run += ls;
         // computed here, in the VALU slot, not where the MFMA slot first reads them
         asm volatile("" : "+v"(P[0]), "+v"(P[1]), "+v"(l_run), "+v"(m_run));
     };
