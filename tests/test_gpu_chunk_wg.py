@@ -71,20 +71,23 @@ def test_agrees_with_the_sliced_kernel_and_is_repeatable():
 
 def test_large_scores_move_the_reference_exponent():
     # Q scaled so that scores spread over hundreds of log2 units and the running maximum keeps jumping
-    # by more than the lag the kernel allows itself: the rescaling path.  At this scale the f16 rounding of
-    # Q alone moves every kernel 1.5e-2 from the f32 oracle, so the check is against the single-pass kernel,
-    # which has the same operands and rescales at every step.
+    # by more than the lag the kernels allow themselves: the rescaling path.  At this scale the f16 rounding
+    # of the Q and K operands moves every kernel 1.5e-2 from the f32 oracle (a score of a few hundred carries
+    # an error of a tenth), so the tight check is between the in-workgroup kernel and the single-pass one:
+    # the same operands, different moments at which the reference exponent moves (the slices start at
+    # different keys), so a mistake in the rescaling of either shows as an error of order one.
     tok, pos0 = 96, 40
     q, kb, vb, stride = chunk_inputs(0xB16_5C0E, tok, pos0, 0)
     q = (q * 12.0).astype(np.float32)
     mono = run_chunk(q, kb, vb, pos0, tok, stride, 1)
     got = run_chunk(q, kb, vb, pos0, tok, stride, 0)
-    ok, _, _ = report("large scores, in-workgroup slices vs single pass", mono, got, 1e-3, 1e-2)
+    ok, _, _ = report("large scores, in-workgroup slices vs single pass", mono, got, *GATE)
     assert ok
     assert np.isfinite(got).all()
     want = orc.attn_chunk_kv(q, kb, vb, N_HEADS, N_KV, HD, pos0, tok, stride, SCALE, n_threads=8)
-    ok, _, _ = report("large scores vs the oracle (f16 Q operands)", want, got, 3e-2, 1e-2)
-    assert ok
+    for name, x in (("in-workgroup slices", got), ("single pass", mono)):
+        ok, _, _ = report(f"large scores, {name} vs the oracle (f16 Q and K operands)", want, x, 3e-2, 1e-2)
+        assert ok
 
 
 def test_q4_cache():
