@@ -1117,15 +1117,20 @@ __global__ void __launch_bounds__(kPfThreads, 1) chunk_wg_kernel(const ChunkArgs
         __builtin_amdgcn_sched_group_barrier(0x008, kWgAheadPv, 0);
     };
 
-    // Two slots per step, each closed by a barrier, every wave in the same slot:
+    // Two slots per step, each closed by a barrier:
     //   V: dequantize K(s+1) into the K tile, request V(s), softmax of step s, dequantize V(s) into the
     //      V tile, request K(s+2)                                                             (VALU)
     //   M: PV of step s, scores of step s+1                                                   (MFMA)
     // K(s) is last read in M(s-1) and V(s-1) as well, so both tiles are free in V(s).  One K or V unit is
-    // in flight per lane: K travels through an M slot, V through the softmax.  (Running waves 4..7 half a
-    // step behind waves 0..3, one set in its VALU slot while the other issues MFMAs as chunk_q8_kernel
-    // does, needs four barriers per step here, because a slice's tiles are single-buffered: 32.7 us
-    // against 31.9 at 672 @ 0.)
+    // in flight per lane: K travels through an M slot, V through the softmax.
+    // Waves 4..7 (slices 2 and 3) run one slot behind waves 0..3 (slices 0 and 1): they pass one barrier
+    // more before their first scores and waves 0..3 one more after their last step, so the two waves of a
+    // SIMD are in opposite slots.  A slice's tiles are touched by its own two waves only, which are in the
+    // same set, so the two barriers per step still separate every write from the reads around it; the Q
+    // rows in the V areas of slices 0 and 1 have been read by every wave before waves 0..3 pass their
+    // first barrier.  (A wave's step is a chain, so the gain is small: 25.6 against 26.0 us at 672 @ 0.)
+    if (wave >= 4)
+        lds_barrier();
     scores(0, std::true_type());
     lds_barrier(); // K(0) may be replaced, and every wave has read its Q: the V tiles may be written
     for (int s = 0; s < nstep; s++) {
@@ -1142,6 +1147,8 @@ __global__ void __launch_bounds__(kPfThreads, 1) chunk_wg_kernel(const ChunkArgs
             scores(s + 1, std::false_type());
         lds_barrier();
     }
+    if (wave < 4)
+        lds_barrier(); // (waves 4..7 are in their last M slot)
 
     // ---- the four slices of a head meet -------------------------------------------------------------
     // Wave `sl` finishes columns 64 sl .. 64 sl + 63 (accumulators 2 sl and 2 sl + 1) of its head.  The
