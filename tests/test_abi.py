@@ -86,6 +86,9 @@ def test_argument_errors_come_before_any_launch(lib):
     # head geometry the kernels are not built for
     rc = lib.hipml_attn_decode_kv(null, one, 0, one, one, one, one, one, one, 24, 4, 128, 64, C.c_float(0.0625), 1, 0, 0)
     assert rc < 0 and b"head_dim" in lib.hipml_attn_last_error()
+    # head_dim 64 is a decode width only (plain fp32 kernels); the chunk entry points are 256 only
+    rc = lib.hipml_attn_chunk_q8_split(null, one, one, one, one, 8, 2, 64, 0, 10, 1, 64, null, null, 1)
+    assert rc < 0 and b"head_dim" in lib.hipml_attn_last_error()
     # a chunk that does not fit the cache
     rc = lib.hipml_attn_chunk_q8_split(null, one, one, one, one, 24, 4, 256, 60, 10, 1, 64, null, null, 1)
     assert rc < 0 and b"does not fit" in lib.hipml_attn_last_error()
