@@ -215,6 +215,7 @@ def bench_prefill(torch, attn, tokens, pos0, steps, warmup, layers, prefix_fill=
     attn_copy_ms = events(attention_copy) if with_copy else None
     flop = prefill_flop(pos0, tokens)
     tf = flop / (attn_ms * 1e-3) / 1e12
+    rows_bytes = 2 * tokens * H * HD * 4 + 2 * KV * (pos0 + tokens) * ROW
     wl = {(672, 0): "prefill672", (2048, 100_000): "chunk100k"}.get((tokens, pos0), "")
     # (the instantiation that reads the cache: <SPLIT, q4_0, over the f16 copy>)
     traffic = measured_traffic(wl, ["chunk_wg_kernel<false, true>"] if splits == 0 else
@@ -241,7 +242,11 @@ def bench_prefill(torch, attn, tokens, pos0, steps, warmup, layers, prefix_fill=
                      "frac": tf / MFMA_F16_PEAK_TF, "traffic": traffic,
                      "kernel": "chunk_wg_kernel" if splits == 0 else
                      "chunk_q8_kernel" + (" + chunk_combine_kernel" if splits >= 2 else ""),
-                     "flop_per_launch": flop, "launch_ms": attn_ms},
+                     "flop_per_launch": flop, "launch_ms": attn_ms,
+                     # the same launch against the other roof: the f32 rows it has to move (Q in, rows out; the
+                     # attention-only launch timed here takes no gate) and the cache rows once, over 8 TB/s
+                     "algorithmic_bytes": rows_bytes,
+                     "hbm_frac": rows_bytes / (attn_ms * 1e-3) / 1e9 / HBM_PEAK_GBS},
     }
 
 
