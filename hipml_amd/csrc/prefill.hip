@@ -27,6 +27,8 @@
 
 #include "common.h"
 
+#include <type_traits>
+
 namespace hipml {
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
@@ -807,6 +809,432 @@ __global__ void __launch_bounds__(kPfThreads, 2) chunk_q8_kernel(const ChunkArgs
     }
 }
 
+// ---- sliced chunk prefill over the f16 copy, 64 tokens per wave ----------------------------------------
+// The kernel above feeds every MFMA one 1-KiB operand from LDS, and a wave cannot ask for them faster than
+// the pipe consumes them.  Here a task is 64 tokens x 1 head: each K and V^T operand read from LDS feeds two
+// MFMAs (one per 32-token half), which halves the LDS operand traffic per MFMA.  That takes all 512 registers of a
+// SIMD for one wave (O: 2 x 8 x 16 = 256 accumulators, Q: 128, scores of this half and of the next: 64,
+// P: 16), so a workgroup is four waves, one per SIMD, and nothing hides a wave's softmax but its own MFMAs:
+// the softmax of one 32-key half is cut into 16 pieces that sit, in program order, between the score MFMAs
+// of the next half.  Every MFMA is written as inline assembly with its accumulator class spelled out (O in
+// accumulation registers, scores in vector registers): left to itself the compiler puts every MFMA result
+// of a 512-register kernel into accumulation registers, which O alone fills.
+// The compiler does not know what the statements are, so it inserts no wait states for them.  What keeps
+// their results safe: a score accumulator is read by vector code one PV product (32 MFMAs) after the MFMA
+// that finished it; O is read by vector code (rescale, epilogue) only behind explicit s_nop padding or two
+// further MFMAs; P and the operands are overwritten long after the MFMAs that read them have issued.
+// Tiles, slices, partial rows and the merge are those of chunk_q8_kernel<true, false, true>.
+constexpr int kT64Tasks = 4;                   // tasks (= waves) per workgroup
+constexpr int kT64Tile = 64;                   // query tokens per task
+constexpr int kT64Threads = 64 * kT64Tasks;
+constexpr int kT64Dma = 9;                     // 1-KiB requests per wave for a K tile (33) or a V^T tile (36)
+constexpr int kT64Lds = 2 * kBufBytesF;        // 141,312
+
+#define HIPML_MFMA_V0(acc, A, B) asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(acc) : "v"(A), "v"(B))
+#define HIPML_MFMA_V(acc, A, B) asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(A), "v"(B))
+// O^T lives in the 256 accumulation registers as state the compiler does not see: token half h, d tile dt in
+// a[(8h + dt) * 16 .. + 15].  The compiler has no use of its own for these registers as long as it spills
+// nothing (it would spill vector registers there first), which the build of this file is checked for.
+#define HIPML_MFMA_O(R, A, B) \
+    asm volatile("v_mfma_f32_32x32x16_f16 a[%2:%3], %0, %1, a[%2:%3]" : : "v"(A), "v"(B), "n"(R), "n"((R) + 15))
+
+template <int R, int N>
+__device__ __forceinline__ void acc_zero()
+{
+    // (the clobber of the last register is what sizes the kernel's accumulation file)
+    asm volatile("v_accvgpr_write_b32 a[%0], 0\n\tv_accvgpr_write_b32 a[%1], 0\n\tv_accvgpr_write_b32 a[%2], 0\n\t"
+                 "v_accvgpr_write_b32 a[%3], 0"
+                 :
+                 : "n"(R), "n"(R + 1), "n"(R + 2), "n"(R + 3)
+                 : "a255");
+    if constexpr (N > 4)
+        acc_zero<R + 4, N - 4>();
+}
+template <int R, int N>
+__device__ __forceinline__ void acc_scale(float c)
+{
+    float t0, t1, t2, t3;
+    asm volatile("v_accvgpr_read_b32 %0, a[%5]\n\tv_accvgpr_read_b32 %1, a[%6]\n\tv_accvgpr_read_b32 %2, a[%7]\n\t"
+                 "v_accvgpr_read_b32 %3, a[%8]\n\t"
+                 "v_mul_f32 %0, %0, %4\n\tv_mul_f32 %1, %1, %4\n\tv_mul_f32 %2, %2, %4\n\tv_mul_f32 %3, %3, %4\n\t"
+                 "v_accvgpr_write_b32 a[%5], %0\n\tv_accvgpr_write_b32 a[%6], %1\n\tv_accvgpr_write_b32 a[%7], %2\n\t"
+                 "v_accvgpr_write_b32 a[%8], %3"
+                 : "=&v"(t0), "=&v"(t1), "=&v"(t2), "=&v"(t3)
+                 : "v"(c), "n"(R), "n"(R + 1), "n"(R + 2), "n"(R + 3));
+    if constexpr (N > 4)
+        acc_scale<R + 4, N - 4>(c);
+}
+template <int R>
+__device__ __forceinline__ float4v acc_read4()
+{
+    float4v x;
+    asm volatile("v_accvgpr_read_b32 %0, a[%4]\n\tv_accvgpr_read_b32 %1, a[%5]\n\tv_accvgpr_read_b32 %2, a[%6]\n\t"
+                 "v_accvgpr_read_b32 %3, a[%7]"
+                 : "=v"(x[0]), "=v"(x[1]), "=v"(x[2]), "=v"(x[3])
+                 : "n"(R), "n"(R + 1), "n"(R + 2), "n"(R + 3));
+    return x;
+}
+
+__global__ void __launch_bounds__(kT64Threads, 1) __attribute__((amdgpu_waves_per_eu(1, 1)))
+chunk_f16_t64_kernel(const ChunkArgs a)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const int wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const int ln = lane & 31; // MFMA column: token within a 32-token half
+    const int lh = lane >> 5; // k half-group
+
+    // blockIdx.x -> (kv head, key slice, task block), as in chunk_q8_kernel (every block has a.splits slices)
+    int kvh, split, tb;
+    {
+        const int combos = a.n_kv * a.splits;
+        const int bid = blockIdx.x;
+        int combo;
+        if (combos % 8 == 0) {
+            const int per = combos / 8;
+            const int xcd = bid & 7, j = bid >> 3;
+            combo = xcd + 8 * (j % per);
+            tb = j / per;
+        } else if (8 % combos == 0) {
+            const int xcd = bid & 7, j = bid >> 3;
+            const int share = 8 / combos;
+            combo = xcd % combos;
+            tb = j * share + xcd / combos;
+        } else {
+            combo = bid % combos;
+            tb = bid / combos;
+        }
+        kvh = combo % a.n_kv;
+        split = combo / a.n_kv;
+        if (tb >= a.nblock)
+            return; // uniform over the workgroup
+    }
+    const int nsp = a.splits;
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave); // (scalar: what follows from it stays in scalar registers)
+    const int task = tb * kT64Tasks + wave_u;
+    const bool task_valid = task < a.ntask;
+    const int tt = (task_valid ? task : a.ntask - 1) / a.group;
+    const int hq = (task_valid ? task : a.ntask - 1) - tt * a.group;
+    const int head = kvh * a.group + hq;
+    const int t0 = tt * kT64Tile;
+
+    const int last_task = (tb * kT64Tasks + kT64Tasks - 1 < a.ntask ? tb * kT64Tasks + kT64Tasks - 1 : a.ntask - 1);
+    const int tt_last = last_task / a.group;
+    const int last_tok = ((tt_last + 1) * kT64Tile < a.tokens ? (tt_last + 1) * kT64Tile : a.tokens) - 1;
+    const int seq_block = a.pos0 + last_tok + 1;
+    const int tiles_block = (seq_block + kKTile - 1) / kKTile;
+    const int klo = (int)((long long)tiles_block * split / nsp) * kKTile;
+    int khi = (int)((long long)tiles_block * (split + 1) / nsp) * kKTile;
+    khi = khi < seq_block ? khi : seq_block;
+    const int ntile = khi > klo ? (khi - klo + kKTile - 1) / kKTile : 0;
+
+    // K tile t of the slice lives in K buffer t & 1, its V^T tile in V^T buffer t & 1; each arrives as
+    // nine 1-KiB requests per wave (the last ones repeat the tile's last KiB; a tile past the slice's last
+    // repeats that one), so that the waits below are constants.
+    const uint32_t lds_at = lds_address(lds);
+    // request j of nine for tile t (the K tile or the V^T tile)
+    auto dma_req = [&](int t, bool v_tile, int j) {
+        const int tc = t < ntile ? t : ntile - 1;
+        const size_t tile = (size_t)kvh * a.tile_stride + (klo / kKTile + tc);
+        const uint8_t *src = v_tile ? a.vt + tile * kVtTileBytes : a.k16 + tile * kKTileBytes;
+        const int last = (v_tile ? kVtTileBytes : kKTileBytes) / 1024 - 1;
+        const uint32_t dst = lds_at + (t & 1) * kBufBytesF + (v_tile ? kKTileBytes : 0);
+        int i = wave_u + kT64Tasks * j;
+        i = i < last ? i : last;
+        dma16(dst + i * 1024, src + i * 1024, lane * 16);
+    };
+    auto dma_tile = [&](int t, bool v_tile) {
+#pragma unroll
+        for (int j = 0; j < kT64Dma; j++)
+            dma_req(t, v_tile, j);
+    };
+    if (ntile > 0) {
+        dma_tile(0, false);
+        dma_tile(0, true);
+    }
+
+    // ---- Q^T operand: per 32-token half, 16 k-steps of 8 f16 (d = ks*16 + lh*8 + j), all in registers.
+    // Rows are fetched whole, converted and turned round in this wave's corner of the second tile buffer.
+    half8 Q[2][16];
+    {
+        uint8_t *qt = lds + kBufBytesF + wave * (32 * kKRow);
+        const float *qh = a.q + (size_t)head * kHeadDim + lane * 4;
+        const size_t tok_stride = (size_t)a.n_head * kHeadDim;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+#pragma unroll
+            for (int b = 0; b < 2; b++) {
+                float4v f[16];
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    const int tr = t0 + h * 32 + b * 16 + i;
+                    f[i] = __builtin_nontemporal_load(
+                        reinterpret_cast<const float4v *>(qh + (size_t)(tr < a.tokens ? tr : a.tokens - 1) * tok_stride));
+                }
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    half4 x;
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+                        x[j] = (_Float16)f[i][j];
+                    *reinterpret_cast<half4 *>(qt + (b * 16 + i) * kKRow + lane * 8) = x;
+                }
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // this wave's own writes
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int ks = 0; ks < 16; ks++)
+                Q[h][ks] = *reinterpret_cast<const half8 *>(qt + ln * kKRow + ks * 32 + lh * 16);
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // read before the next half overwrites the corner
+            __builtin_amdgcn_wave_barrier();
+        }
+    }
+    __syncthreads(); // every wave has its Q, tile 0 has landed (no load is outstanding): the second buffer is free
+    if (ntile > 0)
+        dma_tile(1, false);
+
+    acc_zero<0, 256>();
+    float m_run[2] = {-INFINITY, -INFINITY}, l_run[2] = {0.0f, 0.0f};
+    float mneg[2] = {0.0f, 0.0f}, ls[2] = {0.0f, 0.0f};
+    float16v S[2], N[2]; // scores of the half whose softmax runs now, and of the next one
+    half8 P[2][2];
+
+    // The softmax of a 32-key half is spread over the MFMAs around it.  Its maxima are taken from the finished
+    // scores N while the PV product of the half before runs (max_piece, masking included); the step that follows
+    // first moves the reference exponent where a maximum has outgrown it (lazily, as chunk_q8_kernel does: the
+    // only place O is rescaled, behind that step's first two MFMAs) and then takes two of a lane's 32
+    // exponentials after each pair of score MFMAs.
+    // A wave issues in order: behind two MFMAs in a row nothing goes out until the first has left the pipe (32
+    // cycles), and vector work that follows the pair for longer than the second one runs leaves the pipe idle.
+    // So every MFMA is followed by its own slot of at most ~28 cycles of other work: one exponential with its
+    // multiply-add and sum, or one LDS read, or one request, or a third of a maximum.
+    float mt[2] = {-INFINITY, -INFINITY}, mx = 0.0f;
+    auto max_part = [&](int t, int hk, int h, int part) { // scores N of half hk of tile t, token half h
+        if (part == 0) {
+            const int k0 = klo + t * kKTile + hk * 32;
+            const int tok0 = a.pos0 + t0 + h * 32;
+            if ((k0 + 31 > tok0) || (k0 + 32 > khi)) { // (uniform over the wave)
+                // (the empty statement keeps this a branch: turned into selects, the 80 instructions would run
+                // for every half, and only the halves on the diagonal and at the end of the slice need them)
+                asm volatile("" ::: "memory");
+                const int my_last = tok0 + ln;
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    const int kg = k0 + (i >> 2) * 8 + lh * 4 + (i & 3);
+                    N[h][i] = (kg <= my_last && kg < khi) ? N[h][i] : -INFINITY;
+                }
+            }
+            mx = fmaxf(fmaxf(N[h][0], N[h][1]), N[h][2]);
+            mx = fmaxf(fmaxf(mx, N[h][3]), N[h][4]);
+            mx = fmaxf(fmaxf(mx, N[h][5]), N[h][6]);
+            mx = fmaxf(mx, N[h][7]);
+        } else if (part == 1) {
+            mx = fmaxf(fmaxf(mx, N[h][8]), N[h][9]);
+            mx = fmaxf(fmaxf(mx, N[h][10]), N[h][11]);
+            mx = fmaxf(fmaxf(mx, N[h][12]), N[h][13]);
+            mx = fmaxf(fmaxf(mx, N[h][14]), N[h][15]);
+        } else {
+            mt[h] = xor32_max(mx) * a.scale_log2;
+        }
+    };
+    // softmax of S, slot p of 32: slot 1 (behind the second MFMA: O is at rest) moves the reference exponent
+    // where a maximum has outgrown it, slots 2..31 take the 32 exponentials of a lane
+    auto exp_slot = [&](int p) {
+        if (p == 1) {
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                if (__any(mt[h] > m_run[h] + kPfLazy)) {
+                    const float m_new = fmaxf(m_run[h], mt[h]);
+                    const float corr = m_new == -INFINITY ? 1.0f : __builtin_amdgcn_exp2f(m_run[h] - m_new);
+                    l_run[h] *= corr;
+                    if (h == 0)
+                        acc_scale<0, 128>(corr);
+                    else
+                        acc_scale<128, 128>(corr);
+                    m_run[h] = m_new;
+                }
+                mneg[h] = m_run[h] == -INFINITY ? 0.0f : -m_run[h];
+                ls[h] = 0.0f;
+            }
+        } else if (p >= 2) {
+            const int lo = (p - 2) * 32 / 30, hi = (p - 1) * 32 / 30;
+#pragma unroll
+            for (int v = lo; v < hi; v++) {
+                const int h = v >> 4, i = v & 15;
+                const float e = __builtin_amdgcn_exp2f(fmaf(S[h][i], a.scale_log2, mneg[h]));
+                ls[h] += e;
+                P[h][i >> 3][i & 7] = (_Float16)e;
+            }
+            if (p == 31) {
+                l_run[0] += ls[0];
+                l_run[1] += ls[1];
+            }
+        }
+    };
+    // Scores of half hk of tile t into N (MFMA), the exponentials of S in the slots (SOFT); each K operand
+    // feeds the MFMAs of both token halves and is read from LDS two steps ahead.
+    auto step = [&](auto mfma_tag, auto soft_tag, int t, int hk) {
+        constexpr bool MFMA = decltype(mfma_tag)::value, SOFT = decltype(soft_tag)::value;
+        const uint8_t *Kh = lds + (t & 1) * kBufBytesF + (hk * 32 + ln) * kKRow + lh * 16;
+        half8 A0, A1;
+        if constexpr (MFMA) {
+            A0 = *reinterpret_cast<const half8 *>(Kh);
+            A1 = *reinterpret_cast<const half8 *>(Kh + 32);
+        }
+#pragma unroll
+        for (int ks = 0; ks < 16; ks++) {
+            half8 A2 = A0;
+            if constexpr (MFMA) {
+                if (ks + 2 < 16)
+                    A2 = *reinterpret_cast<const half8 *>(Kh + (ks + 2) * 32);
+                if (ks == 0)
+                    HIPML_MFMA_V0(N[0], A0, Q[0][ks]);
+                else
+                    HIPML_MFMA_V(N[0], A0, Q[0][ks]);
+            }
+            if constexpr (SOFT)
+                exp_slot(2 * ks);
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (MFMA) {
+                if (ks == 0)
+                    HIPML_MFMA_V0(N[1], A0, Q[1][ks]);
+                else
+                    HIPML_MFMA_V(N[1], A0, Q[1][ks]);
+                A0 = A1;
+                A1 = A2;
+            }
+            if constexpr (SOFT)
+                exp_slot(2 * ks + 1);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    // O^T += V^T . P^T for half hk of tile t: each V^T operand feeds both token halves.  The slot behind the
+    // first MFMA of a pair reads the operand of two steps on; the slots behind the second ones carry this wave's
+    // nine requests for tile dt (its V^T tile if dv) and, MAXP, the maxima of the scores N of the half
+    // (nt, nhk) that follows.
+    auto pv = [&](auto max_tag, int t, int hk, int nt, int nhk, int dt, bool dv) {
+        constexpr bool MAXP = decltype(max_tag)::value;
+        const uint8_t *Vt = lds + (t & 1) * kBufBytesF + kKTileBytes + ln * kVtRow + (hk * 32 + lh * 8) * 2;
+        half8 A0 = *reinterpret_cast<const half8 *>(Vt);
+        half8 A1 = *reinterpret_cast<const half8 *>(Vt + 32 * kVtRow);
+#define HIPML_PV_STEP(s)                                                                                        \
+    {                                                                                                           \
+        half8 A2 = A0;                                                                                          \
+        HIPML_MFMA_O(((s) & 7) * 16, A0, P[0][(s) >> 3]);                                                       \
+        if ((s) + 2 < 16)                                                                                       \
+            A2 = *reinterpret_cast<const half8 *>(Vt + (((s) + 2) & 7) * 32 * kVtRow + (((s) + 2) >> 3) * 32); \
+        __builtin_amdgcn_sched_barrier(0);                                                                      \
+        HIPML_MFMA_O(128 + ((s) & 7) * 16, A0, P[1][(s) >> 3]);                                                 \
+        if constexpr ((s) < kT64Dma)                                                                            \
+            dma_req(dt, dv, (s));                                                                               \
+        else if constexpr (MAXP && (s) < kT64Dma + 6)                                                           \
+            max_part(nt, nhk, ((s) - kT64Dma) / 3, ((s) - kT64Dma) % 3);                                        \
+        __builtin_amdgcn_sched_barrier(0);                                                                      \
+        A0 = A1;                                                                                                \
+        A1 = A2;                                                                                                \
+    }
+        HIPML_PV_STEP(0) HIPML_PV_STEP(1) HIPML_PV_STEP(2) HIPML_PV_STEP(3) HIPML_PV_STEP(4) HIPML_PV_STEP(5)
+        HIPML_PV_STEP(6) HIPML_PV_STEP(7) HIPML_PV_STEP(8) HIPML_PV_STEP(9) HIPML_PV_STEP(10) HIPML_PV_STEP(11)
+        HIPML_PV_STEP(12) HIPML_PV_STEP(13) HIPML_PV_STEP(14) HIPML_PV_STEP(15)
+#undef HIPML_PV_STEP
+    };
+    const std::true_type yes;
+    const std::false_type no;
+
+    // Per tile t: [scores(t, 1) with the exponentials of (t, 0); PV(t, 0), requesting V^T(t + 1) into the buffer
+    // of V^T(t - 1)]; K(t + 1) has landed: barrier A; [scores(t + 1, 0) with the exponentials of (t, 1); PV(t, 1),
+    // requesting K(t + 2) into the buffer of K(t), which every wave finished with before barrier A]; V^T(t + 1)
+    // has landed: barrier B (after it every wave has finished with V^T(t)).  Requests outstanding at barrier A,
+    // oldest first: K(t + 1), V^T(t + 1); at barrier B: V^T(t + 1), K(t + 2): the wait is vmcnt(9) both times.
+    if (ntile > 0) {
+        step(yes, no, 0, 0);
+        asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); // these scores were finished just now
+#pragma unroll
+        for (int h = 0; h < 2; h++)
+#pragma unroll
+            for (int part = 0; part < 3; part++)
+                max_part(0, 0, h, part);
+        S[0] = N[0];
+        S[1] = N[1];
+    }
+    for (int t = 0; t < ntile; t++) {
+        step(yes, yes, t, 1);
+        pv(yes, t, 0, t, 1, t + 1, true);
+        S[0] = N[0];
+        S[1] = N[1];
+        asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
+        lds_barrier();
+        if (t + 1 < ntile) {
+            step(yes, yes, t + 1, 0);
+            pv(yes, t, 1, t + 1, 0, t + 2, false);
+        } else {
+            asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); // O may be rescaled right behind the MFMAs of PV(t, 0)
+            step(no, yes, t + 1, 0);
+            pv(no, t, 1, t + 1, 0, t + 2, false);
+        }
+        S[0] = N[0];
+        S[1] = N[1];
+        asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
+        lds_barrier();
+    }
+    // the tile buffers are about to be reused, and O is about to be read
+    asm volatile("s_waitcnt vmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+    lds_barrier();
+
+    // ---- epilogue: partial rows leave through this wave's corner of LDS, as in chunk_q8_kernel ----------
+    constexpr int kPitch = 512 + 16;
+    uint8_t *mine = lds + wave * (32 * kPitch);
+    const int l32 = lane & 31, rsel = lane >> 5;
+    auto half_rows = [&](auto h_tag, auto hf_tag) {
+        // 128 columns (d tiles 4 hf .. 4 hf + 3) of token half h into this wave's corner
+        constexpr int h = decltype(h_tag)::value, hf = decltype(hf_tag)::value;
+        constexpr int R = (h * 8 + hf * 4) * 16;
+#define HIPML_ROW_PIECE(dl, g)                                                                                   \
+    *reinterpret_cast<float4v *>(mine + ln * kPitch + ((dl) * 32 + (g) * 8 + lh * 4) * 4) = acc_read4<R + (dl) * 16 + (g) * 4>();
+        HIPML_ROW_PIECE(0, 0) HIPML_ROW_PIECE(0, 1) HIPML_ROW_PIECE(0, 2) HIPML_ROW_PIECE(0, 3)
+        HIPML_ROW_PIECE(1, 0) HIPML_ROW_PIECE(1, 1) HIPML_ROW_PIECE(1, 2) HIPML_ROW_PIECE(1, 3)
+        HIPML_ROW_PIECE(2, 0) HIPML_ROW_PIECE(2, 1) HIPML_ROW_PIECE(2, 2) HIPML_ROW_PIECE(2, 3)
+        HIPML_ROW_PIECE(3, 0) HIPML_ROW_PIECE(3, 1) HIPML_ROW_PIECE(3, 2) HIPML_ROW_PIECE(3, 3)
+#undef HIPML_ROW_PIECE
+    };
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        const float lsum = l_run[h] + __shfl_xor(l_run[h], 32);
+        const int tbase = t0 + h * 32;
+#pragma unroll
+        for (int hf = 0; hf < 2; hf++) {
+            if (h == 0 && hf == 0)
+                half_rows(I0(), I0());
+            else if (h == 0)
+                half_rows(I0(), I1());
+            else if (hf == 0)
+                half_rows(I1(), I0());
+            else
+                half_rows(I1(), I1());
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int r2 = 0; r2 < 16; r2++) {
+                const int r = r2 * 2 + rsel;
+                const float4v x = *reinterpret_cast<const float4v *>(mine + r * kPitch + l32 * 16);
+                if (task_valid && tbase + r < a.tokens) {
+                    const size_t prow = ((size_t)split * a.qslots + (tbase + r)) * a.n_head + head;
+                    *reinterpret_cast<float4v *>(a.part_acc + prow * kHeadDim + hf * 128 + l32 * 4) = x;
+                }
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            __builtin_amdgcn_wave_barrier();
+        }
+        if (task_valid && tbase + ln < a.tokens && lh == 0) {
+            const size_t row = ((size_t)split * a.qslots + (tbase + ln)) * a.n_head + head;
+            a.part_ml[row * 2] = m_run[h];
+            a.part_ml[row * 2 + 1] = lsum;
+        }
+    }
+}
+
 // ---- chunk prefill with the key split inside the workgroup -----------------------------------------
 // Near position 0 a chunk has few keys per token and little to do in total (672 tokens at depth 0:
 // 5.6 GFLOP, 1.5 MB of cache), but as many Q and output rows as at any depth.  The kernel above then
@@ -1517,6 +1945,9 @@ int prefill_init()
         e = hipFuncSetAttribute(reinterpret_cast<const void *>(&chunk_q8_kernel<true, false, true>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, kPfLdsF);
     if (e == hipSuccess)
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&chunk_f16_t64_kernel),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, kT64Lds);
+    if (e == hipSuccess)
         e = hipFuncSetAttribute(reinterpret_cast<const void *>(&kv_f16_tiles_kernel<false>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, kBufBytes);
     if (e == hipSuccess)
@@ -1624,7 +2055,17 @@ int launch_chunk_q8(hipStream_t st, const float *q, const uint8_t *kc, const uin
                            reinterpret_cast<const float4v *>(out), static_cast<half4 *>(out16), n4);
         return launched("attn_chunk_rows_f16");
     }
-    if (kv_f16)
+    if (kv_f16 && a.uniform) {
+        // 64 tokens per wave: its own task blocks (4 tasks of 64 tokens), every one with `splits` slices
+        ChunkArgs b = a;
+        b.ntask = (tokens + kT64Tile - 1) / kT64Tile * a.group;
+        b.nblock = (b.ntask + kT64Tasks - 1) / kT64Tasks;
+        const int combos = n_kv * a.splits;
+        unsigned g64 = (unsigned)(combos * b.nblock);
+        if (combos % 8 != 0 && 8 % combos == 0)
+            g64 = (unsigned)(8 * ((b.nblock + 8 / combos - 1) / (8 / combos)));
+        hipLaunchKernelGGL(chunk_f16_t64_kernel, dim3(g64, 1, 1), dim3(kT64Threads, 1, 1), kT64Lds, st, b);
+    } else if (kv_f16)
         hipLaunchKernelGGL((chunk_q8_kernel<true, false, true>), dim3(grid, 1, 1), block, kPfLdsF, st, a);
     else if (q4)
         hipLaunchKernelGGL((chunk_q8_kernel<true, true>), dim3(grid, 1, 1), block, kPfLds, st, a);
