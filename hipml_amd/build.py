@@ -31,6 +31,40 @@ def hipcc() -> str:
     raise RuntimeError("hipcc not found")
 
 
+# Kernels that keep state in the accumulation registers behind the compiler's back (every use of those
+# registers is inside their inline assembly): (source, substring of the mangled kernel name).
+HAND_PLACED_ACC = [("prefill.hip", "chunk_f16_t64_kernel")]
+
+
+def check_hand_placed_acc(cc: str, flags: list[str], src: str, kernel: str) -> None:
+    """Fail the build if the compiler itself touches an accumulation register in `kernel` (it parks
+    vector registers there under pressure, which would overwrite the kernel's hand-placed state)."""
+    import re
+    cmd = [cc] + COMMON + flags + ["-S", "--cuda-device-only", os.path.join(CSRC, src), "-o", "-"]
+    text = subprocess.run(cmd, check=True, capture_output=True, text=True).stdout.split("\n")
+    start = [i for i, l in enumerate(text) if re.match(r"^_Z\w*" + kernel + r"\w*:", l)]
+    if not start:
+        raise RuntimeError(f"{src}: kernel {kernel} not found in the generated assembly")
+    in_asm, n_inside = False, 0
+    for l in text[start[0]:]:
+        if l.startswith(".Lfunc_end"):
+            break
+        if "ASMSTART" in l:
+            in_asm = True
+        elif "ASMEND" in l:
+            in_asm = False
+        else:
+            code = l.split(";")[0]
+            acc = re.search(r"\ba\[?\d", code) or "accvgpr" in code
+            if acc and in_asm:
+                n_inside += 1
+            elif acc:
+                raise RuntimeError(f"{src}: the compiler uses accumulation registers of its own in {kernel}: "
+                                   f"'{code.strip()}'")
+    if n_inside == 0:
+        raise RuntimeError(f"{src}: no accumulation register found in {kernel}: the check looks at the wrong text")
+
+
 def build_library(verbose: bool = False, extra: list[str] | None = None) -> str:
     """Compile every translation unit and link the shared library; returns its path."""
     cc = hipcc()
@@ -42,6 +76,9 @@ def build_library(verbose: bool = False, extra: list[str] | None = None) -> str:
             print(" ".join(cmd), flush=True)
         subprocess.run(cmd, check=True)
         objs.append(obj)
+        for hsrc, kernel in HAND_PLACED_ACC:
+            if hsrc == src:
+                check_hand_placed_acc(cc, flags + (extra or []), src, kernel)
     cmd = [cc, "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", LIB] + objs
     if verbose:
         print(" ".join(cmd), flush=True)

@@ -830,13 +830,27 @@ constexpr int kT64Threads = 64 * kT64Tasks;
 constexpr int kT64Dma = 9;                     // 1-KiB requests per wave for a K tile (33) or a V^T tile (36)
 constexpr int kT64Lds = 2 * kBufBytesF;        // 141,312
 
-#define HIPML_MFMA_V0(acc, A, B) asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(acc) : "v"(A), "v"(B))
-#define HIPML_MFMA_V(acc, A, B) asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(A), "v"(B))
+// All 256 accumulation registers as a clobber list.  Every MFMA statement of the kernel below carries it, so
+// the compiler can keep nothing of its own in them from one MFMA to the next (under register pressure it
+// would otherwise park vector registers there, on top of O).
+#define HIPML_A10(t) "a" #t "0", "a" #t "1", "a" #t "2", "a" #t "3", "a" #t "4", "a" #t "5", "a" #t "6", "a" #t "7", "a" #t "8", "a" #t "9"
+#define HIPML_ACC_ALL                                                                                            \
+    HIPML_A10(), HIPML_A10(1), HIPML_A10(2), HIPML_A10(3), HIPML_A10(4), HIPML_A10(5), HIPML_A10(6), HIPML_A10(7),  \
+        HIPML_A10(8), HIPML_A10(9), HIPML_A10(10), HIPML_A10(11), HIPML_A10(12), HIPML_A10(13), HIPML_A10(14),      \
+        HIPML_A10(15), HIPML_A10(16), HIPML_A10(17), HIPML_A10(18), HIPML_A10(19), HIPML_A10(20), HIPML_A10(21),    \
+        HIPML_A10(22), HIPML_A10(23), HIPML_A10(24), "a250", "a251", "a252", "a253", "a254", "a255"
+#define HIPML_MFMA_V0(acc, A, B) \
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(acc) : "v"(A), "v"(B) : HIPML_ACC_ALL)
+#define HIPML_MFMA_V(acc, A, B) \
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(A), "v"(B) : HIPML_ACC_ALL)
 // O^T lives in the 256 accumulation registers as state the compiler does not see: token half h, d tile dt in
-// a[(8h + dt) * 16 .. + 15].  The compiler has no use of its own for these registers as long as it spills
-// nothing (it would spill vector registers there first), which the build of this file is checked for.
+// a[(8h + dt) * 16 .. + 15].  The build checks the generated code of this kernel for accumulation registers
+// outside these statements (hipml_amd/build.py).
 #define HIPML_MFMA_O(R, A, B) \
-    asm volatile("v_mfma_f32_32x32x16_f16 a[%2:%3], %0, %1, a[%2:%3]" : : "v"(A), "v"(B), "n"(R), "n"((R) + 15))
+    asm volatile("v_mfma_f32_32x32x16_f16 a[%2:%3], %0, %1, a[%2:%3]"                                            \
+                 :                                                                                               \
+                 : "v"(A), "v"(B), "n"(R), "n"((R) + 15)                                                         \
+                 : HIPML_ACC_ALL)
 
 template <int R, int N>
 __device__ __forceinline__ void acc_zero()
@@ -1061,9 +1075,12 @@ chunk_f16_t64_kernel(const ChunkArgs a)
 #pragma unroll
             for (int v = lo; v < hi; v++) {
                 const int h = v >> 4, i = v & 15;
-                const float e = __builtin_amdgcn_exp2f(fmaf(S[h][i], a.scale_log2, mneg[h]));
-                ls[h] += e;
-                P[h][i >> 3][i & 7] = (_Float16)e;
+                P[h][i >> 3][i & 7] = (_Float16)__builtin_amdgcn_exp2f(fmaf(S[h][i], a.scale_log2, mneg[h]));
+                if (i & 1) {
+                    // the sum takes the probabilities as the PV product sees them (f16), two per instruction
+                    const half2v pr = {P[h][i >> 3][(i & 7) - 1], P[h][i >> 3][i & 7]};
+                    ls[h] = __builtin_amdgcn_fdot2(pr, half2v{(_Float16)1.0f, (_Float16)1.0f}, ls[h], false);
+                }
             }
             if (p == 31) {
                 l_run[0] += ls[0];
