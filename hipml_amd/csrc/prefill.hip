@@ -1051,8 +1051,25 @@ chunk_f16_t64_kernel(const ChunkArgs a)
             mt[h] = xor32_max(mx) * a.scale_log2;
         }
     };
-    // softmax of S, slot p of 32: slot 1 (behind the second MFMA: O is at rest) moves the reference exponent
-    // where a maximum has outgrown it, slots 2..31 take the 32 exponentials of a lane
+    // Softmax of S.  A lane's 32 exponentials are taken in the order the PV product needs them: first the 16
+    // of its first k-step (keys 0..15 of the half: P[h][0]), then the 16 of the second.  Exponential v of that
+    // order, with its multiply-add, conversion and (every second time) the sum of a pair:
+    auto exp_value = [&](int v) {
+        const int h = (v >> 3) & 1, i = (v >> 4) * 8 + (v & 7);
+        P[h][i >> 3][i & 7] = (_Float16)__builtin_amdgcn_exp2f(fmaf(S[h][i], a.scale_log2, mneg[h]));
+        if (i & 1) {
+            // the sum takes the probabilities as the PV product sees them (f16), two per instruction
+            const half2v pr = {P[h][i >> 3][(i & 7) - 1], P[h][i >> 3][i & 7]};
+            ls[h] = __builtin_amdgcn_fdot2(pr, half2v{(_Float16)1.0f, (_Float16)1.0f}, ls[h], false);
+        }
+    };
+    // Behind one MFMA a wave gets four or five vector instructions through before the next MFMA is held up
+    // (an exponential counts double), so the 32 exponentials are spread: the score step carries the first
+    // kExpStep (slots 2..31), the PV product that follows takes the last kExpPv in its first slots; it does
+    // not read them before its second half (pv below).  Slot 1 of the step (behind the second MFMA: O is at
+    // rest) moves the reference exponent where a maximum has outgrown it, the only place O is rescaled.
+    // (Measured at 2,048 @ 100,000: 24 | 8 4.05 ms, 22 | 10 4.07, 20 | 12 4.09, 18 | 14 4.07; 32 | 0 4.13.)
+    constexpr int kExpStep = 24, kExpPv = 32 - kExpStep; // (kExpPv even, at most 14)
     auto exp_slot = [&](int p) {
         if (p == 1) {
 #pragma unroll
@@ -1071,21 +1088,10 @@ chunk_f16_t64_kernel(const ChunkArgs a)
                 ls[h] = 0.0f;
             }
         } else if (p >= 2) {
-            const int lo = (p - 2) * 32 / 30, hi = (p - 1) * 32 / 30;
+            const int lo = (p - 2) * kExpStep / 30, hi = (p - 1) * kExpStep / 30;
 #pragma unroll
-            for (int v = lo; v < hi; v++) {
-                const int h = v >> 4, i = v & 15;
-                P[h][i >> 3][i & 7] = (_Float16)__builtin_amdgcn_exp2f(fmaf(S[h][i], a.scale_log2, mneg[h]));
-                if (i & 1) {
-                    // the sum takes the probabilities as the PV product sees them (f16), two per instruction
-                    const half2v pr = {P[h][i >> 3][(i & 7) - 1], P[h][i >> 3][i & 7]};
-                    ls[h] = __builtin_amdgcn_fdot2(pr, half2v{(_Float16)1.0f, (_Float16)1.0f}, ls[h], false);
-                }
-            }
-            if (p == 31) {
-                l_run[0] += ls[0];
-                l_run[1] += ls[1];
-            }
+            for (int v = lo; v < hi; v++)
+                exp_value(v);
         }
     };
     // Scores of half hk of tile t into N (MFMA), the exponentials of S in the slots (SOFT); each K operand
@@ -1126,8 +1132,9 @@ chunk_f16_t64_kernel(const ChunkArgs a)
         }
     };
     // O^T += V^T . P^T for half hk of tile t: each V^T operand feeds both token halves.  The slot behind the
-    // first MFMA of a pair reads the operand of two steps on; the slots behind the second ones carry this wave's
-    // nine requests for tile dt (its V^T tile if dv) and, MAXP, the maxima of the scores N of the half
+    // first MFMA of a pair reads the operand of two steps on; the first kExpPv slots take the exponentials that
+    // the second eight steps read, the second slots after them carry this wave's nine requests for tile dt (its
+    // V^T tile if dv), and the first slots of the last six steps, MAXP, the maxima of the scores N of the half
     // (nt, nhk) that follows.
     auto pv = [&](auto max_tag, int t, int hk, int nt, int nhk, int dt, bool dv) {
         constexpr bool MAXP = decltype(max_tag)::value;
@@ -1140,12 +1147,20 @@ chunk_f16_t64_kernel(const ChunkArgs a)
         HIPML_MFMA_O(((s) & 7) * 16, A0, P[0][(s) >> 3]);                                                       \
         if ((s) + 2 < 16)                                                                                       \
             A2 = *reinterpret_cast<const half8 *>(Vt + (((s) + 2) & 7) * 32 * kVtRow + (((s) + 2) >> 3) * 32); \
+        if constexpr (2 * (s) < kExpPv)                                                                         \
+            exp_value(kExpStep + 2 * (s));                                                                      \
+        if constexpr (MAXP && (s) >= 10)                                                                        \
+            max_part(nt, nhk, ((s) - 10) / 3, ((s) - 10) % 3);                                                  \
         __builtin_amdgcn_sched_barrier(0);                                                                      \
         HIPML_MFMA_O(128 + ((s) & 7) * 16, A0, P[1][(s) >> 3]);                                                 \
-        if constexpr ((s) < kT64Dma)                                                                            \
-            dma_req(dt, dv, (s));                                                                               \
-        else if constexpr (MAXP && (s) < kT64Dma + 6)                                                           \
-            max_part(nt, nhk, ((s) - kT64Dma) / 3, ((s) - kT64Dma) % 3);                                        \
+        if constexpr (2 * (s) + 1 < kExpPv)                                                                     \
+            exp_value(kExpStep + 2 * (s) + 1);                                                                  \
+        else if constexpr ((s) - kExpPv / 2 < kT64Dma)                                                          \
+            dma_req(dt, dv, (s) - kExpPv / 2);                                                                  \
+        if constexpr (2 * (s) + 2 == kExpPv) {                                                                  \
+            l_run[0] += ls[0];                                                                                  \
+            l_run[1] += ls[1];                                                                                  \
+        }                                                                                                       \
         __builtin_amdgcn_sched_barrier(0);                                                                      \
         A0 = A1;                                                                                                \
         A1 = A2;                                                                                                \

@@ -1,0 +1,136 @@
+"""The sliced chunk kernel over the f16 copy with 64 tokens per wave (chunk_f16_t64_kernel).
+
+hipml_attn_chunk_kv_f16 runs it whenever the keys are cut into slices and every task block gets all of them
+(uniform(...) below restates the launcher's rule), which is the case deep in a prefix.  Its accumulators live in
+registers the compiler does not manage and its softmax is spread over the slots between its MFMAs, so the cases
+here go for what that could break: token counts that are no multiple of 64, task counts that are no multiple of
+4, every mapping of workgroups to (KV head, slice), the diagonal inside the last slice, slices that end inside
+a tile, and scores large enough to move the reference exponent again and again.  Expected values: the CPU
+oracle over the same cache bytes, at the chunk gate of the reference (2e-3 / 1e-2)."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+from oracle import binding as orc  # noqa: E402
+from hipml_amd import attn  # noqa: E402
+from gpu_util import HD, SCALE, ROW, dev, host, report  # noqa: E402
+from test_gpu_prefill import GATE  # noqa: E402
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _init():
+    attn.init(0)
+
+
+def uniform(tok, pos0, splits, group):
+    # the launcher's rule: task blocks of 8 tasks of 32 tokens; a block whose last token sees fewer key tiles
+    # than splits * slice_tiles gets fewer slices, and then the kernel of 32 tokens per wave runs
+    ntask = (tok + 31) // 32 * group
+    tiles_last = (pos0 + tok + 63) // 64
+    slice_tiles = (tiles_last + splits - 1) // splits
+    for tb in range((ntask + 7) // 8):
+        last_task = min(tb * 8 + 7, ntask - 1)
+        last_tok = min((last_task // group + 1) * 32, tok) - 1
+        tiles = (pos0 + last_tok + 1 + 63) // 64
+        if min(splits, max(1, (tiles + slice_tiles - 1) // slice_tiles)) != splits:
+            return False
+    return True
+
+
+def inputs(seed, tok, pos0, pad, n_heads, n_kv, q_scale=1.0, k_ramp=0.0):
+    stride = pos0 + tok + pad
+    r = orc.Rng(seed)
+    q = (r.normal_array((tok, n_heads, HD)) * q_scale).astype(np.float32)
+    k = r.normal_array((n_kv, stride, HD))
+    if k_ramp:
+        # keys grow with their position, so the maxima keep growing along the prefix
+        k = (k * (1.0 + k_ramp * np.arange(stride, dtype=np.float32) / stride)[None, :, None]).astype(np.float32)
+    v = r.normal_array((n_kv, stride, HD))
+    kb = orc.quantize(0, k).reshape(n_kv, stride, ROW)
+    vb = orc.quantize(0, v).reshape(n_kv, stride, ROW)
+    return q, kb, vb, stride
+
+
+def run(q, kb, vb, pos0, tok, stride, splits, n_heads, n_kv, gate=None):
+    copy = attn.kv_f16_alloc(stride, n_kv)
+    copy.fill_(0xFF)  # f16 NaN wherever the conversion does not write
+    attn.kv_f16_rows(0, dev(kb), dev(vb), copy, n_kv, HD, stride, 0, pos0 + tok)
+    out = torch.full((tok, n_heads, HD), float("nan"), dtype=torch.float32, device="cuda")
+    acc, ml = attn.chunk_scratch(tok, n_heads, splits)
+    acc.fill_(float("nan"))
+    ml.fill_(float("nan"))
+    attn.chunk_attention_kv_f16(dev(q), copy, None if gate is None else dev(gate), out, None, n_heads, n_kv, HD,
+                                pos0, tok, stride, acc, ml, splits)
+    torch.cuda.synchronize()
+    return host(out)
+
+
+@pytest.mark.parametrize("tok,pos0,pad,splits,n_heads,n_kv", [
+    (100, 5000, 7, 4, 24, 4),    # 36 tokens in the last tile of 64; 12 tasks = 3 workgroups per (KV head, slice)
+    (65, 3000, 0, 4, 24, 4),     # one token in the second tile
+    (200, 3000, 1, 3, 24, 4),    # 12 (KV head, slice) pairs: neither a multiple nor a divisor of the 8 XCDs
+    (70, 2000, 0, 2, 24, 4),     # 8 pairs
+    (128, 4096, 0, 2, 6, 1),     # 2 pairs, one KV head: each pair spread over 4 XCDs
+    (64, 2500, 5, 5, 8, 2),      # 4 heads per KV head: 4 tasks = exactly one workgroup; 10 pairs
+    (96, 2200, 0, 4, 12, 4),     # 3 heads per KV head: 6 tasks, the second workgroup half empty
+    (300, 9000, 3, 8, 24, 4),    # 8 slices
+])
+def test_against_the_oracle(tok, pos0, pad, splits, n_heads, n_kv):
+    assert uniform(tok, pos0, splits, n_heads // n_kv)
+    q, kb, vb, stride = inputs(0x7640_0000 + tok * 131 + pos0, tok, pos0, pad, n_heads, n_kv)
+    want = orc.attn_chunk_kv(q, kb, vb, n_heads, n_kv, HD, pos0, tok, stride, SCALE, n_threads=8)
+    got = run(q, kb, vb, pos0, tok, stride, splits, n_heads, n_kv)
+    ok, _, _ = report(f"64-token chunk kernel {tok}@{pos0} pad {pad} splits {splits} heads {n_heads}/{n_kv}", want,
+                      got, *GATE)
+    assert ok
+    assert np.isfinite(got).all()
+
+
+def test_gate_is_applied_by_the_merge():
+    tok, pos0, splits, n_heads, n_kv = 130, 4000, 4, 24, 4
+    assert uniform(tok, pos0, splits, n_heads // n_kv)
+    q, kb, vb, stride = inputs(0x7641_6A7E, tok, pos0, 2, n_heads, n_kv)
+    gate = orc.Rng(0x6A7E_7641).normal_array((tok, n_heads, HD))
+    plain = run(q, kb, vb, pos0, tok, stride, splits, n_heads, n_kv)
+    gated = run(q, kb, vb, pos0, tok, stride, splits, n_heads, n_kv, gate=gate)
+    two = torch.empty((tok, n_heads, HD), dtype=torch.float32, device="cuda")
+    attn.q_gate(dev(plain), dev(gate), two)
+    torch.cuda.synchronize()
+    assert np.array_equal(gated.view(np.uint32), host(two).view(np.uint32))
+
+
+def test_growing_maxima_move_the_reference_exponent():
+    # Q scaled and the keys growing along the prefix: the maxima outgrow the reference exponent many times
+    # in every slice, so O is rescaled in its registers again and again.  At this scale the f16 rounding of
+    # the operands moves any kernel ~1.5e-2 from the f32 oracle; the tight check is against the kernel of 32
+    # tokens per wave over the same copy (unsplit: one pass over the keys), which rounds the same operands
+    # and rescales at other moments.
+    tok, pos0, splits, n_heads, n_kv = 128, 3000, 4, 24, 4
+    assert uniform(tok, pos0, splits, n_heads // n_kv)
+    q, kb, vb, stride = inputs(0x7642_B16, tok, pos0, 0, n_heads, n_kv, q_scale=8.0, k_ramp=2.0)
+    got = run(q, kb, vb, pos0, tok, stride, splits, n_heads, n_kv)
+    assert np.isfinite(got).all()
+    copy = attn.kv_f16_alloc(stride, n_kv)
+    attn.kv_f16_rows(0, dev(kb), dev(vb), copy, n_kv, HD, stride, 0, pos0 + tok)
+    mono = torch.full((tok, n_heads, HD), float("nan"), dtype=torch.float32, device="cuda")
+    attn.chunk_attention_kv_f16(dev(q), copy, None, mono, None, n_heads, n_kv, HD, pos0, tok, stride, None, None, 1)
+    torch.cuda.synchronize()
+    ok, _, _ = report("growing maxima, 64-token kernel vs single pass over the same copy", host(mono), got, *GATE)
+    assert ok
+    want = orc.attn_chunk_kv(q, kb, vb, n_heads, n_kv, HD, pos0, tok, stride, SCALE, n_threads=8)
+    ok, _, _ = report("growing maxima, 64-token kernel vs the oracle (f16 Q and K operands)", want, got, 3e-2, 1e-2)
+    assert ok
+
+
+def test_same_bits_on_every_call():
+    # the accumulators are state in registers no compiler tracks: a second call, after another launch has
+    # used the chip, must give the same bits
+    tok, pos0, splits, n_heads, n_kv = 192, 6000, 4, 24, 4
+    q, kb, vb, stride = inputs(0x7643_0001, tok, pos0, 0, n_heads, n_kv)
+    first = run(q, kb, vb, pos0, tok, stride, splits, n_heads, n_kv)
+    other = inputs(0x7643_0002, 64, 1000, 0, n_heads, n_kv)
+    run(other[0], other[1], other[2], 1000, 64, other[3], 4, n_heads, n_kv)
+    again = run(q, kb, vb, pos0, tok, stride, splits, n_heads, n_kv)
+    assert np.array_equal(first.view(np.uint32), again.view(np.uint32))
