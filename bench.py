@@ -49,7 +49,7 @@ def decode_bytes(seq_total: int) -> float:
     return float(2 * KV * seq_total * ROW)
 
 
-def measured_traffic(workload: str, kernels):
+def measured_traffic(workload: str, kernels, largest=()):
     """HBM bytes per launch (read + written) of the named kernels, from the committed
     counter runs in profiles/hbm_traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled
     by a plain copy of known size); None when that file has no entry."""
@@ -62,6 +62,10 @@ def measured_traffic(workload: str, kernels):
     for name, v in t.items():
         if any(k in name for k in kernels):
             total += v["read_bytes"] + v["written_bytes"]
+            seen = True
+        elif any(k in name for k in largest):
+            # a kernel that the run also launches at other sizes: its largest dispatch is the one meant
+            total += v.get("max_read_bytes", v["read_bytes"]) + v.get("max_written_bytes", v["written_bytes"])
             seen = True
     return total if seen else None
 
@@ -218,13 +222,21 @@ def bench_prefill(torch, attn, tokens, pos0, steps, warmup, layers, prefix_fill=
     rows_bytes = 2 * tokens * H * HD * 4 + 2 * KV * (pos0 + tokens) * ROW
     wl = {(672, 0): "prefill672", (2048, 100_000): "chunk100k"}.get((tokens, pos0), "")
     # (the instantiation that reads the cache: <SPLIT, q4_0, over the f16 copy>)
-    traffic = measured_traffic(wl, ["chunk_wg_kernel<false, true>"] if splits == 0 else
-                               ["chunk_q8_kernel<true, false, false>", "chunk_q8_kernel<false, false, false>",
-                                "chunk_combine_kernel"])
+    # A scratch sized for more slices than the sliced kernel would use: the call writes the live rows of the
+    # cache as f16 tiles into the tail of the scratch and runs `slices` slices of the 64-token kernel over them.
+    tiles_path = splits > slices >= 2
+    if splits == 0:
+        traffic = measured_traffic(wl, ["chunk_wg_kernel<false, true>"])
+    elif tiles_path:
+        traffic = measured_traffic(wl, ["chunk_f16_t64_kernel", "chunk_combine_kernel"], ["kv_f16_tiles_kernel<false>"])
+    else:
+        traffic = measured_traffic(wl, ["chunk_q8_kernel<true, false, false>", "chunk_q8_kernel<false, false, false>",
+                                        "chunk_combine_kernel"])
     return {
         "workload": f"prefill {tokens}@{pos0}: rope + q8_0 append + causal GQA attention + gate, "
                     f"1 layer, {H}q/{KV}kv heads, head_dim {HD}",
         "tokens": tokens, "pos0": pos0, "splits": splits, "slices_over_f16_copy": slices, "layers_rotated": layers,
+        "scratch_slices": max(splits, slices), "slices_run": slices if tiles_path else splits,
         "ms_per_step": wall_ms,
         "tok_per_s": tokens / (wall_ms * 1e-3),
         "ms_per_step_separate_launches": unfused_ms,
@@ -241,6 +253,7 @@ def bench_prefill(torch, attn, tokens, pos0, steps, warmup, layers, prefix_fill=
         "roofline": {"bound": "mfma", "achieved": tf, "peak": MFMA_F16_PEAK_TF, "unit": "TFLOP/s",
                      "frac": tf / MFMA_F16_PEAK_TF, "traffic": traffic,
                      "kernel": "chunk_wg_kernel" if splits == 0 else
+                     "kv_f16_tiles_kernel + chunk_f16_t64_kernel + chunk_combine_kernel" if tiles_path else
                      "chunk_q8_kernel" + (" + chunk_combine_kernel" if splits >= 2 else ""),
                      "flop_per_launch": flop, "launch_ms": attn_ms,
                      # the same launch against the other roof: the f32 rows it has to move (Q in, rows out; the

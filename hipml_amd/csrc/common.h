@@ -115,6 +115,9 @@ int launch_chunk_q8(hipStream_t st, const float *q, const uint8_t *kc, const uin
 // The f16 copy of a cache that launch_chunk_q8 can read instead of the cache (kv_f16): its size for
 // `stride` rows per KV head, and the conversion of the 64-key tiles that hold rows [start, start + rows).
 size_t kv_f16_bytes(int stride, int n_kv);
+// The scratch slice count that lets a sliced chunk over the cache of `slices` slices run over f16 tiles made in
+// the tail of its scratch (launch_chunk_q8 takes that path by itself when the count it is given allows it).
+int chunk_tiles_splits(int pos0, int tokens, int n_head, int n_kv, int slices);
 int launch_kv_f16_rows(hipStream_t st, const uint8_t *kc, const uint8_t *vc, void *copy, int n_kv, int stride,
                        int start, int rows, int q4);
 

@@ -1938,23 +1938,29 @@ size_t kv_f16_bytes(int stride, int n_kv)
     return (size_t)n_kv * tiles * kBufBytesF;
 }
 
+// Tiles tile0 .. of a copy with tile_stride tiles per KV head, from cache rows below seq_end.
+static int launch_kv_f16_tiles(hipStream_t st, const uint8_t *kc, const uint8_t *vc, void *copy, int n_kv, int stride,
+                               int tile_stride, int start, int seq_end, int q4)
+{
+    uint8_t *k16 = static_cast<uint8_t *>(copy);
+    uint8_t *vt = k16 + (size_t)n_kv * tile_stride * kKTileBytes;
+    const int tile0 = start / kKTile, tile1 = (seq_end + kKTile - 1) / kKTile;
+    const dim3 grid((unsigned)(tile1 - tile0), (unsigned)n_kv, 1);
+    if (q4)
+        hipLaunchKernelGGL(kv_f16_tiles_kernel<true>, grid, dim3(256, 1, 1), kBufBytes, st, kc, vc, k16, vt, stride,
+                           tile0, seq_end, tile_stride);
+    else
+        hipLaunchKernelGGL(kv_f16_tiles_kernel<false>, grid, dim3(256, 1, 1), kBufBytes, st, kc, vc, k16, vt, stride,
+                           tile0, seq_end, tile_stride);
+    return launched("kv_f16_rows");
+}
+
 int launch_kv_f16_rows(hipStream_t st, const uint8_t *kc, const uint8_t *vc, void *copy, int n_kv, int stride,
                        int start, int rows, int q4)
 {
     if (rows < 1)
         return 0;
-    const int tile_stride = (stride + kKTile - 1) / kKTile;
-    uint8_t *k16 = static_cast<uint8_t *>(copy);
-    uint8_t *vt = k16 + (size_t)n_kv * tile_stride * kKTileBytes;
-    const int tile0 = start / kKTile, tile1 = (start + rows + kKTile - 1) / kKTile;
-    const dim3 grid((unsigned)(tile1 - tile0), (unsigned)n_kv, 1);
-    if (q4)
-        hipLaunchKernelGGL(kv_f16_tiles_kernel<true>, grid, dim3(256, 1, 1), kBufBytes, st, kc, vc, k16, vt, stride,
-                           tile0, start + rows, tile_stride);
-    else
-        hipLaunchKernelGGL(kv_f16_tiles_kernel<false>, grid, dim3(256, 1, 1), kBufBytes, st, kc, vc, k16, vt, stride,
-                           tile0, start + rows, tile_stride);
-    return launched("kv_f16_rows");
+    return launch_kv_f16_tiles(st, kc, vc, copy, n_kv, stride, (stride + kKTile - 1) / kKTile, start, start + rows, q4);
 }
 
 int prefill_init()
@@ -2003,11 +2009,55 @@ int prefill_init()
     return 0;
 }
 
+// Deep in a prefix a sliced chunk over the cache runs faster as two steps: the live rows of the cache are first
+// written out as f16 tiles (what hipml_kv_f16_rows makes) into the tail of the caller's partial-row scratch, and
+// the attention then runs over those with the 64-token kernel and fewer slices.  That needs a scratch sized for
+// more slices than the attention uses: `splits` (the count the scratch was sized for) must cover `*use` slices
+// of partial rows plus the tiles, which start at byte *tiles_at of part_acc.  hipml_attn_chunk_splits returns
+// such a count where the detour pays (the pass over the cache costs 1.5 us per 1,000 rows, the kernel of 32
+// tokens per wave with its own dequantization 15 % of the attention); with any smaller count the chunk runs as
+// before.
+bool chunk_tiles_plan(int pos0, int tokens, int n_head, int n_kv, int splits, int *use, size_t *tiles_at)
+{
+    if (tokens < 768 || pos0 < 8 * tokens || splits < 3)
+        return false;
+    const int s = hipml_attn_chunk_slices(pos0, tokens, n_kv);
+    if (s < 2)
+        return false;
+    const size_t per_slice = (size_t)((tokens + 31) / 32 * 32) * n_head * kHeadDim * sizeof(float);
+    const size_t tiles = (size_t)n_kv * ((pos0 + tokens + kKTile - 1) / kKTile) * kBufBytesF;
+    if ((size_t)splits * per_slice < (size_t)s * per_slice + tiles)
+        return false;
+    *use = s;
+    *tiles_at = (size_t)s * per_slice;
+    return true;
+}
+
+int chunk_tiles_splits(int pos0, int tokens, int n_head, int n_kv, int slices)
+{
+    const size_t per_slice = (size_t)((tokens + 31) / 32 * 32) * n_head * kHeadDim * sizeof(float);
+    const size_t tiles = (size_t)n_kv * ((pos0 + tokens + kKTile - 1) / kKTile) * kBufBytesF;
+    return slices + (int)((tiles + per_slice - 1) / per_slice);
+}
+
 int launch_chunk_q8(hipStream_t st, const float *q, const uint8_t *kc, const uint8_t *vc,
                     float *out, int n_head, int n_kv, int pos0, int tokens, int stride,
                     float *part_acc, float *part_ml, int splits, const float *gate, int q4, void *out16,
                     const void *kv_f16, const float *rope_tab)
 {
+    {
+        int use;
+        size_t tiles_at;
+        if (kv_f16 == nullptr && rope_tab == nullptr &&
+            chunk_tiles_plan(pos0, tokens, n_head, n_kv, splits, &use, &tiles_at)) {
+            const int live_tiles = (pos0 + tokens + kKTile - 1) / kKTile;
+            uint8_t *tiles = reinterpret_cast<uint8_t *>(part_acc) + tiles_at;
+            if (int rc = launch_kv_f16_tiles(st, kc, vc, tiles, n_kv, stride, live_tiles, 0, pos0 + tokens, q4))
+                return rc;
+            return launch_chunk_q8(st, q, kc, vc, out, n_head, n_kv, pos0, tokens, live_tiles * kKTile, part_acc,
+                                   part_ml, use, gate, 0, out16, tiles, nullptr);
+        }
+    }
     // rope_tab != nullptr (splits == 0 only): q holds unrotated rows, the kernel rotates them as it loads them
     ChunkArgs a;
     // kv_f16 != nullptr: K and V are read from the f16 copy of the cache (kc, vc unused)

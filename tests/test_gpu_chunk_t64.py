@@ -134,3 +134,51 @@ def test_same_bits_on_every_call():
     run(other[0], other[1], other[2], 1000, 64, other[3], 4, n_heads, n_kv)
     again = run(q, kb, vb, pos0, tok, stride, splits, n_heads, n_kv)
     assert np.array_equal(first.view(np.uint32), again.view(np.uint32))
+
+
+@pytest.mark.parametrize("dtype", [0, 1])
+def test_cache_entry_point_makes_its_tiles_in_the_scratch(dtype):
+    # hipml_attn_chunk_splits sizes the scratch of a long chunk deep in a prefix for the slices plus the live
+    # rows as f16 tiles; hipml_attn_chunk_q8_split then converts the rows there and runs the 64-token kernel
+    # over them: the same bits as hipml_attn_chunk_kv_f16 over a copy made beforehand with the same number of
+    # slices, and the oracle's values on sampled rows.  One slice fewer in the scratch and the call runs the
+    # kernel that dequantizes for itself: same values within the gate.
+    n_heads, n_kv, tok, pos0 = 24, 4, 800, 6500
+    stride = pos0 + tok + 12
+    splits, slices = attn.chunk_splits(pos0, tok, n_kv), attn.chunk_slices(pos0, tok, n_kv)
+    assert slices >= 2 and splits > slices and uniform(tok, pos0, slices, n_heads // n_kv)
+    r = orc.Rng(0x7644_0000 + dtype)
+    q = r.normal_array((tok, n_heads, HD))
+    kb = orc.quantize(dtype, r.normal_array((n_kv, stride, HD))).reshape(n_kv, stride, -1)
+    vb = orc.quantize(dtype, r.normal_array((n_kv, stride, HD))).reshape(n_kv, stride, -1)
+    gate = r.normal_array((tok, n_heads, HD))
+
+    def over_cache(n):
+        acc, ml = attn.chunk_scratch(tok, n_heads, n)
+        acc.fill_(float("nan"))
+        ml.fill_(float("nan"))
+        out = torch.full((tok, n_heads, HD), float("nan"), dtype=torch.float32, device="cuda")
+        attn.chunk_attention_q8_split_gate(dev(q), dev(kb), dev(vb), dev(gate), out, n_heads, n_kv, HD, pos0, tok,
+                                           1 + dtype, stride, acc, ml, n)
+        torch.cuda.synchronize()
+        return host(out)
+
+    got = over_cache(splits)
+    copy = attn.kv_f16_alloc(stride, n_kv)
+    attn.kv_f16_rows(dtype, dev(kb), dev(vb), copy, n_kv, HD, stride, 0, pos0 + tok)
+    acc, ml = attn.chunk_scratch(tok, n_heads, slices)
+    ref = torch.full((tok, n_heads, HD), float("nan"), dtype=torch.float32, device="cuda")
+    attn.chunk_attention_kv_f16(dev(q), copy, dev(gate), ref, None, n_heads, n_kv, HD, pos0, tok, stride, acc, ml,
+                                slices)
+    torch.cuda.synchronize()
+    assert np.array_equal(got.view(np.uint32), host(ref).view(np.uint32))
+    rows = np.array([0, 1, 63, 64, 399, 767, 799], dtype=np.int32)
+    want = orc.attn_chunk_kv(q, kb, vb, n_heads, n_kv, HD, pos0, tok, stride, SCALE, dtype=dtype, rows=rows,
+                             n_threads=8)
+    want = want / (1.0 + np.exp(-gate[rows].astype(np.float64)))
+    tol = GATE if dtype == 0 else (3e-2, 3e-2)
+    ok, _, _ = report(f"chunk {tok}@{pos0} over tiles made in the scratch, cache dtype {dtype}", want, got[rows], *tol)
+    assert ok
+    less = over_cache(splits - 1)
+    ok, _, _ = report("the same chunk with a scratch too small for the tiles", got, less, *GATE)
+    assert ok
