@@ -62,6 +62,7 @@ constexpr int kVtRow = 144;
 constexpr int kKTileBytes = kKTile * kKRow;              // 33,792
 constexpr int kVtTileBytes = kHeadDim * kVtRow;          // 36,864
 constexpr int kBufBytesF = kKTileBytes + kVtTileBytes;   // 70,656
+constexpr int kTilesLds = kKTile * kVRow;                // 34,816: one staged tile of kv_f16_tiles_kernel (the V pitch is the larger)
 constexpr int kPfLdsF = 2 * kBufBytesF;                  // 141,312: no Q steps parked, the staging registers are free
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kPfLazy = 8.0f; // growth of a maximum (log2 units) that moves the reference exponent of chunk_q8_kernel
@@ -1868,7 +1869,7 @@ __global__ void __launch_bounds__(256) rows_f16_kernel(const float4v *__restrict
 }
 
 // The f16 copy of 64-key tiles of a cache: what a chunk workgroup would stage for itself, made once.
-// grid (tiles, n_kv); tile = tile0 + blockIdx.x; rows at or past seq_end repeat row seq_end - 1 (the
+// grid (tiles, n_kv, 2); tile = tile0 + blockIdx.x; rows at or past seq_end repeat row seq_end - 1 (the
 // attention kernels mask them; a later call that brings the rows overwrites the tile).
 // The K rows leave as they lie in LDS; the V tile leaves through the transposing reads of the PV
 // product, so row d of the copy holds, for every 16 keys, the eight values of k-group 0 and the eight
@@ -1879,12 +1880,15 @@ __global__ void __launch_bounds__(256) kv_f16_tiles_kernel(const uint8_t *__rest
                                                            uint8_t *__restrict__ vt, int stride, int tile0,
                                                            int seq_end, int tile_stride)
 {
+    // grid (tiles, n_kv, 2): blockIdx.z = 0 makes the K tile, 1 the V^T tile (35 KB of LDS either way: four
+    // workgroups per CU, which this pass needs more than anything else: it is all latency)
     typedef typename HalfOf<Q4>::type Half;
     constexpr int kRowBytes = Q4 ? hipml::kRowBytesQ4 : hipml::kRowBytes;
     constexpr int kUnitBytes = Q4 ? 36 : 68;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int tile = tile0 + blockIdx.x;
     const int kvh = blockIdx.y;
+    const bool v_tile = blockIdx.z != 0;
     const int su = threadIdx.x;
     const int lane = su & 63, wave = su >> 6;
     // thread -> (row, unit) as in the chunk kernel's staging: conflict-free 128-bit LDS writes
@@ -1893,28 +1897,23 @@ __global__ void __launch_bounds__(256) kv_f16_tiles_kernel(const uint8_t *__rest
     int key = tile * kKTile + srow;
     key = key < seq_end ? key : seq_end - 1;
     const size_t src = ((size_t)kvh * stride + key) * kRowBytes + spr * kUnitBytes;
-    Half hk0, hk1, hv0, hv1;
-    load_half0(hk0, kc + src);
-    load_half1(hk1, kc + src);
-    load_half0(hv0, vc + src);
-    load_half1(hv1, vc + src);
-    uint8_t *kd = lds + srow * kKRow + spr * 128;
-    uint8_t *vd = lds + kVOff + srow * kVRow + spr * 128;
-    stage_block0(hk0, kd);
-    stage_block1(hk1, kd);
-    stage_block0(hv0, vd);
-    stage_block1(hv1, vd);
+    const uint8_t *from_cache = (v_tile ? vc : kc) + src;
+    Half h0, h1;
+    load_half0(h0, from_cache);
+    load_half1(h1, from_cache);
+    uint8_t *sd = lds + srow * (v_tile ? kVRow : kKRow) + spr * 128;
+    stage_block0(h0, sd);
+    stage_block1(h1, sd);
     __syncthreads();
     const size_t at = (size_t)kvh * tile_stride + tile;
-    {
+    if (!v_tile) {
         const uint4v *from = reinterpret_cast<const uint4v *>(lds);
         uint4v *to = reinterpret_cast<uint4v *>(k16 + at * kKTileBytes);
         for (int i = su; i < kKTileBytes / 16; i += 256)
             to[i] = from[i];
-    }
-    {
+    } else {
         const int ln = lane & 31, lh = lane >> 5, gl = lane & 15;
-        const int vtr_off = kVOff + (gl >> 2) * kVRow + (((lane >> 4) & 1) * 16 + (gl & 3) * 4) * 2;
+        const int vtr_off = (gl >> 2) * kVRow + (((lane >> 4) & 1) * 16 + (gl & 3) * 4) * 2;
         uint8_t *to = vt + at * kVtTileBytes;
 #pragma unroll
         for (int o8 = 0; o8 < 8; o8++) {
@@ -1945,12 +1944,12 @@ static int launch_kv_f16_tiles(hipStream_t st, const uint8_t *kc, const uint8_t 
     uint8_t *k16 = static_cast<uint8_t *>(copy);
     uint8_t *vt = k16 + (size_t)n_kv * tile_stride * kKTileBytes;
     const int tile0 = start / kKTile, tile1 = (seq_end + kKTile - 1) / kKTile;
-    const dim3 grid((unsigned)(tile1 - tile0), (unsigned)n_kv, 1);
+    const dim3 grid((unsigned)(tile1 - tile0), (unsigned)n_kv, 2);
     if (q4)
-        hipLaunchKernelGGL(kv_f16_tiles_kernel<true>, grid, dim3(256, 1, 1), kBufBytes, st, kc, vc, k16, vt, stride,
+        hipLaunchKernelGGL(kv_f16_tiles_kernel<true>, grid, dim3(256, 1, 1), kTilesLds, st, kc, vc, k16, vt, stride,
                            tile0, seq_end, tile_stride);
     else
-        hipLaunchKernelGGL(kv_f16_tiles_kernel<false>, grid, dim3(256, 1, 1), kBufBytes, st, kc, vc, k16, vt, stride,
+        hipLaunchKernelGGL(kv_f16_tiles_kernel<false>, grid, dim3(256, 1, 1), kTilesLds, st, kc, vc, k16, vt, stride,
                            tile0, seq_end, tile_stride);
     return launched("kv_f16_rows");
 }
@@ -1987,10 +1986,10 @@ int prefill_init()
                                 hipFuncAttributeMaxDynamicSharedMemorySize, kT64Lds);
     if (e == hipSuccess)
         e = hipFuncSetAttribute(reinterpret_cast<const void *>(&kv_f16_tiles_kernel<false>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, kBufBytes);
+                                hipFuncAttributeMaxDynamicSharedMemorySize, kTilesLds);
     if (e == hipSuccess)
         e = hipFuncSetAttribute(reinterpret_cast<const void *>(&kv_f16_tiles_kernel<true>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, kBufBytes);
+                                hipFuncAttributeMaxDynamicSharedMemorySize, kTilesLds);
     if (e == hipSuccess)
         e = hipFuncSetAttribute(reinterpret_cast<const void *>(&chunk_wg_kernel<false, false>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, kWgLds);
