@@ -24,6 +24,10 @@
 // The same kernel also runs over an f16 copy of the cache (template parameter F16): then nothing is
 // dequantized or staged by the waves, whole tiles come in through global_load_lds, and the V tile is
 // stored transposed so that the PV operands are plain 128-bit reads.  kv_f16_tiles_kernel makes that copy.
+//
+// Deep in a prefix the sliced chunk over such tiles is served by chunk_f16_t64_kernel instead: 64 tokens per
+// wave, one wave per SIMD, O in the accumulation registers (see there); the cache entry points reach it for
+// long chunks by making the tiles in their scratch first (chunk_tiles_plan).
 
 #include "common.h"
 

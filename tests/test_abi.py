@@ -48,8 +48,16 @@ def test_split_policies(lib):
     assert attn.batch_splits(100, 4, 16) == 1
     # prefill: no key slices once the task blocks fill the chip; slices keep n_kv*splits on the XCDs
     assert attn.chunk_splits(0, 8192, 4) == 1
-    s = attn.chunk_splits(100_000, 2048, 4)
+    s = attn.chunk_slices(100_000, 2048, 4)
     assert s > 1 and (4 * s) % 8 == 0
+    # long chunks deep in a prefix: the scratch is sized for the slices that run plus the live rows as f16
+    # tiles (70,656 bytes per KV head and 64 rows) in whole slices of partial rows (2,048 x 24 x 256 f32)
+    tiles = 4 * ((100_000 + 2048 + 63) // 64) * 70_656
+    per_slice = 2048 * 24 * 256 * 4
+    assert attn.chunk_splits(100_000, 2048, 4) == s + (tiles + per_slice - 1) // per_slice == 13
+    assert attn.chunk_splits(100_000, 767, 4) == attn.chunk_slices(100_000, 767, 4)   # too short to pay
+    assert attn.chunk_splits(8 * 1024 - 1, 1024, 4) == attn.chunk_slices(8 * 1024 - 1, 1024, 4)  # not deep enough
+    assert attn.chunk_splits(8 * 1024, 1024, 4) > attn.chunk_slices(8 * 1024, 1024, 4) >= 2
     assert attn.chunk_slices(0, 1, 4) >= 1
     # near position 0 the keys are cut inside the workgroups (0); deep chunks and long ones are not
     assert attn.chunk_splits(0, 672, 4) == 0 and attn.chunk_splits(0, 1, 4) == 0
