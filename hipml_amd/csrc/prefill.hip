@@ -951,16 +951,34 @@ chunk_f16_t64_kernel(const ChunkArgs a)
     // nine 1-KiB requests per wave (the last ones repeat the tile's last KiB; a tile past the slice's last
     // repeats that one), so that the waits below are constants.
     const uint32_t lds_at = lds_address(lds);
-    // request j of nine for tile t (the K tile or the V^T tile)
+    // Request j of nine for tile t (the K tile or the V^T tile): KiB i = wave + 4 j of the tile.  The per-lane
+    // offsets and the KiB offsets are made once (a request in the loop is then three instructions: LDS
+    // address into m0, the wait state m0 asks for, the load), and the K tile's last request repeats KiB 32
+    // for the waves whose ninth would lie behind the tile.
+    uint32_t voff[kT64Dma];
+    int soff[kT64Dma];
+#pragma unroll
+    for (int j = 0; j < kT64Dma; j++) {
+        soff[j] = (wave_u + kT64Tasks * j) * 1024;
+        voff[j] = lane * 16 + soff[j];
+    }
+    const int soff_k8 = (wave_u + kT64Tasks * 8 < kKTileBytes / 1024 ? wave_u + kT64Tasks * 8 : kKTileBytes / 1024 - 1) * 1024;
+    const uint32_t voff_k8 = lane * 16 + soff_k8;
     auto dma_req = [&](int t, bool v_tile, int j) {
         const int tc = t < ntile ? t : ntile - 1;
         const size_t tile = (size_t)kvh * a.tile_stride + (klo / kKTile + tc);
         const uint8_t *src = v_tile ? a.vt + tile * kVtTileBytes : a.k16 + tile * kKTileBytes;
-        const int last = (v_tile ? kVtTileBytes : kKTileBytes) / 1024 - 1;
         const uint32_t dst = lds_at + (t & 1) * kBufBytesF + (v_tile ? kKTileBytes : 0);
-        int i = wave_u + kT64Tasks * j;
-        i = i < last ? i : last;
-        dma16(dst + i * 1024, src + i * 1024, lane * 16);
+        const bool last_k = !v_tile && j == kT64Dma - 1;
+        const uint32_t at = __builtin_amdgcn_readfirstlane(dst);
+        const int so = __builtin_amdgcn_readfirstlane(last_k ? soff_k8 : soff[j]);
+        const uint64_t p = (uint64_t)(uintptr_t)src;
+        const uint64_t pu = (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)p) |
+                            ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(p >> 32)) << 32);
+        asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3"
+                     :
+                     : "s"(at), "s"(so), "v"(last_k ? voff_k8 : voff[j]), "s"(pu)
+                     : "memory", "scc");
     };
     auto dma_tile = [&](int t, bool v_tile) {
 #pragma unroll
