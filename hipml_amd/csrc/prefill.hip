@@ -2158,15 +2158,17 @@ int launch_chunk_q8(hipStream_t st, const float *q, const uint8_t *kc, const uin
                            reinterpret_cast<const float4v *>(out), static_cast<half4 *>(out16), n4);
         return launched("attn_chunk_rows_f16");
     }
-    if (kv_f16 && a.uniform) {
-        // 64 tokens per wave: its own task blocks (4 tasks of 64 tokens), every one with `splits` slices
-        ChunkArgs b = a;
-        b.ntask = (tokens + kT64Tile - 1) / kT64Tile * a.group;
-        b.nblock = (b.ntask + kT64Tasks - 1) / kT64Tasks;
-        const int combos = n_kv * a.splits;
-        unsigned g64 = (unsigned)(combos * b.nblock);
-        if (combos % 8 != 0 && 8 % combos == 0)
-            g64 = (unsigned)(8 * ((b.nblock + 8 / combos - 1) / (8 / combos)));
+    // 64 tokens per wave: its own task blocks (4 tasks of 64 tokens), every one with `splits` slices.  Both
+    // kernels run one workgroup per CU, so the hardware starts them in rounds of 256; where the other cut of
+    // the tokens needs a round more (672 tokens are 10.5 tiles of 64: 17 blocks per KV head and slice against
+    // 16), the kernel of 32 tokens per wave keeps the chunk.
+    ChunkArgs b = a;
+    b.ntask = (tokens + kT64Tile - 1) / kT64Tile * a.group;
+    b.nblock = (b.ntask + kT64Tasks - 1) / kT64Tasks;
+    unsigned g64 = (unsigned)(n_kv * a.splits * b.nblock);
+    if ((n_kv * a.splits) % 8 != 0 && 8 % (n_kv * a.splits) == 0)
+        g64 = (unsigned)(8 * ((b.nblock + 8 / (n_kv * a.splits) - 1) / (8 / (n_kv * a.splits))));
+    if (kv_f16 && a.uniform && (g64 + 255) / 256 <= (grid + 255) / 256) {
         hipLaunchKernelGGL(chunk_f16_t64_kernel, dim3(g64, 1, 1), dim3(kT64Threads, 1, 1), kT64Lds, st, b);
     } else if (kv_f16)
         hipLaunchKernelGGL((chunk_q8_kernel<true, false, true>), dim3(grid, 1, 1), block, kPfLdsF, st, a);

@@ -1,7 +1,8 @@
 """The sliced chunk kernel over the f16 copy with 64 tokens per wave (chunk_f16_t64_kernel).
 
-hipml_attn_chunk_kv_f16 runs it whenever the keys are cut into slices and every task block gets all of them
-(uniform(...) below restates the launcher's rule), which is the case deep in a prefix.  Its accumulators live in
+hipml_attn_chunk_kv_f16 runs it whenever the keys are cut into slices, every task block gets all of them and
+its cut of the tokens needs no extra round of workgroups (uniform(...) and no_extra_round(...) below restate the
+launcher's rules), which is the case deep in a prefix.  Its accumulators live in
 registers the compiler does not manage and its softmax is spread over the slots between its MFMAs, so the cases
 here go for what that could break: token counts that are no multiple of 64, task counts that are no multiple of
 4, every mapping of workgroups to (KV head, slice), the diagonal inside the last slice, slices that end inside
@@ -37,6 +38,20 @@ def uniform(tok, pos0, splits, group):
         if min(splits, max(1, (tiles + slice_tiles - 1) // slice_tiles)) != splits:
             return False
     return True
+
+
+def no_extra_round(tok, splits, n_heads, n_kv):
+    # the launcher's second rule: the cut into tasks of 64 tokens must not need a round of 256 workgroups more
+    # than the cut into tasks of 32 (672 tokens: 17 blocks per KV head and slice against 16)
+    group, pairs = n_heads // n_kv, n_kv * splits
+
+    def grid(blocks):
+        if pairs % 8 != 0 and 8 % pairs == 0:
+            return 8 * ((blocks + 8 // pairs - 1) // (8 // pairs))
+        return pairs * blocks
+    g32 = grid(((tok + 31) // 32 * group + 7) // 8)
+    g64 = grid(((tok + 63) // 64 * group + 3) // 4)
+    return (g64 + 255) // 256 <= (g32 + 255) // 256
 
 
 def inputs(seed, tok, pos0, pad, n_heads, n_kv, q_scale=1.0, k_ramp=0.0):
@@ -78,7 +93,7 @@ def run(q, kb, vb, pos0, tok, stride, splits, n_heads, n_kv, gate=None):
     (300, 9000, 3, 8, 24, 4),    # 8 slices
 ])
 def test_against_the_oracle(tok, pos0, pad, splits, n_heads, n_kv):
-    assert uniform(tok, pos0, splits, n_heads // n_kv)
+    assert uniform(tok, pos0, splits, n_heads // n_kv) and no_extra_round(tok, splits, n_heads, n_kv)
     q, kb, vb, stride = inputs(0x7640_0000 + tok * 131 + pos0, tok, pos0, pad, n_heads, n_kv)
     want = orc.attn_chunk_kv(q, kb, vb, n_heads, n_kv, HD, pos0, tok, stride, SCALE, n_threads=8)
     got = run(q, kb, vb, pos0, tok, stride, splits, n_heads, n_kv)
@@ -147,6 +162,7 @@ def test_cache_entry_point_makes_its_tiles_in_the_scratch(dtype):
     stride = pos0 + tok + 12
     splits, slices = attn.chunk_splits(pos0, tok, n_kv), attn.chunk_slices(pos0, tok, n_kv)
     assert slices >= 2 and splits > slices and uniform(tok, pos0, slices, n_heads // n_kv)
+    assert no_extra_round(tok, slices, n_heads, n_kv) and not no_extra_round(672, 4, 24, 4)
     r = orc.Rng(0x7644_0000 + dtype)
     q = r.normal_array((tok, n_heads, HD))
     kb = orc.quantize(dtype, r.normal_array((n_kv, stride, HD))).reshape(n_kv, stride, -1)
