@@ -2035,12 +2035,13 @@ int prefill_init()
 // the attention then runs over those with the 64-token kernel and fewer slices.  That needs a scratch sized for
 // more slices than the attention uses: `splits` (the count the scratch was sized for) must cover `*use` slices
 // of partial rows plus the tiles, which start at byte *tiles_at of part_acc.  hipml_attn_chunk_splits returns
-// such a count where the detour pays (the pass over the cache costs 1.5 us per 1,000 rows, the kernel of 32
-// tokens per wave with its own dequantization 15 % of the attention); with any smaller count the chunk runs as
-// before.
+// such a count where the detour pays (the pass over the cache costs 1.3 us per 1,000 rows, the kernel of 32
+// tokens per wave with its own dequantization 15 % of the attention; measured gain, 2,048 tokens at depth
+// 2,048 / 8,192 / 16,384 / 100,000: 13 / 10 / 11 / 13 %, 1,024 tokens at 2,048 / 8,192: 3 / 4 %, 768 tokens at
+// 3,072 / 6,144: 0.5 / 3 %); with any smaller count the chunk runs as before.
 bool chunk_tiles_plan(int pos0, int tokens, int n_head, int n_kv, int splits, int *use, size_t *tiles_at)
 {
-    if (tokens < 768 || pos0 < 8 * tokens || splits < 3)
+    if (tokens < 768 || pos0 < tokens || splits < 3)
         return false;
     const int s = hipml_attn_chunk_slices(pos0, tokens, n_kv);
     if (s < 2)

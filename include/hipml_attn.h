@@ -79,7 +79,7 @@ int hipml_attn_batch_splits(int stride, int n_kv, int slots);
  * crates/hipml-model/src/gpu/attn_tile.rs:138-151.  0 (chunks near position 0: pos0 + tokens <=
  * 1,792 and pos0 <= 2 * tokens) selects the kernel that cuts the keys inside its workgroups and
  * needs no scratch; 1 the single-pass kernel; n >= 2 that kernel over n key slices with scratch
- * and a merge launch.  For long chunks deep in a prefix (tokens >= 768, pos0 >= 8 * tokens) n is larger
+ * and a merge launch.  For long chunks behind a prefix at least as long (tokens >= 768, pos0 >= tokens) n is larger
  * than the number of slices that run (hipml_attn_chunk_slices): the chunk entry points then write the
  * live rows of the cache as f16 tiles (70,656 bytes per KV head and 64 rows) into the tail of part_acc
  * and run the attention over those, which is faster than dequantizing inside the attention (2,048 tokens
@@ -340,7 +340,7 @@ int hipml_attn_decode_kv_noalloc(hipml_stream_t stream, const int32_t *step, int
  * workgroup per 32 tokens x 2 heads; made for chunks near position 0, correct at any depth);
  * both ignore the scratch.  Otherwise part_acc is f32
  * [splits][ceil32(tokens)][n_head][head_dim] and part_ml [..][2]; how that memory is used is the
- * library's business (with a count from hipml_attn_chunk_splits for a long chunk deep in a prefix,
+ * library's business (with a count from hipml_attn_chunk_splits for a long chunk behind a prefix,
  * fewer slices run and the rest of part_acc holds the cache rows as f16 tiles for the length of the
  * call), and nothing beyond those sizes is touched.
  * Replaces AttnLayer::chunk_attention_q8_split -> attn_chunk_wmma_f16 /
