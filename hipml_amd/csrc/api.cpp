@@ -358,7 +358,7 @@ int hipml_attn_chunk_splits(int pos0, int tokens, int n_kv)
     // Long chunks behind a prefix at least as long: a scratch sized for this many slices also holds the live rows as f16 tiles,
     // and the call then runs `slices` slices of the 64-token kernel over those (2,048 @ 100,000: 13 for 4
     // slices, 4.1 against 4.7 ms).  Heads per KV head are taken as 6, as in hipml_attn_chunk_slices.
-    if (slices >= 2 && tokens >= 768 && pos0 >= tokens) {
+    if (slices >= 2 && chunk_tiles_pay(pos0, tokens)) {
         const int with_tiles = chunk_tiles_splits(pos0, tokens, 6 * n_kv, n_kv, slices);
         if (with_tiles <= 64)
             return with_tiles;

@@ -118,6 +118,7 @@ size_t kv_f16_bytes(int stride, int n_kv);
 // The scratch slice count that lets a sliced chunk over the cache of `slices` slices run over f16 tiles made in
 // the tail of its scratch (launch_chunk_q8 takes that path by itself when the count it is given allows it).
 int chunk_tiles_splits(int pos0, int tokens, int n_head, int n_kv, int slices);
+bool chunk_tiles_pay(int pos0, int tokens); // the shapes for which hipml_attn_chunk_splits asks for that count
 int launch_kv_f16_rows(hipStream_t st, const uint8_t *kc, const uint8_t *vc, void *copy, int n_kv, int stride,
                        int start, int rows, int q4);
 

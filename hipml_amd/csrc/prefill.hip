@@ -930,17 +930,41 @@ chunk_f16_t64_kernel(const ChunkArgs a)
     }
     const int nsp = a.splits;
     const int wave_u = __builtin_amdgcn_readfirstlane(wave); // (scalar: what follows from it stays in scalar registers)
+    // Tasks of one KV head, in order: the whole 64-token tiles, one task per head (its halves are the tile's
+    // two 32-token halves); then the rest of the tokens: more than 32 make one more such tile with a ragged
+    // second half, up to 32 make tasks of 32 tokens x 2 heads (the halves are two heads of the same tokens;
+    // they share the K/V operands all the same), so that 672 tokens x 6 heads are 63 tasks = 16 workgroups per
+    // KV head and slice, not 66 = 17.  Half h of this wave's task: tokens th0[h] .. th0[h] + 31 of head hd[h].
     const int task = tb * kT64Tasks + wave_u;
     const bool task_valid = task < a.ntask;
-    const int tt = (task_valid ? task : a.ntask - 1) / a.group;
-    const int hq = (task_valid ? task : a.ntask - 1) - tt * a.group;
-    const int head = kvh * a.group + hq;
-    const int t0 = tt * kT64Tile;
+    const int rem = a.tokens % kT64Tile;
+    const int whole = (a.tokens / kT64Tile + (rem > 32 ? 1 : 0)) * a.group; // tasks of 64 tokens x 1 head
+    auto last_token_of = [&](int k) { // of task k (the last one any of its halves holds)
+        const int end = k < whole ? (k / a.group + 1) * kT64Tile : a.tokens;
+        return (end < a.tokens ? end : a.tokens) - 1;
+    };
+    int th0[2], hd[2];
+    bool half_valid[2];
+    {
+        const int k = task_valid ? task : a.ntask - 1;
+        if (k < whole) {
+            const int tt = k / a.group, hq = k - tt * a.group;
+            th0[0] = tt * kT64Tile;
+            th0[1] = tt * kT64Tile + 32;
+            hd[0] = hd[1] = kvh * a.group + hq;
+            half_valid[0] = half_valid[1] = task_valid;
+        } else {
+            const int j = k - whole;
+            th0[0] = th0[1] = a.tokens - rem;
+            hd[0] = kvh * a.group + 2 * j;
+            hd[1] = kvh * a.group + (2 * j + 1 < a.group ? 2 * j + 1 : a.group - 1);
+            half_valid[0] = task_valid;
+            half_valid[1] = task_valid && 2 * j + 1 < a.group;
+        }
+    }
 
     const int last_task = (tb * kT64Tasks + kT64Tasks - 1 < a.ntask ? tb * kT64Tasks + kT64Tasks - 1 : a.ntask - 1);
-    const int tt_last = last_task / a.group;
-    const int last_tok = ((tt_last + 1) * kT64Tile < a.tokens ? (tt_last + 1) * kT64Tile : a.tokens) - 1;
-    const int seq_block = a.pos0 + last_tok + 1;
+    const int seq_block = a.pos0 + last_token_of(last_task) + 1;
     const int tiles_block = (seq_block + kKTile - 1) / kKTile;
     const int klo = (int)((long long)tiles_block * split / nsp) * kKTile;
     int khi = (int)((long long)tiles_block * (split + 1) / nsp) * kKTile;
@@ -995,16 +1019,16 @@ chunk_f16_t64_kernel(const ChunkArgs a)
     half8 Q[2][16];
     {
         uint8_t *qt = lds + kBufBytesF + wave * (32 * kKRow);
-        const float *qh = a.q + (size_t)head * kHeadDim + lane * 4;
         const size_t tok_stride = (size_t)a.n_head * kHeadDim;
 #pragma unroll
         for (int h = 0; h < 2; h++) {
+            const float *qh = a.q + (size_t)hd[h] * kHeadDim + lane * 4;
 #pragma unroll
             for (int b = 0; b < 2; b++) {
                 float4v f[16];
 #pragma unroll
                 for (int i = 0; i < 16; i++) {
-                    const int tr = t0 + h * 32 + b * 16 + i;
+                    const int tr = th0[h] + b * 16 + i;
                     f[i] = __builtin_nontemporal_load(
                         reinterpret_cast<const float4v *>(qh + (size_t)(tr < a.tokens ? tr : a.tokens - 1) * tok_stride));
                 }
@@ -1049,7 +1073,7 @@ chunk_f16_t64_kernel(const ChunkArgs a)
     auto max_part = [&](int t, int hk, int h, int part) { // scores N of half hk of tile t, token half h
         if (part == 0) {
             const int k0 = klo + t * kKTile + hk * 32;
-            const int tok0 = a.pos0 + t0 + h * 32;
+            const int tok0 = a.pos0 + th0[h];
             if ((k0 + 31 > tok0) || (k0 + 32 > khi)) { // (uniform over the wave)
                 // (the empty statement keeps this a branch: turned into selects, the 80 instructions would run
                 // for every half, and only the halves on the diagonal and at the end of the slice need them)
@@ -1257,7 +1281,8 @@ chunk_f16_t64_kernel(const ChunkArgs a)
 #pragma unroll
     for (int h = 0; h < 2; h++) {
         const float lsum = l_run[h] + __shfl_xor(l_run[h], 32);
-        const int tbase = t0 + h * 32;
+        const int tbase = th0[h], head = hd[h];
+        const bool task_valid = half_valid[h];
 #pragma unroll
         for (int hf = 0; hf < 2; hf++) {
             if (h == 0 && hf == 0)
@@ -2039,9 +2064,17 @@ int prefill_init()
 // tokens per wave with its own dequantization 15 % of the attention; measured gain, 2,048 tokens at depth
 // 2,048 / 8,192 / 16,384 / 100,000: 13 / 10 / 11 / 13 %, 1,024 tokens at 2,048 / 8,192: 3 / 4 %, 768 tokens at
 // 3,072 / 6,144: 0.5 / 3 %); with any smaller count the chunk runs as before.
+// Where the detour pays: chunks of 768 tokens or more behind a prefix at least as long, and chunks of 640 or
+// more (the 672 tokens of the usual prefill chunk) behind a prefix of eight times their length (672 tokens at
+// depth 672 / 2,048 / 8,192 / 32,768 / 100,000: -3 / -3 / +5 / +7 / +6 %).
+bool chunk_tiles_pay(int pos0, int tokens)
+{
+    return (tokens >= 768 && pos0 >= tokens) || (tokens >= 640 && pos0 >= 8 * tokens);
+}
+
 bool chunk_tiles_plan(int pos0, int tokens, int n_head, int n_kv, int splits, int *use, size_t *tiles_at)
 {
-    if (tokens < 768 || pos0 < tokens || splits < 3)
+    if (!chunk_tiles_pay(pos0, tokens) || splits < 3)
         return false;
     const int s = hipml_attn_chunk_slices(pos0, tokens, n_kv);
     if (s < 2)
@@ -2161,10 +2194,12 @@ int launch_chunk_q8(hipStream_t st, const float *q, const uint8_t *kc, const uin
     }
     // 64 tokens per wave: its own task blocks (4 tasks of 64 tokens), every one with `splits` slices.  Both
     // kernels run one workgroup per CU, so the hardware starts them in rounds of 256; where the other cut of
-    // the tokens needs a round more (672 tokens are 10.5 tiles of 64: 17 blocks per KV head and slice against
-    // 16), the kernel of 32 tokens per wave keeps the chunk.
+    // the tokens needs a round more, the kernel of 32 tokens per wave keeps the chunk.
     ChunkArgs b = a;
-    b.ntask = (tokens + kT64Tile - 1) / kT64Tile * a.group;
+    {
+        const int rem = tokens % kT64Tile; // (up to 32 left-over tokens: tasks of 32 tokens x 2 heads, see the kernel)
+        b.ntask = (tokens / kT64Tile + (rem > 32 ? 1 : 0)) * a.group + (rem > 0 && rem <= 32 ? (a.group + 1) / 2 : 0);
+    }
     b.nblock = (b.ntask + kT64Tasks - 1) / kT64Tasks;
     unsigned g64 = (unsigned)(n_kv * a.splits * b.nblock);
     if ((n_kv * a.splits) % 8 != 0 && 8 % (n_kv * a.splits) == 0)

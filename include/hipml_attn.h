@@ -79,7 +79,8 @@ int hipml_attn_batch_splits(int stride, int n_kv, int slots);
  * crates/hipml-model/src/gpu/attn_tile.rs:138-151.  0 (chunks near position 0: pos0 + tokens <=
  * 1,792 and pos0 <= 2 * tokens) selects the kernel that cuts the keys inside its workgroups and
  * needs no scratch; 1 the single-pass kernel; n >= 2 that kernel over n key slices with scratch
- * and a merge launch.  For long chunks behind a prefix at least as long (tokens >= 768, pos0 >= tokens) n is larger
+ * and a merge launch.  For long chunks behind a prefix at least as long (tokens >= 768 and pos0 >= tokens, or tokens >= 640
+ * and pos0 >= 8 * tokens) n is larger
  * than the number of slices that run (hipml_attn_chunk_slices): the chunk entry points then write the
  * live rows of the cache as f16 tiles (70,656 bytes per KV head and 64 rows) into the tail of part_acc
  * and run the attention over those, which is faster than dequantizing inside the attention (2,048 tokens

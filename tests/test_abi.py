@@ -55,9 +55,12 @@ def test_split_policies(lib):
     tiles = 4 * ((100_000 + 2048 + 63) // 64) * 70_656
     per_slice = 2048 * 24 * 256 * 4
     assert attn.chunk_splits(100_000, 2048, 4) == s + (tiles + per_slice - 1) // per_slice == 13
-    assert attn.chunk_splits(100_000, 767, 4) == attn.chunk_slices(100_000, 767, 4)   # too short to pay
     assert attn.chunk_splits(2047, 2048, 4) == attn.chunk_slices(2047, 2048, 4)  # prefix shorter than the chunk
     assert attn.chunk_splits(2048, 2048, 4) > attn.chunk_slices(2048, 2048, 4) >= 2
+    # the usual 672-token chunk: from eight times its length on
+    assert attn.chunk_splits(8 * 672 - 1, 672, 4) == attn.chunk_slices(8 * 672 - 1, 672, 4)
+    assert attn.chunk_splits(32768, 672, 4) > attn.chunk_slices(32768, 672, 4) >= 2
+    assert attn.chunk_splits(100_000, 639, 4) == attn.chunk_slices(100_000, 639, 4)
     assert attn.chunk_slices(0, 1, 4) >= 1
     # near position 0 the keys are cut inside the workgroups (0); deep chunks and long ones are not
     assert attn.chunk_splits(0, 672, 4) == 0 and attn.chunk_splits(0, 1, 4) == 0
