@@ -319,6 +319,8 @@ def bench_decode(torch, attn, seq, steps, warmup, layers, dtype=0):
         "workload": f"decode 1 query @ depth {seq}, {'q8_0' if dtype == 0 else 'q4_0'} cache, "
                     f"split-K {splits} + merge",
         "seq": seq, "splits": splits, "layers_rotated": layers,
+        # (the scratch is sized for `splits`; over q8_0 one sequence runs at most one workgroup per CU)
+        "splits_run": min(splits, max(256 // KV, 1)) if dtype == 0 else splits,
         "us_per_layer": us,
         "us_per_layer_gate_fused": tg.ms * 1e3 / (steps * layers),
         "us_per_layer_gate_separate": ts.ms * 1e3 / (steps * layers),

@@ -253,13 +253,14 @@ const char *hipml_attn_version(void) { return "hipml-attn-mi355x 0.2 (gfx950)"; 
 int hipml_attn_decode_splits(int seq, int n_kv)
 {
     // One workgroup of four waves walks 32-key tiles; give every workgroup at least one tile per
-    // wave (128 keys) and stop at one workgroup per CU (256) across the KV heads: the merge then
-    // reads half the partials of two workgroups per CU, and the rows stream no slower (measured at
-    // depth 32,768: 19.2 us per layer with 64 splits, 20.4 with 128; at 131,072: 51.9 against 52.5).
+    // wave (128 keys) and stop at two workgroups per CU (512) across the KV heads.  That is the scratch
+    // the q4_0 kernel wants (depth 32,768: 20.4 us per layer with 128 splits, 23.5 with 64); over q8_0
+    // the launch uses half of it, one workgroup per CU: the merge then reads half the partials, and the
+    // rows stream no slower (19.2 us with 64 splits, 20.4 with 128; at 131,072: 51.9 against 52.5).
     if (seq < 1 || n_kv < 1)
         return 1;
     int by_work = (seq + 127) / 128;
-    int by_cus = 256 / n_kv;
+    int by_cus = 512 / n_kv;
     if (by_cus < 1)
         by_cus = 1;
     int s = by_work < by_cus ? by_work : by_cus;

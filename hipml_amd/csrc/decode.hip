@@ -1905,10 +1905,26 @@ static int launch_decode_hd(hipStream_t st, const DecodeLaunch &L)
     return launched("attn_decode_kv_hd_reduce");
 }
 
-int launch_decode_q8(hipStream_t st, const DecodeLaunch &L)
+int launch_decode_q8(hipStream_t st, const DecodeLaunch &given)
 {
-    if (L.head_dim != kHeadDim)
-        return launch_decode_hd(st, L);
+    if (given.head_dim != kHeadDim)
+        return launch_decode_hd(st, given);
+    DecodeLaunch L = given;
+    // q8_0: the kernel that streams raw rows into LDS (its tile addressing is 32-bit per KV head);
+    // q4_0, the fp32-class variant and caches of more than 4 GiB per KV head: the staged kernel
+    // the kernel that moves raw rows addresses a KV head's rows and the Q rows with 32-bit byte offsets
+    const bool raw_rows = !L.q4 && !L.exact && (size_t)L.stride * kRowBytes < ((size_t)1 << 32) &&
+                          ((size_t)L.total_rows * L.q_slot + (size_t)L.n_heads * kHeadDim) * sizeof(float) <
+                              ((size_t)1 << 32);
+    // One sequence: the raw-row kernel is at its best with one workgroup per CU (19.2 us per layer at depth
+    // 32,768 with 64 splits of 4 KV heads, 20.4 with 128), the staged kernel with two (q4_0 there: 20.4 us
+    // with 128 splits, 23.5 with 64).  The split policy sizes the scratch for two; the raw-row kernel then
+    // cuts the keys into half as many splits and leaves the rest of the scratch alone (the layout of the
+    // partials is the kernels' own; every row of a verify group is cut the same way as its plain decode).
+    if (raw_rows && L.slots == 1) {
+        const int one_per_cu = 256 / L.n_kv > 1 ? 256 / L.n_kv : 1;
+        L.splits = L.splits < one_per_cu ? L.splits : one_per_cu;
+    }
     DecodeArgs a;
     a.q = L.q;
     a.k = L.k;
@@ -1930,12 +1946,6 @@ int launch_decode_q8(hipStream_t st, const DecodeLaunch &L)
     memset(a.kvslot, 0, sizeof(a.kvslot));
     memset(a.head0, 0, sizeof(a.head0));
     memset(a.nhead, 0, sizeof(a.nhead));
-    // q8_0: the kernel that streams raw rows into LDS (its tile addressing is 32-bit per KV head);
-    // q4_0, the fp32-class variant and caches of more than 4 GiB per KV head: the staged kernel
-    // the kernel that moves raw rows addresses a KV head's rows and the Q rows with 32-bit byte offsets
-    const bool raw_rows = !L.q4 && !L.exact && (size_t)L.stride * kRowBytes < ((size_t)1 << 32) &&
-                          ((size_t)L.total_rows * L.q_slot + (size_t)L.n_heads * kHeadDim) * sizeof(float) <
-                              ((size_t)1 << 32);
     // Work items: a slot whose rows x heads fit 8 columns is one item; a wider one (rows of an
     // MTP-verify slot) is cut by heads into as few items of at most 16 columns as will do, of equal
     // width where the heads divide that way (3 rows x 6 heads: two items of 9 columns).

@@ -70,7 +70,9 @@ const char *hipml_attn_version(void);
 
 /* Key splits for single-sequence decode on MI355X.  Same role as
  * DeepKv::splits, crates/hipml-model/src/gpu/deep_kv.rs:102-110, retuned for
- * 256 CUs.  Scratch is [n_heads][splits][head_dim] + [n_heads][splits][2] f32. */
+ * 256 CUs.  Scratch is [n_heads][splits][head_dim] + [n_heads][splits][2] f32.  The count is what the q4_0
+ * kernel wants (two workgroups per CU); over q8_0 a single-sequence launch given more than 256 / n_kv splits
+ * runs that many (one workgroup per CU, its optimum) inside the same scratch. */
 int hipml_attn_decode_splits(int seq, int n_kv);
 /* Key splits for batched decode.  Same role as attn_splits,
  * crates/hipml-model/src/gpu/batch/kv.rs:39-42. */
