@@ -177,13 +177,17 @@ def test_cache_entry_point_makes_its_tiles_in_the_scratch(dtype):
     gate = r.normal_array((tok, n_heads, HD))
 
     def over_cache(n):
-        acc, ml = attn.chunk_scratch(tok, n_heads, n)
-        acc.fill_(float("nan"))
-        ml.fill_(float("nan"))
+        # the scratch as the count sizes it, with a guard behind each part: the tiles must end inside it
+        qslots, guard = (tok + 31) // 32 * 32, 1 << 20
+        flat = torch.full((n * qslots * n_heads * HD + guard,), float("nan"), dtype=torch.float32, device="cuda")
+        flat[-guard:] = 12345.0
+        ml = torch.full((n * qslots * n_heads * 2 + guard,), float("nan"), dtype=torch.float32, device="cuda")
+        ml[-guard:] = 12345.0
         out = torch.full((tok, n_heads, HD), float("nan"), dtype=torch.float32, device="cuda")
         attn.chunk_attention_q8_split_gate(dev(q), dev(kb), dev(vb), dev(gate), out, n_heads, n_kv, HD, pos0, tok,
-                                           1 + dtype, stride, acc, ml, n)
+                                           1 + dtype, stride, flat, ml, n)
         torch.cuda.synchronize()
+        assert bool((flat[-guard:] == 12345.0).all()) and bool((ml[-guard:] == 12345.0).all())
         return host(out)
 
     got = over_cache(splits)
