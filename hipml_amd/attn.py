@@ -45,6 +45,7 @@ EXPORTS = [
     "hipml_attn_chunk_kv_f16",
     "hipml_attn_front_rows_f32", "hipml_attn_front_rows_encode_f32",
     "hipml_attn_decode_kv_noalloc", "hipml_rope_allow_device_angles",
+    "hipml_attn_decode_one_launch",
 ]
 
 
@@ -101,6 +102,7 @@ def lib() -> C.CDLL:
                                               sz, sz]),
             "hipml_attn_decode_kv_noalloc": (i, [vp, vp, i, vp, vp, vp, vp, i, i, i, i, f, i, sz, sz]),
             "hipml_rope_allow_device_angles": (i, [i]),
+            "hipml_attn_decode_one_launch": (i, [i]),
             "hipml_attn_decode_batch_cols_gate": (i, [vp, i, vp, vp, vp, vp, vp, vp, vp, vp, i, i, i,
                                                       i, f, i, sz, sz, sz, sz, i, vp]),
             "hipml_attn_chunk_q8_split": (i, [vp, vp, vp, vp, vp, i, i, i, i, i, i, i, vp, vp, i]),
@@ -382,6 +384,12 @@ def attn_decode_kv_noalloc(step, dtype, q, k, v, out, n_heads, n_kv, head_dim, s
     _check(lib().hipml_attn_decode_kv_noalloc(_stream(stream), _p(step), dtype, _p(q), _p(k), _p(v),
                                               _p(out), n_heads, n_kv, head_dim, stride, scale, splits,
                                               k_off, v_off))
+
+
+def decode_one_launch(on: int = -1) -> int:
+    """Process-wide: 1 = a single sequence over q8_0 merges its key splits inside the one launch, 0 (the
+    default) = in a second launch; a negative value only reads the mode.  Returns the mode before the call."""
+    return int(lib().hipml_attn_decode_one_launch(int(on)))
 
 
 def attn_decode_batch_cols_gate(dtype, pos, q, k_cache, v_cache, part_acc, part_ml, out, gate,

@@ -814,6 +814,8 @@ int hipml_attn_decode_kv_noalloc(hipml_stream_t stream, const int32_t *step, int
                                 head_dim, stride, scale, splits, k_off, v_off);
 }
 
+int hipml_attn_decode_one_launch(int on) { return decode_one_launch(on); }
+
 int hipml_attn_decode_kv_cols(hipml_stream_t stream, int dtype, const int32_t *pos,
                               const float *q, const void *k, const void *v, float *part_acc,
                               float *part_ml, float *out, int n_heads, int n_kv, int head_dim,

@@ -105,6 +105,9 @@ int decode_init();
 // hipml_attn_init with `device` current), and hand it out as the partial buffers of one call.
 int decode_static_init(int device);
 int decode_static_partials(int n_heads, int splits, float **part_acc, float **part_ml);
+// The process-wide choice between split + merge launches (0) and one launch whose workgroups merge their
+// partials themselves (1) for a single sequence over q8_0; on < 0 only reads it.  Returns the old value.
+int decode_one_launch(int on);
 
 // Raise the prefill kernels' dynamic LDS limit (once per process; called by hipml_attn_init).
 int prefill_init();

@@ -41,7 +41,10 @@
 
 #include "common.h"
 
+#include <atomic>
+#include <mutex>
 #include <stddef.h>
+#include <stdlib.h>
 #include <string.h>
 #include <type_traits>
 
@@ -89,6 +92,12 @@ struct DecodeArgs {
                      // the kernel decides the same per item for launches with several
     float scale_log2; // scale * log2(e) * 2^24
     size_t kv_slot_bytes, acc_slot, ml_slot, q_slot;
+    // merge > 0: the workgroups of a plain launch merge their partials themselves (decode_merge_tail),
+    // in groups of `merge` splits first; `tickets` are that launch's arrival counters
+    float *out;
+    const float *gate;
+    unsigned int *tickets;
+    int merge;
     // Work items (grid.y).  A slot whose rows x heads fit the columns of one workgroup (16; the raw-row
     // kernel runs items of up to 8 columns through its narrow body and wider ones through its wide
     // one) is one item; a wider one (2-4 MTP rows x 6 heads) is cut by heads into
@@ -220,7 +229,7 @@ __device__ __forceinline__ float quad_rows(float v)
 
 // The work of one workgroup: which KV head, work item and key split it serves.
 struct Work {
-    int kvh, split, nsp;                    // KV head, split index, splits of this item that have workers
+    int kvh, split, nsp, item;              // KV head, split index, splits of this item that have workers, item index
     int slot, row0, ncols, group, head0;    // the item: cache slot, first query row, rows, heads, first head
     int hbase, nvalid;                      // first head overall, (row, head) columns of the item
 };
@@ -368,6 +377,7 @@ __device__ __forceinline__ bool find_work(const DecodeArgs &a, int lane, Work &w
     wk.kvh = kvh;
     wk.split = split;
     wk.nsp = nsp;
+    wk.item = item;
     wk.slot = slot;
     wk.row0 = row0;
     wk.ncols = ncols;
@@ -874,6 +884,34 @@ __device__ __forceinline__ void dma16(uint32_t lds_at, const uint8_t *base, uint
                      : "memory");
 }
 
+// Device-scope accesses to the split partials.  A workgroup that merges partials (decode_merge_tail) reads
+// what workgroups on other XCDs, behind other L2 caches, have written while the same kernel runs.  A fence
+// would make that safe by writing back and invalidating a whole L2, once per wave: measured, it turned a
+// 19-us launch into one of 65 us.  Instead every access to a partial carries device scope itself (relaxed
+// atomic accesses of 64 bits: stores that are acknowledged once they are visible to the whole device, loads
+// that do not take a line another XCD may have changed from the local caches), and the order is kept by
+// waiting for the stores' acknowledgements before the ticket is drawn.
+__device__ __forceinline__ void store_dev(float *p, float2 v)
+{
+    __hip_atomic_store(reinterpret_cast<unsigned long long *>(p), __builtin_bit_cast(unsigned long long, v),
+                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void store_dev(float *p, float4v v)
+{
+    store_dev(p, (float2){v[0], v[1]});
+    store_dev(p + 2, (float2){v[2], v[3]});
+}
+__device__ __forceinline__ float2 load_dev2(const float *p)
+{
+    return __builtin_bit_cast(float2, __hip_atomic_load(reinterpret_cast<const unsigned long long *>(p),
+                                                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+}
+__device__ __forceinline__ float4v load_dev4(const float *p)
+{
+    const float2 a = load_dev2(p), b = load_dev2(p + 2);
+    return (float4v){a.x, a.y, b.x, b.y};
+}
+
 // A operand of a score MFMA from a raw key row: the 8 payload bytes [8 lg, 8 lg + 8) of block c as
 // f16 (b + 128) * 2^-24; `row_lg` = row + 8 lg.  LDS reads that are not aligned to their size run at a
 // fraction of the rate of aligned ones (measured: 35-64 against 2-3 cycles per ds_read_b64 over the
@@ -1037,8 +1075,7 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Work 
             const int col = threadIdx.x / group;
             const int head = hbase + (threadIdx.x - col * group);
             float *pm = a.part_ml + (size_t)(row0 + col) * a.ml_slot + ((size_t)head * a.splits + split) * 2;
-            pm[0] = -INFINITY;
-            pm[1] = 0.0f;
+            store_dev(pm, (float2){-INFINITY, 0.0f});
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // nothing may land in LDS after the wave has gone
         return; // uniform over the workgroup
@@ -1414,13 +1451,153 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Work 
                     const float2 x1 = *reinterpret_cast<const float2 *>(row + col0 + dd + 2);
                     acc += ((float4v){x0.x, x0.y, x1.x, x1.y} - off) * wgt[w];
                 }
-                *reinterpret_cast<float4v *>(pa + dd) = acc;
+                if (a.merge > 0)
+                    store_dev(pa + dd, acc);
+                else
+                    *reinterpret_cast<float4v *>(pa + dd) = acc;
             }
             if (threadIdx.x % kDRuns == 0) {
                 float *pm = a.part_ml + (size_t)(row0 + col) * a.ml_slot + slice * 2;
-                pm[0] = ms;
-                pm[1] = lsum;
+                if (a.merge > 0)
+                    store_dev(pm, (float2){ms, lsum});
+                else
+                    *reinterpret_cast<float2 *>(pm) = (float2){ms, lsum};
             }
+        }
+    }
+}
+
+// ---- the splits merged by the workgroups themselves ---------------------------------------------------
+// A plain launch of one sequence needs no second launch.  A workgroup that has written its partial takes
+// a ticket of its group of kMergeGroup consecutive splits.  Whoever draws a group's last ticket finds every
+// partial of the group in memory, folds them into one (in split order, so the result does not depend on
+// who came last), writes that over the group's first partial and takes a ticket of the (item, KV head);
+// whoever draws the last of those folds the groups' partials and writes the output rows, gated if the call
+// says so.  Nobody waits for anybody: a workgroup that is not last leaves.  Two levels keep a fold at a few
+// dozen KB (the 64 partials of a KV head with 6 heads are 384 KB, which one CU takes 3 us to read).
+// The counters (`tickets`: per (item, KV head) one per group, then one for the groups) live in library
+// memory, start at zero and are put back to zero by the workgroup that draws the last ticket, so a
+// captured launch can be replayed; launches that share counters must not overlap.
+constexpr int kMergeGroup = 8;
+constexpr int kMergeMaxSplits = 128; // beyond: the merge kernels
+
+// Thread 0 draws from `counter` once every thread's device-scope stores so far are visible to the device;
+// returns (uniformly) whether this workgroup drew ticket `count` - 1: then every other drawer's stores are.
+typedef volatile __attribute__((address_space(3))) unsigned int *LdsFlag;
+__device__ __forceinline__ bool last_ticket(unsigned int *counter, unsigned int count, LdsFlag flag)
+{
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // this thread's stores have been acknowledged
+    __syncthreads(); // (also: everybody has read the flag of an earlier draw and is done with the LDS it lies in)
+    if (threadIdx.x == 0) {
+        const unsigned int drawn = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const bool last = drawn + 1 == count;
+        if (last)
+            __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *flag = last ? 1u : 0u;
+    }
+    __syncthreads();
+    return *flag != 0;
+}
+
+// (m, sum, KRUN values of d) of the partials first, first + step, ... (`count` of them) folded in that order:
+// M = max m_j over the partials that saw a key (sum > 0), w_j = 2^(m_j - M), L = sum l_j w_j, A = sum acc_j w_j.
+template <int KRUN>
+__device__ __forceinline__ void fold_partials(const float *pa, const float *pm, int first, int step, int count,
+                                              float &M, float &L, float4v (&A)[KRUN / 4])
+{
+    const float4v z = {0, 0, 0, 0};
+    float2 v[8];
+    float4v x[8][KRUN / 4];
+    auto fetch = [&](int j0) {
+#pragma unroll
+        for (int jj = 0; jj < 8; jj++) {
+            const int j = j0 + jj < count ? j0 + jj : count - 1; // (past the end: the last one again, weight 0)
+            const size_t s = (size_t)first + (size_t)j * step;
+            v[jj] = load_dev2(pm + s * 2);
+#pragma unroll
+            for (int i = 0; i < KRUN / 4; i++)
+                x[jj][i] = load_dev4(pa + s * kHeadDim + 4 * i);
+        }
+    };
+    fetch(0);
+    M = -INFINITY;
+#pragma unroll
+    for (int jj = 0; jj < 8; jj++)
+        M = jj < count && v[jj].y > 0.0f ? fmaxf(M, v[jj].x) : M;
+    for (int j = 8; j < count; j++) {
+        const float2 u = load_dev2(pm + ((size_t)first + (size_t)j * step) * 2);
+        M = u.y > 0.0f ? fmaxf(M, u.x) : M;
+    }
+    L = 0.0f;
+#pragma unroll
+    for (int i = 0; i < KRUN / 4; i++)
+        A[i] = z;
+    for (int j0 = 0; j0 < count; j0 += 8) {
+        if (j0 > 0)
+            fetch(j0);
+#pragma unroll
+        for (int jj = 0; jj < 8; jj++) {
+            const bool live = j0 + jj < count && v[jj].y > 0.0f; // (false for NaN as well)
+            const float w = live ? __builtin_amdgcn_exp2f(v[jj].x - M) : 0.0f;
+            L = fmaf(live ? v[jj].y : 0.0f, w, L);
+            // a partial without a key holds whatever the scratch held: select, not multiply
+#pragma unroll
+            for (int i = 0; i < KRUN / 4; i++)
+                A[i] += w > 0.0f ? x[jj][i] * w : z;
+        }
+    }
+}
+
+template <bool WIDE>
+__device__ __forceinline__ void decode_merge_tail(const DecodeArgs &a, const Work &wk)
+{
+    constexpr int kCols = WIDE ? 16 : 8;
+    constexpr int kDRuns = kThreads / kCols, kRun = kHeadDim / kDRuns; // as the partials were written
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds_all[];
+    const LdsFlag flag = (LdsFlag)lds_all;
+    const int ngroup = (a.splits + kMergeGroup - 1) / kMergeGroup;
+    const int g0 = wk.split / kMergeGroup * kMergeGroup;
+    const int gsize = a.splits - g0 < kMergeGroup ? a.splits - g0 : kMergeGroup;
+    unsigned int *tk = a.tickets + (size_t)(wk.item * a.n_kv + wk.kvh) * (ngroup + 1);
+    if (!last_ticket(tk + g0 / kMergeGroup, (unsigned)gsize, flag))
+        return;
+    const int nc = threadIdx.x / kDRuns;
+    const int d0 = (threadIdx.x % kDRuns) * kRun;
+    const bool mine = nc < wk.nvalid;
+    const int col = mine ? nc / wk.group : 0;
+    const int head = wk.hbase + (mine ? nc - col * wk.group : 0);
+    float *pa = a.part_acc + (size_t)(wk.row0 + col) * a.acc_slot + (size_t)head * a.splits * kHeadDim + d0;
+    float *pm = a.part_ml + (size_t)(wk.row0 + col) * a.ml_slot + (size_t)head * a.splits * 2;
+    float M = -INFINITY, L = 0.0f;
+    float4v A[kRun / 4];
+    if (mine)
+        fold_partials<kRun>(pa, pm, g0, 1, gsize, M, L, A);
+    if (ngroup > 1) {
+        if (mine) {
+#pragma unroll
+            for (int i = 0; i < kRun / 4; i++)
+                store_dev(pa + (size_t)g0 * kHeadDim + 4 * i, A[i]);
+            if (threadIdx.x % kDRuns == 0)
+                store_dev(pm + (size_t)g0 * 2, (float2){M, L});
+        }
+        if (!last_ticket(tk + ngroup, (unsigned)ngroup, flag))
+            return;
+        if (mine)
+            fold_partials<kRun>(pa, pm, 0, kMergeGroup, ngroup, M, L, A);
+    }
+    if (mine) {
+        const size_t at = (size_t)(wk.row0 + col) * a.q_slot + (size_t)head * kHeadDim + d0;
+        const float inv = L > 0.0f ? 1.0f / L : 0.0f;
+#pragma unroll
+        for (int i = 0; i < kRun / 4; i++) {
+            float4v r = A[i] * inv;
+            if (!(L > 0.0f))
+                r = (float4v){0, 0, 0, 0};
+            if (a.gate != nullptr) {
+                const float4v gt = *reinterpret_cast<const float4v *>(a.gate + at + 4 * i);
+                r = (float4v){gated(r[0], gt[0]), gated(r[1], gt[1]), gated(r[2], gt[2]), gated(r[3], gt[3])};
+            }
+            *reinterpret_cast<float4v *>(a.out + at + 4 * i) = r;
         }
     }
 }
@@ -1431,10 +1608,15 @@ __global__ void __launch_bounds__(kThreads, 2) decode_q8_kernel(const DecodeArgs
     Work wk;
     if (!find_work(a, threadIdx.x & 63, wk))
         return;
-    if (wk.nvalid > 8) // uniform over the workgroup
+    if (wk.nvalid > 8) { // uniform over the workgroup
         decode_body_dma<true>(a, wk);
-    else
+        if (a.merge > 0)
+            decode_merge_tail<true>(a, wk);
+    } else {
         decode_body_dma<false>(a, wk);
+        if (a.merge > 0)
+            decode_merge_tail<false>(a, wk);
+    }
 }
 
 // Wave-wide reductions without LDS: DPP inside a row of 16 lanes, then the two row-swap
@@ -1680,6 +1862,8 @@ static __device__ __align__(256) float scratch[kStaticSlices * (kHeadDim + 2)];
 constexpr int kMaxDevices = 64;
 static float *g_scratch_ptr[kMaxDevices]; // device address of `scratch` on each initialised GPU
 
+static int decode_tickets_init(int device);
+
 // Called by hipml_attn_init with `device` current.
 int decode_static_init(int device)
 {
@@ -1691,7 +1875,81 @@ int decode_static_init(int device)
         return fail(e != hipSuccess ? (int)e : HIPML_ATTN_E_STATE, "hipGetSymbolAddress(scratch) failed: %d (%s)",
                     (int)e, hipGetErrorString(e));
     g_scratch_ptr[device] = ptr;
+    return decode_tickets_init(device);
+}
+
+// ---- arrival counters of the launches whose workgroups merge their own partials ---------------------
+// (decode_merge_tail).  Launches that may run at the same time need counters of their own, and launches
+// on one stream never do, so a launch takes the slot of its stream: the first kTicketStreams streams a
+// device sees get one each, for good; launches on further streams go the way of two launches.  A launch
+// that is being captured into a graph takes the next slot of a ring instead, because a graph may be
+// replayed on any stream and beside eager launches of the stream it was captured on: two graphs whose
+// captured launches are kTicketRing launches apart share slots and must not be replayed at the same time.
+// Every GPU the library is initialised on holds one copy of the array (512 KiB), zero when the module is
+// loaded; a kernel leaves the counters it used at zero.
+// Whether they do is a setting of the process, off unless asked for: measured on MI355X the device-scope
+// round trips of one level of this merge (stores acknowledged, ticket, loads: ~1.2 us each) cost as much as
+// the launch of the merge kernel they replace, so the two launches are the faster form at every depth.
+static std::atomic<int> g_one_launch{[] {
+    const char *e = getenv("HIPML_DECODE_ONE_LAUNCH");
+    return e != nullptr && e[0] != '\0' && e[0] != '0' ? 1 : 0;
+}()};
+int decode_one_launch(int on)
+{
+    return on < 0 ? g_one_launch.load(std::memory_order_relaxed) : g_one_launch.exchange(on != 0 ? 1 : 0);
+}
+
+constexpr int kTicketStreams = 32, kTicketRing = 96;
+constexpr int kTicketsPerSlot = 1024;
+static __device__ __align__(256) unsigned int tickets[(kTicketStreams + kTicketRing) * kTicketsPerSlot];
+static unsigned int *g_tickets_ptr[kMaxDevices];
+static std::mutex g_ticket_mu;
+static hipStream_t g_ticket_stream[kMaxDevices][kTicketStreams];
+static int g_ticket_streams[kMaxDevices];
+static unsigned int g_ticket_ring[kMaxDevices];
+
+static int decode_tickets_init(int device)
+{
+    unsigned int *ptr = nullptr;
+    const hipError_t e = hipGetSymbolAddress(reinterpret_cast<void **>(&ptr), HIP_SYMBOL(tickets));
+    if (e != hipSuccess || ptr == nullptr)
+        return fail(e != hipSuccess ? (int)e : HIPML_ATTN_E_STATE, "hipGetSymbolAddress(tickets) failed: %d (%s)",
+                    (int)e, hipGetErrorString(e));
+    std::lock_guard<std::mutex> lock(g_ticket_mu);
+    g_tickets_ptr[device] = ptr;
     return 0;
+}
+
+// The counters a launch of `need` of them on `st` may use, or nullptr: then the launch leaves the merge
+// to a second one.  Allocates nothing and launches nothing.
+static unsigned int *decode_tickets(hipStream_t st, int need)
+{
+    if (g_one_launch.load(std::memory_order_relaxed) == 0 || need > kTicketsPerSlot)
+        return nullptr;
+    int device = -1;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices)
+        return nullptr;
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(st, &capture) != hipSuccess) {
+        (void)hipGetLastError(); // (the launch itself will report what is wrong with the stream)
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(g_ticket_mu);
+    unsigned int *base = g_tickets_ptr[device];
+    if (base == nullptr)
+        return nullptr;
+    if (capture != hipStreamCaptureStatusNone)
+        return base + (size_t)(kTicketStreams + g_ticket_ring[device]++ % kTicketRing) * kTicketsPerSlot;
+    int n = g_ticket_streams[device], i = 0;
+    while (i < n && g_ticket_stream[device][i] != st)
+        i++;
+    if (i == n) {
+        if (n == kTicketStreams)
+            return nullptr;
+        g_ticket_stream[device][n] = st;
+        g_ticket_streams[device] = n + 1;
+    }
+    return base + (size_t)i * kTicketsPerSlot;
 }
 
 // The current device's copy of the array, cut into the two partial buffers of a decode call of
@@ -1982,6 +2240,18 @@ int launch_decode_q8(hipStream_t st, const DecodeLaunch &given)
     a.workers = L.slots > 1 && items > 1 && items <= 64 && 2 * items <= window ? window : 0;
     const dim3 grid = a.workers > 0 ? dim3((unsigned)(L.n_kv * a.workers), 1, 1)
                                     : dim3((unsigned)(L.n_kv * L.splits), (unsigned)items, 1);
+    // One sequence over q8_0 rows: the workgroups merge their partials themselves, if this stream has
+    // counters for them (one row and the rows of a verify group alike, so that a column of a group stays
+    // bit for bit the plain decode of its row).
+    a.out = L.out;
+    a.gate = L.gate;
+    a.tickets = nullptr;
+    a.merge = 0;
+    if (raw_rows && L.slots == 1 && a.workers == 0 && L.splits <= kMergeMaxSplits) {
+        const int ngroup = (L.splits + kMergeGroup - 1) / kMergeGroup;
+        a.tickets = decode_tickets(st, items * L.n_kv * (ngroup + 1));
+        a.merge = a.tickets != nullptr ? kMergeGroup : 0;
+    }
     if (raw_rows)
         hipLaunchKernelGGL(decode_q8_kernel, grid, dim3(kThreads, 1, 1), kDmaLds, st, a);
     else if (L.q4)
@@ -1989,7 +2259,7 @@ int launch_decode_q8(hipStream_t st, const DecodeLaunch &given)
     else
         hipLaunchKernelGGL((decode_staged_kernel<false, true>), grid, dim3(kThreads, 1, 1), decode_lds_bytes(1), st, a);
     int rc = launched(L.q4 ? "attn_decode_kv_q4" : "attn_decode_kv_q8");
-    if (rc)
+    if (rc || a.merge > 0)
         return rc;
     // Up to 128 splits (every launch the split policies make): the one-barrier merge.  One sequence
     // (a query row, or the rows of a verify group: the same merge, so that a column of a group is

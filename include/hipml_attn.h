@@ -334,6 +334,21 @@ int hipml_attn_decode_kv_noalloc(hipml_stream_t stream, const int32_t *step, int
                                  int head_dim, int stride, float scale, int splits, size_t k_off,
                                  size_t v_off);
 
+/* How a single sequence over a q8_0 cache (hipml_attn_decode_kv, _gate, _noalloc, _cols) merges its key
+ * splits.  0 (the default): a second launch, as in the reference (attn_decode_kv_reduce,
+ * crates/hipml-kernels/kernels/attn_decode_kv.hip:491-532).  1: the workgroups of the one launch merge
+ * them: each takes a ticket when its partial is in memory, the last of eight neighbouring splits folds
+ * those, the last of those groups folds the groups and writes `out`; nobody waits, nothing is allocated
+ * (the counters are library memory, one set per stream for the first 32 streams of a device and a ring
+ * of 96 for launches under capture; launches that share a set must not overlap).  Same tolerance class,
+ * not the same bits as mode 0; a verify column still has the bits of its row's plain decode in the same
+ * mode.  Measured on MI355X it is the slower form at every depth (depth 32,768: 23.3 against 20.0 us
+ * per layer; 8,192: 15.7 against 11.4; 673: 10.1 against 9.6): one level of such a merge is three
+ * dependent device-scope round trips of ~1.2 us, as much as the launch it saves.  It has no counterpart
+ * in the reference and is kept so that this figure can be measured again.  on < 0 only reads the mode;
+ * returns the mode before the call.  Environment: HIPML_DECODE_ONE_LAUNCH=1 sets the initial mode. */
+int hipml_attn_decode_one_launch(int on);
+
 /* ---- causal chunk prefill over a q8_0 / q4_0 cache -------------------------------- */
 
 /* tokens query rows at positions pos0..pos0+tokens-1 attend keys [0, pos0+t]
