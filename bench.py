@@ -15,8 +15,15 @@ decode with MTP-verify slots), each with its own roofline object.
 
 roofline.achieved = algorithmic FLOP (prefill) or K+V cache bytes (decode) per
 attention launch / the attention launch's mean duration measured with HIP
-events on the launch stream.  cpu_baseline = the CPU oracle (a scalar restatement
-of the reference's CPU path) timed on this host on the stated sample.
+events on the launch stream.  roofline.achievable = what a kernel that does
+nothing else reaches on this box in the same run: a pure read of the same bytes
+in the decode kernel's access pattern, or a loop of independent MFMAs (the
+library's measurement-only entry points hipml_bench_*).  Every figure is the mean
+over at least --steps steps and at least 200 ms of timed GPU work (the reference
+sizes its repetitions the same way, crates/hipml-kernels/src/kvbench.rs:160-163);
+`timed_ms` and `steps_timed` say what was timed.  cpu_baseline = the CPU oracle (a
+scalar restatement of the reference's CPU path) timed on this host on the stated
+sample.
 """
 from __future__ import annotations
 
@@ -36,6 +43,8 @@ SCALE = 1.0 / 16.0
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E, published
 MFMA_F16_PEAK_TF = 2500.0  # MI355X dense fp16 MFMA, published
 LAYERS = 16                # distinct layer caches a pass rotates over
+MIN_TIMED_MS = 200.0       # every figure is a mean over at least this much timed GPU work
+MFMA_FLOP_PER_CYCLE = 256 * 4 * 1024.0  # dense f16: 256 CUs x 4 SIMDs x 32x32x16x2 FLOP per 32 cycles
 
 
 def prefill_flop(pos0: int, tokens: int) -> float:
@@ -88,6 +97,83 @@ class Timer:
         self.ms = self.a.elapsed_time(self.b)
 
 
+def timed(torch, fn, steps, warm=3, wall=False, min_ms=MIN_TIMED_MS):
+    """Mean duration of fn(i) in ms over max(steps, what fills `min_ms`) calls, by HIP events on the launch
+    stream (wall: by the host clock between two synchronisations); returns (ms per call, ms timed, calls)."""
+    for i in range(warm):
+        fn(i)
+    probe = max(1, min(steps, 8))
+    with Timer(torch) as t:
+        for i in range(probe):
+            fn(i)
+    n = max(steps, int(1.1 * min_ms / max(t.ms / probe, 1e-4)) + 1)
+    while True:
+        if wall:
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for i in range(n):
+                fn(i)
+            torch.cuda.synchronize()
+            total = (time.perf_counter() - t0) * 1e3
+        else:
+            with Timer(torch) as t:
+                for i in range(n):
+                    fn(i)
+            total = t.ms
+        if total >= min_ms:
+            break
+        n = int(n * 1.2 * min_ms / max(total, 1e-3)) + 1  # (the short run was slower per call than the long one)
+    return total / n, total, n
+
+
+def counters(workload: str, kernel: str):
+    """Clock and MFMA-busy share of `kernel` in the committed counter run of `workload`
+    (profiles/mfma_counters.json: rocprofv3 --pmc on this benchmark's --only legs), or {}."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "mfma_counters.json")) as f:
+            t = json.load(f).get(workload, {})
+    except OSError:
+        return {}
+    for name, v in t.items():
+        if kernel in name:
+            return {"clock_ghz": v.get("clock_ghz"), "mfma_busy": v.get("mfma_busy"),
+                    "clock_source": "profiles/mfma_counters.json (GRBM_GUI_ACTIVE / 8 / kernel duration)"}
+    return {}
+
+
+def mfma_yardstick(torch, attn, steps=4):
+    """A loop of independent v_mfma_f32_32x32x16_f16 on one wave per SIMD of every CU: the rate the MFMA
+    pipes reach with nothing else to do, and the clock the chip holds under that load."""
+    wgs, iters = 256, 20000
+    sink = torch.zeros(4, dtype=torch.float32, device="cuda")
+    clocks = torch.zeros(2, dtype=torch.int64, device="cuda")
+    ms, total, n = timed(torch, lambda i: attn.bench_mfma_f16(wgs, iters, sink, clocks), steps)
+    flop = wgs * 4 * iters * 8 * 32768.0
+    c = clocks.cpu().tolist()
+    ghz = c[0] / max(c[1], 1) * 0.1
+    tf = flop / (ms * 1e-3) / 1e12
+    return {"workload": "256 workgroups x 4 waves (one per SIMD) x 20,000 x 8 independent v_mfma_f32_32x32x16_f16",
+            "tflops": tf, "frac_of_peak": tf / MFMA_F16_PEAK_TF, "clock_ghz": ghz,
+            "frac_at_that_clock": tf * 1e12 / (MFMA_FLOP_PER_CYCLE * ghz * 1e9),
+            "ms_per_launch": ms, "timed_ms": total, "steps_timed": n}
+
+
+def stream_yardstick(torch, attn, pairs, bytes_each, steps):
+    """One launch per (k, v) pair that only reads bytes_each bytes of each, rotating over the pairs: GB/s of
+    the better of the two load forms, with both times."""
+    sink = torch.zeros(4, dtype=torch.int32, device="cuda")
+    bytes_each = bytes_each // 8704 * 8704
+    res = {}
+    for mode, name in ((0, "global_load_lds"), (1, "register_loads")):
+        def one(i, mode=mode):
+            k, v = pairs[i % len(pairs)]
+            attn.bench_stream_read(k, v, bytes_each, mode, sink)
+        ms, total, n = timed(torch, one, steps * len(pairs), warm=len(pairs))
+        res[name] = {"us_per_launch": ms * 1e3, "gbs": 2 * bytes_each / (ms * 1e-3) / 1e9, "timed_ms": total}
+    best = max(res.values(), key=lambda r: r["gbs"])
+    return {"achievable": best["gbs"], "bytes_per_launch": 2 * bytes_each, **{k: v for k, v in res.items()}}
+
+
 def fill_cache_normal(torch, attn, k_cache, v_cache, stride, rows, gen, dtype=0):
     """Quantize N(0,1) rows into a [KV][stride][272] (q8_0) or [..][144] (q4_0, dtype 1) cache pair
     with the library's own append kernel, in slabs so the f32 source stays small."""
@@ -104,7 +190,7 @@ def fill_cache_normal(torch, attn, k_cache, v_cache, stride, rows, gen, dtype=0)
 # prefill: rope + append + attention + gate
 # ---------------------------------------------------------------------------------------
 
-def bench_prefill(torch, attn, tokens, pos0, steps, warmup, layers, prefix_fill=True):
+def bench_prefill(torch, attn, tokens, pos0, steps, warmup, layers, prefix_fill=True, mfma=None):
     stride = (pos0 + tokens + 63) // 64 * 64
     gen = torch.Generator(device="cuda")
     gen.manual_seed(0x5EED0002 + pos0)
@@ -188,60 +274,81 @@ def bench_prefill(torch, attn, tokens, pos0, steps, warmup, layers, prefix_fill=
         attention(i)
         attn.q_gate(out, gate, out)
 
-    def wall(fn):
-        for i in range(warmup):
-            fn(i)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for i in range(steps):
-            fn(i)
-        torch.cuda.synchronize()
-        return (time.perf_counter() - t0) * 1e3 / steps
-
-    unfused_ms = wall(step_unfused)
-    wall_ms = wall(step)
+    unfused_ms, _, _ = timed(torch, step_unfused, steps, warmup, wall=True)
+    wall_ms, wall_total, wall_n = timed(torch, step, steps, warmup, wall=True)
     # the f16 copy of the cache serves long prefixes: the sliced kernel over it is not what a chunk near
     # position 0 would run (splits == 0), so that leg is left out there
     with_copy = splits != 0
-    copy_ms = wall(step_copy) if with_copy else None
-    copy_rebuilt_ms = wall(lambda i: step_copy(i, True)) if with_copy else None
+    copy_ms = timed(torch, step_copy, steps, warmup, wall=True)[0] if with_copy else None
+    copy_rebuilt_ms = timed(torch, lambda i: step_copy(i, True), steps, warmup, wall=True)[0] if with_copy else None
 
     # the attention launch alone, HIP events on the launch stream
-    def events(fn):
-        for i in range(min(warmup, 3)):
-            fn(i)
-        with Timer(torch) as t:
-            for i in range(steps):
-                fn(i)
-        return t.ms / steps
-
-    attn_ms = events(attention)
-    attn_copy_ms = events(attention_copy) if with_copy else None
+    attn_ms, attn_total, attn_n = timed(torch, attention, steps, min(warmup, 3))
+    attn_copy_ms = timed(torch, attention_copy, steps, min(warmup, 3))[0] if with_copy else None
     flop = prefill_flop(pos0, tokens)
     tf = flop / (attn_ms * 1e-3) / 1e12
-    rows_bytes = 2 * tokens * H * HD * 4 + 2 * KV * (pos0 + tokens) * ROW
-    wl = {(672, 0): "prefill672", (2048, 100_000): "chunk100k"}.get((tokens, pos0), "")
-    # (the instantiation that reads the cache: <SPLIT, q4_0, over the f16 copy>)
     # A scratch sized for more slices than the sliced kernel would use: the call writes the live rows of the
     # cache as f16 tiles into the tail of the scratch and runs `slices` slices of the 64-token kernel over them.
     tiles_path = splits > slices >= 2
+    # What an engine gets that keeps the reference's own scratch: 8 slices, allocated once
+    # (crates/hipml-model/src/gpu/prefill.rs:159-166, gpu/attn_tile.rs:122-151): no room for the tiles, so the
+    # call runs the kernel that dequantizes for itself.
+    ref_scratch = None
+    if tiles_path:
+        ref_splits = 8
+
+        def attention_ref(i):
+            k, v = caches[i % layers]
+            q, kx, vx, gate, out = acts[i % layers]
+            attn.chunk_attention_q8_split(q, k, v, out, H, KV, HD, pos0, tokens, 1, stride, acc, ml, ref_splits)
+        ref_ms, ref_total, _ = timed(torch, attention_ref, steps, min(warmup, 3))
+        ref_scratch = {"note": "the same attention launch with the scratch an unchanged reference engine allocates "
+                               "(8 slices): chunk_q8_kernel<split> + chunk_combine_kernel, no f16 tiles",
+                       "splits": ref_splits, "attn_ms": ref_ms, "timed_ms": ref_total,
+                       "frac": flop / (ref_ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TF}
+    # The same calls with every layer cache registered once (hipml_kv_f16_attach, what an engine does where it
+    # allocates the cache): the library keeps the f16 tiles itself, the append converts the chunk's rows and the
+    # attention through the reference's entry point reads them; no tiles are made per call.
+    shadow = None
+    if with_copy:
+        for (k, v), c in zip(caches, copies):
+            attn.kv_f16_attach(0, k, v, c, KV, HD, stride, pos0)
+        try:
+            sh_ms, sh_total, sh_n = timed(torch, step, steps, warmup, wall=True)
+            sh_attn_ms, sh_attn_total, sh_attn_n = timed(torch, attention, steps, min(warmup, 3))
+        finally:
+            for k, v in caches:
+                attn.kv_f16_detach(k)
+        shadow = {"note": "every layer cache registered once with hipml_kv_f16_attach: rope + append (which converts "
+                          "the chunk's rows) + hipml_attn_chunk_q8_split_gate reading the library-kept f16 tiles",
+                  "ms_per_step": sh_ms, "tok_per_s": tokens / (sh_ms * 1e-3), "timed_ms": sh_total, "steps_timed": sh_n,
+                  "attn_ms": sh_attn_ms, "attn_timed_ms": sh_attn_total,
+                  "attn_frac": flop / (sh_attn_ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TF,
+                  "slices_run": min(max(splits, slices), slices)}
+    rows_bytes = 2 * tokens * H * HD * 4 + 2 * KV * (pos0 + tokens) * ROW
+    wl = {(672, 0): "prefill672", (2048, 100_000): "chunk100k"}.get((tokens, pos0), "")
+    # (the attention-only launch timed here takes no gate and rotated query rows: <q4_0 false, in-kernel RoPE false>)
     if splits == 0:
-        traffic = measured_traffic(wl, ["chunk_wg_kernel<false, true>"])
+        kernel, traffic = "chunk_wg_kernel", measured_traffic(wl, ["chunk_wg_kernel<false, false>"])
     elif tiles_path:
+        kernel = "chunk_f16_t64_kernel"
         traffic = measured_traffic(wl, ["chunk_f16_t64_kernel", "chunk_combine_kernel"], ["kv_f16_tiles_kernel<false>"])
     else:
+        kernel = "chunk_q8_kernel"
         traffic = measured_traffic(wl, ["chunk_q8_kernel<true, false, false>", "chunk_q8_kernel<false, false, false>",
                                         "chunk_combine_kernel"])
-    return {
+    res = {
         "workload": f"prefill {tokens}@{pos0}: rope + q8_0 append + causal GQA attention + gate, "
                     f"1 layer, {H}q/{KV}kv heads, head_dim {HD}",
         "tokens": tokens, "pos0": pos0, "splits": splits, "slices_over_f16_copy": slices, "layers_rotated": layers,
         "scratch_slices": max(splits, slices), "slices_run": slices if tiles_path else splits,
-        "ms_per_step": wall_ms,
+        "ms_per_step": wall_ms, "timed_ms": wall_total, "steps_timed": wall_n,
         "tok_per_s": tokens / (wall_ms * 1e-3),
         "ms_per_step_separate_launches": unfused_ms,
         "attn_ms": attn_ms,
         "attn_tok_per_s": tokens / (attn_ms * 1e-3),
+        "reference_scratch_8_slices": ref_scratch,
+        "attached_f16_shadow": shadow,
         "over_f16_copy": None if not with_copy else {
             "note": "the same step with the attention reading an f16 copy of the cache that the step keeps "
                     "current (hipml_kv_f16_rows for the chunk's rows after the append, then "
@@ -252,22 +359,46 @@ def bench_prefill(torch, attn, tokens, pos0, steps, warmup, layers, prefix_fill=
             "copy_bytes_per_layer": attn.kv_f16_bytes(stride, KV)},
         "roofline": {"bound": "mfma", "achieved": tf, "peak": MFMA_F16_PEAK_TF, "unit": "TFLOP/s",
                      "frac": tf / MFMA_F16_PEAK_TF, "traffic": traffic,
+                     "achievable": None if mfma is None else mfma["tflops"],
+                     "frac_of_achievable": None if mfma is None else tf / mfma["tflops"],
+                     **counters(wl, kernel),
                      "kernel": "chunk_wg_kernel" if splits == 0 else
                      "kv_f16_tiles_kernel + chunk_f16_t64_kernel + chunk_combine_kernel" if tiles_path else
                      "chunk_q8_kernel" + (" + chunk_combine_kernel" if splits >= 2 else ""),
-                     "flop_per_launch": flop, "launch_ms": attn_ms,
+                     "flop_per_launch": flop, "launch_ms": attn_ms, "timed_ms": attn_total, "steps_timed": attn_n,
                      # the same launch against the other roof: the f32 rows it has to move (Q in, rows out; the
                      # attention-only launch timed here takes no gate) and the cache rows once, over 8 TB/s
                      "algorithmic_bytes": rows_bytes,
                      "hbm_frac": rows_bytes / (attn_ms * 1e-3) / 1e9 / HBM_PEAK_GBS},
     }
+    if tiles_path and shadow is not None:
+        # Deep in a prefix the entry's figures are those of an engine that has registered its caches (the
+        # integration this library documents); what the same calls cost without that is kept beside them.
+        res["tiles_made_per_call_in_the_scratch"] = {
+            "note": "no shadow registered, scratch sized by hipml_attn_chunk_splits: every call writes the live "
+                    "rows as f16 tiles into the tail of the scratch first (kv_f16_tiles_kernel)",
+            "ms_per_step": wall_ms, "attn_ms": attn_ms, "timed_ms": attn_total, "frac": tf / MFMA_F16_PEAK_TF,
+            "traffic": traffic}
+        tfs = flop / (shadow["attn_ms"] * 1e-3) / 1e12
+        res.update({"ms_per_step": shadow["ms_per_step"], "timed_ms": shadow["timed_ms"],
+                    "steps_timed": shadow["steps_timed"], "tok_per_s": shadow["tok_per_s"],
+                    "attn_ms": shadow["attn_ms"], "attn_tok_per_s": tokens / (shadow["attn_ms"] * 1e-3)})
+        res["workload"] += "; every layer cache registered once with hipml_kv_f16_attach"
+        res["roofline"].update({
+            "achieved": tfs, "frac": tfs / MFMA_F16_PEAK_TF,
+            "frac_of_achievable": None if mfma is None else tfs / mfma["tflops"],
+            "traffic": measured_traffic(wl, ["chunk_f16_t64_kernel", "chunk_combine_kernel"]),
+            "kernel": "chunk_f16_t64_kernel + chunk_combine_kernel (f16 tiles kept by the library)",
+            "launch_ms": shadow["attn_ms"], "timed_ms": shadow["attn_timed_ms"],
+            "hbm_frac": rows_bytes / (shadow["attn_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS})
+    return res
 
 
 # ---------------------------------------------------------------------------------------
 # decode
 # ---------------------------------------------------------------------------------------
 
-def bench_decode(torch, attn, seq, steps, warmup, layers, dtype=0):
+def bench_decode(torch, attn, seq, steps, warmup, layers, dtype=0, one_launch=False):
     row = ROW if dtype == 0 else 144
     stride = seq
     gen = torch.Generator(device="cuda")
@@ -286,48 +417,57 @@ def bench_decode(torch, attn, seq, steps, warmup, layers, dtype=0):
     stepbuf = torch.tensor([seq - 1, seq, 0, 0, seq - 1, seq - 1, seq - 1, seq - 1],
                            dtype=torch.int32, device="cuda")
 
-    def one_pass():
-        for k, v in caches:
-            attn.attn_decode_kv(stepbuf, dtype, q, k, v, acc, ml, out, H, KV, HD, stride, SCALE, splits)
+    def plain(i):
+        k, v = caches[i % layers]
+        attn.attn_decode_kv(stepbuf, dtype, q, k, v, acc, ml, out, H, KV, HD, stride, SCALE, splits)
 
-    for _ in range(warmup):
-        one_pass()
-    with Timer(torch) as t:
-        for _ in range(steps):
-            one_pass()
-    us = t.ms * 1e3 / (steps * layers)
+    calls = steps * layers
+    ms, total, n = timed(torch, plain, calls, warmup * layers)
+    us = ms * 1e3
     # the same with the sigmoid output gate: in the merge kernel, and as the separate launch it replaces
     gate = torch.randn((H, HD), device="cuda", generator=gen)
-    for _ in range(warmup):
-        for k, v in caches:
-            attn.attn_decode_kv_gate(stepbuf, dtype, q, k, v, acc, ml, out, gate, H, KV, HD, stride, SCALE, splits)
-    with Timer(torch) as tg:
-        for _ in range(steps):
-            for k, v in caches:
-                attn.attn_decode_kv_gate(stepbuf, dtype, q, k, v, acc, ml, out, gate, H, KV, HD, stride, SCALE,
-                                         splits)
-    with Timer(torch) as ts:
-        for _ in range(steps):
-            for k, v in caches:
-                attn.attn_decode_kv(stepbuf, dtype, q, k, v, acc, ml, out, H, KV, HD, stride, SCALE, splits)
-                attn.q_gate(out, gate, out, H * HD)
+
+    def gated(i):
+        k, v = caches[i % layers]
+        attn.attn_decode_kv_gate(stepbuf, dtype, q, k, v, acc, ml, out, gate, H, KV, HD, stride, SCALE, splits)
+
+    def gate_apart(i):
+        plain(i)
+        attn.q_gate(out, gate, out, H * HD)
+
+    tg = timed(torch, gated, calls, layers)[0] * 1e3
+    ts = timed(torch, gate_apart, calls, layers)[0] * 1e3
+    # the form whose workgroups merge the key splits themselves (one launch instead of two; q8_0 only)
+    one_launch_us = None
+    if one_launch and dtype == 0:
+        before = attn.decode_one_launch(1)
+        try:
+            one_launch_us = timed(torch, plain, calls, layers)[0] * 1e3
+        finally:
+            attn.decode_one_launch(before)
     nbytes = decode_bytes(seq) * row // ROW
     gbs = nbytes / (us * 1e-6) / 1e9
     traffic = measured_traffic({8192: "decode8k", 32768: "decode32k"}.get(seq, "") if dtype == 0 else "",
-                               ["decode_q8_kernel", "decode_reduce_kernel"])
+                               ["decode_q8_kernel", "decode_reduce"])
+    # what a launch that only reads the same bytes reaches on this box, same rotation over the layer caches
+    ys = stream_yardstick(torch, attn, caches, KV * stride * row, steps)
     return {
         "workload": f"decode 1 query @ depth {seq}, {'q8_0' if dtype == 0 else 'q4_0'} cache, "
                     f"split-K {splits} + merge",
         "seq": seq, "splits": splits, "layers_rotated": layers,
         # (the scratch is sized for `splits`; over q8_0 one sequence runs at most one workgroup per CU)
         "splits_run": min(splits, max(256 // KV, 1)) if dtype == 0 else splits,
-        "us_per_layer": us,
-        "us_per_layer_gate_fused": tg.ms * 1e3 / (steps * layers),
-        "us_per_layer_gate_separate": ts.ms * 1e3 / (steps * layers),
+        "us_per_layer": us, "timed_ms": total, "steps_timed": n,
+        "us_per_layer_gate_fused": tg,
+        "us_per_layer_gate_separate": ts,
+        "us_per_layer_one_launch": one_launch_us,
+        "pure_read": ys,
         "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": gbs / HBM_PEAK_GBS, "traffic": traffic,
-                     "kernel": "decode_q8_kernel + decode_reduce_kernel",
-                     "bytes_per_launch": nbytes, "launch_us": us},
+                     "achievable": ys["achievable"], "frac_of_achievable": gbs / ys["achievable"],
+                     "kernel": "decode_q8_kernel + decode_reduce128_kernel" if dtype == 0 else
+                     "decode_staged_kernel + decode_reduce128_kernel",
+                     "bytes_per_launch": nbytes, "launch_us": us, "timed_ms": total, "steps_timed": n},
     }
 
 
@@ -380,31 +520,32 @@ def bench_batch(torch, attn, steps, warmup, layers):
     acc = torch.empty((rows, H, splits, HD), device="cuda")
     ml = torch.empty((rows, H, splits, 2), device="cuda")
 
-    def one_pass():
-        for k, v in caches:
-            attn.attn_decode_batch_cols(0, pos_d, q, k, v, acc, ml, out, H, KV, HD, stride, SCALE,
-                                        splits, slot_bytes, H * splits * HD, H * splits * 2, H * HD,
-                                        cols)
+    def one(i):
+        k, v = caches[i % layers]
+        attn.attn_decode_batch_cols(0, pos_d, q, k, v, acc, ml, out, H, KV, HD, stride, SCALE,
+                                    splits, slot_bytes, H * splits * HD, H * splits * 2, H * HD,
+                                    cols)
 
-    for _ in range(warmup):
-        one_pass()
-    with Timer(torch) as t:
-        for _ in range(steps):
-            one_pass()
-    us = t.ms * 1e3 / (steps * layers)
+    ms, total, n = timed(torch, one, steps * layers, warmup * layers)
+    us = ms * 1e3
     live = sum(d + c for d, c in zip(depths, cols))
     nbytes = decode_bytes(live)
     gbs = nbytes / (us * 1e-6) / 1e9
-    traffic = measured_traffic("batch16", ["decode_q8_kernel", "decode_reduce_kernel"])
+    traffic = measured_traffic("batch16", ["decode_q8_kernel", "decode_reduce"])
+    # the pure read of as many bytes (the first half of them from each of a layer's two arrays)
+    flat = [(k.reshape(-1), v.reshape(-1)) for k, v in caches]
+    ys = stream_yardstick(torch, attn, flat, int(nbytes) // 2, steps)
     return {
         "workload": f"batched decode, {slots} slots, depths U[512,16384] (seeded), "
                     f"slots 0..3 carry 3 query rows (MTP verify), one launch",
         "slots": slots, "rows": rows, "live_rows": live, "splits": splits, "layers_rotated": layers,
-        "us_per_layer": us,
+        "us_per_layer": us, "timed_ms": total, "steps_timed": n,
+        "pure_read": ys,
         "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": gbs / HBM_PEAK_GBS, "traffic": traffic,
-                     "kernel": "decode_q8_kernel + decode_reduce_kernel",
-                     "bytes_per_launch": nbytes, "launch_us": us},
+                     "achievable": ys["achievable"], "frac_of_achievable": gbs / ys["achievable"],
+                     "kernel": "decode_q8_kernel + decode_reduce128_kernel",
+                     "bytes_per_launch": nbytes, "launch_us": us, "timed_ms": total, "steps_timed": n},
     }
 
 
@@ -436,21 +577,17 @@ def bench_batch_layer(torch, attn, steps, layers):
     y = torch.empty((slots, m), device="cuda")
     attn.rope_table(THETA, NROT, stride + 64)
 
-    def one_pass():
-        for kv, w in zip(kvs, ws):
-            kv.front_append(qg, kx, vx, q, gate, qw, kw, NROT, THETA, 1e-6, pos)
-            kv.decode(pos, q, out, SCALE, gate=gate)
-            attn.gemv_q8_0_rows(w, out, y, m, k, slots)
+    def one(i):
+        kv, w = kvs[i % layers], ws[i % layers]
+        kv.front_append(qg, kx, vx, q, gate, qw, kw, NROT, THETA, 1e-6, pos)
+        kv.decode(pos, q, out, SCALE, gate=gate)
+        attn.gemv_q8_0_rows(w, out, y, m, k, slots)
 
-    for _ in range(3):
-        one_pass()
-    with Timer(torch) as t:
-        for _ in range(steps):
-            one_pass()
+    ms, total, n = timed(torch, one, steps * layers, 3 * layers)
     return {"workload": f"batched step, {slots} sequences at depths U[512,16384] (seeded), one row each: front "
-                        f"end with append + attention with gate + W_o, {layers} layers per pass (4 launches "
+                        f"end with append + attention with gate + W_o, {layers} layers rotated (4 launches "
                         f"per layer)",
-            "us_per_layer": t.ms * 1e3 / (steps * layers), "live_rows": sum(depths) + slots}
+            "us_per_layer": ms * 1e3, "timed_ms": total, "steps_timed": n, "live_rows": sum(depths) + slots}
 
 
 def bench_front(torch, attn, tokens, steps):
@@ -465,16 +602,13 @@ def bench_front(torch, attn, tokens, steps):
     q = torch.empty((tokens, H, HD), device="cuda")
     gate = torch.empty((tokens, H, HD), device="cuda")
     attn.rope_table(THETA, NROT, max(tokens, 1024))
-    for _ in range(3):
-        attn.chunk_front(qg, k, q, gate, qw, kw, H, KV, HD, NROT, THETA, 1e-6, 0, tokens)
-    with Timer(torch) as t:
-        for _ in range(steps):
-            attn.chunk_front(qg, k, q, gate, qw, kw, H, KV, HD, NROT, THETA, 1e-6, 0, tokens)
-    us = t.ms * 1e3 / steps
+    ms, total, n = timed(torch, lambda i: attn.chunk_front(qg, k, q, gate, qw, kw, H, KV, HD, NROT, THETA, 1e-6, 0,
+                                                            tokens), steps)
+    us = ms * 1e3
     nbytes = tokens * (H * 2 * HD + 2 * H * HD + 2 * KV * HD) * 4  # qg read, q + gate written, k both
     gbs = nbytes / (us * 1e-6) / 1e9
     return {"workload": f"attention front end, {tokens} rows: q|gate split + head RMS norm + RoPE",
-            "us": us, "bytes": nbytes,
+            "us": us, "bytes": nbytes, "timed_ms": total, "steps_timed": n,
             "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": gbs / HBM_PEAK_GBS, "traffic": None, "kernel": "front_kernel"}}
 
@@ -534,20 +668,14 @@ def bench_decode_layer(torch, attn, seq, steps, layers):
         one_pass()
         one_pass(False)
         graph.replay()
-    with Timer(torch) as te:
-        for _ in range(steps):
-            one_pass()
-    with Timer(torch) as ts:
-        for _ in range(steps):
-            one_pass(False)
-    with Timer(torch) as tg:
-        for _ in range(steps):
-            graph.replay()
+    te, total, n = timed(torch, lambda i: one_pass(), steps, 0)
+    ts = timed(torch, lambda i: one_pass(False), steps, 0)[0]
+    tg = timed(torch, lambda i: graph.replay(), steps, 0)[0]
     return {"workload": f"decode token @ depth {seq}: front end with append + attention with gate + W_o, "
                         f"{layers} layers per pass (4 launches per layer)",
-            "us_per_layer_eager": te.ms * 1e3 / (steps * layers),
-            "us_per_layer_graph_replay": tg.ms * 1e3 / (steps * layers),
-            "us_per_layer_eager_front_and_append_apart": ts.ms * 1e3 / (steps * layers)}
+            "us_per_layer_eager": te * 1e3 / layers, "timed_ms": total, "steps_timed": n * layers,
+            "us_per_layer_graph_replay": tg * 1e3 / layers,
+            "us_per_layer_eager_front_and_append_apart": ts * 1e3 / layers}
 
 
 def bench_chunk_layer(torch, attn, tokens, pos0, steps, layers):
@@ -600,12 +728,10 @@ def bench_chunk_layer(torch, attn, tokens, pos0, steps, layers):
 
     res = {}
     for name, fn in (("us_per_layer", fused), ("us_per_layer_separate_calls", apart)):
-        for i in range(3):
-            fn(i)
-        with Timer(torch) as t:
-            for i in range(steps):
-                fn(i)
-        res[name] = t.ms * 1e3 / steps
+        ms, total, n = timed(torch, fn, steps)
+        res[name] = ms * 1e3
+        if name == "us_per_layer":
+            res["timed_ms"], res["steps_timed"] = total, n
     return {"workload": f"chunk {tokens}@{pos0} through front end with append + gated attention (f16 rows) "
                         f"+ W_o GEMM, {layers} layers rotated (4 launches per layer)", **res,
             "tok_per_s": tokens / (res["us_per_layer"] * 1e-6)}
@@ -627,26 +753,23 @@ def bench_gemv(torch, attn, rows, steps, layers, m=5120, k=6144):
     ws = [random_q8_0_weights(torch, m, k, gen) for _ in range(layers)]
     x = torch.randn((rows, k), device="cuda", generator=gen) * 0.5
     y = torch.empty((rows, m), device="cuda")
-    for w in ws:
-        attn.gemv_q8_0_rows(w, x, y, m, k, rows)
-    with Timer(torch) as t:
-        for _ in range(steps):
-            for w in ws:
-                attn.gemv_q8_0_rows(w, x, y, m, k, rows)
-    us = t.ms * 1e3 / (steps * layers)
+    ms, total, n = timed(torch, lambda i: attn.gemv_q8_0_rows(ws[i % layers], x, y, m, k, rows), steps * layers, layers)
+    us = ms * 1e3
     # algorithmic bytes: the weights once, however many passes the kernel makes over them
     nbytes = m * (k // 32) * 34
     gbs = nbytes / (us * 1e-6) / 1e9
     return {"workload": f"W_o projection, Q8_0 {m}x{k}, {rows} activation rows",
-            "us_per_layer": us, "weight_bytes": m * (k // 32) * 34, "layers_rotated": layers,
+            "us_per_layer": us, "timed_ms": total, "steps_timed": n, "weight_bytes": m * (k // 32) * 34,
+            "layers_rotated": layers,
             "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": gbs / HBM_PEAK_GBS,
-                         "traffic": measured_traffic("gemv1" if rows == 1 else "", ["gemv_q8_rows_kernel"]),
+                         "traffic": measured_traffic({1: "gemv1", 24: "gemv24"}.get(rows, ""),
+                                                     ["gemv_q8_rows_kernel", "gemv_q8_tile_kernel"]),
                          "kernel": "gemv_q8_rows_kernel" if rows <= 2 else "gemv_q8_tile_kernel",
                          "bytes_per_launch": nbytes, "launch_us": us}}
 
 
-def bench_gemm(torch, attn, tokens, steps, layers, m=5120, k=6144):
+def bench_gemm(torch, attn, tokens, steps, layers, m=5120, k=6144, mfma=None):
     """Output side of a prefill chunk: y = W_o (out * sigmoid(gate)), [tokens][6144] x W_o^T (Q8_0) on
     MFMA with f16 operands."""
     gen = torch.Generator(device="cuda")
@@ -656,28 +779,23 @@ def bench_gemm(torch, attn, tokens, steps, layers, m=5120, k=6144):
     y = torch.empty((tokens, m), device="cuda")
     gate = torch.randn((tokens, k), device="cuda", generator=gen)
     x16 = torch.empty((tokens, k), dtype=torch.float16, device="cuda")
-    for w in ws:
-        attn.gemm_q8_0_f16(w, x, y, m, k, tokens)
-        attn.output_chunk_q8_0(w, x, gate, y, m, k, tokens, x16)
-    with Timer(torch) as t32:
-        for _ in range(steps):
-            for w in ws:
-                attn.gemm_q8_0_f16(w, x, y, m, k, tokens)
+    t32 = timed(torch, lambda i: attn.gemm_q8_0_f16(ws[i % layers], x, y, m, k, tokens), steps * layers, layers)[0]
     # the whole output side: gate + rounding to f16 in one pass, then the GEMM over f16 rows
-    with Timer(torch) as t:
-        for _ in range(steps):
-            for w in ws:
-                attn.output_chunk_q8_0(w, x, gate, y, m, k, tokens, x16)
-    us = t.ms * 1e3 / (steps * layers)
+    ms, total, n = timed(torch, lambda i: attn.output_chunk_q8_0(ws[i % layers], x, gate, y, m, k, tokens, x16),
+                         steps * layers, layers)
+    us = ms * 1e3
     flop = 2.0 * tokens * m * k
     tf = flop / (us * 1e-6) / 1e12
+    wl = "gemm672" if tokens == 672 else ""
     return {"workload": f"W_o projection of a chunk, Q8_0 {m}x{k}, {tokens} tokens",
-            "us_per_layer": us, "us_per_layer_f32_rows_no_gate": t32.ms * 1e3 / (steps * layers),
+            "us_per_layer": us, "timed_ms": total, "steps_timed": n, "us_per_layer_f32_rows_no_gate": t32 * 1e3,
             "flop": flop, "layers_rotated": layers,
             "roofline": {"bound": "mfma", "achieved": tf, "peak": MFMA_F16_PEAK_TF, "unit": "TFLOP/s",
                          "frac": tf / MFMA_F16_PEAK_TF,
-                         "traffic": measured_traffic("gemm672" if tokens == 672 else "",
-                                                     ["gate_f16_kernel", "gemm_q8_f16_kernel<true>"]),
+                         "achievable": None if mfma is None else mfma["tflops"],
+                         "frac_of_achievable": None if mfma is None else tf / mfma["tflops"],
+                         **counters(wl, "gemm_q8_f16_kernel<true"),
+                         "traffic": measured_traffic(wl, ["gate_f16_kernel", "gemm_q8_f16_kernel<true"]),
                          "kernel": "gate_f16_kernel + gemm_q8_f16_kernel",
                          "flop_per_launch": flop, "launch_us": us}}
 
@@ -688,11 +806,9 @@ def bench_copycal(torch, steps):
     n = 64 << 20
     a = torch.empty(n, dtype=torch.uint8, device="cuda")
     b = torch.ones(n, dtype=torch.uint8, device="cuda")
-    with Timer(torch) as t:
-        for _ in range(steps):
-            a.copy_(b)
+    ms, total, cnt = timed(torch, lambda i: a.copy_(b), steps)
     return {"workload": "device copy", "bytes_read": n, "bytes_written": n,
-            "us_per_copy": t.ms * 1e3 / steps}
+            "us_per_copy": ms * 1e3, "timed_ms": total, "steps_timed": cnt}
 
 
 # ---------------------------------------------------------------------------------------
@@ -745,11 +861,12 @@ def cpu_decode(orc, seq):
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--steps", type=int, default=200,
+                    help="steps of the headline workload to time at least (more are timed until 200 ms are full)")
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--main-only", action="store_true", help="skip the 'also' workloads")
     ap.add_argument("--only", default="", help="run one workload alone (prefill672, decode8k, "
-                    "decode32k, decode128k, chunk100k, batch16, front672, decode32k_q4, gemv1, gemv4, gemv16, gemm672, gemm2048, layer32k, layer672, blayer16, copycal) for profiling; prints its object")
+                    "decode32k, decode128k, chunk100k, batch16, mfma, front672, decode32k_q4, gemv1, gemv4, gemv16, gemm672, gemm2048, layer32k, layer672, blayer16, copycal) for profiling; prints its object")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -767,40 +884,46 @@ def main() -> int:
     attn.init(0)
     K, W = args.steps, args.warmup
 
+    # (--steps is a lower bound on what every figure is averaged over; figures that would be timed for less
+    # than MIN_TIMED_MS at that count repeat until they have been)
     if args.only:
+        mf = lambda: mfma_yardstick(torch, attn)
         fn = {
-            "prefill672": lambda: bench_prefill(torch, attn, 672, 0, K, W, LAYERS),
+            "prefill672": lambda: bench_prefill(torch, attn, 672, 0, K, W, LAYERS, mfma=mf()),
             "decode8k": lambda: bench_decode(torch, attn, 8192, K, W, LAYERS),
-            "decode32k": lambda: bench_decode(torch, attn, 32768, K, W, LAYERS),
+            "decode32k": lambda: bench_decode(torch, attn, 32768, K, W, LAYERS, one_launch=True),
             "decode128k": lambda: bench_decode(torch, attn, 131072, K, W, LAYERS),
-            "chunk100k": lambda: bench_prefill(torch, attn, 2048, 100_000, max(K, 10), W, 2),
+            "chunk100k": lambda: bench_prefill(torch, attn, 2048, 100_000, K, W, 2, mfma=mf()),
             "batch16": lambda: bench_batch(torch, attn, K, W, 4),
             "copycal": lambda: bench_copycal(torch, K),
-            "front672": lambda: bench_front(torch, attn, 672, max(K, 20)),
-            "decode32k_q4": lambda: bench_decode(torch, attn, 32768, max(K, 20), 3, LAYERS, 1),
-            "gemv1": lambda: bench_gemv(torch, attn, 1, max(K // 4, 10), LAYERS),
-            "gemv4": lambda: bench_gemv(torch, attn, 4, max(K // 4, 10), LAYERS),
-            "gemv16": lambda: bench_gemv(torch, attn, 16, max(K // 4, 10), LAYERS),
-            "gemv24": lambda: bench_gemv(torch, attn, 24, max(K // 4, 10), LAYERS),
-            "gemv64": lambda: bench_gemv(torch, attn, 64, max(K // 4, 10), LAYERS),
-            "gemv128": lambda: bench_gemv(torch, attn, 128, max(K // 4, 10), LAYERS),
-            "gemm24": lambda: bench_gemm(torch, attn, 24, max(K // 4, 10), LAYERS),
-            "gemm128": lambda: bench_gemm(torch, attn, 128, max(K // 4, 10), LAYERS),
-            "layer32k": lambda: bench_decode_layer(torch, attn, 32768, max(K // 4, 10), LAYERS),
-            "blayer16": lambda: bench_batch_layer(torch, attn, max(K // 10, 10), 4),
-            "layer672": lambda: bench_chunk_layer(torch, attn, 672, 0, max(K // 10, 10), 4),
-            "gemm672": lambda: bench_gemm(torch, attn, 672, max(K // 10, 10), 4),
-            "gemm2048": lambda: bench_gemm(torch, attn, 2048, max(K // 20, 10), 4),
+            "mfma": mf,
+            "front672": lambda: bench_front(torch, attn, 672, K),
+            "decode32k_q4": lambda: bench_decode(torch, attn, 32768, K, 3, LAYERS, 1),
+            "gemv1": lambda: bench_gemv(torch, attn, 1, K, LAYERS),
+            "gemv4": lambda: bench_gemv(torch, attn, 4, K, LAYERS),
+            "gemv16": lambda: bench_gemv(torch, attn, 16, K, LAYERS),
+            "gemv24": lambda: bench_gemv(torch, attn, 24, K, LAYERS),
+            "gemv64": lambda: bench_gemv(torch, attn, 64, K, LAYERS),
+            "gemv128": lambda: bench_gemv(torch, attn, 128, K, LAYERS),
+            "gemm24": lambda: bench_gemm(torch, attn, 24, K, LAYERS),
+            "gemm128": lambda: bench_gemm(torch, attn, 128, K, LAYERS),
+            "layer32k": lambda: bench_decode_layer(torch, attn, 32768, K, LAYERS),
+            "blayer16": lambda: bench_batch_layer(torch, attn, K, 4),
+            "layer672": lambda: bench_chunk_layer(torch, attn, 672, 0, K, 4),
+            "gemm672": lambda: bench_gemm(torch, attn, 672, K, 4, mfma=mf()),
+            "gemm2048": lambda: bench_gemm(torch, attn, 2048, K, 4, mfma=mf()),
         }[args.only]
         print(json.dumps(fn()))
         return 0
 
-    main_r = bench_prefill(torch, attn, 672, 0, K, W, LAYERS)
+    mfma = mfma_yardstick(torch, attn)
+    main_r = bench_prefill(torch, attn, 672, 0, K, W, LAYERS, mfma=mfma)
     line = {
         "metric": "prefill_attn_tok_per_s",
         "value": main_r["tok_per_s"],
         "unit": "tok/s",
         "n_gpus": 1, "steps": K, "warmup": W,
+        "steps_timed": main_r["steps_timed"], "timed_ms": main_r["timed_ms"],
         "ms_per_step": main_r["ms_per_step"],
         "higher_is_better": True,
         "scaling": "weak",
@@ -816,34 +939,34 @@ def main() -> int:
 
     if not args.main_only:
         also = {}
-        d_steps = max(K // 4, 10)
-        also["decode_8192"] = bench_decode(torch, attn, 8192, d_steps, max(W // 4, 2), LAYERS)
+        d_steps = 1  # passes over the 16 layer caches: the 200 ms rule sets the count
+        also["mfma_32x32x16_f16"] = mfma
+        also["decode_8192"] = bench_decode(torch, attn, 8192, d_steps, 2, LAYERS)
         torch.cuda.empty_cache()
-        also["decode_32768"] = bench_decode(torch, attn, 32768, d_steps, max(W // 4, 2), LAYERS)
+        also["decode_32768"] = bench_decode(torch, attn, 32768, d_steps, 2, LAYERS, one_launch=True)
         torch.cuda.empty_cache()
         # beyond the two benchmark depths: shows what the same kernel does once launch and ramp-up
         # stop dominating (285 MB per layer)
-        also["decode_131072"] = bench_decode(torch, attn, 131072, max(d_steps // 4, 10), 2, LAYERS)
+        also["decode_131072"] = bench_decode(torch, attn, 131072, d_steps, 2, LAYERS)
         torch.cuda.empty_cache()
-        also["chunk_2048_at_100000"] = bench_prefill(torch, attn, 2048, 100_000,
-                                                     max(K // 20, 10), 2, 2)
+        also["chunk_2048_at_100000"] = bench_prefill(torch, attn, 2048, 100_000, 10, 2, 2, mfma=mfma)
         torch.cuda.empty_cache()
-        also["front_672"] = bench_front(torch, attn, 672, d_steps)
-        also["decode_32768_q4_0"] = bench_decode(torch, attn, 32768, d_steps, max(W // 4, 2), LAYERS, 1)
-        also["batch16_mtp"] = bench_batch(torch, attn, d_steps, max(W // 4, 2), 4)
+        also["front_672"] = bench_front(torch, attn, 672, 20)
+        also["decode_32768_q4_0"] = bench_decode(torch, attn, 32768, d_steps, 2, LAYERS, 1)
+        also["batch16_mtp"] = bench_batch(torch, attn, d_steps, 2, 4)
         torch.cuda.empty_cache()
         # the step after the path: output projection over Q8_0 weights (decode rows, then a chunk)
         also["wo_rows_1"] = bench_gemv(torch, attn, 1, d_steps, LAYERS)
         also["wo_rows_4"] = bench_gemv(torch, attn, 4, d_steps, LAYERS)
         also["wo_rows_24"] = bench_gemv(torch, attn, 24, d_steps, LAYERS)  # the batch of 16 slots with 4 verify groups
         torch.cuda.empty_cache()
-        also["wo_chunk_672"] = bench_gemm(torch, attn, 672, max(K // 20, 10), 4)
+        also["wo_chunk_672"] = bench_gemm(torch, attn, 672, 10, 4, mfma=mfma)
         torch.cuda.empty_cache()
         also["decode_layer_32768"] = bench_decode_layer(torch, attn, 32768, d_steps, LAYERS)
         torch.cuda.empty_cache()
-        also["chunk_layer_672"] = bench_chunk_layer(torch, attn, 672, 0, max(K // 10, 10), 4)
+        also["chunk_layer_672"] = bench_chunk_layer(torch, attn, 672, 0, 10, 4)
         torch.cuda.empty_cache()
-        also["batch_layer_16"] = bench_batch_layer(torch, attn, max(K // 10, 10), 4)
+        also["batch_layer_16"] = bench_batch_layer(torch, attn, d_steps, 4)
         torch.cuda.empty_cache()
         line["also"] = also
 

@@ -46,6 +46,8 @@ EXPORTS = [
     "hipml_attn_front_rows_f32", "hipml_attn_front_rows_encode_f32",
     "hipml_attn_decode_kv_noalloc", "hipml_rope_allow_device_angles",
     "hipml_attn_decode_one_launch",
+    "hipml_bench_stream_read", "hipml_bench_mfma_f16",
+    "hipml_kv_f16_attach", "hipml_kv_f16_detach",
 ]
 
 
@@ -103,6 +105,10 @@ def lib() -> C.CDLL:
             "hipml_attn_decode_kv_noalloc": (i, [vp, vp, i, vp, vp, vp, vp, i, i, i, i, f, i, sz, sz]),
             "hipml_rope_allow_device_angles": (i, [i]),
             "hipml_attn_decode_one_launch": (i, [i]),
+            "hipml_kv_f16_attach": (i, [vp, i, vp, vp, vp, i, i, i, i]),
+            "hipml_kv_f16_detach": (i, [vp]),
+            "hipml_bench_stream_read": (i, [vp, vp, vp, sz, i, vp]),
+            "hipml_bench_mfma_f16": (i, [vp, i, i, vp, vp]),
             "hipml_attn_decode_batch_cols_gate": (i, [vp, i, vp, vp, vp, vp, vp, vp, vp, vp, i, i, i,
                                                       i, f, i, sz, sz, sz, sz, i, vp]),
             "hipml_attn_chunk_q8_split": (i, [vp, vp, vp, vp, vp, i, i, i, i, i, i, i, vp, vp, i]),
@@ -386,6 +392,27 @@ def attn_decode_kv_noalloc(step, dtype, q, k, v, out, n_heads, n_kv, head_dim, s
                                               k_off, v_off))
 
 
+def kv_f16_attach(dtype, k_cache, v_cache, kv_f16, n_kv, head_dim, stride, rows=0, stream=None):
+    """Register kv_f16 as the f16 shadow of (k_cache, v_cache): the library keeps it current through its own
+    append entry points and the chunk attention over the cache reads it.  Detach before freeing either."""
+    _check(lib().hipml_kv_f16_attach(_stream(stream), dtype, _p(k_cache), _p(v_cache), _p(kv_f16), n_kv, head_dim,
+                                     stride, rows))
+
+
+def kv_f16_detach(k_cache):
+    _check(lib().hipml_kv_f16_detach(_p(k_cache)))
+
+
+def bench_stream_read(a, b, bytes_each, mode, sink, stream=None):
+    """Measurement only: one launch that reads `bytes_each` bytes of each of a and b in the decode kernel's pattern."""
+    _check(lib().hipml_bench_stream_read(_stream(stream), _p(a), _p(b), bytes_each, mode, _p(sink)))
+
+
+def bench_mfma_f16(workgroups, iters, sink, clocks=None, stream=None):
+    """Measurement only: workgroups x 4 waves x iters x 8 independent 32x32x16 f16 MFMAs."""
+    _check(lib().hipml_bench_mfma_f16(_stream(stream), workgroups, iters, _p(sink), _p(clocks)))
+
+
 def decode_one_launch(on: int = -1) -> int:
     """Process-wide: 1 = a single sequence over q8_0 merges its key splits inside the one launch, 0 (the
     default) = in a second launch; a negative value only reads the mode.  Returns the mode before the call."""
@@ -521,7 +548,8 @@ class DeepKv:
                                     dtype=torch.float32, device=device)
         self.part_ml = torch.empty((max_cols, n_heads, self.max_splits, 2), dtype=torch.float32,
                                    device=device)
-        self.f16 = None  # the optional f16 copy of the rows (enable_f16_copy)
+        self.f16 = None  # the optional f16 copy of the rows (enable_f16_copy, attach_f16)
+        self._attached = False
 
     def enable_f16_copy(self, live: int = 0, stream=None):
         """Keep an f16 copy of this cache for chunk prefill over long prefixes (chunk_attention_kv_f16
@@ -529,6 +557,25 @@ class DeepKv:
         if self.f16 is None:
             self.f16 = kv_f16_alloc(self.seq, self.n_kv, self.k.device)
         self.sync_f16(0, live, stream)
+
+    def attach_f16(self, live: int = 0, stream=None):
+        """Hand the f16 copy to the library (hipml_kv_f16_attach): appends through the library keep it current
+        and `chunk_attention_q8_split*` over this cache reads it; no sync_f16 calls are needed."""
+        if self.f16 is None:
+            self.f16 = kv_f16_alloc(self.seq, self.n_kv, self.k.device)
+        kv_f16_attach(self.dtype, self.k, self.v, self.f16, self.n_kv, self.head_dim, self.seq, live, stream)
+        self._attached = True
+
+    def detach_f16(self):
+        if self._attached:
+            self._attached = False
+            kv_f16_detach(self.k)
+
+    def __del__(self):
+        try:
+            self.detach_f16()
+        except Exception:  # (interpreter shutdown: the library may be gone)
+            pass
 
     def sync_f16(self, start: int, rows: int, stream=None):
         """After rows [start, start + rows) were appended (or restored): bring the copy up to date."""

@@ -22,6 +22,7 @@ SOURCES = [
     ("decode.hip", []),
     ("prefill.hip", []),
     ("proj.hip", []),
+    ("yardstick.hip", []),
     ("api.cpp", ["-x", "hip"]),
 ]
 

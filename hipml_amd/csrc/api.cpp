@@ -132,6 +132,85 @@ static int check_aligned16(const void *p, const char *name)
             return fail(HIPML_ATTN_E_NULL, "%s is NULL", #p);                                        \
     } while (0)
 
+// ---- f16 shadows of caches ------------------------------------------------------------------------
+// A cache registered with hipml_kv_f16_attach has an f16 tile copy that this library keeps: every entry
+// point that writes rows of the cache at positions the host knows converts those rows right behind its own
+// launch, the ones whose positions live in device memory mark the shadow stale (the next chunk attention
+// over the cache then converts every live row once), and the chunk attention over the cache reads the
+// tiles instead of making them per call.  The bookkeeping is host state, updated when a call is issued
+// (or captured), not when a captured graph is replayed.
+struct KvShadow {
+    const uint8_t *kc, *vc;
+    void *copy;
+    int n_kv, stride, q4;
+    int valid;  // rows [0, valid) of the copy match the cache
+    bool stale; // rows were written at positions only the device knows
+};
+constexpr int kMaxShadows = 1024;
+static std::mutex g_shadow_mu;
+static KvShadow g_shadows[kMaxShadows];
+static int g_nshadows = 0;
+
+static int shadow_index(const void *kc) // (lock held)
+{
+    for (int i = 0; i < g_nshadows; i++)
+        if (g_shadows[i].kc == kc)
+            return i;
+    return -1;
+}
+
+// Rows [start, start + rows) of the cache at kc have been written by a launch already issued on st.
+static int shadow_rows_written(hipStream_t st, const void *kc, int start, int rows)
+{
+    if (rows <= 0)
+        return 0;
+    KvShadow sh;
+    {
+        std::lock_guard<std::mutex> lock(g_shadow_mu);
+        const int i = shadow_index(kc);
+        if (i < 0)
+            return 0;
+        sh = g_shadows[i];
+        if (sh.stale || start > sh.valid)
+            return 0; // (the chunk attention converts from `valid` on, or everything, when it needs the rows)
+        g_shadows[i].valid = sh.valid > start + rows ? sh.valid : start + rows;
+    }
+    return launch_kv_f16_rows(st, sh.kc, sh.vc, sh.copy, sh.n_kv, sh.stride, start, rows, sh.q4);
+}
+
+// Rows of the caches inside [base, base + bytes) have been written at positions only the device knows.
+static void shadow_rows_unknown(const void *base, size_t bytes)
+{
+    std::lock_guard<std::mutex> lock(g_shadow_mu);
+    const uint8_t *lo = static_cast<const uint8_t *>(base);
+    for (int i = 0; i < g_nshadows; i++)
+        if (g_shadows[i].kc >= lo && g_shadows[i].kc < lo + (bytes > 0 ? bytes : 1))
+            g_shadows[i].stale = true;
+}
+
+// The shadow the chunk attention over (kc, vc) may read for rows [0, need), brought up to date on st;
+// false: there is none (or it belongs to another geometry).
+static bool shadow_for_chunk(hipStream_t st, const void *kc, const void *vc, int n_kv, int stride, int q4, int need,
+                             const void **copy, int *rc)
+{
+    KvShadow sh;
+    int from;
+    {
+        std::lock_guard<std::mutex> lock(g_shadow_mu);
+        const int i = shadow_index(kc);
+        if (i < 0 || g_shadows[i].vc != vc || g_shadows[i].n_kv != n_kv || g_shadows[i].stride != stride ||
+            g_shadows[i].q4 != q4)
+            return false;
+        sh = g_shadows[i];
+        from = sh.stale ? 0 : (sh.valid < need ? sh.valid : need);
+        g_shadows[i].stale = false;
+        g_shadows[i].valid = sh.stale || sh.valid < need ? need : sh.valid;
+    }
+    *copy = sh.copy;
+    *rc = from < need ? launch_kv_f16_rows(st, sh.kc, sh.vc, sh.copy, sh.n_kv, sh.stride, from, need - from, sh.q4) : 0;
+    return true;
+}
+
 static int decode_common(hipStream_t st, int dtype, const int32_t *pos, const float *q, const void *k,
                          const void *v, float *part_acc, float *part_ml, float *out, int n_heads,
                          int n_kv, int head_dim, int stride, float scale, int splits,
@@ -236,6 +315,8 @@ int hipml_attn_init(int device)
         rc = prefill_init();
     if (rc == 0)
         rc = proj_init();
+    if (rc == 0)
+        rc = yardstick_init();
     if (before != device)
         (void)hipSetDevice(before);
     if (rc)
@@ -598,6 +679,7 @@ int hipml_attn_front_encode_f32(hipml_stream_t stream, const int32_t *step, int 
         return rc;
     if (s0 < 0 || s1 < 0 || s2 < 0 || s3 < 0)
         return fail(HIPML_ATTN_E_RANGE, "negative M-RoPE section");
+    shadow_rows_unknown(k_cache, 1);
     return launch_front(as_stream(stream), qg, q, gate, k, q_norm, k_norm, n_heads, n_kv, n_rot, s0, s1,
                         s2, s3, step + 4, 0, 1, theta_base, eps, g_rope, dtype, v,
                         static_cast<uint8_t *>(k_cache), static_cast<uint8_t *>(v_cache), step, 0, stride);
@@ -624,10 +706,11 @@ int hipml_attn_chunk_front_encode_f32(hipml_stream_t stream, int dtype, const fl
                     pos0 + tokens, stride);
     if (tokens == 0)
         return 0;
-    return launch_front(as_stream(stream), qg, q, gate, k, q_norm, k_norm, n_heads, n_kv, n_rot, 0, 0, 0,
-                        0, nullptr, pos0, tokens, theta_base, eps, g_rope, dtype, v,
-                        static_cast<uint8_t *>(k_cache), static_cast<uint8_t *>(v_cache), nullptr, pos0,
-                        stride);
+    rc = launch_front(as_stream(stream), qg, q, gate, k, q_norm, k_norm, n_heads, n_kv, n_rot, 0, 0, 0,
+                      0, nullptr, pos0, tokens, theta_base, eps, g_rope, dtype, v,
+                      static_cast<uint8_t *>(k_cache), static_cast<uint8_t *>(v_cache), nullptr, pos0,
+                      stride);
+    return rc ? rc : shadow_rows_written(as_stream(stream), k_cache, pos0, tokens);
 }
 
 // The batched engine's front end: row r belongs to sequence r and rotates at text position pos[2 r].
@@ -669,6 +752,7 @@ int hipml_attn_front_rows_encode_f32(hipml_stream_t stream, int dtype, const flo
         return fail(HIPML_ATTN_E_RANGE, "slots %d is negative", slots);
     if (slots == 0)
         return 0;
+    shadow_rows_unknown(k_cache, slot_bytes * (size_t)slots);
     return launch_front(as_stream(stream), qg, q, gate, k, q_norm, k_norm, n_heads, n_kv, n_rot, 0, 0, 0,
                         0, nullptr, 0, slots, theta_base, eps, g_rope, dtype, v,
                         static_cast<uint8_t *>(k_cache), static_cast<uint8_t *>(v_cache), nullptr, 0, stride,
@@ -684,6 +768,7 @@ int hipml_kv_encode(hipml_stream_t stream, const int32_t *step, int dtype, const
     int rc = check_encode(dtype, k_in, v_in, k_cache, v_cache, n_kv, head_dim, stride);
     if (rc)
         return rc;
+    shadow_rows_unknown(k_cache, 1);
     return launch_kv_encode(as_stream(stream), dtype, k_in, v_in, static_cast<uint8_t *>(k_cache),
                                static_cast<uint8_t *>(v_cache), n_kv, head_dim, stride, step, 0, 0,
                                1, 0, 0, 1);
@@ -703,9 +788,10 @@ int hipml_kv_encode_bulk(hipml_stream_t stream, int dtype, const float *k_f32, c
     if ((long long)start + rows > stride)
         return fail(HIPML_ATTN_E_RANGE, "rows [%d, %d) do not fit a cache of %d rows per head",
                     start, start + rows, stride);
-    return launch_kv_encode(as_stream(stream), dtype, k_f32, v_f32, static_cast<uint8_t *>(k_cache),
-                               static_cast<uint8_t *>(v_cache), n_kv, head_dim, stride, nullptr, 0,
-                               0, rows, start, src0, rows);
+    rc = launch_kv_encode(as_stream(stream), dtype, k_f32, v_f32, static_cast<uint8_t *>(k_cache),
+                          static_cast<uint8_t *>(v_cache), n_kv, head_dim, stride, nullptr, 0,
+                          0, rows, start, src0, rows);
+    return rc ? rc : shadow_rows_written(as_stream(stream), k_cache, start, rows);
 }
 
 int hipml_rope_encode_chunk_f32(hipml_stream_t stream, float *q, float *k, const float *v, void *k_cache,
@@ -731,9 +817,10 @@ int hipml_rope_encode_chunk_f32(hipml_stream_t stream, float *q, float *k, const
                     pos0 + tokens, stride);
     if (tokens == 0)
         return 0;
-    return launch_rope_encode_chunk(as_stream(stream), dtype, q, k, v, static_cast<uint8_t *>(k_cache),
-                                    static_cast<uint8_t *>(v_cache), n_head, n_kv, n_rot, theta_base, pos0,
-                                    tokens, stride, g_rope);
+    rc = launch_rope_encode_chunk(as_stream(stream), dtype, q, k, v, static_cast<uint8_t *>(k_cache),
+                                  static_cast<uint8_t *>(v_cache), n_head, n_kv, n_rot, theta_base, pos0,
+                                  tokens, stride, g_rope);
+    return rc ? rc : shadow_rows_written(as_stream(stream), k_cache, pos0, tokens);
 }
 
 int hipml_kv_encode_rows(hipml_stream_t stream, int dtype, const float *k_f32, const float *v_f32,
@@ -747,6 +834,7 @@ int hipml_kv_encode_rows(hipml_stream_t stream, int dtype, const float *k_f32, c
         return rc;
     if (slots < 0)
         return fail(HIPML_ATTN_E_RANGE, "slots %d is negative", slots);
+    shadow_rows_unknown(k_cache, slot_bytes * (size_t)(slots > 0 ? slots : 0));
     return launch_kv_encode(as_stream(stream), dtype, k_f32, v_f32, static_cast<uint8_t *>(k_cache),
                                static_cast<uint8_t *>(v_cache), n_kv, head_dim, stride, pos, 2,
                                slot_bytes, slots, 0, 0, slots);
@@ -772,9 +860,10 @@ int hipml_kv_rows_copy(hipml_stream_t stream, int dtype, const void *k_src, cons
     if ((rc = check_aligned16(k_src, "k_src")) || (rc = check_aligned16(v_src, "v_src")) ||
         (rc = check_aligned16(k_dst, "k_dst")) || (rc = check_aligned16(v_dst, "v_dst")))
         return rc;
-    return launch_kv_rows_copy(as_stream(stream), dtype, static_cast<const uint8_t *>(k_src),
-                               static_cast<const uint8_t *>(v_src), static_cast<uint8_t *>(k_dst),
-                               static_cast<uint8_t *>(v_dst), n_kv, src_stride, dst_stride, rows);
+    rc = launch_kv_rows_copy(as_stream(stream), dtype, static_cast<const uint8_t *>(k_src),
+                             static_cast<const uint8_t *>(v_src), static_cast<uint8_t *>(k_dst),
+                             static_cast<uint8_t *>(v_dst), n_kv, src_stride, dst_stride, rows);
+    return rc ? rc : shadow_rows_written(as_stream(stream), k_dst, 0, rows);
 }
 
 // ---- decode ------------------------------------------------------------------------------------
@@ -981,6 +1070,19 @@ static int chunk_q8_common(hipml_stream_t stream, const float *q, const void *kc
         return 0;
     if ((rc = require_init()))
         return rc;
+    // a cache with a registered f16 shadow: the sliced attention reads its tiles (as many slices as the policy
+    // gives a chunk over such a copy, within what the scratch was sized for)
+    if (splits >= 2 && kv_f16 == nullptr && rope_tab == nullptr) {
+        const void *copy = nullptr;
+        if (shadow_for_chunk(as_stream(stream), kc, vc, n_kv, stride, dtype == 2 ? 1 : 0, pos0 + tokens, &copy, &rc)) {
+            if (rc)
+                return rc;
+            const int slices = hipml_attn_chunk_slices(pos0, tokens, n_kv);
+            kv_f16 = copy;
+            splits = slices < splits ? (slices < 1 ? 1 : slices) : splits;
+            dtype = 1; // (the tiles are f16 whatever the cache holds)
+        }
+    }
     return launch_chunk_q8(as_stream(stream), q, static_cast<const uint8_t *>(kc),
                            static_cast<const uint8_t *>(vc), out, n_head, n_kv, pos0, tokens,
                            stride, part_acc, part_ml, splits, want_gate ? gate : nullptr, dtype == 2 ? 1 : 0,
@@ -1083,6 +1185,36 @@ int hipml_kv_f16_rows(hipml_stream_t stream, int dtype, const void *k_cache, con
                               static_cast<const uint8_t *>(v_cache), kv_f16, n_kv, stride, start, rows, dtype);
 }
 
+int hipml_kv_f16_attach(hipml_stream_t stream, int dtype, const void *k_cache, const void *v_cache, void *kv_f16,
+                        int n_kv, int head_dim, int stride, int rows)
+{
+    // (the checks and the conversion of the rows the cache holds already)
+    int rc = hipml_kv_f16_rows(stream, dtype, k_cache, v_cache, kv_f16, n_kv, head_dim, stride, 0, rows);
+    if (rc)
+        return rc;
+    std::lock_guard<std::mutex> lock(g_shadow_mu);
+    int i = shadow_index(k_cache);
+    if (i < 0) {
+        if (g_nshadows == kMaxShadows)
+            return fail(HIPML_ATTN_E_RANGE, "%d caches have an f16 shadow already", kMaxShadows);
+        i = g_nshadows++;
+    }
+    g_shadows[i] = KvShadow{static_cast<const uint8_t *>(k_cache), static_cast<const uint8_t *>(v_cache), kv_f16,
+                            n_kv, stride, dtype, rows, false};
+    return 0;
+}
+
+int hipml_kv_f16_detach(const void *k_cache)
+{
+    clear_error();
+    std::lock_guard<std::mutex> lock(g_shadow_mu);
+    const int i = shadow_index(k_cache);
+    if (i < 0)
+        return fail(HIPML_ATTN_E_STATE, "no f16 shadow is registered for this cache");
+    g_shadows[i] = g_shadows[--g_nshadows];
+    return 0;
+}
+
 int hipml_attn_chunk_kv_f16(hipml_stream_t stream, const float *q, const void *kv_f16, const float *gate,
                             float *out, void *out16, int n_head, int n_kv, int head_dim, int pos0, int tokens,
                             int stride, float *part_acc, float *part_ml, int splits)
@@ -1174,6 +1306,41 @@ int hipml_attn_output_chunk_q8_0(hipml_stream_t stream, const void *wo, const fl
         return rc;
     return launch_gemm_q8_f16(as_stream(stream), static_cast<const uint8_t *>(wo), attn_out, gate, y, m, k,
                               tokens, x16);
+}
+
+// ---- measurement only --------------------------------------------------------------------------
+
+int hipml_bench_stream_read(hipml_stream_t stream, const void *a, const void *b, size_t bytes_each, int mode,
+                            void *sink)
+{
+    clear_error();
+    REQUIRE_PTR(a);
+    REQUIRE_PTR(b);
+    REQUIRE_PTR(sink);
+    if (mode != 0 && mode != 1)
+        return fail(HIPML_ATTN_E_RANGE, "mode %d: 0 (global memory to LDS) or 1 (register loads)", mode);
+    if (bytes_each == 0 || bytes_each % (32 * kRowBytes) != 0 || bytes_each / (32 * kRowBytes) > 0x7fffffffu)
+        return fail(HIPML_ATTN_E_RANGE, "bytes_each %zu must be a positive multiple of %d", bytes_each, 32 * kRowBytes);
+    int rc;
+    if ((rc = check_aligned16(a, "a")) || (rc = check_aligned16(b, "b")) || (rc = require_init()))
+        return rc;
+    return launch_bench_stream(as_stream(stream), static_cast<const uint8_t *>(a), static_cast<const uint8_t *>(b),
+                               bytes_each, mode, static_cast<uint32_t *>(sink));
+}
+
+int hipml_bench_mfma_f16(hipml_stream_t stream, int workgroups, int iters, void *sink, void *clocks)
+{
+    clear_error();
+    REQUIRE_PTR(sink);
+    if (workgroups < 1 || workgroups > (1 << 20) || iters < 1)
+        return fail(HIPML_ATTN_E_RANGE, "workgroups %d / iters %d out of range", workgroups, iters);
+    if (((uintptr_t)clocks & 7) != 0)
+        return fail(HIPML_ATTN_E_RANGE, "clocks must be 8-byte aligned");
+    int rc = require_init();
+    if (rc)
+        return rc;
+    return launch_bench_mfma(as_stream(stream), workgroups, iters, static_cast<float *>(sink),
+                             static_cast<unsigned long long *>(clocks));
 }
 
 } // extern "C"

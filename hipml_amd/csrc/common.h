@@ -135,4 +135,10 @@ int launch_gemm_q8_f16(hipStream_t st, const uint8_t *w, const float *x, const f
 // Raise the projection kernels' dynamic LDS limit (once per process; called by hipml_attn_init).
 int proj_init();
 
+// Measurement-only kernels (yardstick.hip): a pure read of two arrays in the decode kernel's access pattern
+// (mode 0: global_load_lds, 1: register loads), and a loop of independent MFMAs on one wave per SIMD.
+int yardstick_init();
+int launch_bench_stream(hipStream_t st, const uint8_t *a, const uint8_t *b, size_t bytes_each, int mode, uint32_t *sink);
+int launch_bench_mfma(hipStream_t st, int workgroups, int iters, float *sink, unsigned long long *clocks);
+
 } // namespace hipml

@@ -1,0 +1,163 @@
+// Measurement-only kernels: what the memory system and the MFMA pipes of this chip deliver to a kernel that
+// does nothing else, in the access pattern and instruction mix of the attention kernels.  The benchmark
+// prints their rates as `achievable` beside the published peaks; nothing on the attention path calls them.
+// (The reference prints its bandwidth yardstick beside every decode number:
+// crates/hipml-kernels/src/kvbench.rs:209-249, kernels/bw_probe.hip, kernels/stream_read.hip.)
+
+#include "common.h"
+
+namespace hipml {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef float float16v __attribute__((ext_vector_type(16)));
+typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
+
+constexpr int kYsWaves = 4;
+constexpr int kYsThreads = 64 * kYsWaves;
+constexpr int kYsPiece = 32 * kRowBytes; // 8,704 bytes: the 32 cache rows a decode wave asks for at a time
+constexpr int kYsPieceReq = 9;           // requests of 64 lanes x 16 bytes per piece (the last one half a wave)
+constexpr int kYsLds = kYsWaves * 2 * kYsPiece; // 69,632
+
+// One launch reads `pieces` pieces of each of two arrays once.  Piece g belongs to workgroup (g / 4) % grid,
+// wave g % 4, as the decode kernel deals its key tiles; a wave keeps one piece of each array in flight and
+// asks for the next one of an array when the previous one of that array has arrived.
+// LDS_ROAD: global_load_lds_dwordx4 (non-temporal) into two per-wave buffers, the decode kernel's road;
+// otherwise non-temporal 128-bit loads into registers.
+template <bool LDS_ROAD>
+__global__ void __launch_bounds__(kYsThreads, 2) stream_read_kernel(const uint8_t *a, const uint8_t *b, int pieces,
+                                                                    uint32_t *sink)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[]; // kYsLds bytes: two pieces per wave
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int lane = threadIdx.x & 63;
+    const int first = blockIdx.x * kYsWaves + wave, step = gridDim.x * kYsWaves;
+    uint4v acc = {0, 0, 0, 0};
+    if (LDS_ROAD) {
+        const uint32_t at = __builtin_amdgcn_readfirstlane(
+            (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void *)(lds + wave * 2 * kYsPiece));
+        auto request = [&](const uint8_t *src, uint32_t lds_to) {
+            const uint32_t lds_at = __builtin_amdgcn_readfirstlane(lds_to);
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt"
+                             :
+                             : "s"(lds_at + j * 1024), "v"(lane * 16), "s"(src + j * 1024)
+                             : "memory");
+            if (lane < 32)
+                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt"
+                             :
+                             : "s"(lds_at + 8192), "v"(lane * 16), "s"(src + 8192)
+                             : "memory");
+        };
+        if (first < pieces) {
+            request(a + (size_t)first * kYsPiece, at);
+            request(b + (size_t)first * kYsPiece, at + kYsPiece);
+        }
+        for (int g = first; g < pieces; g += step) {
+            const bool more = g + step < pieces;
+            asm volatile("s_waitcnt vmcnt(9)" ::: "memory"); // this piece of `a` is in LDS
+            if (more)
+                request(a + (size_t)(g + step) * kYsPiece, at);
+            if (more)
+                asm volatile("s_waitcnt vmcnt(9)" ::: "memory"); // this piece of `b`
+            else
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            if (more)
+                request(b + (size_t)(g + step) * kYsPiece, at + kYsPiece);
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        acc[0] = *reinterpret_cast<const uint32_t *>(lds + wave * 2 * kYsPiece + lane * 4);
+    } else {
+        for (int g = first; g < pieces; g += step) {
+            const uint8_t *pa = a + (size_t)g * kYsPiece + lane * 16, *pb = b + (size_t)g * kYsPiece + lane * 16;
+            uint4v x[2 * kYsPieceReq];
+#pragma unroll
+            for (int j = 0; j < kYsPieceReq; j++) {
+                const bool in = j < 8 || lane < 32;
+                x[2 * j] = in ? __builtin_nontemporal_load(reinterpret_cast<const uint4v *>(pa + j * 1024)) : acc;
+                x[2 * j + 1] = in ? __builtin_nontemporal_load(reinterpret_cast<const uint4v *>(pb + j * 1024)) : acc;
+            }
+#pragma unroll
+            for (int j = 0; j < 2 * kYsPieceReq; j++)
+                acc ^= x[j];
+        }
+    }
+    if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x9E3779B9u) // (keeps the loads; practically never true)
+        sink[0] = acc[0];
+}
+
+// Every wave issues `iters` x 8 independent v_mfma_f32_32x32x16_f16 back to back, one wave per SIMD (the
+// arrangement of the long-chunk kernel).  Wave 0 of workgroup 0 also reads the core clock counter and the
+// constant 100 MHz counter around its loop: clocks[0] = core cycles, clocks[1] = 100 MHz ticks.
+__global__ void __launch_bounds__(kYsThreads, 1) mfma_loop_kernel(int iters, float *sink, unsigned long long *clocks)
+{
+    // eight operand pairs of pseudo-random values in (-1, 1): consecutive MFMAs see different bits, as the
+    // attention kernels' do (a loop over one constant operand pair draws less power and holds a higher clock)
+    half8 x[8], y[8];
+    uint32_t h = 0x9E3779B9u * (threadIdx.x + 1u);
+#pragma unroll
+    for (int t = 0; t < 8; t++)
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            h = h * 1664525u + 1013904223u;
+            x[t][j] = (_Float16)((float)(int)(h >> 8 & 0xffff) * (1.0f / 32768.0f) - 1.0f);
+            h = h * 1664525u + 1013904223u;
+            y[t][j] = (_Float16)((float)(int)(h >> 8 & 0xffff) * (1.0f / 32768.0f) - 1.0f);
+        }
+    float16v acc[8];
+#pragma unroll
+    for (int t = 0; t < 8; t++)
+#pragma unroll
+        for (int i = 0; i < 16; i++)
+            acc[t][i] = 0.0f;
+    const unsigned long long c0 = __builtin_readcyclecounter();
+    const unsigned long long r0 = __builtin_amdgcn_s_memrealtime();
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+        for (int t = 0; t < 8; t++)
+            acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(x[t], y[t], acc[t], 0, 0, 0);
+    }
+    float s = 0.0f;
+#pragma unroll
+    for (int t = 0; t < 8; t++)
+#pragma unroll
+        for (int i = 0; i < 16; i++)
+            s += acc[t][i];
+    const unsigned long long c1 = __builtin_readcyclecounter();
+    const unsigned long long r1 = __builtin_amdgcn_s_memrealtime();
+    if (s == 12345.678f) // (keeps the MFMAs; never true for these operands)
+        sink[0] = s;
+    if (clocks != nullptr && blockIdx.x == 0 && threadIdx.x == 0) {
+        clocks[0] = c1 - c0;
+        clocks[1] = r1 - r0;
+    }
+}
+
+int yardstick_init()
+{
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&stream_read_kernel<true>),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, kYsLds);
+    if (e != hipSuccess)
+        return fail((int)e, "hipFuncSetAttribute(yardstick LDS) failed: %d (%s)", (int)e, hipGetErrorString(e));
+    return 0;
+}
+
+int launch_bench_stream(hipStream_t st, const uint8_t *a, const uint8_t *b, size_t bytes_each, int mode, uint32_t *sink)
+{
+    const int pieces = (int)(bytes_each / kYsPiece);
+    const dim3 grid(256, 1, 1), block(kYsThreads, 1, 1);
+    if (mode == 0)
+        hipLaunchKernelGGL(stream_read_kernel<true>, grid, block, kYsLds, st, a, b, pieces, sink);
+    else
+        hipLaunchKernelGGL(stream_read_kernel<false>, grid, block, 0, st, a, b, pieces, sink);
+    return launched("bench_stream_read");
+}
+
+int launch_bench_mfma(hipStream_t st, int workgroups, int iters, float *sink, unsigned long long *clocks)
+{
+    hipLaunchKernelGGL(mfma_loop_kernel, dim3((unsigned)workgroups, 1, 1), dim3(kYsThreads, 1, 1), 0, st, iters, sink,
+                       clocks);
+    return launched("bench_mfma_f16");
+}
+
+} // namespace hipml

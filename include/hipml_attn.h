@@ -442,6 +442,29 @@ int hipml_attn_chunk_kv_f16(hipml_stream_t stream, const float *q, const void *k
                             int head_dim, int pos0, int tokens, int stride, float *part_acc,
                             float *part_ml, int splits);
 
+/* The same copy kept by the library, behind the reference's own entry points.  hipml_kv_f16_attach registers
+ * kv_f16 (hipml_kv_f16_bytes(stride, n_kv) bytes, 16-byte aligned) as the f16 shadow of the cache
+ * (k_cache, v_cache) and converts its rows [0, rows) on `stream`.  From then on, without any change to the
+ * calls the reference's engine makes per chunk (crates/hipml-model/src/gpu/attn_tile.rs:53-82):
+ *   - the entry points that write rows of that cache at positions the host knows (hipml_kv_encode_bulk,
+ *     hipml_rope_encode_chunk_f32, hipml_attn_chunk_front_encode_f32, hipml_kv_rows_copy as destination)
+ *     convert those rows right behind their own launch;
+ *   - the ones whose positions live in device memory (hipml_kv_encode, hipml_attn_front_encode_f32,
+ *     hipml_kv_encode_rows, hipml_attn_front_rows_encode_f32) mark the shadow stale, and the next chunk
+ *     attention over the cache converts every live row once (0.13 ms per 100,000 rows);
+ *   - hipml_attn_chunk_q8_split, _gate and _gate_f16 over (k_cache, v_cache) with the registered stride,
+ *     n_kv and format and splits >= 2 read the tiles: min(splits, hipml_attn_chunk_slices) slices, no
+ *     tiles made per call in the scratch (2,048 tokens at depth 100,000: 4.06 against 4.19 ms).
+ * The bookkeeping is host state that changes when a call is issued or captured, not when a captured
+ * graph is replayed.  Rows written into the cache by any other means (a device copy, another library)
+ * must be followed by hipml_kv_f16_rows for those rows.  hipml_kv_f16_detach must be called before
+ * either buffer is freed; it is HIPML_ATTN_E_STATE for a cache that has no shadow.  At most 1,024 caches
+ * per process.  No counterpart in the reference: its DeepKv::new (crates/hipml-model/src/gpu/deep_kv.rs:41-83)
+ * is where an engine would allocate the copy and attach it. */
+int hipml_kv_f16_attach(hipml_stream_t stream, int dtype, const void *k_cache, const void *v_cache,
+                        void *kv_f16, int n_kv, int head_dim, int stride, int rows);
+int hipml_kv_f16_detach(const void *k_cache);
+
 /* ---- output gate ------------------------------------------------------------ */
 
 /* y[i] = x[i] * sigmoid(gate[i]); y may alias x.  Replaces
@@ -497,6 +520,26 @@ int hipml_gemm_q8_0_f16(hipml_stream_t stream, const void *w, const float *x, fl
  * crates/hipml-kernels/src/attn_gpu/imp/attn_chunk.rs:343-397. */
 int hipml_attn_output_chunk_q8_0(hipml_stream_t stream, const void *wo, const float *attn_out,
                                  const float *gate, float *y, int m, int k, int tokens, void *x16);
+
+/* ---- measurement only: yardsticks for the benchmark ----------------------------------------------
+ * Not part of the attention path and without a counterpart in the reference's launchers; they stand where the
+ * reference's bandwidth probes do (crates/hipml-kernels/kernels/bw_probe.hip, stream_read.hip, printed beside
+ * every decode figure by crates/hipml-kernels/src/kvbench.rs:209-249).  Both launch asynchronously on
+ * `stream`, allocate nothing and write at most the few bytes named below. */
+
+/* One launch of 256 workgroups that reads bytes_each bytes (a positive multiple of 8,704 = 32 cache rows)
+ * of each of `a` and `b` once, dealt to workgroups and waves as the decode kernel deals the K and V rows of
+ * a cache, and does nothing with them.  mode 0: global memory straight into LDS (global_load_lds_dwordx4,
+ * non-temporal), the decode kernel's road; mode 1: non-temporal 128-bit loads into registers.  `sink`:
+ * 4 bytes of device memory (never written in practice; it keeps the loads alive). */
+int hipml_bench_stream_read(hipml_stream_t stream, const void *a, const void *b, size_t bytes_each, int mode,
+                            void *sink);
+/* `workgroups` workgroups of four waves, one per SIMD, each wave issuing iters x 8 independent
+ * v_mfma_f32_32x32x16_f16: workgroups x 4 x iters x 8 x 32,768 FLOP per launch.  `sink`: 4 bytes of device
+ * memory (as above).  `clocks`: NULL or 16 bytes of device memory that receive, from one wave, the core
+ * clock cycles and the ticks of the constant 100 MHz counter its loop took (the clock the chip ran at
+ * under this load is their ratio x 100 MHz). */
+int hipml_bench_mfma_f16(hipml_stream_t stream, int workgroups, int iters, void *sink, void *clocks);
 
 #ifdef __cplusplus
 }
