@@ -4,6 +4,7 @@
 
 #include "common.h"
 
+#include <atomic>
 #include <math.h>
 #include <mutex>
 #include <stdarg.h>
@@ -14,12 +15,12 @@ namespace hipml {
 
 static thread_local char g_err[512] = "";
 // The registered RoPE table is a device pointer, so there is one registration per device: the entry
-// points work on a snapshot of the current device's, taken under the lock when they start
-// (clear_error), and the two calls that change it write under the same lock.
+// points that rotate work on a snapshot of the current device's, taken under the lock when they start
+// (snapshot_rope), and the two calls that change it write under the same lock.
 static RopeTable g_rope_dev[64];
 static std::mutex g_rope_mu;
 static thread_local RopeTable g_rope = {nullptr, 0.0f, 0, 0, 0};
-static bool g_inited[64]; // per device: hipml_attn_init has run with that device current
+static std::atomic<bool> g_inited[64]; // per device: hipml_attn_init has run with that device current
 
 static int rope_device()
 {
@@ -38,20 +39,23 @@ int fail(int code, const char *fmt, ...)
     return code;
 }
 
-// Start of every entry point: no message, and no error left over from an earlier runtime call of
-// the caller's (launched() below reads the runtime's last error after each launch).
-void clear_error()
+// Start of every entry point: no message.
+void clear_error() { g_err[0] = '\0'; }
+
+// Entry points that rotate work on a snapshot of the current device's RoPE registration.
+static void snapshot_rope()
 {
-    g_err[0] = '\0';
-    (void)hipGetLastError();
     const int device = rope_device();
     std::lock_guard<std::mutex> lock(g_rope_mu);
     g_rope = g_rope_dev[device];
 }
 
+static thread_local hipError_t g_launch_status = hipSuccess;
+void set_launch_status(hipError_t e) { g_launch_status = e; }
+
 int launched(const char *what)
 {
-    hipError_t e = hipGetLastError();
+    const hipError_t e = g_launch_status;
     if (e == hipSuccess)
         return 0;
     snprintf(g_err, sizeof(g_err), "%s launch failed: %d (%s)", what, (int)e, hipGetErrorString(e));
@@ -534,6 +538,7 @@ int hipml_mrope_f32(hipml_stream_t stream, const float *x, float *y, int n_heads
                     float theta_base)
 {
     clear_error();
+    snapshot_rope();
     REQUIRE_PTR(x);
     REQUIRE_PTR(y);
     REQUIRE_PTR(pos);
@@ -551,6 +556,7 @@ int hipml_mrope_rows_f32(hipml_stream_t stream, const float *x, float *y, int n_
                          const int32_t *pos, int rows, float theta_base)
 {
     clear_error();
+    snapshot_rope();
     REQUIRE_PTR(x);
     REQUIRE_PTR(y);
     REQUIRE_PTR(pos);
@@ -569,6 +575,7 @@ int hipml_rope_chunk_f32(hipml_stream_t stream, float *q, float *k, int n_head, 
                          int head_dim, int n_rot, float theta_base, int pos0, int tokens)
 {
     clear_error();
+    snapshot_rope();
     REQUIRE_PTR(q);
     REQUIRE_PTR(k);
     int rc = check_rope(n_head, head_dim, n_rot, theta_base);
@@ -615,6 +622,7 @@ int hipml_attn_front_f32(hipml_stream_t stream, const float *qg, float *q, float
                          const int32_t *pos, float theta_base, float eps)
 {
     clear_error();
+    snapshot_rope();
     REQUIRE_PTR(pos);
     int rc = check_front(qg, q, gate, k, q_norm, k_norm, n_heads, n_kv, head_dim, n_rot, theta_base, eps);
     if (rc)
@@ -631,6 +639,7 @@ int hipml_attn_chunk_front_f32(hipml_stream_t stream, const float *qg, float *k,
                                int pos0, int tokens)
 {
     clear_error();
+    snapshot_rope();
     int rc = check_front(qg, q, gate, k, q_norm, k_norm, n_heads, n_kv, head_dim, n_rot, theta_base, eps);
     if (rc)
         return rc;
@@ -671,6 +680,7 @@ int hipml_attn_front_encode_f32(hipml_stream_t stream, const int32_t *step, int 
                                 float eps, int stride)
 {
     clear_error();
+    snapshot_rope();
     REQUIRE_PTR(step);
     int rc = check_front(qg, q, gate, k, q_norm, k_norm, n_heads, n_kv, head_dim, n_rot, theta_base, eps);
     if (rc == 0)
@@ -692,6 +702,7 @@ int hipml_attn_chunk_front_encode_f32(hipml_stream_t stream, int dtype, const fl
                                       int pos0, int tokens, int stride)
 {
     clear_error();
+    snapshot_rope();
     int rc = check_front(qg, q, gate, k, q_norm, k_norm, n_heads, n_kv, head_dim, n_rot, theta_base, eps);
     if (rc == 0)
         rc = check_encode(dtype, k, v, k_cache, v_cache, n_kv, head_dim, stride);
@@ -720,6 +731,7 @@ int hipml_attn_front_rows_f32(hipml_stream_t stream, const float *qg, float *k, 
                               int rows)
 {
     clear_error();
+    snapshot_rope();
     REQUIRE_PTR(pos);
     int rc = check_front(qg, q, gate, k, q_norm, k_norm, n_heads, n_kv, head_dim, n_rot, theta_base, eps);
     if (rc)
@@ -742,6 +754,7 @@ int hipml_attn_front_rows_encode_f32(hipml_stream_t stream, int dtype, const flo
                                      int stride, const int32_t *pos, size_t slot_bytes, int slots)
 {
     clear_error();
+    snapshot_rope();
     REQUIRE_PTR(pos);
     int rc = check_front(qg, q, gate, k, q_norm, k_norm, n_heads, n_kv, head_dim, n_rot, theta_base, eps);
     if (rc == 0)
@@ -799,6 +812,7 @@ int hipml_rope_encode_chunk_f32(hipml_stream_t stream, float *q, float *k, const
                                 float theta_base, int pos0, int tokens, int dtype, int stride)
 {
     clear_error();
+    snapshot_rope();
     // (q may be NULL: only the K rows are rotated, for a caller whose attention call rotates the query rows)
     int rc = check_rope(n_head, head_dim, n_rot, theta_base);
     if (rc == 0)
@@ -1024,13 +1038,12 @@ int hipml_attn_decode_batch_cols_gate(hipml_stream_t stream, int dtype, const in
 
 // ---- chunk prefill ---------------------------------------------------------------------------------
 
-static int chunk_q8_common(hipml_stream_t stream, const float *q, const void *kc, const void *vc,
-                           float *out, const float *gate, bool want_gate, int n_head, int n_kv,
-                           int head_dim, int pos0, int tokens, int dtype, int stride, float *part_acc,
-                           float *part_ml, int splits, void *out16 = nullptr, bool want_f16 = false,
-                           const void *kv_f16 = nullptr, const float *rope_tab = nullptr)
+// Everything chunk_q8_common can refuse, without a launch: the entry point that rotates q in place first
+// runs these checks before it touches q.
+static int chunk_q8_validate(const float *q, const void *kc, const void *vc, float *out, const float *gate,
+                             bool want_gate, int n_head, int n_kv, int head_dim, int pos0, int tokens, int dtype,
+                             int stride, float *part_acc, float *part_ml, int splits, void *out16, bool want_f16)
 {
-    clear_error();
     REQUIRE_PTR(q);
     REQUIRE_PTR(kc);
     REQUIRE_PTR(vc);
@@ -1066,9 +1079,19 @@ static int chunk_q8_common(hipml_stream_t stream, const float *q, const void *kc
         return rc;
     if (want_gate && (rc = check_aligned16(gate, "gate")))
         return rc;
-    if (tokens == 0)
-        return 0;
-    if ((rc = require_init()))
+    return tokens == 0 ? 0 : require_init();
+}
+
+static int chunk_q8_common(hipml_stream_t stream, const float *q, const void *kc, const void *vc,
+                           float *out, const float *gate, bool want_gate, int n_head, int n_kv,
+                           int head_dim, int pos0, int tokens, int dtype, int stride, float *part_acc,
+                           float *part_ml, int splits, void *out16 = nullptr, bool want_f16 = false,
+                           const void *kv_f16 = nullptr, const float *rope_tab = nullptr)
+{
+    clear_error();
+    int rc = chunk_q8_validate(q, kc, vc, out, gate, want_gate, n_head, n_kv, head_dim, pos0, tokens, dtype, stride,
+                               part_acc, part_ml, splits, out16, want_f16);
+    if (rc || tokens == 0)
         return rc;
     // a cache with a registered f16 shadow: the sliced attention reads its tiles (as many slices as the policy
     // gives a chunk over such a copy, within what the scratch was sized for)
@@ -1122,6 +1145,7 @@ int hipml_attn_chunk_rope_q8(hipml_stream_t stream, float *q, const void *kc, co
                              float *part_ml, int splits)
 {
     clear_error();
+    snapshot_rope();
     REQUIRE_PTR(q);
     int rc = check_rope(n_head, head_dim, n_rot, theta_base);
     if (rc)
@@ -1134,6 +1158,10 @@ int hipml_attn_chunk_rope_q8(hipml_stream_t stream, float *q, const void *kc, co
     // kernel gets them rotated in place first.
     const bool in_kernel = splits == 0 && n_rot == 64 && head_dim == kHeadDim &&
                            (long long)pos0 + tokens <= g_rope.max_pos;
+    // nothing may be refused once q has been rotated in place: a corrected retry would rotate it again
+    if ((rc = chunk_q8_validate(q, kc, vc, out, gate, gate != nullptr, n_head, n_kv, head_dim, pos0, tokens, dtype,
+                                stride, part_acc, part_ml, splits, out16, out16 != nullptr)))
+        return rc;
     if (!in_kernel && tokens > 0) {
         if ((rc = check_aligned16(q, "q")))
             return rc;

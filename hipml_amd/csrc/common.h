@@ -21,11 +21,34 @@ constexpr int kMaxGroup = 8;      // query heads per KV head
 
 // Record `msg` for hipml_attn_last_error() and return `code`.
 int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
-// Translate the launch status of the most recent kernel launch on this thread.
+// Translate the status of this thread's most recent HIPML_LAUNCH: the return code of that launch call itself,
+// so an error the caller's own earlier HIP calls left pending is neither consumed nor mistaken for ours.
 int launched(const char *what);
+void set_launch_status(hipError_t e);
 void clear_error();
 
 #ifdef __HIPCC__
+} // namespace hipml
+#include <tuple>
+#include <utility>
+namespace hipml {
+template <typename Tuple, size_t... I>
+inline void launch_pointers(Tuple &vals, void **ptrs, std::index_sequence<I...>)
+{
+    ((ptrs[I] = static_cast<void *>(&std::get<I>(vals))), ...);
+}
+// kernel<<<grid, block, lds, st>>>(args...) with the status kept for launched().
+template <typename... KArgs, typename... Args>
+inline void launch_kernel(void (*kernel)(KArgs...), dim3 grid, dim3 block, size_t lds, hipStream_t st, Args &&...args)
+{
+    static_assert(sizeof...(KArgs) == sizeof...(Args), "one argument per kernel parameter");
+    std::tuple<KArgs...> vals(static_cast<KArgs>(std::forward<Args>(args))...);
+    void *ptrs[sizeof...(KArgs) > 0 ? sizeof...(KArgs) : 1];
+    launch_pointers(vals, ptrs, std::index_sequence_for<KArgs...>{});
+    set_launch_status(hipLaunchKernel(reinterpret_cast<const void *>(kernel), grid, block, ptrs, lds, st));
+}
+#define HIPML_LAUNCH(kernel, grid, block, lds, st, ...) ::hipml::launch_kernel(kernel, grid, block, lds, st, __VA_ARGS__)
+
 // The sigmoid output gate (crates/hipml-core/src/ops.rs:354-360): x / (1 + e^-g).  Every kernel that gates
 // writes it through this one expression, so a fused call and the attention followed by the stand-alone
 // gate kernel give the same bits.  The exponential is one v_exp_f32 of g * -log2(e) and the quotient one

@@ -1860,7 +1860,7 @@ int decode_init()
 constexpr size_t kStaticSlices = 4096; // (head, split) pairs: n_heads * splits of a call
 static __device__ __align__(256) float scratch[kStaticSlices * (kHeadDim + 2)];
 constexpr int kMaxDevices = 64;
-static float *g_scratch_ptr[kMaxDevices]; // device address of `scratch` on each initialised GPU
+static std::atomic<float *> g_scratch_ptr[kMaxDevices]; // device address of `scratch` on each initialised GPU
 
 static int decode_tickets_init(int device);
 
@@ -1960,13 +1960,13 @@ int decode_static_partials(int n_heads, int splits, float **part_acc, float **pa
     const hipError_t e = hipGetDevice(&device);
     if (e != hipSuccess)
         return fail((int)e, "hipGetDevice failed: %d (%s)", (int)e, hipGetErrorString(e));
-    if (device < 0 || device >= kMaxDevices || g_scratch_ptr[device] == nullptr)
+    if (device < 0 || device >= kMaxDevices || g_scratch_ptr[device].load() == nullptr)
         return fail(HIPML_ATTN_E_STATE, "hipml_attn_init has not been called for device %d", device);
     if (n_heads < 1 || splits < 1 || (size_t)n_heads * (size_t)splits > kStaticSlices)
         return fail(HIPML_ATTN_E_RANGE,
                     "n_heads %d x splits %d: the built-in scratch holds at most %zu (head, split) partials",
                     n_heads, splits, kStaticSlices);
-    float *ptr = g_scratch_ptr[device];
+    float *ptr = g_scratch_ptr[device].load();
     *part_acc = ptr;
     *part_ml = ptr + (size_t)n_heads * (size_t)splits * kHeadDim;
     return 0;
@@ -2153,13 +2153,13 @@ static int launch_decode_hd(hipStream_t st, const DecodeLaunch &L)
     if (L.head_dim != 64)
         return fail(HIPML_ATTN_E_SHAPE, "head_dim %d: 256 and 64 are built", L.head_dim);
     if (L.q4)
-        hipLaunchKernelGGL((decode_hd_kernel<64, true>), grid, block, 0, st, a);
+        HIPML_LAUNCH((decode_hd_kernel<64, true>), grid, block, 0, st, a);
     else
-        hipLaunchKernelGGL((decode_hd_kernel<64, false>), grid, block, 0, st, a);
+        HIPML_LAUNCH((decode_hd_kernel<64, false>), grid, block, 0, st, a);
     int rc = launched("attn_decode_kv_hd");
     if (rc)
         return rc;
-    hipLaunchKernelGGL(decode_hd_reduce_kernel<64>, rgrid, dim3(64, 1, 1), 0, st, a);
+    HIPML_LAUNCH(decode_hd_reduce_kernel<64>, rgrid, dim3(64, 1, 1), 0, st, a);
     return launched("attn_decode_kv_hd_reduce");
 }
 
@@ -2253,11 +2253,11 @@ int launch_decode_q8(hipStream_t st, const DecodeLaunch &given)
         a.merge = a.tickets != nullptr ? kMergeGroup : 0;
     }
     if (raw_rows)
-        hipLaunchKernelGGL(decode_q8_kernel, grid, dim3(kThreads, 1, 1), kDmaLds, st, a);
+        HIPML_LAUNCH(decode_q8_kernel, grid, dim3(kThreads, 1, 1), kDmaLds, st, a);
     else if (L.q4)
-        hipLaunchKernelGGL((decode_staged_kernel<true, false>), grid, dim3(kThreads, 1, 1), decode_lds_bytes(1), st, a);
+        HIPML_LAUNCH((decode_staged_kernel<true, false>), grid, dim3(kThreads, 1, 1), decode_lds_bytes(1), st, a);
     else
-        hipLaunchKernelGGL((decode_staged_kernel<false, true>), grid, dim3(kThreads, 1, 1), decode_lds_bytes(1), st, a);
+        HIPML_LAUNCH((decode_staged_kernel<false, true>), grid, dim3(kThreads, 1, 1), decode_lds_bytes(1), st, a);
     int rc = launched(L.q4 ? "attn_decode_kv_q4" : "attn_decode_kv_q8");
     if (rc || a.merge > 0)
         return rc;
@@ -2269,31 +2269,31 @@ int launch_decode_q8(hipStream_t st, const DecodeLaunch &given)
     if (L.splits <= 128 && L.slots == 1) {
         const dim3 grid((unsigned)L.n_heads * 16, (unsigned)L.total_rows, 1);
         if (L.splits <= 64)
-            hipLaunchKernelGGL((decode_reduce128_kernel<4, 1>), grid, dim3(256, 1, 1), 0, st, L.part_acc, L.part_ml,
+            HIPML_LAUNCH((decode_reduce128_kernel<4, 1>), grid, dim3(256, 1, 1), 0, st, L.part_acc, L.part_ml,
                                L.out, L.gate, L.splits, L.acc_slot, L.ml_slot, L.q_slot);
         else
-            hipLaunchKernelGGL((decode_reduce128_kernel<4, 2>), grid, dim3(256, 1, 1), 0, st, L.part_acc, L.part_ml,
+            HIPML_LAUNCH((decode_reduce128_kernel<4, 2>), grid, dim3(256, 1, 1), 0, st, L.part_acc, L.part_ml,
                                L.out, L.gate, L.splits, L.acc_slot, L.ml_slot, L.q_slot);
     } else if (L.splits <= 128) {
         const dim3 grid((unsigned)L.n_heads * 4, (unsigned)L.total_rows, 1);
         if (L.splits <= 16)
-            hipLaunchKernelGGL((decode_reduce128_kernel<16, 1>), grid, dim3(256, 1, 1), 0, st, L.part_acc, L.part_ml,
+            HIPML_LAUNCH((decode_reduce128_kernel<16, 1>), grid, dim3(256, 1, 1), 0, st, L.part_acc, L.part_ml,
                                L.out, L.gate, L.splits, L.acc_slot, L.ml_slot, L.q_slot);
         else if (L.splits <= 32)
-            hipLaunchKernelGGL((decode_reduce128_kernel<16, 2>), grid, dim3(256, 1, 1), 0, st, L.part_acc, L.part_ml,
+            HIPML_LAUNCH((decode_reduce128_kernel<16, 2>), grid, dim3(256, 1, 1), 0, st, L.part_acc, L.part_ml,
                                L.out, L.gate, L.splits, L.acc_slot, L.ml_slot, L.q_slot);
         else if (L.splits <= 64)
-            hipLaunchKernelGGL((decode_reduce128_kernel<16, 4>), grid, dim3(256, 1, 1), 0, st, L.part_acc, L.part_ml,
+            HIPML_LAUNCH((decode_reduce128_kernel<16, 4>), grid, dim3(256, 1, 1), 0, st, L.part_acc, L.part_ml,
                                L.out, L.gate, L.splits, L.acc_slot, L.ml_slot, L.q_slot);
         else
-            hipLaunchKernelGGL((decode_reduce128_kernel<16, 8>), grid, dim3(256, 1, 1), 0, st, L.part_acc, L.part_ml,
+            HIPML_LAUNCH((decode_reduce128_kernel<16, 8>), grid, dim3(256, 1, 1), 0, st, L.part_acc, L.part_ml,
                                L.out, L.gate, L.splits, L.acc_slot, L.ml_slot, L.q_slot);
     }
     else if (L.slots == 1)
-        hipLaunchKernelGGL(decode_reduce_kernel<4>, dim3((unsigned)L.n_heads * 16, (unsigned)L.total_rows, 1), dim3(256, 1, 1), 0,
+        HIPML_LAUNCH(decode_reduce_kernel<4>, dim3((unsigned)L.n_heads * 16, (unsigned)L.total_rows, 1), dim3(256, 1, 1), 0,
                            st, L.part_acc, L.part_ml, L.out, L.gate, L.splits, L.acc_slot, L.ml_slot, L.q_slot);
     else
-        hipLaunchKernelGGL(decode_reduce_kernel<16>,
+        HIPML_LAUNCH(decode_reduce_kernel<16>,
                            dim3((unsigned)L.n_heads * 4, (unsigned)L.total_rows, 1), dim3(256, 1, 1), 0,
                            st, L.part_acc, L.part_ml, L.out, L.gate, L.splits, L.acc_slot, L.ml_slot, L.q_slot);
     return launched("attn_decode_kv_reduce");

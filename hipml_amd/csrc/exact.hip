@@ -139,7 +139,7 @@ int launch_kv_encode(hipStream_t st, int q4, const float *k, const float *v, uin
     // grid.y is limited to 65535: walk long chunks in slices.
     for (int u0 = 0; u0 < units; u0 += 32768) {
         const int n = units - u0 < 32768 ? units - u0 : 32768;
-        hipLaunchKernelGGL(q4 ? kv_encode_q4_kernel : kv_encode_q8_kernel, dim3(n_kv, n, 1),
+        HIPML_LAUNCH(q4 ? kv_encode_q4_kernel : kv_encode_q8_kernel, dim3(n_kv, n, 1),
                            dim3(block, 1, 1), 0, st, k, v, kc + (size_t)u0 * slot_bytes,
                            vc + (size_t)u0 * slot_bytes, n_kv, head_dim, stride,
                            pos ? pos + (size_t)u0 * pos_stride : nullptr, pos_stride, slot_bytes,
@@ -268,7 +268,7 @@ int launch_mrope(hipStream_t st, const float *x, float *y, int n_heads, int head
     for (int r0 = 0; r0 < rows; r0 += 32768) {
         const int n = rows - r0 < 32768 ? rows - r0 : 32768;
         const size_t off = (size_t)r0 * n_heads * head_dim;
-        hipLaunchKernelGGL(mrope_kernel, dim3(n_heads, n, 1), dim3(64, 1, 1), 0, st, x + off,
+        HIPML_LAUNCH(mrope_kernel, dim3(n_heads, n, 1), dim3(64, 1, 1), 0, st, x + off,
                            y + off, n_heads, head_dim, n_rot, s0, s1, s2, s3,
                            pos + (size_t)r0 * pos_stride, pos_stride, text, theta, t, tab_rows);
         int rc = launched("mrope_f32");
@@ -287,7 +287,7 @@ int launch_rope_chunk(hipStream_t st, float *q, float *k, int n_head, int n_kv, 
     for (int t0 = 0; t0 < tokens; t0 += slab) {
         const int n = tokens - t0 < slab ? tokens - t0 : slab;
         const long long rows = (long long)n * (n_head + n_kv);
-        hipLaunchKernelGGL(rope_chunk_kernel, dim3((unsigned)((rows + 7) / 8), 1, 1), dim3(256, 1, 1), 0,
+        HIPML_LAUNCH(rope_chunk_kernel, dim3((unsigned)((rows + 7) / 8), 1, 1), dim3(256, 1, 1), 0,
                            st, q + (size_t)t0 * n_head * head_dim, k + (size_t)t0 * n_kv * head_dim,
                            n_head, n_kv, head_dim, n_rot, theta, pos0 + t0, n, t, tab_rows);
         int rc = launched("rope_chunk_f32");
@@ -471,10 +471,10 @@ int launch_rope_encode_chunk(hipStream_t st, int q4, float *q, float *k, const f
         float *kk = k + (size_t)t0 * n_kv * kHeadDim;
         const float *vv = v + (size_t)t0 * n_kv * kHeadDim;
         if (q4)
-            hipLaunchKernelGGL(rope_encode_chunk_kernel<true>, grid, dim3(256, 1, 1), 0, st, qq, kk, vv, kc, vc,
+            HIPML_LAUNCH(rope_encode_chunk_kernel<true>, grid, dim3(256, 1, 1), 0, st, qq, kk, vv, kc, vc,
                                n_head, n_kv, n_rot, theta, pos0 + t0, n, stride, q_blocks, t, tab_rows);
         else
-            hipLaunchKernelGGL(rope_encode_chunk_kernel<false>, grid, dim3(256, 1, 1), 0, st, qq, kk, vv, kc, vc,
+            HIPML_LAUNCH(rope_encode_chunk_kernel<false>, grid, dim3(256, 1, 1), 0, st, qq, kk, vv, kc, vc,
                                n_head, n_kv, n_rot, theta, pos0 + t0, n, stride, q_blocks, t, tab_rows);
         int rc = launched("rope_encode_chunk");
         if (rc)
@@ -666,7 +666,7 @@ int launch_front(hipStream_t st, const float *qg, float *q, float *gate, float *
                                 vc ? vc + (rowpos ? (size_t)r0 * slot_bytes : 0) : nullptr, step, start + r0,
                                 stride};
         auto kern = enc < 0 ? front_kernel<0> : enc == 0 ? front_kernel<1> : front_kernel<2>;
-        hipLaunchKernelGGL(kern, dim3(grid, 1, 1), dim3(256, 1, 1), 0, st,
+        HIPML_LAUNCH(kern, dim3(grid, 1, 1), dim3(256, 1, 1), 0, st,
                            qg + (size_t)r0 * n_heads * 2 * kHeadDim, q + (size_t)r0 * n_heads * kHeadDim,
                            gate + (size_t)r0 * n_heads * kHeadDim, k + (size_t)r0 * n_kv * kHeadDim, qw, kw,
                            n_heads, n_kv, n_rot, s0, s1, s2, s3, pos, pos0 + r0, n, theta, eps, t, tab_rows, ap);
@@ -715,7 +715,7 @@ int launch_q_gate(hipStream_t st, const float *x, const float *gate, float *y, s
     size_t n4 = aligned ? n / 4 : 0;
     if (n4 > 0) {
         const size_t blocks = (n4 + 255) / 256;
-        hipLaunchKernelGGL(q_gate_kernel4, dim3((unsigned)blocks, 1, 1), dim3(256, 1, 1), 0, st,
+        HIPML_LAUNCH(q_gate_kernel4, dim3((unsigned)blocks, 1, 1), dim3(256, 1, 1), 0, st,
                            reinterpret_cast<const float4 *>(x),
                            reinterpret_cast<const float4 *>(gate), reinterpret_cast<float4 *>(y),
                            n4);
@@ -726,7 +726,7 @@ int launch_q_gate(hipStream_t st, const float *x, const float *gate, float *y, s
     const size_t done = n4 * 4;
     if (done < n) {
         const size_t blocks = (n - done + 255) / 256;
-        hipLaunchKernelGGL(q_gate_kernel1, dim3((unsigned)blocks, 1, 1), dim3(256, 1, 1), 0, st, x,
+        HIPML_LAUNCH(q_gate_kernel1, dim3((unsigned)blocks, 1, 1), dim3(256, 1, 1), 0, st, x,
                            gate, y, done, n);
         return launched("q_gate_f32");
     }
@@ -761,7 +761,7 @@ int launch_kv_rows_copy(hipStream_t st, int q4, const uint8_t *k_src, const uint
     size_t blocks = (span16 + 255) / 256;
     if (blocks > 512)
         blocks = 512; // 2,048 workgroups over K, V and four heads fill the chip; the rest is the loop
-    hipLaunchKernelGGL(kv_rows_copy_kernel, dim3((unsigned)blocks, (unsigned)n_kv, 2), dim3(256, 1, 1), 0, st,
+    HIPML_LAUNCH(kv_rows_copy_kernel, dim3((unsigned)blocks, (unsigned)n_kv, 2), dim3(256, 1, 1), 0, st,
                        reinterpret_cast<const uint4 *>(k_src), reinterpret_cast<const uint4 *>(v_src),
                        reinterpret_cast<uint4 *>(k_dst), reinterpret_cast<uint4 *>(v_dst),
                        (size_t)src_stride * row16, (size_t)dst_stride * row16, span16);

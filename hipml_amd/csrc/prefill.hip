@@ -869,10 +869,23 @@ __device__ __forceinline__ void acc_zero()
     if constexpr (N > 4)
         acc_zero<R + 4, N - 4>();
 }
-template <int R, int N>
+// (The reads of accumulation registers below carry their own wait states: an MFMA of 8 passes needs 11 between
+// its issue and a read of its result by another unit, and the compiler inserts none for statements it cannot
+// read.  s_nop 10 in the same statement as the first read makes that independent of what is scheduled between
+// this statement and the MFMA before it.)
+template <int R, int N, bool FIRST = true>
 __device__ __forceinline__ void acc_scale(float c)
 {
     float t0, t1, t2, t3;
+    if constexpr (FIRST)
+        asm volatile("s_nop 10\n\tv_accvgpr_read_b32 %0, a[%5]\n\tv_accvgpr_read_b32 %1, a[%6]\n\t"
+                     "v_accvgpr_read_b32 %2, a[%7]\n\tv_accvgpr_read_b32 %3, a[%8]\n\t"
+                     "v_mul_f32 %0, %0, %4\n\tv_mul_f32 %1, %1, %4\n\tv_mul_f32 %2, %2, %4\n\tv_mul_f32 %3, %3, %4\n\t"
+                     "v_accvgpr_write_b32 a[%5], %0\n\tv_accvgpr_write_b32 a[%6], %1\n\tv_accvgpr_write_b32 a[%7], %2\n\t"
+                     "v_accvgpr_write_b32 a[%8], %3"
+                     : "=&v"(t0), "=&v"(t1), "=&v"(t2), "=&v"(t3)
+                     : "v"(c), "n"(R), "n"(R + 1), "n"(R + 2), "n"(R + 3));
+    else
     asm volatile("v_accvgpr_read_b32 %0, a[%5]\n\tv_accvgpr_read_b32 %1, a[%6]\n\tv_accvgpr_read_b32 %2, a[%7]\n\t"
                  "v_accvgpr_read_b32 %3, a[%8]\n\t"
                  "v_mul_f32 %0, %0, %4\n\tv_mul_f32 %1, %1, %4\n\tv_mul_f32 %2, %2, %4\n\tv_mul_f32 %3, %3, %4\n\t"
@@ -881,14 +894,14 @@ __device__ __forceinline__ void acc_scale(float c)
                  : "=&v"(t0), "=&v"(t1), "=&v"(t2), "=&v"(t3)
                  : "v"(c), "n"(R), "n"(R + 1), "n"(R + 2), "n"(R + 3));
     if constexpr (N > 4)
-        acc_scale<R + 4, N - 4>(c);
+        acc_scale<R + 4, N - 4, false>(c);
 }
 template <int R>
 __device__ __forceinline__ float4v acc_read4()
 {
     float4v x;
-    asm volatile("v_accvgpr_read_b32 %0, a[%4]\n\tv_accvgpr_read_b32 %1, a[%5]\n\tv_accvgpr_read_b32 %2, a[%6]\n\t"
-                 "v_accvgpr_read_b32 %3, a[%7]"
+    asm volatile("s_nop 10\n\tv_accvgpr_read_b32 %0, a[%4]\n\tv_accvgpr_read_b32 %1, a[%5]\n\t"
+                 "v_accvgpr_read_b32 %2, a[%6]\n\tv_accvgpr_read_b32 %3, a[%7]"
                  : "=v"(x[0]), "=v"(x[1]), "=v"(x[2]), "=v"(x[3])
                  : "n"(R), "n"(R + 1), "n"(R + 2), "n"(R + 3));
     return x;
@@ -1227,7 +1240,8 @@ chunk_f16_t64_kernel(const ChunkArgs a)
     // oldest first: K(t + 1), V^T(t + 1); at barrier B: V^T(t + 1), K(t + 2): the wait is vmcnt(9) both times.
     if (ntile > 0) {
         step(yes, no, 0, 0);
-        asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); // these scores were finished just now
+        // these scores were finished just now (the statement owns N, so no read of them can move above it)
+        asm volatile("s_nop 15\n\ts_nop 15" : "+v"(N[0]), "+v"(N[1])::"memory");
 #pragma unroll
         for (int h = 0; h < 2; h++)
 #pragma unroll
@@ -1993,10 +2007,10 @@ static int launch_kv_f16_tiles(hipStream_t st, const uint8_t *kc, const uint8_t 
     const int tile0 = start / kKTile, tile1 = (seq_end + kKTile - 1) / kKTile;
     const dim3 grid((unsigned)(tile1 - tile0), (unsigned)n_kv, 2);
     if (q4)
-        hipLaunchKernelGGL(kv_f16_tiles_kernel<true>, grid, dim3(256, 1, 1), kTilesLds, st, kc, vc, k16, vt, stride,
+        HIPML_LAUNCH(kv_f16_tiles_kernel<true>, grid, dim3(256, 1, 1), kTilesLds, st, kc, vc, k16, vt, stride,
                            tile0, seq_end, tile_stride);
     else
-        hipLaunchKernelGGL(kv_f16_tiles_kernel<false>, grid, dim3(256, 1, 1), kTilesLds, st, kc, vc, k16, vt, stride,
+        HIPML_LAUNCH(kv_f16_tiles_kernel<false>, grid, dim3(256, 1, 1), kTilesLds, st, kc, vc, k16, vt, stride,
                            tile0, seq_end, tile_stride);
     return launched("kv_f16_rows");
 }
@@ -2112,6 +2126,15 @@ int launch_chunk_q8(hipStream_t st, const float *q, const uint8_t *kc, const uin
             return launch_chunk_q8(st, q, kc, vc, out, n_head, n_kv, pos0, tokens, live_tiles * kKTile, part_acc,
                                    part_ml, use, gate, 0, out16, tiles, nullptr);
         }
+        // A count that was meant to hold the tiles but does not (hipml_attn_chunk_splits assumes 6 heads per KV
+        // head; fewer make the partial rows, and with them the room per slice, smaller): the extra slices are
+        // not slices to run.  The kernel that dequantizes for itself gets the count it would have been given.
+        if (kv_f16 == nullptr && rope_tab == nullptr && splits >= 3 && chunk_tiles_pay(pos0, tokens) &&
+            n_head / n_kv < 6) {
+            const int s = hipml_attn_chunk_slices(pos0, tokens, n_kv);
+            if (s >= 2 && s < splits && splits == chunk_tiles_splits(pos0, tokens, 6 * n_kv, n_kv, s))
+                splits = s;
+        }
     }
     // rope_tab != nullptr (splits == 0 only): q holds unrotated rows, the kernel rotates them as it loads them
     ChunkArgs a;
@@ -2144,13 +2167,13 @@ int launch_chunk_q8(hipStream_t st, const float *q, const uint8_t *kc, const uin
         const unsigned wgs = (unsigned)((tokens + kQTile - 1) / kQTile * n_kv * ((a.group + 1) / 2));
         a.rope_tab = rope_tab;
         if (q4 && rope_tab)
-            hipLaunchKernelGGL((chunk_wg_kernel<true, true>), dim3(wgs, 1, 1), dim3(kPfThreads, 1, 1), kWgLds, st, a);
+            HIPML_LAUNCH((chunk_wg_kernel<true, true>), dim3(wgs, 1, 1), dim3(kPfThreads, 1, 1), kWgLds, st, a);
         else if (q4)
-            hipLaunchKernelGGL((chunk_wg_kernel<true, false>), dim3(wgs, 1, 1), dim3(kPfThreads, 1, 1), kWgLds, st, a);
+            HIPML_LAUNCH((chunk_wg_kernel<true, false>), dim3(wgs, 1, 1), dim3(kPfThreads, 1, 1), kWgLds, st, a);
         else if (rope_tab)
-            hipLaunchKernelGGL((chunk_wg_kernel<false, true>), dim3(wgs, 1, 1), dim3(kPfThreads, 1, 1), kWgLds, st, a);
+            HIPML_LAUNCH((chunk_wg_kernel<false, true>), dim3(wgs, 1, 1), dim3(kPfThreads, 1, 1), kWgLds, st, a);
         else
-            hipLaunchKernelGGL((chunk_wg_kernel<false, false>), dim3(wgs, 1, 1), dim3(kPfThreads, 1, 1), kWgLds, st, a);
+            HIPML_LAUNCH((chunk_wg_kernel<false, false>), dim3(wgs, 1, 1), dim3(kPfThreads, 1, 1), kWgLds, st, a);
         return launched(q4 ? "attn_chunk_q4_wg" : "attn_chunk_q8_wg");
     }
     // slices per block: the last block (most keys) gets `splits`, a block with fewer key tiles gets
@@ -2179,16 +2202,16 @@ int launch_chunk_q8(hipStream_t st, const float *q, const uint8_t *kc, const uin
     }
     if (splits < 2) {
         if (kv_f16)
-            hipLaunchKernelGGL((chunk_q8_kernel<false, false, true>), dim3(grid, 1, 1), block, kPfLdsF, st, a);
+            HIPML_LAUNCH((chunk_q8_kernel<false, false, true>), dim3(grid, 1, 1), block, kPfLdsF, st, a);
         else if (q4)
-            hipLaunchKernelGGL((chunk_q8_kernel<false, true>), dim3(grid, 1, 1), block, kPfLds, st, a);
+            HIPML_LAUNCH((chunk_q8_kernel<false, true>), dim3(grid, 1, 1), block, kPfLds, st, a);
         else
-            hipLaunchKernelGGL(chunk_q8_kernel<false>, dim3(grid, 1, 1), block, kPfLds, st, a);
+            HIPML_LAUNCH(chunk_q8_kernel<false>, dim3(grid, 1, 1), block, kPfLds, st, a);
         int rc = launched(kv_f16 ? "attn_chunk_f16" : q4 ? "attn_chunk_q4" : "attn_chunk_q8");
         if (rc || out16 == nullptr)
             return rc;
         const size_t n4 = (size_t)tokens * n_head * kHeadDim / 4;
-        hipLaunchKernelGGL(rows_f16_kernel, dim3((unsigned)((n4 + 255) / 256), 1, 1), dim3(256, 1, 1), 0, st,
+        HIPML_LAUNCH(rows_f16_kernel, dim3((unsigned)((n4 + 255) / 256), 1, 1), dim3(256, 1, 1), 0, st,
                            reinterpret_cast<const float4v *>(out), static_cast<half4 *>(out16), n4);
         return launched("attn_chunk_rows_f16");
     }
@@ -2205,17 +2228,17 @@ int launch_chunk_q8(hipStream_t st, const float *q, const uint8_t *kc, const uin
     if ((n_kv * a.splits) % 8 != 0 && 8 % (n_kv * a.splits) == 0)
         g64 = (unsigned)(8 * ((b.nblock + 8 / (n_kv * a.splits) - 1) / (8 / (n_kv * a.splits))));
     if (kv_f16 && a.uniform && (g64 + 255) / 256 <= (grid + 255) / 256) {
-        hipLaunchKernelGGL(chunk_f16_t64_kernel, dim3(g64, 1, 1), dim3(kT64Threads, 1, 1), kT64Lds, st, b);
+        HIPML_LAUNCH(chunk_f16_t64_kernel, dim3(g64, 1, 1), dim3(kT64Threads, 1, 1), kT64Lds, st, b);
     } else if (kv_f16)
-        hipLaunchKernelGGL((chunk_q8_kernel<true, false, true>), dim3(grid, 1, 1), block, kPfLdsF, st, a);
+        HIPML_LAUNCH((chunk_q8_kernel<true, false, true>), dim3(grid, 1, 1), block, kPfLdsF, st, a);
     else if (q4)
-        hipLaunchKernelGGL((chunk_q8_kernel<true, true>), dim3(grid, 1, 1), block, kPfLds, st, a);
+        HIPML_LAUNCH((chunk_q8_kernel<true, true>), dim3(grid, 1, 1), block, kPfLds, st, a);
     else
-        hipLaunchKernelGGL(chunk_q8_kernel<true>, dim3(grid, 1, 1), block, kPfLds, st, a);
+        HIPML_LAUNCH(chunk_q8_kernel<true>, dim3(grid, 1, 1), block, kPfLds, st, a);
     int rc = launched(kv_f16 ? "attn_chunk_f16_split" : q4 ? "attn_chunk_q4_split" : "attn_chunk_q8_split");
     if (rc)
         return rc;
-    hipLaunchKernelGGL(chunk_combine_kernel, dim3((unsigned)tokens, (unsigned)((n_head + 3) / 4), 1),
+    HIPML_LAUNCH(chunk_combine_kernel, dim3((unsigned)tokens, (unsigned)((n_head + 3) / 4), 1),
                        dim3(256, 1, 1), 0, st, part_acc, part_ml, out, gate, n_head, a.qslots, a.splits, a.group,
                        a.ntask, tokens, pos0, a.slice_tiles, a.uniform, static_cast<_Float16 *>(out16));
     return launched("attn_chunk_combine");

@@ -475,7 +475,7 @@ static int launch_gemv_tile_steps(hipStream_t st, const uint8_t *w, const float 
     const size_t lds = (size_t)WAVES * TILES * XT * 64 * sizeof(float4v);
     auto kern = gemv_q8_tile_kernel<WAVES, TILES, XT, STEPS>;
     const dim3 grid((unsigned)((m + 16 * TILES - 1) / (16 * TILES)), (unsigned)((rows + 16 * XT - 1) / (16 * XT)), 1);
-    hipLaunchKernelGGL(kern, grid, dim3(64 * WAVES, 1, 1), lds, st, w, x, y, m, k, rows);
+    HIPML_LAUNCH(kern, grid, dim3(64 * WAVES, 1, 1), lds, st, w, x, y, m, k, rows);
     return launched("gemv_q8_0_rows");
 }
 
@@ -497,7 +497,7 @@ static int launch_gemv_xg(hipStream_t st, const uint8_t *w, const float *x, floa
     const size_t lds = (size_t)(k >> 5) * rp * 128 + (size_t)WAVES * TILES * 32 * sizeof(float4v);
     auto kern = gemv_q8_rows_kernel<WAVES, TILES, CH, XG>;
     const dim3 grid((unsigned)((m + 16 * TILES - 1) / (16 * TILES)), (unsigned)((rows + rp - 1) / rp), 1);
-    hipLaunchKernelGGL(kern, grid, dim3(64 * WAVES, 1, 1), lds, st, w, x, y, m, k, rows, rp);
+    HIPML_LAUNCH(kern, grid, dim3(64 * WAVES, 1, 1), lds, st, w, x, y, m, k, rows, rp);
     return launched("gemv_q8_0_rows");
 }
 
@@ -874,20 +874,20 @@ int launch_gemm_q8_f16(hipStream_t st, const uint8_t *w, const float *x, const f
 {
     const dim3 grid((unsigned)((m + kGemmM - 1) / kGemmM), (unsigned)((tokens + kGemmT - 1) / kGemmT), 1);
     if (x16 == nullptr) {
-        hipLaunchKernelGGL((gemm_q8_f16_kernel<false, kGemmWaves>), grid, dim3(64 * (kGemmWaves + kGemmCWaves), 1, 1), kGemmLds,
+        HIPML_LAUNCH((gemm_q8_f16_kernel<false, kGemmWaves>), grid, dim3(64 * (kGemmWaves + kGemmCWaves), 1, 1), kGemmLds,
                            st, w, x, y, m, k, tokens);
         return launched("gemm_q8_0_f16");
     }
     if (x != nullptr) {
         const size_t n8 = (size_t)tokens * k / 8;
-        hipLaunchKernelGGL(gate_f16_kernel, dim3((unsigned)((n8 + 255) / 256), 1, 1), dim3(256, 1, 1), 0, st,
+        HIPML_LAUNCH(gate_f16_kernel, dim3((unsigned)((n8 + 255) / 256), 1, 1), dim3(256, 1, 1), 0, st,
                            reinterpret_cast<const float4v *>(x), reinterpret_cast<const float4v *>(gate),
                            static_cast<half8 *>(x16), n8);
         int rc = launched("gate_f16");
         if (rc)
             return rc;
     }
-    hipLaunchKernelGGL((gemm_q8_f16_kernel<true, kGemmWaves>), grid, dim3(64 * (kGemmWaves + kGemmCWaves), 1, 1), kGemmLds, st, w,
+    HIPML_LAUNCH((gemm_q8_f16_kernel<true, kGemmWaves>), grid, dim3(64 * (kGemmWaves + kGemmCWaves), 1, 1), kGemmLds, st, w,
                        x16, y, m, k, tokens);
     return launched("gemm_q8_0_f16");
 }

@@ -147,15 +147,15 @@ int launch_bench_stream(hipStream_t st, const uint8_t *a, const uint8_t *b, size
     const int pieces = (int)(bytes_each / kYsPiece);
     const dim3 grid(256, 1, 1), block(kYsThreads, 1, 1);
     if (mode == 0)
-        hipLaunchKernelGGL(stream_read_kernel<true>, grid, block, kYsLds, st, a, b, pieces, sink);
+        HIPML_LAUNCH(stream_read_kernel<true>, grid, block, kYsLds, st, a, b, pieces, sink);
     else
-        hipLaunchKernelGGL(stream_read_kernel<false>, grid, block, 0, st, a, b, pieces, sink);
+        HIPML_LAUNCH(stream_read_kernel<false>, grid, block, 0, st, a, b, pieces, sink);
     return launched("bench_stream_read");
 }
 
 int launch_bench_mfma(hipStream_t st, int workgroups, int iters, float *sink, unsigned long long *clocks)
 {
-    hipLaunchKernelGGL(mfma_loop_kernel, dim3((unsigned)workgroups, 1, 1), dim3(kYsThreads, 1, 1), 0, st, iters, sink,
+    HIPML_LAUNCH(mfma_loop_kernel, dim3((unsigned)workgroups, 1, 1), dim3(kYsThreads, 1, 1), 0, st, iters, sink,
                        clocks);
     return launched("bench_mfma_f16");
 }

@@ -112,23 +112,27 @@ def test_argument_errors_come_before_any_launch(lib):
     assert e.value.code == rc
 
 
-def test_launching_entry_points_ask_for_init_first(lib):
+def test_launching_entry_points_ask_for_init_first():
     # the MFMA kernels need the LDS limit that hipml_attn_init raises; without it a call with valid
-    # arguments is refused with a message instead of failing inside the launch
+    # arguments is refused with a message instead of failing inside the launch.  In a process of its own, so
+    # that no earlier test has initialised the library (with or without a GPU: the check comes before any launch).
+    import subprocess
+    import sys
     from hipml_amd import attn
-    if attn_inited():
-        pytest.skip("the library was initialised earlier in this process")
-    one = C.c_void_p(16)
-    rc = lib.hipml_gemv_q8_0_rows(None, one, one, one, 64, 64, 1)
-    assert rc == -6 and b"hipml_attn_init" in lib.hipml_attn_last_error()
-    rc = lib.hipml_attn_decode_kv(None, one, 0, one, one, one, one, one, one, 24, 4, 256, 64,
-                                  C.c_float(0.0625), 1, 0, 0)
-    assert rc == -6 and b"hipml_attn_init" in lib.hipml_attn_last_error()
-
-
-def attn_inited():
-    import torch
-    return torch.cuda.is_available()
+    code = f"""
+import ctypes as C
+lib = C.CDLL({attn.LIB_PATH!r})
+lib.hipml_attn_last_error.restype = C.c_char_p
+one = C.c_void_p(16)
+rc = lib.hipml_gemv_q8_0_rows(None, one, one, one, 64, 64, 1)
+assert rc == -6 and b"hipml_attn_init" in lib.hipml_attn_last_error(), (rc, lib.hipml_attn_last_error())
+rc = lib.hipml_attn_decode_kv(None, one, 0, one, one, one, one, one, one, 24, 4, 256, 64, C.c_float(0.0625), 1,
+                              C.c_size_t(0), C.c_size_t(0))
+assert rc == -6 and b"hipml_attn_init" in lib.hipml_attn_last_error(), (rc, lib.hipml_attn_last_error())
+print("refused before init")
+"""
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0 and "refused before init" in r.stdout, r.stdout + r.stderr
 
 
 def test_header_is_plain_c_and_links_from_c(tmp_path):

@@ -53,6 +53,37 @@ def test_noalloc_decode_matches_decode_with_caller_scratch_twice():
     assert orc.compare(ref, got.ravel(), *KERNEL_CLASS)[0]
 
 
+def test_noalloc_decode_allocates_nothing_and_replays_from_a_graph():
+    # its namesake property: the device's free memory is the same before and after the calls; and the use it is
+    # for: captured into a HIP graph and replayed, with eager work between the replays
+    attn.init(0)
+    q, kb, vb = _case(0x70A110C4, 24, 4, 2000, 2048)
+    qd, kd, vd = dev(q), dev(kb), dev(vb)
+    step = step_buffer(1999, 2000)
+    eager = torch.full((24, HD), float("nan"), dtype=torch.float32, device="cuda")
+    out = torch.full((24, HD), float("nan"), dtype=torch.float32, device="cuda")
+    attn.attn_decode_kv_noalloc(step, 0, qd, kd, vd, eager, 24, 4, HD, 2048, SCALE, 16)  # (first call: code is loaded)
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info()
+    for _ in range(3):
+        attn.attn_decode_kv_noalloc(step, 0, qd, kd, vd, eager, 24, 4, HD, 2048, SCALE, 16)
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after == free_before
+    ref = orc.attn_decode_kv(q, kb, vb, 24, 4, HD, 2000, SCALE, stride=2048)
+    assert orc.compare(ref, host(eager).ravel(), *KERNEL_CLASS)[0]
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        attn.attn_decode_kv_noalloc(step, 0, qd, kd, vd, out, 24, 4, HD, 2048, SCALE, 16)
+    for i in range(3):
+        out.fill_(float("nan"))
+        attn.attn_decode_kv_noalloc(step, 0, qd, kd, vd, eager, 24, 4, HD, 2048, SCALE, 16)  # eager work between
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), f"replay {i}"
+
+
 def test_noalloc_decode_rejects_more_partials_than_the_array_holds():
     attn.init(0)
     q, kb, vb = _case(0x70A110C3, 24, 4, 64, 64)
