@@ -39,12 +39,11 @@ def hipcc() -> str:
 HAND_PLACED_ACC = [("prefill.hip", "chunk_f16_t64_kernel")]
 
 
-def check_hand_placed_acc(cc: str, flags: list[str], src: str, kernel: str) -> None:
-    """Fail the build if the compiler itself touches an accumulation register in `kernel` (it parks
-    vector registers there under pressure, which would overwrite the kernel's hand-placed state)."""
+def scan_hand_placed_acc(text: list[str], src: str, kernel: str) -> int:
+    """The check itself, over the lines of generated assembly: raises if `kernel` is missing, if code outside
+    its inline-assembly statements (the compiler's own) names an accumulation register, or if no statement
+    does (the scan looks at the wrong text); returns the number of lines inside statements that do."""
     import re
-    cmd = [cc] + COMMON + flags + ["-S", "--cuda-device-only", os.path.join(CSRC, src), "-o", "-"]
-    text = subprocess.run(cmd, check=True, capture_output=True, text=True).stdout.split("\n")
     start = [i for i, l in enumerate(text) if re.match(r"^_Z\w*" + kernel + r"\w*:", l)]
     if not start:
         raise RuntimeError(f"{src}: kernel {kernel} not found in the generated assembly")
@@ -66,6 +65,15 @@ def check_hand_placed_acc(cc: str, flags: list[str], src: str, kernel: str) -> N
                                    f"'{code.strip()}'")
     if n_inside == 0:
         raise RuntimeError(f"{src}: no accumulation register found in {kernel}: the check looks at the wrong text")
+    return n_inside
+
+
+def check_hand_placed_acc(cc: str, flags: list[str], src: str, kernel: str) -> None:
+    """Fail the build if the compiler itself touches an accumulation register in `kernel` (it parks
+    vector registers there under pressure, which would overwrite the kernel's hand-placed state)."""
+    cmd = [cc] + COMMON + flags + ["-S", "--cuda-device-only", os.path.join(CSRC, src), "-o", "-"]
+    text = subprocess.run(cmd, check=True, capture_output=True, text=True).stdout.split("\n")
+    scan_hand_placed_acc(text, src, kernel)
 
 
 def build_library(verbose: bool = False, extra: list[str] | None = None) -> str:

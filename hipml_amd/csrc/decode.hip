@@ -58,6 +58,36 @@ typedef int int2v __attribute__((ext_vector_type(2)));
 typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
 typedef uint32_t uint4a4 __attribute__((ext_vector_type(4), aligned(4)));
 
+// ---- phase stamps (instrumented builds only: -DHIPML_DECODE_STAMPS, see hipml_amd/decode_phases.py) ------
+// Wave 0 of every workgroup of decode_q8_kernel keeps the 100 MHz counter's value at up to kStampsPerWg points
+// in scalar registers and writes them out when the kernel is done with its own memory traffic (a store in
+// between would count among the requests the kernel's explicit waits are sized for).  Off, the macros are empty.
+constexpr int kStampsPerWg = 12, kStampWgs = 4096;
+#ifdef HIPML_DECODE_STAMPS
+static __device__ unsigned long long decode_stamps[kStampWgs * kStampsPerWg];
+struct Stamps { unsigned long long t[kStampsPerWg]; };
+#define HIPML_STAMPS_DECL Stamps stamps_ = {}
+#define HIPML_STAMP(st, i) ((st).t[i] = __builtin_amdgcn_s_memrealtime())
+#define HIPML_STAMPS_ARG , Stamps &stamps_
+#define HIPML_STAMPS_PASS , stamps_
+__device__ __forceinline__ void stamps_out(const Stamps &st)
+{
+    const unsigned wg = blockIdx.x + gridDim.x * blockIdx.y;
+    if (threadIdx.x == 0 && wg < kStampWgs)
+        for (int i = 0; i < kStampsPerWg; i++)
+            decode_stamps[wg * kStampsPerWg + i] = st.t[i];
+}
+int decode_read_stamps(unsigned long long *host, size_t n)
+{
+    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(decode_stamps), (n < (size_t)kStampWgs * kStampsPerWg ? n : (size_t)kStampWgs * kStampsPerWg) * sizeof(unsigned long long));
+}
+#else
+#define HIPML_STAMPS_DECL
+#define HIPML_STAMP(st, i) ((void)0)
+#define HIPML_STAMPS_ARG
+#define HIPML_STAMPS_PASS
+#endif
+
 constexpr int kMaxItems = 4 * kMaxSlots;               // work items of one launch (see DecodeArgs)
 constexpr int kTileKeys = 32;                         // keys per wave tile
 constexpr int kLdsRow = 288;                          // 256 payload bytes + 32 pad (bank spread)
@@ -942,7 +972,7 @@ __device__ __forceinline__ half8 raw_k_operand(const uint8_t *row_lg, int c)
 // is a real one, the two f16 halves of Q are two B operands and two MFMAs per block, and the raw Q rows
 // (16 KB) pass through the waves' V rows before the first V rows are requested.
 template <bool WIDE>
-__device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Work &wk)
+__device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Work &wk HIPML_STAMPS_ARG)
 {
     static_assert(kWaves * 2 * kScaleBytes <= kDmaQLds, "the scale tables reuse the Q staging area");
     constexpr int kCols = WIDE ? 16 : 8; // columns of an item
@@ -1067,6 +1097,7 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Work 
     issue(false, 0);
     if (!WIDE)
         issue(true, 0);
+    HIPML_STAMP(stamps_, 2); // the first requests have left
 
     const int hi = seq_max; // keys at or past it are masked
     if (split * kWaves * kTileKeys >= hi) {
@@ -1150,6 +1181,7 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Work 
         __syncthreads();
     }
     // (the staging area is the waves' scale tables from here on)
+    HIPML_STAMP(stamps_, 3); // Q operands in registers
 
     // per-column causal bound (MTP rows see one more key each)
     const int seq_n = qcol < nvalid ? seqc[qcol / group] : 0;
@@ -1201,6 +1233,10 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Work 
         // scores of tile t and V(t + 1) after its PV.
         // ---- K rows of this tile are in LDS once only the 9 loads of its V rows are outstanding
         asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
+#ifdef HIPML_DECODE_STAMPS
+        if (t == 0)
+            HIPML_STAMP(stamps_, 4); // K rows of the wave's first tile in LDS
+#endif
         build_scales(Kraw, sK, key0, partial);
 
         // ---- scores ----------------------------------------------------------------------------
@@ -1308,6 +1344,10 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Work 
             asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
         else
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#ifdef HIPML_DECODE_STAMPS
+        if (!more)
+            HIPML_STAMP(stamps_, 5); // V rows of the wave's last tile in LDS
+#endif
         build_scales(Vraw, sV, key0, partial);
 
         // ---- O^T += V^T . P' -------------------------------------------------------------------
@@ -1351,6 +1391,7 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Work 
             issue(true, t + 1);
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // (a wave without a tile still has its first K rows in flight)
+    HIPML_STAMP(stamps_, 6); // the wave's last tile is done
 
     // ---- merge the four waves and write the split's partial -------------------------------
     // Run j of O^T: lane holds byte columns 16j + lg*4 + i of the key rows for column n = lane%16.
@@ -1549,7 +1590,7 @@ __device__ __forceinline__ void fold_partials(const float *pa, const float *pm, 
 }
 
 template <bool WIDE>
-__device__ __forceinline__ void decode_merge_tail(const DecodeArgs &a, const Work &wk)
+__device__ __forceinline__ void decode_merge_tail(const DecodeArgs &a, const Work &wk HIPML_STAMPS_ARG)
 {
     constexpr int kCols = WIDE ? 16 : 8;
     constexpr int kDRuns = kThreads / kCols, kRun = kHeadDim / kDRuns; // as the partials were written
@@ -1559,7 +1600,9 @@ __device__ __forceinline__ void decode_merge_tail(const DecodeArgs &a, const Wor
     const int g0 = wk.split / kMergeGroup * kMergeGroup;
     const int gsize = a.splits - g0 < kMergeGroup ? a.splits - g0 : kMergeGroup;
     unsigned int *tk = a.tickets + (size_t)(wk.item * a.n_kv + wk.kvh) * (ngroup + 1);
-    if (!last_ticket(tk + g0 / kMergeGroup, (unsigned)gsize, flag))
+    const bool last1 = last_ticket(tk + g0 / kMergeGroup, (unsigned)gsize, flag);
+    HIPML_STAMP(stamps_, 8); // the ticket of the group has come back
+    if (!last1)
         return;
     const int nc = threadIdx.x / kDRuns;
     const int d0 = (threadIdx.x % kDRuns) * kRun;
@@ -1580,7 +1623,10 @@ __device__ __forceinline__ void decode_merge_tail(const DecodeArgs &a, const Wor
             if (threadIdx.x % kDRuns == 0)
                 store_dev(pm + (size_t)g0 * 2, (float2){M, L});
         }
-        if (!last_ticket(tk + ngroup, (unsigned)ngroup, flag))
+        HIPML_STAMP(stamps_, 9); // the group's partials folded and stored
+        const bool last2 = last_ticket(tk + ngroup, (unsigned)ngroup, flag);
+        HIPML_STAMP(stamps_, 10); // the ticket of the KV head has come back
+        if (!last2)
             return;
         if (mine)
             fold_partials<kRun>(pa, pm, 0, kMergeGroup, ngroup, M, L, A);
@@ -1605,18 +1651,28 @@ __device__ __forceinline__ void decode_merge_tail(const DecodeArgs &a, const Wor
 // One workgroup = one (KV head, key split, work item); the item's width picks the body.
 __global__ void __launch_bounds__(kThreads, 2) decode_q8_kernel(const DecodeArgs a)
 {
+    HIPML_STAMPS_DECL;
+    HIPML_STAMP(stamps_, 0); // the wave's first instruction
     Work wk;
     if (!find_work(a, threadIdx.x & 63, wk))
         return;
+    HIPML_STAMP(stamps_, 1); // work item found
     if (wk.nvalid > 8) { // uniform over the workgroup
-        decode_body_dma<true>(a, wk);
+        decode_body_dma<true>(a, wk HIPML_STAMPS_PASS);
+        HIPML_STAMP(stamps_, 7); // partial stored (not yet acknowledged)
         if (a.merge > 0)
-            decode_merge_tail<true>(a, wk);
+            decode_merge_tail<true>(a, wk HIPML_STAMPS_PASS);
     } else {
-        decode_body_dma<false>(a, wk);
+        decode_body_dma<false>(a, wk HIPML_STAMPS_PASS);
+        HIPML_STAMP(stamps_, 7);
         if (a.merge > 0)
-            decode_merge_tail<false>(a, wk);
+            decode_merge_tail<false>(a, wk HIPML_STAMPS_PASS);
     }
+#ifdef HIPML_DECODE_STAMPS
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    HIPML_STAMP(stamps_, 11); // everything this wave stored has been acknowledged
+    stamps_out(stamps_);
+#endif
 }
 
 // Wave-wide reductions without LDS: DPP inside a row of 16 lanes, then the two row-swap
@@ -2300,3 +2356,9 @@ int launch_decode_q8(hipStream_t st, const DecodeLaunch &given)
 }
 
 } // namespace hipml
+
+#ifdef HIPML_DECODE_STAMPS
+// Instrumented builds only: the stamps of the most recent decode_q8_kernel launch, [workgroup][12] ticks of the
+// 100 MHz counter (0 where a workgroup did not pass a point); returns a hipError_t.
+extern "C" int hipml_dbg_decode_stamps(unsigned long long *host, size_t n) { return hipml::decode_read_stamps(host, n); }
+#endif

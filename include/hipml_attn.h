@@ -66,7 +66,12 @@ int hipml_attn_init(int device);
 const char *hipml_attn_last_error(void);
 const char *hipml_attn_version(void);
 
-/* ---- split policies (host arithmetic, no GPU) ---------------------------- */
+/* ---- split policies (host arithmetic, no GPU) ----------------------------
+ * The three policies are tuned for the chip and the model this library is built for and say so nowhere in
+ * their arguments: 256 CUs in 8 XCDs (one or two workgroups per CU, windows of 256 or 512 workgroups), and 6
+ * query heads per KV head wherever a count depends on the heads (the chunk policies size task blocks and
+ * the tiles' room in the scratch for 6).  Other head groupings work with the counts they return; they are
+ * merely not the measured optimum there. */
 
 /* Key splits for single-sequence decode on MI355X.  Same role as
  * DeepKv::splits, crates/hipml-model/src/gpu/deep_kv.rs:102-110, retuned for
@@ -88,7 +93,18 @@ int hipml_attn_batch_splits(int stride, int n_kv, int slots);
  * and run the attention over those, which is faster than dequantizing inside the attention (2,048 tokens
  * at depth 100,000: n = 13 for 4 slices, 654 MB of scratch, 4.1 against 4.7 ms).  A caller that passes a
  * smaller n (the reference's own policy gives 8) gets n slices of the kernel that dequantizes for itself:
- * the scratch is never written beyond the n slices it was sized for. */
+ * the scratch is never written beyond the n slices it was sized for.
+ * How that count grows: the partial rows are ceil32(tokens) * n_heads * 1,024 bytes per slice (50.3 MB at
+ * 2,048 tokens and 24 heads), the tiles n_kv * ceil((pos0 + tokens) / 64) * 70,656 bytes (4.4 MB per 1,000
+ * rows of depth at 4 KV heads), so n = slices + ceil(tiles / partial rows of one slice): 2,048-token chunks
+ * at depth 32,768 / 100,000 / 200,000 / 400,000: 8 / 13 / 22 / 40, i.e. 0.40 / 0.65 / 1.1 / 2.0 GB.  The
+ * reference caps its scratch at 1 GiB (crates/hipml-model/src/gpu/prefill.rs:159-166); an engine that keeps
+ * that cap passes the count its allocation holds, and from ~195,000 positions on that is the kernel that
+ * dequantizes for itself again.  Counts above 64 are never returned (the plain slice count is, instead).
+ * An engine that registers its caches with hipml_kv_f16_attach needs none of this: the tiles then live
+ * in the cache's own shadow, the count only has to cover the slices that run (hipml_attn_chunk_slices:
+ * 4 at these shapes), and 8 is always enough.
+ * NOTE: unlike the reference's split_count, which is at least 1, this returns 0 near position 0. */
 int hipml_attn_chunk_splits(int pos0, int tokens, int n_kv);
 /* The slice count (>= 1) for callers that want the sliced kernel whatever the shape, and for
  * hipml_attn_chunk_kv_f16, which has no in-workgroup variant: what hipml_attn_chunk_splits
