@@ -140,6 +140,71 @@ struct DecodeArgs {
     uint8_t nhead[kMaxItems];  // heads of the item
 };
 
+// What a workgroup needs before it can ask for its first rows.  decode_q8_kernel takes these as leading scalar
+// kernel arguments, which arrive in registers with the wave (the argument structure behind them is fetched from
+// memory: a round trip of ~0.4 us before "work item found" while everything sat there); the staged kernels fill
+// the same view from the structure.
+struct Front {
+    const uint8_t *k, *v; // (a launch with one item: already at that item's slot)
+    const float *q;
+    const int32_t *pos;
+    int stride, splits, workers, items;
+    int i0_row0, i0_cols, i0_slot, i0_head0, i0_nhead;
+    int group, n_kv, stream_once;
+    uint32_t q_slot;
+    uint32_t karg_at; // where the argument structure lies in the kernel-argument segment
+};
+__device__ __forceinline__ Front front_of(const DecodeArgs &a)
+{
+    Front f;
+    f.k = a.k;
+    f.v = a.v;
+    f.q = a.q;
+    f.pos = a.pos;
+    f.stride = a.stride;
+    f.splits = a.splits;
+    f.workers = a.workers;
+    f.items = a.items;
+    f.i0_row0 = a.i0_row0;
+    f.i0_cols = a.i0_cols;
+    f.i0_slot = a.i0_slot;
+    f.i0_head0 = a.i0_head0;
+    f.i0_nhead = a.i0_nhead;
+    f.group = a.group;
+    f.n_kv = a.n_kv;
+    f.stream_once = a.stream_once;
+    f.q_slot = (uint32_t)a.q_slot;
+    f.karg_at = 0;
+    return f;
+}
+// The leading arguments of decode_q8_kernel, packed on the host (pack_front) and taken apart here.
+struct FrontWords { uint32_t wi, item0, geom; };
+__device__ __forceinline__ Front front_of(const uint8_t *k, const uint8_t *v, const float *q, const int32_t *pos, int stride,
+                                          int splits, uint32_t wi, uint32_t item0, uint32_t geom, uint32_t q_slot,
+                                          uint32_t karg_at)
+{
+    Front f;
+    f.k = k;
+    f.v = v;
+    f.q = q;
+    f.pos = pos;
+    f.stride = stride;
+    f.splits = splits;
+    f.workers = (int)(wi & 0xffffu);
+    f.items = (int)(wi >> 16);
+    f.i0_row0 = (int)(item0 & 0x3ffu);
+    f.i0_cols = (int)(item0 >> 10 & 7u);
+    f.i0_head0 = (int)(item0 >> 13 & 7u);
+    f.i0_nhead = (int)(item0 >> 16 & 15u);
+    f.i0_slot = (int)(item0 >> 20 & 0xffu);
+    f.group = (int)(geom & 15u);
+    f.n_kv = (int)(geom >> 4 & 0xffffu);
+    f.stream_once = (int)(geom >> 20 & 1u);
+    f.q_slot = q_slot;
+    f.karg_at = karg_at;
+    return f;
+}
+
 // 68 bytes of a key row starting at a block-pair boundary: [s0 | 32 x i8 | s1 | 32 x i8].
 struct Unit {
     uint4v a, b; // dwords 0..7:  s0 and the first 30 bytes of the even block
@@ -265,11 +330,11 @@ struct Work {
 };
 
 // Returns false when this workgroup has nothing to do (uniform over the workgroup).
-__device__ __forceinline__ bool find_work(const DecodeArgs &a, int lane, Work &wk)
+__device__ __forceinline__ bool find_work(const DecodeArgs &a, const Front &f, int lane, Work &wk)
 {
     // ---- which (kv head, item, split) this workgroup is ---------------------------------------
     // Plain launches: grid (n_kv * splits, items), every split of every item gets tiles.
-    // Worker launches (batches, a.workers > 0): grid (n_kv * workers).  The hardware starts the
+    // Worker launches (batches, f.workers > 0): grid (n_kv * workers).  The hardware starts the
     // workgroups of a launch in windows of as many as fit the chip (512 here) and opens the next
     // window only when the whole previous one has finished, so a workgroup with little or nothing to
     // do still holds its place for as long as the longest one of its window.  A batch has items of
@@ -284,25 +349,25 @@ __device__ __forceinline__ bool find_work(const DecodeArgs &a, int lane, Work &w
     // line only where the pointers are first used: two memory round trips one after the other.  A
     // condition over one field of each line asks for both at once (`stride` is positive, checked by
     // the launcher).
-    const bool worker_launch = (a.workers > 0) & (a.stride > 0);
+    const bool worker_launch = (f.workers > 0) & (f.stride > 0);
     if (worker_launch) {
-        kvh = blockIdx.x / a.workers;
-        const int w = blockIdx.x - kvh * a.workers;
+        kvh = blockIdx.x / f.workers;
+        const int w = blockIdx.x - kvh * f.workers;
         // lane i looks at item i (the launcher uses this mode for at most 64 items); item tables
         // are read through the kernel-argument pointer: a lane-indexed read of the by-value
         // argument struct would make the compiler copy its arrays to scratch
         typedef const __attribute__((address_space(4))) uint8_t *KargBytes;
         typedef const __attribute__((address_space(4))) uint16_t *KargHalves;
         const KargBytes ka = (KargBytes)__builtin_amdgcn_kernarg_segment_ptr();
-        const KargHalves t_row0 = (KargHalves)(ka + offsetof(DecodeArgs, row0));
-        const KargBytes t_cols = ka + offsetof(DecodeArgs, cols);
+        const KargHalves t_row0 = (KargHalves)(ka + f.karg_at + offsetof(DecodeArgs, row0));
+        const KargBytes t_cols = ka + f.karg_at + offsetof(DecodeArgs, cols);
         int tiles = 0;
-        if (lane < a.items) {
+        if (lane < f.items) {
             const int r0 = t_row0[lane], nc = t_cols[lane];
             int sm = 0;
             for (int c = 0; c < nc; c++) {
-                int v = a.pos[(size_t)(r0 + c) * 2 + 1];
-                v = v < 0 ? 0 : (v > a.stride ? a.stride : v);
+                int v = f.pos[(size_t)(r0 + c) * 2 + 1];
+                v = v < 0 ? 0 : (v > f.stride ? f.stride : v);
                 sm = v > sm ? v : sm;
             }
             tiles = (sm + kTileKeys - 1) / kTileKeys;
@@ -320,20 +385,20 @@ __device__ __forceinline__ bool find_work(const DecodeArgs &a, int lane, Work &w
         }
         auto share_at = [&](int t) {
             int sh = 0;
-            if (lane < a.items) {
+            if (lane < f.items) {
                 // ceil(tiles / t) through a float quotient (tiles < 2^24: exact or one too many at a
                 // multiple, corrected below); every wave computes the same values
                 sh = (int)((float)tiles / (float)t);
                 sh += sh * t < tiles ? 1 : 0;
                 sh -= (sh - 1) * t >= tiles && sh > 0 ? 1 : 0;
-                sh = sh < 1 ? 1 : (sh < a.splits ? sh : a.splits);
+                sh = sh < 1 ? 1 : (sh < f.splits ? sh : f.splits);
             }
             return sh;
         };
         // T lies between total / workers and total / (workers - items) (each share is below
         // tiles / T + 1), so the search is a few steps
-        const int spare = a.workers - a.items;
-        int lo = (total + a.workers - 1) / a.workers;
+        const int spare = f.workers - f.items;
+        int lo = (total + f.workers - 1) / f.workers;
         lo = lo < 1 ? 1 : lo;
         int hi = spare > 0 ? (total + spare - 1) / spare : (tmax > 1 ? tmax : 1);
         hi = hi < lo ? lo : hi;
@@ -343,7 +408,7 @@ __device__ __forceinline__ bool find_work(const DecodeArgs &a, int lane, Work &w
 #pragma unroll
             for (int off = 32; off > 0; off >>= 1)
                 need += __shfl_xor(need, off);
-            if (need <= a.workers)
+            if (need <= f.workers)
                 hi = mid;
             else
                 lo = mid + 1;
@@ -355,7 +420,7 @@ __device__ __forceinline__ bool find_work(const DecodeArgs &a, int lane, Work &w
             const int up = __shfl_up(end, off);
             end += lane >= off ? up : 0;
         }
-        const unsigned long long hit = __ballot(lane < a.items && w >= end - share && w < end);
+        const unsigned long long hit = __ballot(lane < f.items && w >= end - share && w < end);
         if (hit == 0)
             return false; // more workers than the shares add up to (uniform over the workgroup)
         item = __builtin_ctzll(hit);
@@ -365,10 +430,10 @@ __device__ __forceinline__ bool find_work(const DecodeArgs &a, int lane, Work &w
         nsp = __builtin_amdgcn_readfirstlane(nsp);
         split = __builtin_amdgcn_readfirstlane(split);
     } else {
-        kvh = blockIdx.x / a.splits;
-        split = blockIdx.x - kvh * a.splits;
+        kvh = blockIdx.x / f.splits;
+        split = blockIdx.x - kvh * f.splits;
         item = blockIdx.y;
-        nsp = a.splits;
+        nsp = f.splits;
     }
     // The item tables are byte arrays read with vector loads, and the item is the same for every lane.
     // Taking the values through readfirstlane puts them in scalar registers and, more to the point,
@@ -376,12 +441,12 @@ __device__ __forceinline__ bool find_work(const DecodeArgs &a, int lane, Work &w
     // below come later in the same in-order queue, so a first use behind them would wait for the Q
     // rows as well, and the first tile could only be requested once those had arrived.
     int slot, row0, ncols, group, head0; // group = heads of this item: columns are (row, head) pairs over them
-    if (a.items == 1) {
-        slot = a.i0_slot;
-        row0 = a.i0_row0;
-        ncols = a.i0_cols;
-        group = a.i0_nhead;
-        head0 = a.i0_head0;
+    if (f.items == 1) {
+        slot = f.i0_slot;
+        row0 = f.i0_row0;
+        ncols = f.i0_cols;
+        group = f.i0_nhead;
+        head0 = f.i0_head0;
     } else {
         slot = __builtin_amdgcn_readfirstlane((int)a.kvslot[item]);
         row0 = __builtin_amdgcn_readfirstlane((int)a.row0[item]);
@@ -389,16 +454,16 @@ __device__ __forceinline__ bool find_work(const DecodeArgs &a, int lane, Work &w
         group = __builtin_amdgcn_readfirstlane((int)a.nhead[item]);
         head0 = __builtin_amdgcn_readfirstlane((int)a.head0[item]);
     }
-    const int hbase = kvh * a.group + head0;
+    const int hbase = kvh * f.group + head0;
     const int nvalid = ncols * group;
-    if (a.workers > 0 && split == 0 && nsp < a.splits) {
+    if (f.workers > 0 && split == 0 && nsp < f.splits) {
         // the splits of this item that no worker takes: empty partials, which the merge skips
-        const int empty = a.splits - nsp;
+        const int empty = f.splits - nsp;
         for (int e = threadIdx.x; e < nvalid * empty; e += (int)blockDim.x) {
             const int n = e / empty, sp = nsp + (e - n * empty);
             const int col = n / group;
             const int head = hbase + (n - col * group);
-            float *pm = a.part_ml + (size_t)(row0 + col) * a.ml_slot + ((size_t)head * a.splits + sp) * 2;
+            float *pm = a.part_ml + (size_t)(row0 + col) * a.ml_slot + ((size_t)head * f.splits + sp) * 2;
             pm[0] = -INFINITY;
             pm[1] = 0.0f;
         }
@@ -434,8 +499,9 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
     const int lane = threadIdx.x & 63;
     const int lm = lane & 15; // MFMA row/col within the 16-tile
     const int lg = lane >> 4; // k-group
+    const Front f = front_of(a);
     Work wk;
-    if (!find_work(a, lane, wk))
+    if (!find_work(a, f, lane, wk))
         return;
     const int kvh = wk.kvh, split = wk.split, nsp = wk.nsp, slot = wk.slot, row0 = wk.row0, ncols = wk.ncols,
               group = wk.group, hbase = wk.hbase, nvalid = wk.nvalid;
@@ -444,8 +510,8 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
     uint8_t *sK = tile_lds + kTileBytes;
     uint8_t *sV = sK + kScaleBytes;
 
-    const uint8_t *kbase = a.k + (size_t)slot * a.kv_slot_bytes + (size_t)kvh * a.stride * kRowBytes;
-    const uint8_t *vbase = a.v + (size_t)slot * a.kv_slot_bytes + (size_t)kvh * a.stride * kRowBytes;
+    const uint8_t *kbase = f.k + (size_t)slot * a.kv_slot_bytes + (size_t)kvh * f.stride * kRowBytes;
+    const uint8_t *vbase = f.v + (size_t)slot * a.kv_slot_bytes + (size_t)kvh * f.stride * kRowBytes;
 
     // ---- key tiles of this wave ---------------------------------------------------------------
     // The 32-key tiles of a KV head are dealt round-robin: tile g belongs to split (g / kWaves)
@@ -460,7 +526,7 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
     Unit Kst[2], Vst[2];
     // unit j of a tile: u = lane + 64*j -> tile row u/4, block pair u%4
     const int ur0 = lane >> 2, ur1 = 16 + (lane >> 2), upr = lane & 3;
-    const int last_row = a.stride - 1;
+    const int last_row = f.stride - 1;
     auto issue = [&](Unit (&dst)[2], const uint8_t *base, int t) {
         const int key0 = tile_key0(t);
         int ka = key0 + ur0, kb = key0 + ur1;
@@ -484,7 +550,7 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
         if (n < nvalid) {
             const int col = n / group;
             const int head = n - col * group;
-            const float *qp = a.q + (size_t)(row0 + col) * a.q_slot +
+            const float *qp = f.q + (size_t)(row0 + col) * f.q_slot +
                               (size_t)(hbase + head) * kHeadDim + c * 32 + (l >> 4) * 8;
             qf[k][0] = *reinterpret_cast<const float4v *>(qp);
             qf[k][1] = *reinterpret_cast<const float4v *>(qp + 4);
@@ -501,8 +567,8 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
     int seq_max = 0;
 #pragma unroll
     for (int c = 0; c < kMaxCols; c++) {
-        int s = c < ncols ? a.pos[(size_t)(row0 + c) * 2 + 1] : 0;
-        s = s < 0 ? 0 : (s > a.stride ? a.stride : s);
+        int s = c < ncols ? f.pos[(size_t)(row0 + c) * 2 + 1] : 0;
+        s = s < 0 ? 0 : (s > f.stride ? f.stride : s);
         seqc[c] = s;
         seq_max = s > seq_max ? s : seq_max;
     }
@@ -513,7 +579,7 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
         if ((int)threadIdx.x < nvalid) {
             const int col = threadIdx.x / group;
             const int head = hbase + (threadIdx.x - col * group);
-            float *pm = a.part_ml + (size_t)(row0 + col) * a.ml_slot + ((size_t)head * a.splits + split) * 2;
+            float *pm = a.part_ml + (size_t)(row0 + col) * a.ml_slot + ((size_t)head * f.splits + split) * 2;
             pm[0] = -INFINITY;
             pm[1] = 0.0f;
         }
@@ -809,7 +875,7 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &a)
                 }
                 const int col = ng / group;
                 const int head = hbase + (ng - col * group);
-                const size_t slice = (size_t)head * a.splits + split;
+                const size_t slice = (size_t)head * f.splits + split;
                 float *pa = a.part_acc + (size_t)(row0 + col) * a.acc_slot + slice * kHeadDim + d0;
 #pragma unroll
                 for (int dd = 0; dd < kRun; dd += 4) {
@@ -972,7 +1038,7 @@ __device__ __forceinline__ half8 raw_k_operand(const uint8_t *row_lg, int c)
 // is a real one, the two f16 halves of Q are two B operands and two MFMAs per block, and the raw Q rows
 // (16 KB) pass through the waves' V rows before the first V rows are requested.
 template <bool WIDE>
-__device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Work &wk HIPML_STAMPS_ARG)
+__device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Front &f, const Work &wk HIPML_STAMPS_ARG)
 {
     static_assert(kWaves * 2 * kScaleBytes <= kDmaQLds, "the scale tables reuse the Q staging area");
     constexpr int kCols = WIDE ? 16 : 8; // columns of an item
@@ -994,22 +1060,24 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Work 
     uint8_t *sV = sK + kScaleBytes;
     const uint32_t wave_at = lds_address(wave_lds);
 
-    const uint8_t *kbase = a.k + (size_t)slot * a.kv_slot_bytes + (size_t)kvh * a.stride * kRowBytes;
-    const uint8_t *vbase = a.v + (size_t)slot * a.kv_slot_bytes + (size_t)kvh * a.stride * kRowBytes;
+    // (a launch with one item gets its cache pointers at that item's slot: nothing to fetch for the address)
+    const size_t slot_at = f.items == 1 ? 0 : (size_t)slot * a.kv_slot_bytes;
+    const uint8_t *kbase = f.k + slot_at + (size_t)kvh * f.stride * kRowBytes;
+    const uint8_t *vbase = f.v + slot_at + (size_t)kvh * f.stride * kRowBytes;
 
     // tile g of a KV head belongs to split (g / kWaves) % nsp, wave g % kWaves (see the staged kernel)
     auto tile_key0 = [&](int t) { return ((t * nsp + split) * kWaves + wave) * kTileKeys; };
 
     // ---- one tile of rows = 8,704 contiguous bytes = 8.5 instructions of 1 KiB ------------------
     const uint32_t lane16 = lane * 16;
-    const uint32_t region_last = (uint32_t)a.stride * kRowBytes - 16; // last 16 bytes of a KV head's rows
+    const uint32_t region_last = (uint32_t)f.stride * kRowBytes - 16; // last 16 bytes of a KV head's rows
     auto issue_as = [&](auto once, bool v_rows, int t) {
         constexpr bool kOnce = decltype(once)::value;
         const uint32_t lds_at = wave_at + (v_rows ? kRawTile : 0);
         const uint8_t *region = v_rows ? vbase : kbase;
         const int key0 = tile_key0(t);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // the wave's own reads of the old rows are done
-        if (key0 + kTileKeys <= a.stride) { // (uniform) the tile lies inside the cache
+        if (key0 + kTileKeys <= f.stride) { // (uniform) the tile lies inside the cache
             const uint8_t *src = region + (size_t)key0 * kRowBytes;
 #pragma unroll
             for (int j = 0; j < 8; j++)
@@ -1032,7 +1100,7 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Work 
         }
     };
     // (an item that carries every head of its KV head is its slot's only reader of these rows)
-    const bool once = a.stream_once != 0 || group == a.group;
+    const bool once = f.stream_once != 0 || group == f.group;
     auto issue = [&](bool v_rows, int t) {
         if (once)
             issue_as(std::true_type(), v_rows, t);
@@ -1046,15 +1114,15 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Work 
     int seq_max = 0;
 #pragma unroll
     for (int c = 0; c < kMaxCols; c++) {
-        int s = c < ncols ? a.pos[(size_t)(row0 + c) * 2 + 1] : 0;
-        s = s < 0 ? 0 : (s > a.stride ? a.stride : s);
+        int s = c < ncols ? f.pos[(size_t)(row0 + c) * 2 + 1] : 0;
+        s = s < 0 ? 0 : (s > f.stride ? f.stride : s);
         seqc[c] = s;
         seq_max = s > seq_max ? s : seq_max;
     }
 
-    // ---- the first requests: the Q rows, then K and V rows of tile 0 ---------------------------
+    // ---- the first requests: the Q rows, then the K rows of tile 0 ------------------------------
     // No address here needs anything from device memory (a tile past the live rows costs one load of
-    // rows inside the cache and is masked out), so all 20 requests leave before the first wait.
+    // rows inside the cache and is masked out), so these 11 requests leave before the first wait.
     // The item has at most 8 (row, head) columns.  MFMA column lm < 8 carries the f16 value of Q column
     // lm, MFMA column lm + 8 what that rounding left over (x - f16(x), again as f16): the two halves
     // of a score are added after the block loop, so Q enters with ~22 bits at the price of one
@@ -1080,11 +1148,11 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Work 
         const int head = fcol - col * group;
         const int kg = WIDE ? (lane >> 4) : ((lane >> 3) & 3);
         // (per-lane byte offsets from the uniform base: the Q rows of a launch are far below 4 GB)
-        const uint32_t qoff = (uint32_t)(((size_t)(row0 + col) * a.q_slot + (size_t)(hbase + head) * kHeadDim +
+        const uint32_t qoff = (uint32_t)(((size_t)(row0 + col) * f.q_slot + (size_t)(hbase + head) * kHeadDim +
                                           wave * (kQB * 32) + kg * 8 + (WIDE ? 0 : (lane >> 5) * 4)) *
                                          sizeof(float));
         const uint32_t at = lds_address(Qraw);
-        const uint8_t *qb = reinterpret_cast<const uint8_t *>(a.q);
+        const uint8_t *qb = reinterpret_cast<const uint8_t *>(f.q);
         if (WIDE) {
 #pragma unroll
             for (int i = 0; i < 4; i++)
@@ -1095,8 +1163,6 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Work 
         }
     }
     issue(false, 0);
-    if (!WIDE)
-        issue(true, 0);
     HIPML_STAMP(stamps_, 2); // the first requests have left
 
     const int hi = seq_max; // keys at or past it are masked
@@ -1105,7 +1171,7 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Work 
         if ((int)threadIdx.x < nvalid) {
             const int col = threadIdx.x / group;
             const int head = hbase + (threadIdx.x - col * group);
-            float *pm = a.part_ml + (size_t)(row0 + col) * a.ml_slot + ((size_t)head * a.splits + split) * 2;
+            float *pm = a.part_ml + (size_t)(row0 + col) * a.ml_slot + ((size_t)head * f.splits + split) * 2;
             store_dev(pm, (float2){-INFINITY, 0.0f});
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // nothing may land in LDS after the wave has gone
@@ -1115,11 +1181,8 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Work 
     const int ntile = first_key < hi ? (hi - first_key + step_keys - 1) / step_keys : 0;
 
     // ---- Q operands and the score bias of every block ------------------------------------------
-    // the Q rows are in LDS once only the requests behind them are outstanding: K(0) [and V(0)]
-    if (WIDE)
-        asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
-    else
-        asm volatile("s_waitcnt vmcnt(18)" ::: "memory");
+    // the Q rows are in LDS once only the requests behind them are outstanding: K(0)
+    asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
     float4v qf[kQB][2];
 #pragma unroll
     for (int cc = 0; cc < kQB; cc++)
@@ -1162,8 +1225,12 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Work 
             *reinterpret_cast<float4v *>(CBs + (c * 16 + lm) * 16) = (float4v){cb, cb, cb, cb};
         }
     }
-    if (WIDE)
-        issue(true, 0); // the raw Q values have left the V rows
+    // The V rows of tile 0 are requested only now.  Asked for together with the K rows they make the launch's
+    // first burst 18 MB, which the memory pipeline takes 3 us to accept: the waves sat in those requests while
+    // their Q rows had long arrived, and the first scores, and with them the request for the next K rows, came
+    // that much later (measured: 18.4 against 19.0 us per layer at depth 32,768, 10.3 against 10.9 at 8,192).
+    // (WIDE: the raw Q values have left the V rows by now.)
+    issue(true, 0);
     __syncthreads();
     half8 bh[8], bl[WIDE ? 8 : 1];
 #pragma unroll
@@ -1479,7 +1546,7 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Work 
             }
             const int col = nc / group;
             const int head = hbase + (nc - col * group);
-            const size_t slice = (size_t)head * a.splits + split;
+            const size_t slice = (size_t)head * f.splits + split;
             float *pa = a.part_acc + (size_t)(row0 + col) * a.acc_slot + slice * kHeadDim + d0;
 #pragma unroll
             for (int dd = 0; dd < kRun; dd += 4) {
@@ -1649,21 +1716,34 @@ __device__ __forceinline__ void decode_merge_tail(const DecodeArgs &a, const Wor
 }
 
 // One workgroup = one (KV head, key split, work item); the item's width picks the body.
-__global__ void __launch_bounds__(kThreads, 2) decode_q8_kernel(const DecodeArgs a)
+// The kernel-argument segment of decode_q8_kernel, as the parameter list lays it out.
+struct DecodeKernarg {
+    const uint8_t *k, *v;
+    const float *q;
+    const int32_t *pos;
+    int stride, splits;
+    uint32_t wi, item0, geom, q_slot;
+    DecodeArgs a;
+};
+
+__global__ void __launch_bounds__(kThreads, 2)
+    decode_q8_kernel(const uint8_t *k, const uint8_t *v, const float *q, const int32_t *pos, int stride, int splits,
+                     uint32_t wi, uint32_t item0, uint32_t geom, uint32_t q_slot, const DecodeArgs a)
 {
     HIPML_STAMPS_DECL;
     HIPML_STAMP(stamps_, 0); // the wave's first instruction
+    const Front f = front_of(k, v, q, pos, stride, splits, wi, item0, geom, q_slot, (uint32_t)offsetof(DecodeKernarg, a));
     Work wk;
-    if (!find_work(a, threadIdx.x & 63, wk))
+    if (!find_work(a, f, threadIdx.x & 63, wk))
         return;
     HIPML_STAMP(stamps_, 1); // work item found
     if (wk.nvalid > 8) { // uniform over the workgroup
-        decode_body_dma<true>(a, wk HIPML_STAMPS_PASS);
+        decode_body_dma<true>(a, f, wk HIPML_STAMPS_PASS);
         HIPML_STAMP(stamps_, 7); // partial stored (not yet acknowledged)
         if (a.merge > 0)
             decode_merge_tail<true>(a, wk HIPML_STAMPS_PASS);
     } else {
-        decode_body_dma<false>(a, wk HIPML_STAMPS_PASS);
+        decode_body_dma<false>(a, f, wk HIPML_STAMPS_PASS);
         HIPML_STAMP(stamps_, 7);
         if (a.merge > 0)
             decode_merge_tail<false>(a, wk HIPML_STAMPS_PASS);
@@ -2308,8 +2388,16 @@ int launch_decode_q8(hipStream_t st, const DecodeLaunch &given)
         a.tickets = decode_tickets(st, items * L.n_kv * (ngroup + 1));
         a.merge = a.tickets != nullptr ? kMergeGroup : 0;
     }
-    if (raw_rows)
-        HIPML_LAUNCH(decode_q8_kernel, grid, dim3(kThreads, 1, 1), kDmaLds, st, a);
+    if (raw_rows) {
+        // the leading arguments (see Front): a launch with one item gets its caches at that item's slot
+        const size_t slot_at = items == 1 ? (size_t)a.i0_slot * a.kv_slot_bytes : 0;
+        const uint32_t wi = (uint32_t)a.workers | (uint32_t)items << 16;
+        const uint32_t item0 = (uint32_t)a.i0_row0 | (uint32_t)a.i0_cols << 10 | (uint32_t)a.i0_head0 << 13 |
+                               (uint32_t)a.i0_nhead << 16 | (uint32_t)a.i0_slot << 20;
+        const uint32_t geom = (uint32_t)a.group | (uint32_t)a.n_kv << 4 | (uint32_t)a.stream_once << 20;
+        HIPML_LAUNCH(decode_q8_kernel, grid, dim3(kThreads, 1, 1), kDmaLds, st, a.k + slot_at, a.v + slot_at, a.q, a.pos,
+                     a.stride, a.splits, wi, item0, geom, (uint32_t)a.q_slot, a);
+    }
     else if (L.q4)
         HIPML_LAUNCH((decode_staged_kernel<true, false>), grid, dim3(kThreads, 1, 1), decode_lds_bytes(1), st, a);
     else

@@ -37,10 +37,11 @@ def build() -> str:
 
 
 def run(seq: int, launches: int) -> None:
-    os.environ["HIPML_ATTN_LIB"] = STAMPS_LIB
     import numpy as np
     import torch
     from hipml_amd import attn
+    assert attn._lib is None, "the library is already loaded"
+    attn.LIB_PATH = STAMPS_LIB  # the instrumented build instead of the shipped one
     attn.init(0)
     H, KV, HD, layers = 24, 4, 256, 16
     gen = torch.Generator(device="cuda")
