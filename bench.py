@@ -455,8 +455,9 @@ def bench_decode(torch, attn, seq, steps, warmup, layers, dtype=0, one_launch=Fa
         "workload": f"decode 1 query @ depth {seq}, {'q8_0' if dtype == 0 else 'q4_0'} cache, "
                     f"split-K {splits} + merge",
         "seq": seq, "splits": splits, "layers_rotated": layers,
-        # (the scratch is sized for `splits`; over q8_0 one sequence runs at most one workgroup per CU)
-        "splits_run": min(splits, max(256 // KV, 1)) if dtype == 0 else splits,
+        # (the scratch is sized for `splits`; one sequence runs at most one workgroup per CU over q8_0, and
+        # over q4_0 below 24,576 rows)
+        "splits_run": min(splits, max(256 // KV, 1)) if dtype == 0 or stride < 24576 else splits,
         "us_per_layer": us, "timed_ms": total, "steps_timed": n,
         "us_per_layer_gate_fused": tg,
         "us_per_layer_gate_separate": ts,
@@ -466,7 +467,7 @@ def bench_decode(torch, attn, seq, steps, warmup, layers, dtype=0, one_launch=Fa
                      "frac": gbs / HBM_PEAK_GBS, "traffic": traffic,
                      "achievable": ys["achievable"], "frac_of_achievable": gbs / ys["achievable"],
                      "kernel": "decode_q8_kernel + decode_reduce128_kernel" if dtype == 0 else
-                     "decode_staged_kernel + decode_reduce128_kernel",
+                     "decode_q4_kernel + decode_reduce128_kernel",
                      "bytes_per_launch": nbytes, "launch_us": us, "timed_ms": total, "steps_timed": n},
     }
 

@@ -1034,14 +1034,48 @@ __device__ __forceinline__ half8 raw_k_operand(const uint8_t *row_lg, int c)
     return __builtin_bit_cast(half8, r);
 }
 
+// The same for a q4_0 row: k-group lg of block c = the low (shift 0) or high (shift 4) nibbles of the 8 payload
+// bytes [8 (lg & 1), + 8) of the block; `row_b` = row + 8 (lg & 1).  A payload starts 2 bytes into its 18-byte
+// block: dword aligned in odd blocks, 2 bytes into a dword in even ones, as in a q8_0 row.  The nibble enters as
+// n * 2^-24 (values n - 8: the offset comes off through the score bias, as the q8_0 offset of 128 does).
+__device__ __forceinline__ half8 raw_k_operand_q4(const uint8_t *row_b, int c, int shift)
+{
+    uint4v r;
+    if (c & 1) {
+        const uint32_t *p = reinterpret_cast<const uint32_t *>(row_b + c * kQ4BlockBytes + 2);
+        const uint32_t x0 = (p[0] >> shift) & 0x0f0f0f0fu, x1 = (p[1] >> shift) & 0x0f0f0f0fu;
+        r[0] = __builtin_amdgcn_perm(0u, x0, 0x0c010c00u);
+        r[1] = __builtin_amdgcn_perm(0u, x0, 0x0c030c02u);
+        r[2] = __builtin_amdgcn_perm(0u, x1, 0x0c010c00u);
+        r[3] = __builtin_amdgcn_perm(0u, x1, 0x0c030c02u);
+    } else {
+        const uint32_t *p = reinterpret_cast<const uint32_t *>(row_b + c * kQ4BlockBytes);
+        const uint32_t x0 = (p[0] >> shift) & 0x0f0f0f0fu, x1 = (p[1] >> shift) & 0x0f0f0f0fu,
+                       x2 = (p[2] >> shift) & 0x0f0f0f0fu;
+        r[0] = __builtin_amdgcn_perm(0u, x0, 0x0c030c02u);
+        r[1] = __builtin_amdgcn_perm(0u, x1, 0x0c010c00u);
+        r[2] = __builtin_amdgcn_perm(0u, x1, 0x0c030c02u);
+        r[3] = __builtin_amdgcn_perm(0u, x2, 0x0c010c00u);
+    }
+    return __builtin_bit_cast(half8, r);
+}
+
 // WIDE: the item has 9 to 16 (row, head) columns (rows of an MTP-verify slot).  Then every MFMA column
 // is a real one, the two f16 halves of Q are two B operands and two MFMAs per block, and the raw Q rows
 // (16 KB) pass through the waves' V rows before the first V rows are requested.
-template <bool WIDE>
+template <bool WIDE, bool Q4 = false>
 __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Front &f, const Work &wk HIPML_STAMPS_ARG)
 {
     static_assert(kWaves * 2 * kScaleBytes <= kDmaQLds, "the scale tables reuse the Q staging area");
+    static_assert(!(WIDE && Q4), "q4_0 rows are served in items of at most 8 columns");
     constexpr int kCols = WIDE ? 16 : 8; // columns of an item
+    // q4_0 (Q4): a row is 144 bytes = 9 aligned 16-byte runs, a tile of 32 rows 4,608 bytes = 4.5 requests of
+    // 1 KiB; byte j of a block holds element j in its low and element j + 16 in its high nibble
+    // (crates/hipml-core/src/kv.rs:201-218), values n - 8.
+    constexpr int kRowB = Q4 ? kRowBytesQ4 : kRowBytes;
+    constexpr int kBlkB = Q4 ? kQ4BlockBytes : kQ8BlockBytes;
+    constexpr int kRawT = kTileKeys * kRowB;     // 8,704 / 4,608: one tile of rows as they lie in the cache
+    constexpr int kReq = Q4 ? 5 : 9;             // requests per tile of rows (the last one half a wave)
     constexpr int kDmaWaveLds = kDmaTileLds;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds_all[];
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
@@ -1053,7 +1087,7 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Front
 
     uint8_t *wave_lds = lds_all + wave * kDmaWaveLds;
     uint8_t *Kraw = wave_lds;
-    uint8_t *Vraw = wave_lds + kRawTile;
+    uint8_t *Vraw = wave_lds + kRawT;
     uint8_t *Qst = lds_all + kWaves * kDmaWaveLds;
     uint8_t *CBs = Qst + kDmaQLds;
     uint8_t *sK = Qst + wave * 2 * kScaleBytes;
@@ -1062,40 +1096,40 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Front
 
     // (a launch with one item gets its cache pointers at that item's slot: nothing to fetch for the address)
     const size_t slot_at = f.items == 1 ? 0 : (size_t)slot * a.kv_slot_bytes;
-    const uint8_t *kbase = f.k + slot_at + (size_t)kvh * f.stride * kRowBytes;
-    const uint8_t *vbase = f.v + slot_at + (size_t)kvh * f.stride * kRowBytes;
+    const uint8_t *kbase = f.k + slot_at + (size_t)kvh * f.stride * kRowB;
+    const uint8_t *vbase = f.v + slot_at + (size_t)kvh * f.stride * kRowB;
 
     // tile g of a KV head belongs to split (g / kWaves) % nsp, wave g % kWaves (see the staged kernel)
     auto tile_key0 = [&](int t) { return ((t * nsp + split) * kWaves + wave) * kTileKeys; };
 
     // ---- one tile of rows = 8,704 contiguous bytes = 8.5 instructions of 1 KiB ------------------
     const uint32_t lane16 = lane * 16;
-    const uint32_t region_last = (uint32_t)f.stride * kRowBytes - 16; // last 16 bytes of a KV head's rows
+    const uint32_t region_last = (uint32_t)f.stride * kRowB - 16; // last 16 bytes of a KV head's rows
     auto issue_as = [&](auto once, bool v_rows, int t) {
         constexpr bool kOnce = decltype(once)::value;
-        const uint32_t lds_at = wave_at + (v_rows ? kRawTile : 0);
+        const uint32_t lds_at = wave_at + (v_rows ? kRawT : 0);
         const uint8_t *region = v_rows ? vbase : kbase;
         const int key0 = tile_key0(t);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // the wave's own reads of the old rows are done
         if (key0 + kTileKeys <= f.stride) { // (uniform) the tile lies inside the cache
-            const uint8_t *src = region + (size_t)key0 * kRowBytes;
+            const uint8_t *src = region + (size_t)key0 * kRowB;
 #pragma unroll
-            for (int j = 0; j < 8; j++)
+            for (int j = 0; j < kReq - 1; j++)
                 dma16<kOnce>(lds_at + j * 1024, src + j * 1024, lane16);
             if (lane < 32)
-                dma16<kOnce>(lds_at + 8192, src + 8192, lane16);
+                dma16<kOnce>(lds_at + (kReq - 1) * 1024, src + (kReq - 1) * 1024, lane16);
         } else {
             // the last rows of the cache: bytes past its end are replaced by its last 16 (rows at or
             // past the live length are masked whatever they hold)
-            const uint32_t off0 = (uint32_t)key0 * kRowBytes + lane16;
+            const uint32_t off0 = (uint32_t)key0 * kRowB + lane16;
 #pragma unroll
-            for (int j = 0; j < 8; j++) {
+            for (int j = 0; j < kReq - 1; j++) {
                 const uint32_t o = off0 + j * 1024;
                 dma16<kOnce>(lds_at + j * 1024, region, o < region_last ? o : region_last);
             }
             if (lane < 32) {
-                const uint32_t o = off0 + 8192;
-                dma16<kOnce>(lds_at + 8192, region, o < region_last ? o : region_last);
+                const uint32_t o = off0 + (kReq - 1) * 1024;
+                dma16<kOnce>(lds_at + (kReq - 1) * 1024, region, o < region_last ? o : region_last);
             }
         }
     };
@@ -1165,6 +1199,13 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Front
     issue(false, 0);
     HIPML_STAMP(stamps_, 2); // the first requests have left
 
+    // all but the newest tile of rows have arrived (requests return in the order of issue)
+    auto wait_all_but_one_tile = [] {
+        if (Q4)
+            asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
+        else
+            asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
+    };
     const int hi = seq_max; // keys at or past it are masked
     if (split * kWaves * kTileKeys >= hi) {
         // not one live tile for any wave of this workgroup: leave an empty partial, which the merge skips
@@ -1182,7 +1223,7 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Front
 
     // ---- Q operands and the score bias of every block ------------------------------------------
     // the Q rows are in LDS once only the requests behind them are outstanding: K(0)
-    asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
+    wait_all_but_one_tile();
     float4v qf[kQB][2];
 #pragma unroll
     for (int cc = 0; cc < kQB; cc++)
@@ -1211,7 +1252,7 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Front
             h8[j] = h;
         }
         sum = quad_rows<false>(sum); // over the four k-groups: the block's 32 values of MFMA column lm
-        const float cb = -128.0f / kTwo24 * sum;
+        const float cb = (Q4 ? -8.0f : -128.0f) / kTwo24 * sum; // the offset the K bytes (nibbles) carry
         // (narrow: the wave's own quarter: every lane has read its raw values, LDS works in program order)
         *reinterpret_cast<half8 *>(Qst + (c * 64 + lane) * 16) = h8;
         if (WIDE) {
@@ -1255,16 +1296,26 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Front
 
     // ---- running state ----------------------------------------------------------------------
     float m_run = -INFINITY, l_run = 0.0f;
-    float4v O[kAccs], B7 = {0, 0, 0, 0};
+    // q8_0: 23 accumulators over the 17 runs of a row (see above); q4_0: two per run of its 9, low and high nibbles
+    constexpr int kNAcc = Q4 ? 18 : kAccs;
+    float4v O[kNAcc], B7 = {0, 0, 0, 0};
 #pragma unroll
-    for (int i = 0; i < kAccs; i++)
+    for (int i = 0; i < kNAcc; i++)
         O[i] = (float4v){0, 0, 0, 0};
 
     // V transpose-read address: lane (2r+e) of its 16-lane group supplies key slot r
     // (slot r<4: key lg*4+r, slot r>=4: key 16+lg*4+(r-4)), bytes [8e, 8e+8) of a 16-column run.
     const int tr_r = lm >> 1;
     const int tr_key = (tr_r >> 2) * 16 + lg * 4 + (tr_r & 3);
-    const uint8_t *vtr = Vraw + tr_key * kRowBytes + (lm & 1) * 8;
+    const uint8_t *vtr = Vraw + tr_key * kRowB + (lm & 1) * 8;
+    // q4_0: the block that byte column 16 j + lm of run j belongs to (its scales go with this lane's rows of V^T),
+    // as the offset of that block's 32 scales in the table
+    int q4_scale_at[Q4 ? 9 : 1];
+    if (Q4) {
+#pragma unroll
+        for (int j = 0; j < 9; j++)
+            q4_scale_at[Q4 ? j : 0] = ((16 * j + lm) * 3641 >> 16) * (kTileKeys * 2); // (x / 18 for x < 144)
+    }
     const uint4v bias_bits = {0x00800080u, 0x00800080u, 0x00800080u, 0x00800080u};
     const half8 Abias = __builtin_bit_cast(half8, bias_bits); // eight times 128 * 2^-24
     const int lm2 = lm >> 1; // run 2c carries the scale bytes of block c in rows 2c and 2c+1
@@ -1272,11 +1323,11 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Front
     // the scales of a tile of raw rows -> f16 table [8 blocks][32 keys]; lane = (block, four keys)
     const int sc_c = lane >> 3, sc_k = (lane & 7) * 4;
     auto build_scales = [&](const uint8_t *raw, uint8_t *table, int key0, bool partial) {
-        const uint8_t *p = raw + sc_k * kRowBytes + sc_c * kQ8BlockBytes;
+        const uint8_t *p = raw + sc_k * kRowB + sc_c * kBlkB;
         uint32_t s0 = *reinterpret_cast<const uint16_t *>(p);
-        uint32_t s1 = *reinterpret_cast<const uint16_t *>(p + kRowBytes);
-        uint32_t s2 = *reinterpret_cast<const uint16_t *>(p + 2 * kRowBytes);
-        uint32_t s3 = *reinterpret_cast<const uint16_t *>(p + 3 * kRowBytes);
+        uint32_t s1 = *reinterpret_cast<const uint16_t *>(p + kRowB);
+        uint32_t s2 = *reinterpret_cast<const uint16_t *>(p + 2 * kRowB);
+        uint32_t s3 = *reinterpret_cast<const uint16_t *>(p + 3 * kRowB);
         if (partial) {
             // a row at or past the live length holds whatever the cache holds there: zero scale, so
             // that its zero weight cannot meet a non-finite value
@@ -1298,8 +1349,8 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Front
         const bool partial = key0 + kTileKeys > hi;
         // Requests complete in the order of issue, 9 per tile of rows: K(0) V(0), then K(t + 1) after the
         // scores of tile t and V(t + 1) after its PV.
-        // ---- K rows of this tile are in LDS once only the 9 loads of its V rows are outstanding
-        asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
+        // ---- K rows of this tile are in LDS once only the loads of its V rows are outstanding
+        wait_all_but_one_tile();
 #ifdef HIPML_DECODE_STAMPS
         if (t == 0)
             HIPML_STAMP(stamps_, 4); // K rows of the wave's first tile in LDS
@@ -1318,7 +1369,8 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Front
             const float4v cb4 = *reinterpret_cast<const float4v *>(CBs + (c * 16 + lm) * 16);
 #pragma unroll
             for (int ms = 0; ms < 2; ms++) {
-                const half8 A = raw_k_operand(Kraw + (ms * 16 + lm) * kRowBytes + lg * 8, c);
+                const half8 A = Q4 ? raw_k_operand_q4(Kraw + (ms * 16 + lm) * kRowB + (lg & 1) * 8, c, (lg >> 1) * 4)
+                                   : raw_k_operand(Kraw + (ms * 16 + lm) * kRowB + lg * 8, c);
                 const half4 sk = *reinterpret_cast<const half4 *>(sK + (c * kTileKeys + ms * 16 + lg * 4) * 2);
                 if (WIDE) {
                     const float4v ch = {cb4[0], cb4[0], cb4[0], cb4[0]}, cl = {cb4[1], cb4[1], cb4[1], cb4[1]};
@@ -1401,14 +1453,14 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Front
         }
         if (t > 0 && __any(grew)) { // (the accumulators of the first tile are still zero)
 #pragma unroll
-            for (int i = 0; i < kAccs; i++)
+            for (int i = 0; i < kNAcc; i++)
                 O[i] *= corr;
             B7 *= corr;
         }
 
         // ---- V rows of this tile: all that may still be outstanding are the next tile's K rows
         if (more)
-            asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
+            wait_all_but_one_tile();
         else
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #ifdef HIPML_DECODE_STAMPS
@@ -1418,39 +1470,77 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Front
         build_scales(Vraw, sV, key0, partial);
 
         // ---- O^T += V^T . P' -------------------------------------------------------------------
-        half8 Aprev = Abias; // the run shared with the previous block
+        if constexpr (Q4) {
+            // One transposing read per run gives this lane the bytes of 8 keys in byte column 16 j + lm: their low
+            // nibbles are a row of V^T (element e of the column's block), their high nibbles another (e + 16).
+            // The block scale differs between the columns of a run, so it goes into the A operand: nibble n as
+            // the f16 1024 + n, minus 1032 (exact), times the key's scale of the column's block (one rounding,
+            // where the q8_0 path rounds the weight times the scale); P stays the plain f16 weights.  Columns
+            // that hold scale bytes make rows nobody reads.
+            const half8 Pp = __builtin_shufflevector(ph[0], ph[1], 0, 1, 2, 3, 4, 5, 6, 7);
+            const half2v k1032 = {(_Float16)1032.0f, (_Float16)1032.0f};
 #pragma unroll
-        for (int c = 0; c < 8; c++) {
-            half4 sv[2];
+            for (int j = 0; j < 9; j++) {
+                const int2v raw = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+                    (int2v __attribute__((address_space(3))) *)(vtr + j * 16));
+                const half4 s0 = *reinterpret_cast<const half4 *>(sV + q4_scale_at[Q4 ? j : 0] + lg * 8);
+                const half4 s1 = *reinterpret_cast<const half4 *>(sV + q4_scale_at[Q4 ? j : 0] + (16 + lg * 4) * 2);
+                const half2v sc[4] = {{s0[0], s0[1]}, {s0[2], s0[3]}, {s1[0], s1[1]}, {s1[2], s1[3]}};
 #pragma unroll
-            for (int ms = 0; ms < 2; ms++)
-                sv[ms] = *reinterpret_cast<const half4 *>(sV + (c * kTileKeys + ms * 16 + lg * 4) * 2);
-            // P' = p * block scale, one packed f16 multiply (f16-class weights)
-            const half4 x0 = ph[0] * sv[0];
-            const half4 x1 = ph[1] * sv[1];
-            const half8 Ph = __builtin_shufflevector(x0, x1, 0, 1, 2, 3, 4, 5, 6, 7);
-            if (c == 7)
-                B7 = __builtin_amdgcn_mfma_f32_16x16x32_f16(Abias, Ph, B7, 0, 0, 0);
-            // the runs that hold columns of block c: 2c .. 2c+2 (15 and 16 for block 7)
+                for (int h = 0; h < 2; h++) {
+                    const uint32_t y0 = ((uint32_t)raw[0] >> (4 * h)) & 0x0f0f0f0fu;
+                    const uint32_t y1 = ((uint32_t)raw[1] >> (4 * h)) & 0x0f0f0f0fu;
+                    uint4v r;
+                    r[0] = __builtin_amdgcn_perm(0x64646464u, y0, 0x04010400u);
+                    r[1] = __builtin_amdgcn_perm(0x64646464u, y0, 0x04030402u);
+                    r[2] = __builtin_amdgcn_perm(0x64646464u, y1, 0x04010400u);
+                    r[3] = __builtin_amdgcn_perm(0x64646464u, y1, 0x04030402u);
+                    half8 A;
 #pragma unroll
-            for (int r = 0; r < (c < 7 ? 3 : 2); r++) {
-                const int j = (c < 7 ? 2 * c : 15) + r;
-                half8 A;
-                if (r == 0 && c > 0 && c < 7) {
-                    A = Aprev;
-                } else {
-                    int2v raw = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
-                        (int2v __attribute__((address_space(3))) *)(vtr + j * 16));
-                    if ((j & 1) == 0 && j <= 12) {
-                        // rows j and j+1 of this run are scale bytes: byte 0 enters as 128 * 2^-24
-                        raw[0] = lm2 == j / 2 ? 0 : raw[0];
-                        raw[1] = lm2 == j / 2 ? 0 : raw[1];
+                    for (int w = 0; w < 4; w++) {
+                        const uint32_t bits = r[w]; // (a copy: bit_cast of a vector element reads element 0)
+                        const half2v x = (__builtin_bit_cast(half2v, bits) - k1032) * sc[w];
+                        A[2 * w] = x[0];
+                        A[2 * w + 1] = x[1];
                     }
-                    A = bytes_to_f16_biased<false>(raw);
+                    O[2 * j + h] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, Pp, O[2 * j + h], 0, 0, 0);
                 }
-                O[c * 3 + r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, Ph, O[c * 3 + r], 0, 0, 0);
-                if (r == 2)
-                    Aprev = A;
+            }
+        } else {
+            half8 Aprev = Abias; // the run shared with the previous block
+    #pragma unroll
+            for (int c = 0; c < 8; c++) {
+                half4 sv[2];
+    #pragma unroll
+                for (int ms = 0; ms < 2; ms++)
+                    sv[ms] = *reinterpret_cast<const half4 *>(sV + (c * kTileKeys + ms * 16 + lg * 4) * 2);
+                // P' = p * block scale, one packed f16 multiply (f16-class weights)
+                const half4 x0 = ph[0] * sv[0];
+                const half4 x1 = ph[1] * sv[1];
+                const half8 Ph = __builtin_shufflevector(x0, x1, 0, 1, 2, 3, 4, 5, 6, 7);
+                if (c == 7)
+                    B7 = __builtin_amdgcn_mfma_f32_16x16x32_f16(Abias, Ph, B7, 0, 0, 0);
+                // the runs that hold columns of block c: 2c .. 2c+2 (15 and 16 for block 7)
+    #pragma unroll
+                for (int r = 0; r < (c < 7 ? 3 : 2); r++) {
+                    const int j = (c < 7 ? 2 * c : 15) + r;
+                    half8 A;
+                    if (r == 0 && c > 0 && c < 7) {
+                        A = Aprev;
+                    } else {
+                        int2v raw = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+                            (int2v __attribute__((address_space(3))) *)(vtr + j * 16));
+                        if ((j & 1) == 0 && j <= 12) {
+                            // rows j and j+1 of this run are scale bytes: byte 0 enters as 128 * 2^-24
+                            raw[0] = lm2 == j / 2 ? 0 : raw[0];
+                            raw[1] = lm2 == j / 2 ? 0 : raw[1];
+                        }
+                        A = bytes_to_f16_biased<false>(raw);
+                    }
+                    O[c * 3 + r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, Ph, O[c * 3 + r], 0, 0, 0);
+                    if (r == 2)
+                        Aprev = A;
+                }
             }
         }
         // the V rows are used up
@@ -1494,7 +1584,22 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Front
             return v;
         };
         const int pc = lm & (kCols - 1); // the column this lane parks
-        if (WIDE) {
+        // q4_0: a column's rows are two halves of 144 byte columns (low nibbles, high nibbles), 160 floats apart,
+        // columns 324 floats apart: the lanes of MFMA columns 0..7 write the low halves, those of columns 8..15
+        // (the same values) the high halves, and the sixteen lanes of a k-group cover all 64 banks once per
+        // 128-bit write (4 n mod 64 for n < 8, + 32 for the other half).
+        constexpr int kQ4Half = 160, kQ4Pitch = 2 * kQ4Half + 4;
+        static_assert(!Q4 || kCols * kQ4Pitch * 4 <= kDmaWaveLds, "a wave parks its columns in its own rows");
+        if constexpr (Q4) {
+            const bool first = lm < 8;
+#pragma unroll
+            for (int j = 0; j < 9; j++) {
+                const float4v lo = O[Q4 ? 2 * j : 0], up = O[Q4 ? 2 * j + 1 : 0];
+                const float4v v = {first ? lo[0] : up[0], first ? lo[1] : up[1], first ? lo[2] : up[2],
+                                   first ? lo[3] : up[3]};
+                *reinterpret_cast<float4v *>(wl + pc * kQ4Pitch + (first ? 0 : kQ4Half) + j * 16 + lg * 4) = v;
+            }
+        } else if (WIDE) {
 #pragma unroll
             for (int j = 0; j < kRuns; j++)
                 *reinterpret_cast<float4v *>(wl + pc * kParkPitch + j * 16 + lg * 4) = run_values(j);
@@ -1525,7 +1630,10 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Front
         static_assert(kRun == 16 || kRun == 8, "a thread's values of d lie in one block");
         const int nc = threadIdx.x / kDRuns;
         const int d0 = (threadIdx.x % kDRuns) * kRun;
-        const int col0 = d0 + 2 + 2 * (d0 >> 5); // byte column of d0: 34 bytes per 32 values, scale first
+        // byte column of d0: 34 bytes per 32 values, scale first; q4_0: 18 bytes per 32 values, element e < 16 in
+        // the low half at byte e, element e + 16 in the high half at the same byte
+        const int col0 = Q4 ? (d0 >> 5) * kQ4BlockBytes + 2 + (d0 & 15) + ((d0 >> 4) & 1) * kQ4Half
+                            : d0 + 2 + 2 * (d0 >> 5);
         if (nc < nvalid) {
             float mw[kWaves], lw[kWaves];
             float ms = -INFINITY;
@@ -1542,7 +1650,8 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Front
             for (int w = 0; w < kWaves; w++) {
                 wgt[w] = mw[w] == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(mw[w] - ms);
                 lsum += lw[w] * wgt[w];
-                wgt[w] *= kTwo24;
+                if (!Q4)
+                    wgt[w] *= kTwo24; // (the q8_0 V operands carry 2^-24; the q4_0 ones are real values)
             }
             const int col = nc / group;
             const int head = hbase + (nc - col * group);
@@ -1553,8 +1662,9 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Front
                 float4v acc = {0, 0, 0, 0};
 #pragma unroll
                 for (int w = 0; w < kWaves; w++) {
-                    const float *row = reinterpret_cast<const float *>(lds_all + w * kDmaWaveLds) + nc * kParkPitch;
-                    const float off = row[(d0 >> 5) * kQ8BlockBytes]; // the block's correction row
+                    const float *row = reinterpret_cast<const float *>(lds_all + w * kDmaWaveLds) +
+                                       nc * (Q4 ? kQ4Pitch : kParkPitch);
+                    const float off = Q4 ? 0.0f : row[(d0 >> 5) * kQ8BlockBytes]; // the block's correction row
                     const float2 x0 = *reinterpret_cast<const float2 *>(row + col0 + dd);
                     const float2 x1 = *reinterpret_cast<const float2 *>(row + col0 + dd + 2);
                     acc += ((float4v){x0.x, x0.y, x1.x, x1.y} - off) * wgt[w];
@@ -1753,6 +1863,21 @@ __global__ void __launch_bounds__(kThreads, 2)
     HIPML_STAMP(stamps_, 11); // everything this wave stored has been acknowledged
     stamps_out(stamps_);
 #endif
+}
+
+// The same road for q4_0 rows (items of at most 8 columns: the launcher cuts wider slots by heads).
+__global__ void __launch_bounds__(kThreads, 2)
+    decode_q4_kernel(const uint8_t *k, const uint8_t *v, const float *q, const int32_t *pos, int stride, int splits,
+                     uint32_t wi, uint32_t item0, uint32_t geom, uint32_t q_slot, const DecodeArgs a)
+{
+#ifdef HIPML_DECODE_STAMPS
+    Stamps stamps_ = {}; // (not written out: the stamps are the q8_0 kernel's)
+#endif
+    const Front f = front_of(k, v, q, pos, stride, splits, wi, item0, geom, q_slot, (uint32_t)offsetof(DecodeKernarg, a));
+    Work wk;
+    if (!find_work(a, f, threadIdx.x & 63, wk))
+        return;
+    decode_body_dma<false, true>(a, f, wk HIPML_STAMPS_PASS);
 }
 
 // Wave-wide reductions without LDS: DPP inside a row of 16 lanes, then the two row-swap
@@ -1977,6 +2102,7 @@ int decode_init()
 {
     struct { const void *fn; int bytes; } const kernels[] = {
         {reinterpret_cast<const void *>(&decode_q8_kernel), kDmaLds},
+        {reinterpret_cast<const void *>(&decode_q4_kernel), kDmaLds},
         {reinterpret_cast<const void *>(&decode_staged_kernel<false, true>), decode_lds_bytes(1)},
         {reinterpret_cast<const void *>(&decode_staged_kernel<true, false>), decode_lds_bytes(1)},
     };
@@ -2304,18 +2430,20 @@ int launch_decode_q8(hipStream_t st, const DecodeLaunch &given)
     if (given.head_dim != kHeadDim)
         return launch_decode_hd(st, given);
     DecodeLaunch L = given;
-    // q8_0: the kernel that streams raw rows into LDS (its tile addressing is 32-bit per KV head);
-    // q4_0, the fp32-class variant and caches of more than 4 GiB per KV head: the staged kernel
-    // the kernel that moves raw rows addresses a KV head's rows and the Q rows with 32-bit byte offsets
-    const bool raw_rows = !L.q4 && !L.exact && (size_t)L.stride * kRowBytes < ((size_t)1 << 32) &&
+    // q8_0 and q4_0: the kernel that streams raw rows into LDS (it addresses a KV head's rows and the Q rows
+    // with 32-bit byte offsets); the fp32-class variant and caches of more than 4 GiB per KV head: the staged
+    // kernel
+    const bool raw_rows = !L.exact && (size_t)L.stride * kRowBytes < ((size_t)1 << 32) &&
                           ((size_t)L.total_rows * L.q_slot + (size_t)L.n_heads * kHeadDim) * sizeof(float) <
                               ((size_t)1 << 32);
-    // One sequence: the raw-row kernel is at its best with one workgroup per CU (19.2 us per layer at depth
-    // 32,768 with 64 splits of 4 KV heads, 20.4 with 128), the staged kernel with two (q4_0 there: 20.4 us
-    // with 128 splits, 23.5 with 64).  The split policy sizes the scratch for two; the raw-row kernel then
-    // cuts the keys into half as many splits and leaves the rest of the scratch alone (the layout of the
-    // partials is the kernels' own; every row of a verify group is cut the same way as its plain decode).
-    if (raw_rows && L.slots == 1) {
+    // One sequence over q8_0: the raw-row kernel is at its best with one workgroup per CU (19.2 us per layer at
+    // depth 32,768 with 64 splits of 4 KV heads, 20.4 with 128).  Over q4_0 a workgroup has half the bytes to
+    // wait for and more arithmetic per byte, and two per CU pay from about 24,000 rows on (one / two per CU:
+    // 10.4 / 11.5 us at 8,192, 16.5 / 16.2 at 32,768, 44.1 / 36.1 at 131,072).  The split policy sizes the
+    // scratch for two; a launch that runs one per CU cuts the keys into half as many splits and leaves the rest
+    // of the scratch alone (the layout of the partials is the kernels' own; every row of a verify group is cut
+    // the same way as its plain decode).
+    if (raw_rows && L.slots == 1 && !(L.q4 && L.stride >= 24576)) {
         const int one_per_cu = 256 / L.n_kv > 1 ? 256 / L.n_kv : 1;
         L.splits = L.splits < one_per_cu ? L.splits : one_per_cu;
     }
@@ -2346,7 +2474,9 @@ int launch_decode_q8(hipStream_t st, const DecodeLaunch &given)
     int items = 0;
     for (int s = 0; s < L.slots; s++) {
         const int cols = L.cols[s];
-        const int cap = !raw_rows || cols * a.group > 8 ? 16 : 8;
+        // (the raw-row kernel runs items of up to 8 columns through its narrow body and, over q8_0, wider ones
+        // through its wide one; over q4_0 every item has at most 8)
+        const int cap = raw_rows && L.q4 ? 8 : (!raw_rows || cols * a.group > 8 ? 16 : 8);
         const int per_max = cap / cols;                           // heads per item: 2..16 (cols <= 4)
         const int n_items = (a.group + per_max - 1) / per_max;
         const int base = a.group / n_items, extra = a.group % n_items;
@@ -2383,7 +2513,7 @@ int launch_decode_q8(hipStream_t st, const DecodeLaunch &given)
     a.gate = L.gate;
     a.tickets = nullptr;
     a.merge = 0;
-    if (raw_rows && L.slots == 1 && a.workers == 0 && L.splits <= kMergeMaxSplits) {
+    if (raw_rows && !L.q4 && L.slots == 1 && a.workers == 0 && L.splits <= kMergeMaxSplits) {
         const int ngroup = (L.splits + kMergeGroup - 1) / kMergeGroup;
         a.tickets = decode_tickets(st, items * L.n_kv * (ngroup + 1));
         a.merge = a.tickets != nullptr ? kMergeGroup : 0;
@@ -2395,8 +2525,12 @@ int launch_decode_q8(hipStream_t st, const DecodeLaunch &given)
         const uint32_t item0 = (uint32_t)a.i0_row0 | (uint32_t)a.i0_cols << 10 | (uint32_t)a.i0_head0 << 13 |
                                (uint32_t)a.i0_nhead << 16 | (uint32_t)a.i0_slot << 20;
         const uint32_t geom = (uint32_t)a.group | (uint32_t)a.n_kv << 4 | (uint32_t)a.stream_once << 20;
-        HIPML_LAUNCH(decode_q8_kernel, grid, dim3(kThreads, 1, 1), kDmaLds, st, a.k + slot_at, a.v + slot_at, a.q, a.pos,
-                     a.stride, a.splits, wi, item0, geom, (uint32_t)a.q_slot, a);
+        if (L.q4)
+            HIPML_LAUNCH(decode_q4_kernel, grid, dim3(kThreads, 1, 1), kDmaLds, st, a.k + slot_at, a.v + slot_at, a.q,
+                         a.pos, a.stride, a.splits, wi, item0, geom, (uint32_t)a.q_slot, a);
+        else
+            HIPML_LAUNCH(decode_q8_kernel, grid, dim3(kThreads, 1, 1), kDmaLds, st, a.k + slot_at, a.v + slot_at, a.q,
+                         a.pos, a.stride, a.splits, wi, item0, geom, (uint32_t)a.q_slot, a);
     }
     else if (L.q4)
         HIPML_LAUNCH((decode_staged_kernel<true, false>), grid, dim3(kThreads, 1, 1), decode_lds_bytes(1), st, a);

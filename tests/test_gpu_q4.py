@@ -76,8 +76,11 @@ def test_q4_encode_step_append():
     assert not host(kc)[:, :pos].any() and not host(kc)[:, pos + 1:].any()
 
 
-@pytest.mark.parametrize("seq,pad,splits", [(1, 0, 1), (257, 31, 7), (4100, 0, 16), (8192, 64, None)])
+@pytest.mark.parametrize("seq,pad,splits", [(1, 0, 1), (2, 0, 1), (31, 1, 2), (33, 0, 1), (257, 31, 7), (4100, 0, 16),
+                                            (8192, 64, None), (24575, 0, None), (24576, 0, None), (32768, 0, None),
+                                            (30011, 700, 128)])
 def test_q4_decode_matches_oracle(seq, pad, splits):
+    # (from 24,576 rows on the launch keeps two workgroups per CU; below it runs one)
     stride = seq + pad
     r = orc.Rng(0x0404_0010 + seq)
     q = r.normal_array((N_HEADS, HD))
@@ -98,16 +101,16 @@ def test_q4_decode_matches_oracle(seq, pad, splits):
     assert ok
 
 
-def test_q4_mtp_columns_equal_single_row_decodes():
-    # three query rows of one sequence (MTP verify): row r sees keys 0..pos0+r
-    pos0, cols, stride = 700, 3, 1024
+@pytest.mark.parametrize("pos0,cols,stride,splits", [(700, 3, 1024, 6), (700, 4, 1024, 5), (25000, 4, 25100, 128),
+                                                     (5, 2, 64, 3)])
+def test_q4_mtp_columns_equal_single_row_decodes(pos0, cols, stride, splits):
+    # query rows of one sequence (MTP verify): row r sees keys 0..pos0+r
     seq = pos0 + cols
     r = orc.Rng(0x0404_0020)
     q = r.normal_array((cols, N_HEADS, HD))
     kf = r.normal_array((N_KV, seq, HD))
     vf = r.normal_array((N_KV, seq, HD))
     kb, vb = q4_cache(kf, vf, stride)
-    splits = 6
     acc = torch.empty((cols, N_HEADS, splits, HD), device="cuda")
     ml = torch.empty((cols, N_HEADS, splits, 2), device="cuda")
     out = torch.empty((cols, N_HEADS, HD), device="cuda")
@@ -121,6 +124,12 @@ def test_q4_mtp_columns_equal_single_row_decodes():
                                   stride=stride)
         ok, _, _ = report(f"q4 MTP column {c}", want, host(out)[c].ravel(), *KERNEL_CLASS)
         assert ok
+        # the reference's column check: a column of a verify group has the bits of its plain decode
+        single = torch.empty((N_HEADS, HD), device="cuda")
+        attn.attn_decode_kv(step_buffer(pos0 + c, pos0 + c + 1), Q4, dev(q[c]), dev(kb), dev(vb), acc, ml, single,
+                            N_HEADS, N_KV, HD, stride, SCALE, splits)
+        torch.cuda.synchronize()
+        assert np.array_equal(host(single).view(np.uint32), host(out)[c].view(np.uint32))
 
 
 @pytest.mark.parametrize("tok,pos0,pad,splits", [(37, 29, 5, 1), (37, 29, 5, 4), (200, 0, 0, 3),
