@@ -126,6 +126,26 @@ def timed(torch, fn, steps, warm=3, wall=False, min_ms=MIN_TIMED_MS):
     return total / n, total, n
 
 
+def timed_graph(torch, fn, calls, min_ms=MIN_TIMED_MS):
+    """Mean duration of fn(i) in ms with fn(0) .. fn(calls - 1) captured once in a HIP graph and the graph
+    replayed until `min_ms` of work have been timed (HIP events around the replays): what the launches cost when
+    the host does not issue them one by one -- a call through Python and ctypes takes about 12 us of host time,
+    more than a short launch runs.  Returns (ms per call, ms timed, calls timed)."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for i in range(calls):
+            fn(i)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for i in range(calls):
+            fn(i)
+    ms, total, n = timed(torch, lambda i: graph.replay(), 2, 2, min_ms=min_ms)
+    return ms / calls, total, n * calls
+
+
 def counters(workload: str, kernel: str):
     """Clock and MFMA-busy share of `kernel` in the committed counter run of `workload`
     (profiles/mfma_counters.json: rocprofv3 --pmc on this benchmark's --only legs), or {}."""
@@ -168,7 +188,7 @@ def stream_yardstick(torch, attn, pairs, bytes_each, steps):
         def one(i, mode=mode):
             k, v = pairs[i % len(pairs)]
             attn.bench_stream_read(k, v, bytes_each, mode, sink)
-        ms, total, n = timed(torch, one, steps * len(pairs), warm=len(pairs))
+        ms, total, n = timed_graph(torch, one, 4 * len(pairs))
         res[name] = {"us_per_launch": ms * 1e3, "gbs": 2 * bytes_each / (ms * 1e-3) / 1e9, "timed_ms": total}
     best = max(res.values(), key=lambda r: r["gbs"])
     return {"achievable": best["gbs"], "bytes_per_launch": 2 * bytes_each, **{k: v for k, v in res.items()}}
@@ -276,6 +296,9 @@ def bench_prefill(torch, attn, tokens, pos0, steps, warmup, layers, prefix_fill=
 
     unfused_ms, _, _ = timed(torch, step_unfused, steps, warmup, wall=True)
     wall_ms, wall_total, wall_n = timed(torch, step, steps, warmup, wall=True)
+    # (a short step, issued call by call from Python, is partly the host's time: the same steps replayed from a
+    # HIP graph, for comparison)
+    graph_ms = timed_graph(torch, step, 2 * layers)[0] if wall_ms < 0.2 else None
     # the f16 copy of the cache serves long prefixes: the sliced kernel over it is not what a chunk near
     # position 0 would run (splits == 0), so that leg is left out there
     with_copy = splits != 0
@@ -345,6 +368,7 @@ def bench_prefill(torch, attn, tokens, pos0, steps, warmup, layers, prefix_fill=
         "ms_per_step": wall_ms, "timed_ms": wall_total, "steps_timed": wall_n,
         "tok_per_s": tokens / (wall_ms * 1e-3),
         "ms_per_step_separate_launches": unfused_ms,
+        "ms_per_step_graph_replay": graph_ms,
         "attn_ms": attn_ms,
         "attn_tok_per_s": tokens / (attn_ms * 1e-3),
         "reference_scratch_8_slices": ref_scratch,
@@ -422,7 +446,12 @@ def bench_decode(torch, attn, seq, steps, warmup, layers, dtype=0, one_launch=Fa
         attn.attn_decode_kv(stepbuf, dtype, q, k, v, acc, ml, out, H, KV, HD, stride, SCALE, splits)
 
     calls = steps * layers
-    ms, total, n = timed(torch, plain, calls, warmup * layers)
+    eager_us = timed(torch, plain, calls, warmup * layers)[0] * 1e3
+    # The figures of this entry are replays of a HIP graph that holds 4 passes over the layer caches, as an
+    # engine issues its decode step; issued call by call from Python the same launches are bound by the host at
+    # short depths (us_per_layer_eager).
+    in_graph = 4 * layers
+    ms, total, n = timed_graph(torch, plain, in_graph)
     us = ms * 1e3
     # the same with the sigmoid output gate: in the merge kernel, and as the separate launch it replaces
     gate = torch.randn((H, HD), device="cuda", generator=gen)
@@ -435,20 +464,20 @@ def bench_decode(torch, attn, seq, steps, warmup, layers, dtype=0, one_launch=Fa
         plain(i)
         attn.q_gate(out, gate, out, H * HD)
 
-    tg = timed(torch, gated, calls, layers)[0] * 1e3
-    ts = timed(torch, gate_apart, calls, layers)[0] * 1e3
+    tg = timed_graph(torch, gated, in_graph)[0] * 1e3
+    ts = timed_graph(torch, gate_apart, in_graph)[0] * 1e3
     # the form whose workgroups merge the key splits themselves (one launch instead of two; q8_0 only)
     one_launch_us = None
     if one_launch and dtype == 0:
         before = attn.decode_one_launch(1)
         try:
-            one_launch_us = timed(torch, plain, calls, layers)[0] * 1e3
+            one_launch_us = timed_graph(torch, plain, in_graph)[0] * 1e3
         finally:
             attn.decode_one_launch(before)
     nbytes = decode_bytes(seq) * row // ROW
     gbs = nbytes / (us * 1e-6) / 1e9
-    traffic = measured_traffic({8192: "decode8k", 32768: "decode32k"}.get(seq, "") if dtype == 0 else "",
-                               ["decode_q8_kernel", "decode_reduce"])
+    traffic = measured_traffic({(8192, 0): "decode8k", (32768, 0): "decode32k", (32768, 1): "decode32k_q4"}.get((seq, dtype), ""),
+                               ["decode_q8_kernel", "decode_q4_kernel", "decode_reduce"])
     # what a launch that only reads the same bytes reaches on this box, same rotation over the layer caches
     ys = stream_yardstick(torch, attn, caches, KV * stride * row, steps)
     return {
@@ -459,6 +488,7 @@ def bench_decode(torch, attn, seq, steps, warmup, layers, dtype=0, one_launch=Fa
         # over q4_0 below 24,576 rows)
         "splits_run": min(splits, max(256 // KV, 1)) if dtype == 0 or stride < 24576 else splits,
         "us_per_layer": us, "timed_ms": total, "steps_timed": n,
+        "issued": f"HIP graph of {in_graph} calls, replayed", "us_per_layer_eager": eager_us,
         "us_per_layer_gate_fused": tg,
         "us_per_layer_gate_separate": ts,
         "us_per_layer_one_launch": one_launch_us,
@@ -754,13 +784,16 @@ def bench_gemv(torch, attn, rows, steps, layers, m=5120, k=6144):
     ws = [random_q8_0_weights(torch, m, k, gen) for _ in range(layers)]
     x = torch.randn((rows, k), device="cuda", generator=gen) * 0.5
     y = torch.empty((rows, m), device="cuda")
-    ms, total, n = timed(torch, lambda i: attn.gemv_q8_0_rows(ws[i % layers], x, y, m, k, rows), steps * layers, layers)
+    one = lambda i: attn.gemv_q8_0_rows(ws[i % layers], x, y, m, k, rows)
+    eager_us = timed(torch, one, steps * layers, layers)[0] * 1e3
+    ms, total, n = timed_graph(torch, one, 4 * layers)  # (issued one by one from Python the launch is host-bound)
     us = ms * 1e3
     # algorithmic bytes: the weights once, however many passes the kernel makes over them
     nbytes = m * (k // 32) * 34
     gbs = nbytes / (us * 1e-6) / 1e9
     return {"workload": f"W_o projection, Q8_0 {m}x{k}, {rows} activation rows",
             "us_per_layer": us, "timed_ms": total, "steps_timed": n, "weight_bytes": m * (k // 32) * 34,
+            "issued": f"HIP graph of {4 * layers} calls, replayed", "us_per_layer_eager": eager_us,
             "layers_rotated": layers,
             "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": gbs / HBM_PEAK_GBS,
@@ -867,7 +900,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--main-only", action="store_true", help="skip the 'also' workloads")
     ap.add_argument("--only", default="", help="run one workload alone (prefill672, decode8k, "
-                    "decode32k, decode128k, chunk100k, batch16, mfma, front672, decode32k_q4, gemv1, gemv4, gemv16, gemm672, gemm2048, layer32k, layer672, blayer16, copycal) for profiling; prints its object")
+                    "decode32k, decode32k_one_launch, decode128k, chunk100k, batch16, mfma, front672, decode32k_q4, gemv1, gemv4, gemv16, gemm672, gemm2048, layer32k, layer672, blayer16, copycal) for profiling; prints its object")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -892,7 +925,8 @@ def main() -> int:
         fn = {
             "prefill672": lambda: bench_prefill(torch, attn, 672, 0, K, W, LAYERS, mfma=mf()),
             "decode8k": lambda: bench_decode(torch, attn, 8192, K, W, LAYERS),
-            "decode32k": lambda: bench_decode(torch, attn, 32768, K, W, LAYERS, one_launch=True),
+            "decode32k": lambda: bench_decode(torch, attn, 32768, K, W, LAYERS),
+            "decode32k_one_launch": lambda: bench_decode(torch, attn, 32768, K, W, LAYERS, one_launch=True),
             "decode128k": lambda: bench_decode(torch, attn, 131072, K, W, LAYERS),
             "chunk100k": lambda: bench_prefill(torch, attn, 2048, 100_000, K, W, 2, mfma=mf()),
             "batch16": lambda: bench_batch(torch, attn, K, W, 4),

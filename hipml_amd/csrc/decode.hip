@@ -1105,12 +1105,15 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Front
     // ---- one tile of rows = 8,704 contiguous bytes = 8.5 instructions of 1 KiB ------------------
     const uint32_t lane16 = lane * 16;
     const uint32_t region_last = (uint32_t)f.stride * kRowB - 16; // last 16 bytes of a KV head's rows
-    auto issue_as = [&](auto once, bool v_rows, int t) {
+    auto issue_as = [&](auto once, auto first, bool v_rows, int t) {
         constexpr bool kOnce = decltype(once)::value;
         const uint32_t lds_at = wave_at + (v_rows ? kRawT : 0);
         const uint8_t *region = v_rows ? vbase : kbase;
         const int key0 = tile_key0(t);
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // the wave's own reads of the old rows are done
+        // the wave's own reads of the old rows are done (the launch's first request replaces nothing, and a
+        // wait here would be one for the live lengths, whose scalar loads count on the same counter)
+        if (!decltype(first)::value)
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         if (key0 + kTileKeys <= f.stride) { // (uniform) the tile lies inside the cache
             const uint8_t *src = region + (size_t)key0 * kRowB;
 #pragma unroll
@@ -1137,9 +1140,15 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Front
     const bool once = f.stream_once != 0 || group == f.group;
     auto issue = [&](bool v_rows, int t) {
         if (once)
-            issue_as(std::true_type(), v_rows, t);
+            issue_as(std::true_type(), std::false_type(), v_rows, t);
         else
-            issue_as(std::false_type(), v_rows, t);
+            issue_as(std::false_type(), std::false_type(), v_rows, t);
+    };
+    auto issue_first = [&] {
+        if (once)
+            issue_as(std::true_type(), std::true_type(), false, 0);
+        else
+            issue_as(std::false_type(), std::true_type(), false, 0);
     };
 
     // live lengths of this slot's rows: scalar loads, requested before the first asm statement (the
@@ -1196,7 +1205,7 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Front
             dma16<false>(at + 1024, qb, qoff + 32 * sizeof(float));
         }
     }
-    issue(false, 0);
+    issue_first();
     HIPML_STAMP(stamps_, 2); // the first requests have left
 
     // all but the newest tile of rows have arrived (requests return in the order of issue)
