@@ -299,6 +299,388 @@ __global__ void __launch_bounds__(64 * WAVES, TILES == 1 ? 2 : 1) gemv_q8_rows_k
     }
 }
 
+// ---- gemv_q8_dma_kernel: one to eight activation rows, the weight rows moved into LDS as they lie in memory ----
+//
+// The row kernel above asks for its weights in 12- and 8-byte pieces per lane, which the memory pipeline serves
+// at 10.0 us for the 33.4 MB of a 5120 x 6144 matrix; the same bytes as whole pieces of rows through
+// global_load_lds_dwordx4 need no registers while they travel and arrive sooner.  A workgroup takes `rows_wg`
+// consecutive weight rows (m / 256 where that is 16..32: one workgroup per CU and every CU the same bytes; one or
+// two MFMA tiles of 16 rows); its waves deal the rows' chunks of 256 values (8 blocks, 272 bytes: the smallest
+// piece of a row that starts and ends at a 16-byte boundary) round-robin, and a wave keeps two chunks in flight
+// into a ring of two buffers.  Nothing is shared between the waves until their sums meet, so the loop has no
+// barrier.
+// The activations take the same road as raw f32 and become MFMA operands in place (the 128 bytes of a block's 32
+// floats of one row become 64 bytes of f16 hi halves and 64 of lo halves, x = hi + lo to ~22 bits): with one row,
+// all of a wave's chunks before the loop, while the first weights travel; with more rows, a chunk's values ride
+// behind its weights in the ring and are converted when the chunk has arrived.
+// One v_mfma_f32_16x16x32_f16 per block and tile with A = activations (A rows 0..7 the hi halves of rows 0..7, A
+// rows 8..15 the lo halves), B = 16 weight rows.  Lane (lm, lg) reads its 8 bytes of weight row lm, quarter lg of
+// the block, from the raw rows with dword-aligned reads (even blocks sit 2 bytes past a boundary and are
+// realigned; LDS reads at 2-byte alignment measured four times slower).  The weight bytes enter the MFMA as the
+// f16 subnormals (b + 128) x 2^-24, one v_perm_b32 per pair: exact, and the offset 128 comes out again as
+// 128 x 2^-24 x (sum of the block's activation halves), a number the wave forms once per block and chunk.  The
+// block's scale multiplies the corrected fp32 dot product, as the CPU definition's d * q products summed in
+// fp32; 2^24 multiplies the final sum.
+// A (row, weight row) result is the sum, in a fixed order, of eight chains (chunk c belongs to chain c % 8, a
+// chain adds its blocks in order), hi and lo halves apart until the end: the same operations in the same order
+// whatever RP, the wave count and rows_wg are and whichever rows travel with it, so a verify group's rows have the
+// bits of their plain decodes (crates/hipml-kernels/src/attn_gpu.rs:930-932).
+constexpr int kDmaChunkBytes = 8 * kQ8Block; // 272: one row's share of a chunk
+constexpr int kDmaChains = 8;
+constexpr float kTwo24f = 16777216.0f;
+
+__device__ __forceinline__ uint32_t proj_lds_address(const void *p)
+{
+    return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void *)p;
+}
+
+// 64 lanes x 16 bytes from base + voff (per lane) to LDS address lds_at + 16 * lane; ONCE: read once (weights)
+template <bool ONCE>
+__device__ __forceinline__ void proj_dma16(uint32_t lds_at, const uint8_t *base, uint32_t voff)
+{
+    if (ONCE)
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt"
+                     :
+                     : "s"(lds_at), "v"(voff), "s"(base)
+                     : "memory");
+    else
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                     :
+                     : "s"(lds_at), "v"(voff), "s"(base)
+                     : "memory");
+}
+
+template <int N>
+__device__ __forceinline__ void wait_vm()
+{
+    static_assert(N >= 0 && N < 64, "vmcnt has six bits");
+    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+}
+
+// 8 int8 (two dwords) -> 8 f16 subnormals (b + 128) x 2^-24, exactly
+__device__ __forceinline__ half8 int8x8_to_f16_sub(uint32_t w0, uint32_t w1)
+{
+    const uint32_t x0 = w0 ^ 0x80808080u, x1 = w1 ^ 0x80808080u;
+    uint4v r;
+    r[0] = __builtin_amdgcn_perm(0u, x0, 0x0c010c00u);
+    r[1] = __builtin_amdgcn_perm(0u, x0, 0x0c030c02u);
+    r[2] = __builtin_amdgcn_perm(0u, x1, 0x0c010c00u);
+    r[3] = __builtin_amdgcn_perm(0u, x1, 0x0c030c02u);
+    return __builtin_bit_cast(half8, r);
+}
+
+// The variants: RP activation rows per pass on WAVES waves; NI requests of 64 x 16 bytes per chunk of weights
+// (rows_wg x 17 pieces), which also says how many 16-row tiles cover rows_wg.
+constexpr bool gemv_dma_front(int rp) { return rp == 1; }
+constexpr int gemv_dma_tiles(int ni) { return ni > 5 ? 2 : 1; }
+constexpr int kDmaDepth = 2; // chunks in flight per wave (three measured no faster)
+// a ring entry: the chunk's weights as they arrive (rows_wg x 272 bytes) and, behind them, its activations
+inline int gemv_dma_entry(int rp, int rows_wg) { return rows_wg * kDmaChunkBytes + (gemv_dma_front(rp) ? 0 : rp * 1024); }
+inline int gemv_dma_lds(int rp, int ni, int waves, int rows_wg, int k)
+{
+    const int per_wave = ((k >> 8) + waves - 1) / waves; // chunks of a wave
+    // rings (at least the 1 KB per chain and tile in which the chains' sums meet at the end); front: the waves'
+    // activations, 1 KB per chunk; the waves' offset tables [8 blocks][2 rp] floats per chunk (front: every chunk,
+    // else the ring's two)
+    int ring = kDmaDepth * gemv_dma_entry(rp, rows_wg);
+    const int sums = kDmaChains / waves * gemv_dma_tiles(ni) * 64 * 16;
+    ring = ring > sums ? ring : sums;
+    return waves * ring + (gemv_dma_front(rp) ? waves * per_wave * (1024 + 64) : waves * 2 * 64 * rp);
+}
+
+template <int RP, int NI, int WAVES>
+__global__ void __launch_bounds__(64 * WAVES, 1) gemv_q8_dma_kernel(const uint8_t *__restrict__ w,
+                                                                                 const float *__restrict__ x,
+                                                                                 float *__restrict__ y, int m, int k,
+                                                                                 int rows, int rows_wg)
+{
+    static_assert(RP == 1 || RP == 2 || RP == 4 || RP == 8, "activation rows per pass");
+    static_assert(WAVES == 4 || WAVES == 8, "the eight chains are dealt to four or eight waves");
+    constexpr int kWaves = WAVES;
+    constexpr int kNCh = kDmaChains / kWaves; // chains of a wave
+    constexpr int kNT = gemv_dma_tiles(NI);
+    constexpr bool kFront = gemv_dma_front(RP);
+    constexpr int kDepth = kDmaDepth;
+    constexpr int kReq = NI + (kFront ? 0 : RP); // requests per chunk
+    constexpr int kNJ = RP < 4 ? RP : 4;         // accumulator rows a lane needs
+    constexpr int kUnits = 32 * RP;              // (block, row, quarter) units of 8 activations per chunk
+    constexpr int kPasses = (kUnits + 63) / 64;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int lane = threadIdx.x & 63;
+    const int lm = lane & 15, lg = lane >> 4;
+    const int nb = k >> 5;
+    const int nchunk = nb >> 3;
+    const uint32_t row_bytes = (uint32_t)nb * kQ8Block;
+    const int m0 = blockIdx.x * rows_wg;
+    const int r0 = blockIdx.y * RP;
+    const int nrows = rows - r0 < RP ? rows - r0 : RP;
+    const int pieces = rows_wg * 17;
+    if ((pieces + 63) / 64 != NI)
+        return; // (the launcher's contract: the waits below count NI requests per chunk of weights)
+    const int mine = wave < nchunk ? (nchunk - wave + kWaves - 1) / kWaves : 0; // chunks wave, wave + kWaves, ...
+    const int per_wave = (nchunk + kWaves - 1) / kWaves;
+
+    const int entry = pieces * 16 + (kFront ? 0 : RP * 1024);
+    constexpr int kSums = kNCh * kNT * 64 * 16; // where this wave's chains leave their sums: the head of its ring
+    const int ring_bytes = kDepth * entry > kSums ? kDepth * entry : kSums;
+    uint8_t *ring = lds + wave * ring_bytes;
+    uint8_t *xfront = lds + kWaves * ring_bytes + wave * per_wave * 1024; // (front only)
+    uint8_t *after_x = lds + kWaves * ring_bytes + (kFront ? kWaves * per_wave * 1024 : 0);
+    float *offs = reinterpret_cast<float *>(after_x + wave * (kFront ? per_wave * 64 : 2 * 64 * RP));
+    const uint32_t ring_at = proj_lds_address(ring);
+
+    // ---- requests ---------------------------------------------------------------------------------------------
+    // weights: piece p = 64 j + lane of the chunk: row p / 17 of the workgroup, 16 bytes p % 17 of its 272; rows
+    // past the end of the matrix repeat the last one (never stored)
+    uint32_t woff[NI];
+#pragma unroll
+    for (int j = 0; j < NI; j++) {
+        const int p = j * 64 + lane;
+        const int pr = p / 17, pq = p - pr * 17;
+        const int row = m0 + pr < m ? m0 + pr : m - 1;
+        woff[j] = (uint32_t)row * row_bytes + (uint32_t)pq * 16u;
+    }
+    const uint8_t *xb = reinterpret_cast<const uint8_t *>(x + (size_t)r0 * k);
+    auto issue = [&](int i) {
+        const uint32_t at = ring_at + (uint32_t)((i % kDepth) * entry);
+        const uint32_t c = (uint32_t)(wave + i * kWaves);
+        // activations behind the weights: one request per row, its 256 floats of the chunk as they lie in memory;
+        // rows past the live ones repeat the last
+        if (!kFront) {
+#pragma unroll
+            for (int r = 0; r < RP; r++) {
+                const uint32_t rr = (uint32_t)(r < nrows ? r : nrows - 1);
+                proj_dma16<false>(at + pieces * 16 + r * 1024, xb, rr * (uint32_t)k * 4u + c * 1024u + lane * 16u);
+            }
+        }
+        // (NI = ceil(pieces / 64): every request has a live lane, so each chunk counts NI requests)
+#pragma unroll
+        for (int j = 0; j < NI; j++) {
+            if (j * 64 + lane < pieces)
+                proj_dma16<true>(at + j * 1024, w, woff[j] + c * kDmaChunkBytes);
+        }
+    };
+    if (kFront) {
+        for (int i = 0; i < mine; i++)
+            proj_dma16<false>(proj_lds_address(xfront) + i * 1024, xb, (uint32_t)(wave + i * kWaves) * 1024u + lane * 16u);
+    }
+#pragma unroll
+    for (int i = 0; i < kDepth; i++)
+        if (i < mine)
+            issue(i);
+    // all but the newest `newer` chunks (at most kDepth - 1) have arrived: requests return in order
+    auto wait_chunks = [&](int newer) {
+        if (newer >= 2 && kDepth > 2)
+            wait_vm<(kDepth > 2 ? 2 : 0) * kReq>();
+        else if (newer >= 1)
+            wait_vm<kReq>();
+        else
+            wait_vm<0>();
+    };
+
+    // ---- activations -> operands, in place: unit ((block b, row r), quarter q): 8 floats -> 8 hi and 8 lo halves in
+    // the operand order of the block, and the block's offset terms.  Every unit of an area is read before any is
+    // written (one wave, LDS in program order).
+    auto unit_write = [&](uint8_t *area, float *off, int b, int r, int q, bool on, const float4v &a4, const float4v &b4) {
+        half8 hi, lo;
+        split_hi_lo(a4, b4, hi, lo);
+        float sh = 0.0f, sl = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            sh += (float)hi[e];
+            sl += (float)lo[e];
+        }
+        // over the unit's four quarters (the lanes of a quad)
+        sh += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, sh), 0xB1, 0xf, 0xf, true));
+        sl += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, sl), 0xB1, 0xf, 0xf, true));
+        sh += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, sh), 0x4E, 0xf, 0xf, true));
+        sl += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, sl), 0x4E, 0xf, 0xf, true));
+        if (on) {
+            uint8_t *blk = area + b * (RP * 128) + q * 16;
+            *reinterpret_cast<half8 *>(blk + r * 64) = hi;
+            *reinterpret_cast<half8 *>(blk + (RP + r) * 64) = lo;
+            if (q == 0) {
+                off[b * 2 * RP + r] = sh * (128.0f / kTwo24f);
+                off[b * 2 * RP + RP + r] = sl * (128.0f / kTwo24f);
+            }
+        }
+    };
+    if (kFront) {
+        // two chunks per pass: lanes 0..31 the units of chunk 2 ps, lanes 32..63 those of chunk 2 ps + 1
+        constexpr int kFrontPasses = 2;
+        // only weights are still travelling
+        if (mine >= 2)
+            wait_vm<2 * NI>();
+        else
+            wait_vm<NI>();
+        for (int i0 = 0; i0 < mine; i0 += 2 * kFrontPasses) {
+            float4v a4[kFrontPasses], b4[kFrontPasses];
+#pragma unroll
+            for (int ps = 0; ps < kFrontPasses; ps++) {
+                const int i = i0 + 2 * ps + (lane >> 5);
+                const uint8_t *src = xfront + (i < mine ? i : 0) * 1024 + (lane & 31) * 32;
+                a4[ps] = *reinterpret_cast<const float4v *>(src);
+                b4[ps] = *reinterpret_cast<const float4v *>(src + 16);
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int ps = 0; ps < kFrontPasses; ps++) {
+                const int i = i0 + 2 * ps + (lane >> 5);
+                unit_write(xfront + i * 1024, offs + i * 16, (lane & 31) >> 2, 0, lane & 3, i < mine, a4[ps], b4[ps]);
+            }
+        }
+    }
+
+    float4v acc[kNCh][kNT];
+#pragma unroll
+    for (int s = 0; s < kNCh; s++)
+#pragma unroll
+        for (int t = 0; t < kNT; t++)
+            acc[s][t] = (float4v){0, 0, 0, 0};
+    // A row lm: half lm / 8 (hi, lo) of activation row lm % 8; rows past the live ones repeat a valid slot
+    // (their products are never read)
+    const int arow = (lm & 7) < nrows ? (lm & 7) : nrows - 1;
+    const int xslot = (((lm >> 3) * RP + arow) * 4 + lg) * 16;
+    // the lane's accumulators are C rows 4 lg + j: half lg / 2, activation rows 4 (lg % 2) + j
+    const int obase = (lg >> 1) * RP + ((lg & 1) * 4 < RP ? (lg & 1) * 4 : 0);
+    int wrow[kNT]; // (rows of the second tile past rows_wg repeat the last: never stored)
+#pragma unroll
+    for (int t = 0; t < kNT; t++)
+        wrow[t] = (t * 16 + lm < rows_wg ? t * 16 + lm : rows_wg - 1) * kDmaChunkBytes;
+
+    auto chunk = [&](int i, float4v (&sum)[kNT]) {
+        wait_chunks(mine - 1 - i < kDepth - 1 ? mine - 1 - i : kDepth - 1);
+        uint8_t *buf = ring + (i % kDepth) * entry;
+        uint8_t *xa = kFront ? xfront + i * 1024 : buf + pieces * 16;
+        float *off = offs + (kFront ? i : (i & 1)) * (16 * RP);
+        if (!kFront) {
+            float4v a4[kPasses], b4[kPasses];
+#pragma unroll
+            for (int ps = 0; ps < kPasses; ps++) {
+                const int u = ps * 64 + lane;
+                const int br = u >> 2, q = u & 3;
+                const int b = br / RP, r = br - b * RP;
+                const uint8_t *src = xa + (u < kUnits ? r * 1024 + b * 128 + q * 32 : 0);
+                a4[ps] = *reinterpret_cast<const float4v *>(src);
+                b4[ps] = *reinterpret_cast<const float4v *>(src + 16);
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int ps = 0; ps < kPasses; ps++) {
+                const int u = ps * 64 + lane;
+                const int br = u >> 2, q = u & 3;
+                const int b = br / RP, r = br - b * RP;
+                unit_write(xa, off, b, r, q, u < kUnits, a4[ps], b4[ps]);
+            }
+        }
+        // ---- the chunk's 8 blocks, in two halves: the reads of the second travel while the first is multiplied
+        half8 xop[8];
+        float ofs[8][kNJ];
+        uint32_t qa[8][kNT], qb[8][kNT], qc[4][kNT];
+        _Float16 dh[8][kNT];
+        auto read_block = [&](int b) {
+            xop[b] = *reinterpret_cast<const half8 *>(xa + b * (RP * 128) + xslot);
+#pragma unroll
+            for (int j = 0; j < kNJ; j++)
+                ofs[b][j] = off[b * 2 * RP + obase + j];
+#pragma unroll
+            for (int t = 0; t < kNT; t++) {
+                const uint8_t *blk = buf + wrow[t] + b * kQ8Block;
+                // the lane's 8 bytes sit 2 bytes past a dword boundary in even blocks (three dwords, realigned
+                // below) and at one in odd blocks
+                if ((b & 1) == 0) {
+                    const uint3a4 e = *reinterpret_cast<const uint3a4 *>(blk + lg * 8);
+                    qa[b][t] = e[0];
+                    qb[b][t] = e[1];
+                    qc[b >> 1][t] = e[2];
+                } else {
+                    const uint2a4 o = *reinterpret_cast<const uint2a4 *>(blk + 2 + lg * 8);
+                    qa[b][t] = o[0];
+                    qb[b][t] = o[1];
+                }
+                dh[b][t] = *reinterpret_cast<const _Float16 *>(blk);
+            }
+        };
+        auto math_block = [&](int b) {
+#pragma unroll
+            for (int t = 0; t < kNT; t++) {
+                uint32_t q0 = qa[b][t], q1 = qb[b][t];
+                if ((b & 1) == 0) {
+                    q0 = __builtin_amdgcn_alignbit(qb[b][t], qa[b][t], 16);
+                    q1 = __builtin_amdgcn_alignbit(qc[b >> 1][t], qb[b][t], 16);
+                }
+                const float d = (float)dh[b][t];
+                const half8 wv = int8x8_to_f16_sub(q0, q1);
+                float4v p = {0, 0, 0, 0};
+                p = __builtin_amdgcn_mfma_f32_16x16x32_f16(xop[b], wv, p, 0, 0, 0);
+#pragma unroll
+                for (int j = 0; j < kNJ; j++)
+                    sum[t][j] = fmaf(d, p[j] - ofs[b][j], sum[t][j]);
+            }
+        };
+#pragma unroll
+        for (int b = 0; b < 4; b++)
+            read_block(b);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int b = 4; b < 8; b++)
+            read_block(b);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int b = 0; b < 4; b++)
+            math_block(b);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int b = 4; b < 8; b++)
+            math_block(b);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // the wave's reads of this entry are done
+        if (i + kDepth < mine)
+            issue(i + kDepth);
+    };
+    // chunk wave + i kWaves belongs to chain wave + (i % kNCh) kWaves
+    for (int i0 = 0; i0 < mine; i0 += kNCh) {
+#pragma unroll
+        for (int s = 0; s < kNCh; s++)
+            if (i0 + s < mine)
+                chunk(i0 + s, acc[s]);
+    }
+
+    // ---- the chains' sums meet in their order; lanes lg = 0, 1 hold the hi products of activation rows 4 lg + j,
+    // lanes lg = 2, 3 the lo products ----------------------------------------------------------------------------
+    // (a wave leaves its chains' sums at the head of its own ring, which it has finished reading)
+    auto sums_of = [&](int chain, int t) {
+        return reinterpret_cast<float4v *>(lds + (chain % kWaves) * ring_bytes) + ((chain / kWaves) * kNT + t) * 64;
+    };
+#pragma unroll
+    for (int s = 0; s < kNCh; s++)
+#pragma unroll
+        for (int t = 0; t < kNT; t++)
+            sums_of(wave + s * kWaves, t)[lane] = acc[s][t];
+    __syncthreads();
+    if (threadIdx.x < 32 * kNT) {
+        const int t = threadIdx.x >> 5, l = threadIdx.x & 31; // (weight row 16 t + l % 16, activation rows 4 (l / 16) + j)
+        float4v hi = sums_of(0, t)[l], lo = sums_of(0, t)[32 + l];
+#pragma unroll
+        for (int c = 1; c < kDmaChains; c++) {
+            hi += sums_of(c, t)[l];
+            lo += sums_of(c, t)[32 + l];
+        }
+        const float4v s = (hi + lo) * kTwo24f;
+        const int wr = t * 16 + (l & 15);
+        if (wr < rows_wg && m0 + wr < m) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int r = (l >> 4) * 4 + j;
+                if (r < nrows)
+                    y[(size_t)(r0 + r) * m + m0 + wr] = s[j];
+            }
+        }
+    }
+}
+
 // ---- gemv_q8_tile_kernel: 3 to 128 activation rows (batched decode, verify groups) --------------
 //
 // The same streaming of W as above, with the activations as full 16-row A tiles: A row = activation
@@ -515,8 +897,73 @@ static int launch_gemv_variant(hipStream_t st, const uint8_t *w, const float *x,
     return launch_gemv_xg<WAVES, TILES, CH, 8>(st, w, x, y, m, k, rows, rp);
 }
 
+// the most waves (8, else 4) whose rings and tables fit a CU's LDS; 0: none
+static int gemv_dma_waves(int rp, int ni, int rows_wg, int k)
+{
+    for (int waves = 8; waves >= 4; waves -= 4)
+        if (gemv_dma_lds(rp, ni, waves, rows_wg, k) <= (160 << 10))
+            return waves;
+    return 0;
+}
+
+template <int RP, int NI>
+static int launch_gemv_dma(hipStream_t st, const uint8_t *w, const float *x, float *y, int m, int k, int rows, int rows_wg)
+{
+    const dim3 grid((unsigned)((m + rows_wg - 1) / rows_wg), (unsigned)((rows + RP - 1) / RP), 1);
+    const int waves = gemv_dma_waves(RP, NI, rows_wg, k);
+    const size_t lds = (size_t)gemv_dma_lds(RP, NI, waves, rows_wg, k);
+    if (waves == 8)
+        HIPML_LAUNCH((gemv_q8_dma_kernel<RP, NI, 8>), grid, dim3(512, 1, 1), lds, st, w, x, y, m, k, rows, rows_wg);
+    else
+        HIPML_LAUNCH((gemv_q8_dma_kernel<RP, NI, 4>), grid, dim3(256, 1, 1), lds, st, w, x, y, m, k, rows, rows_wg);
+    return launched("gemv_q8_0_rows");
+}
+
+template <int NI>
+static int launch_gemv_dma_rows(hipStream_t st, const uint8_t *w, const float *x, float *y, int m, int k, int rows, int rows_wg)
+{
+    if (rows == 1)
+        return launch_gemv_dma<1, NI>(st, w, x, y, m, k, rows, rows_wg);
+    if (rows == 2)
+        return launch_gemv_dma<2, NI>(st, w, x, y, m, k, rows, rows_wg);
+    if (rows <= 4)
+        return launch_gemv_dma<4, NI>(st, w, x, y, m, k, rows, rows_wg);
+    return launch_gemv_dma<8, NI>(st, w, x, y, m, k, rows, rows_wg);
+}
+
+// Up to eight rows over the raw-row kernel: rows of whole 256-value chunks at 16-byte boundaries, addressed with
+// 32-bit offsets, and LDS room for every row count (so that all of them take this kernel, or none).  Returns -1
+// where the shape does not qualify (the kernels above serve it).
+static int try_gemv_dma(hipStream_t st, const uint8_t *w, const float *x, float *y, int m, int k, int rows)
+{
+    if (rows > 8 || k % 256 != 0 || (reinterpret_cast<uintptr_t>(w) & 15) != 0 ||
+        (reinterpret_cast<uintptr_t>(x) & 15) != 0 || (size_t)m * (k >> 5) * kQ8Block >= ((size_t)1 << 32) ||
+        (size_t)rows * k * sizeof(float) >= ((size_t)1 << 32))
+        return -1;
+    // the fewest weight rows per workgroup that make one round of the chip's 256 CUs
+    static const int kRowsWg[4] = {16, 20, 24, 32}, kNi[4] = {5, 6, 7, 9};
+    int v = 3;
+    for (int i = 0; i < 4; i++)
+        if ((m + kRowsWg[i] - 1) / kRowsWg[i] <= 256) {
+            v = i;
+            break;
+        }
+    for (int rp = 1; rp <= 8; rp *= 2)
+        if (gemv_dma_waves(rp, kNi[v], kRowsWg[v], k) == 0)
+            return -1;
+    switch (v) {
+    case 0: return launch_gemv_dma_rows<5>(st, w, x, y, m, k, rows, 16);
+    case 1: return launch_gemv_dma_rows<6>(st, w, x, y, m, k, rows, 20);
+    case 2: return launch_gemv_dma_rows<7>(st, w, x, y, m, k, rows, 24);
+    default: return launch_gemv_dma_rows<9>(st, w, x, y, m, k, rows, 32);
+    }
+}
+
 int launch_gemv_q8_rows(hipStream_t st, const uint8_t *w, const float *x, float *y, int m, int k, int rows)
 {
+    const int dma = try_gemv_dma(st, w, x, y, m, k, rows);
+    if (dma >= 0)
+        return dma;
     // three rows or more: full A tiles of 16 or 32 rows (measured at 5120 x 6144, 4 rows: 14.6 us
     // against 16.7 us for the row kernel with two weight tiles per workgroup; 1 row: 13.6 against 12.1)
     if (rows > kGemvMaxRows)
@@ -862,6 +1309,21 @@ int proj_init()
                                 hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLds);
     if (e == hipSuccess)
         e = raise_gemv_lds<8, 1, 6>();
+    auto raise = [&](const void *f) {
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, 160 << 10);
+    };
+#define HIPML_RAISE_DMA(ni) \
+    raise(reinterpret_cast<const void *>(&gemv_q8_dma_kernel<1, ni, 8>)); \
+    raise(reinterpret_cast<const void *>(&gemv_q8_dma_kernel<2, ni, 8>)); \
+    raise(reinterpret_cast<const void *>(&gemv_q8_dma_kernel<4, ni, 8>)); \
+    raise(reinterpret_cast<const void *>(&gemv_q8_dma_kernel<8, ni, 8>)); \
+    raise(reinterpret_cast<const void *>(&gemv_q8_dma_kernel<1, ni, 4>)); \
+    raise(reinterpret_cast<const void *>(&gemv_q8_dma_kernel<2, ni, 4>)); \
+    raise(reinterpret_cast<const void *>(&gemv_q8_dma_kernel<4, ni, 4>)); \
+    raise(reinterpret_cast<const void *>(&gemv_q8_dma_kernel<8, ni, 4>));
+    HIPML_RAISE_DMA(5) HIPML_RAISE_DMA(6) HIPML_RAISE_DMA(7) HIPML_RAISE_DMA(9)
+#undef HIPML_RAISE_DMA
     if (e != hipSuccess)
         return fail((int)e, "hipFuncSetAttribute(projection LDS) failed: %d (%s)", (int)e, hipGetErrorString(e));
     return 0;

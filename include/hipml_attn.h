@@ -504,9 +504,13 @@ int hipml_kv_rows_copy(hipml_stream_t stream, int dtype, const void *k_src, cons
 /* y[r][row] = sum_k W[row][k] * x[r][k] for r < rows: W is m rows of k/32 Q8_0 blocks (34 bytes:
  * f16 scale, 32 int8) at a 4-byte aligned address, x is f32 [rows][k] (16-byte aligned), y is f32
  * [rows][m]; k a multiple of 64 up to 32768, 1 <= rows <= 128.
- * W streams from memory once per 4 rows; fp32 accumulation of exact integer block products (the
- * activations enter as hi + lo f16 halves), so every row has the precision class of the
- * reference's f32 GEMV kernels and row r does not depend on `rows`.
+ * fp32 accumulation of exact integer block products (the activations enter as hi + lo f16 halves), so
+ * every row has the precision class of the reference's f32 GEMV kernels.  Up to 8 rows W streams from
+ * memory once and a row's result has the same bits whatever `rows` is and whichever rows travel with it:
+ * the rows of a verify group match their plain decodes, as the reference's batched GEMVs do
+ * (crates/hipml-kernels/src/attn_gpu.rs:930-932).  From 9 rows on W streams once per 16 or 32 rows and a
+ * row's bits are again the same for every such `rows`, but not those of the call with up to 8.
+ * (W at a 16-byte aligned address and k a multiple of 256 take the fastest road.)
  * Replaces AttnLayer::gemv / gemv_rows / gemv_batched over a Q8_0 ResidentMat (the output
  * projection of apply_output / output_rows, and W_q, W_k, W_v in prepare_rows),
  * crates/hipml-kernels/src/attn_gpu.rs:843-846,967-1023,1066-1117 -> gemv_q8_0 / gemv_q8_0_b,
