@@ -1151,16 +1151,16 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Front
             issue_as(std::false_type(), std::true_type(), false, 0);
     };
 
-    // live lengths of this slot's rows: scalar loads, requested before the first asm statement (the
-    // compiler reads memory it must assume changed with vector loads, and would then wait for all loads)
-    int seqc[kMaxCols];
-    int seq_max = 0;
-#pragma unroll
-    for (int c = 0; c < kMaxCols; c++) {
-        int s = c < ncols ? f.pos[(size_t)(row0 + c) * 2 + 1] : 0;
-        s = s < 0 ? 0 : (s > f.stride ? f.stride : s);
-        seqc[c] = s;
-        seq_max = s > seq_max ? s : seq_max;
+    // live lengths of this slot's rows: lane c asks for that of row row0 + c with the launch's first vector load,
+    // written out so that the wait is this code's own.  Requests return in order, so the wait for the Q rows
+    // below is the wait for this one as well.  (As scalar loads they took 2 us to come back under the launch's
+    // first burst, and every wait for an LDS read is one for outstanding scalar loads too: the Q conversion
+    // stood behind them.  Left to the compiler, a vector load would be waited for with vmcnt(0): it does not
+    // count the requests made in asm statements.)
+    int pos_lane;
+    {
+        const int32_t *pp = f.pos + (size_t)(row0 + (lane < ncols ? lane : 0)) * 2 + 1;
+        asm volatile("global_load_dword %0, %1, off" : "=v"(pos_lane) : "v"(pp) : "memory");
     }
 
     // ---- the first requests: the Q rows, then the K rows of tile 0 ------------------------------
@@ -1215,6 +1215,21 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Front
         else
             asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
     };
+    // the Q rows are in LDS, and the live lengths in their register, once only the requests behind them are
+    // outstanding: K(0)
+    if (Q4)
+        asm volatile("s_waitcnt vmcnt(5)" : "+v"(pos_lane) : : "memory");
+    else
+        asm volatile("s_waitcnt vmcnt(9)" : "+v"(pos_lane) : : "memory");
+    int seqc[kMaxCols];
+    int seq_max = 0;
+#pragma unroll
+    for (int c = 0; c < kMaxCols; c++) {
+        int s = c < ncols ? __builtin_amdgcn_readlane(pos_lane, c) : 0;
+        s = s < 0 ? 0 : (s > f.stride ? f.stride : s);
+        seqc[c] = s;
+        seq_max = s > seq_max ? s : seq_max;
+    }
     const int hi = seq_max; // keys at or past it are masked
     if (split * kWaves * kTileKeys >= hi) {
         // not one live tile for any wave of this workgroup: leave an empty partial, which the merge skips
@@ -1231,8 +1246,6 @@ __device__ __forceinline__ void decode_body_dma(const DecodeArgs &a, const Front
     const int ntile = first_key < hi ? (hi - first_key + step_keys - 1) / step_keys : 0;
 
     // ---- Q operands and the score bias of every block ------------------------------------------
-    // the Q rows are in LDS once only the requests behind them are outstanding: K(0)
-    wait_all_but_one_tile();
     float4v qf[kQB][2];
 #pragma unroll
     for (int cc = 0; cc < kQB; cc++)
