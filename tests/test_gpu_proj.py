@@ -113,6 +113,37 @@ def test_ragged_shapes_and_scales():
         assert np.max(np.abs(got - exact)) <= max(2 * np.max(np.abs(want - exact)), 1e-5)
 
 
+@pytest.mark.parametrize("m,k", [(1, 256), (17, 512), (33, 768), (100, 2304), (5121, 1024), (6150, 512), (8200, 256),
+                                 (300, 8192)])
+def test_raw_row_kernel_over_ragged_shapes(m, k):
+    # k a multiple of 256 and up to 8 rows take the kernel that moves the weight rows into LDS as they lie: fewer
+    # rows than a workgroup takes, a last workgroup with a single row, 20 / 24 / 32 rows per workgroup (m above 4,096
+    # / 5,120 / 6,144), one chunk per row (seven of eight waves idle), nine chunks (uneven shares), 32 chunks; real
+    # scales.  Every row count against the oracle, and a row's bits the same whatever travels with it.
+    r = orc.Rng(0x0D3A + m + k)
+    w = orc.random_q8_0_bytes(r, m * k // 32).reshape(-1, 34)
+    scales = (r.uniform_array(w.shape[0]) * 0.05 + 0.001).astype(np.float16)
+    w[:, :2] = scales.view(np.uint8).reshape(-1, 2)
+    w = w.ravel()
+    x = r.normal_array((8, k))
+    want = orc.gemm_q8_0(w, x, 8, m, k, n_threads=8)
+    blocks = w.reshape(m, k // 32, 34)
+    dense = (blocks[:, :, :2].copy().view(np.float16).astype(np.float64)
+             * blocks[:, :, 2:].view(np.int8).astype(np.float64)).reshape(m, k)
+    exact = x.astype(np.float64) @ dense.T
+    alone = [run_gemv(w, x[i], m, k, 1)[0] for i in range(8)]
+    for rows in (1, 2, 3, 4, 5, 7, 8):
+        got = run_gemv(w, x[:rows], m, k, rows)
+        ok, _, _ = report(f"raw-row {m}x{k} rows={rows}", want[:rows], got, 2e-3, 3e-2)
+        assert ok
+        # as close to the float64 value as a sequential fp32 sum is, or 21 bits of the largest output (the
+        # activations enter with ~22 bits, and the offset of the weight bytes is taken out again in fp32)
+        bound = max(2 * np.max(np.abs(want[:rows] - exact[:rows])), 2e-6 * np.max(np.abs(exact[:rows])) + 1e-5)
+        assert np.max(np.abs(got - exact[:rows])) <= bound
+        for i in range(rows):
+            assert np.array_equal(got[i], alone[i]), f"rows={rows} row {i}"
+
+
 def test_argument_errors():
     w = torch.zeros(34 * 4, dtype=torch.uint8, device="cuda")
     x = torch.zeros(64, device="cuda")
