@@ -681,6 +681,205 @@ __global__ void __launch_bounds__(64 * WAVES, 1) gemv_q8_dma_kernel(const uint8_
     }
 }
 
+// ---- gemv_q8_dma_tile_kernel: 9 to 64 activation rows over the same stream of raw weight rows ------------------
+//
+// More rows than the kernel above holds operands for.  The workgroups are the same (rows_wg consecutive weight
+// rows, one workgroup per CU, eight waves), but the waves walk the chunks together: for a chunk of 256 values the
+// workgroup fetches its weight rows and the same 256 values of every activation row as raw f32 (1 KB per row, all
+// through global_load_lds_dwordx4, the requests dealt to the waves), and wave w multiplies block w of the chunk.  So
+// a workgroup reads every activation once, from LDS.
+// Lane (row lm, quarter lg) of an A tile reads its 8 floats and splits them into hi and lo halves in registers;
+// a block and tile is two chained MFMAs (hi, then lo into the same fp32 sums) per weight tile, the weights exactly as
+// f16 integers (1024 + u trick), the block scale applied to the fp32 dot product.  The activation rows lie 1,040
+// bytes apart in LDS, so the 16 rows of a tile start in 16 different banks.
+// Two rings: kDW chunks of weights and kDX chunks of activations are in flight, two barriers per chunk.  Vector
+// memory returns in order, so a wave that waits for its activation requests of a chunk also waits for every weight
+// request it made before them: the activations of chunk c + kDX are asked for before the weights of chunk c + kDW,
+// and the wait counts the activation requests behind it only.
+// A (row, weight row) result is the sum in wave order of eight chains (block b of every chunk belongs to chain b):
+// the same whatever the number of rows, and other bits than those of the kernel for up to 8 rows.
+constexpr int kTileRowPitch = 1040;
+// (chunks of activations / of weights in flight, measured at 5120 x 6144 over 16 / 24 / 32 / 64 rows: 2 / 3: 17.5 / 23.4 /
+// 23.5 / 39.8 us; 2 / 4: 17.9 / 29.0 / 29.1 / 41.4; 3 / 6: 18.3 / 25.5 / 25.6 / -; the tile kernel below: 19.6 / 25.8 / 29.7 /
+// 54.5)
+constexpr int gemv_tile_dx(int) { return 2; }
+constexpr int gemv_tile_dw(int) { return 3; }
+inline int gemv_dma_tile_lds(int xt, int ni, int rows_wg)
+{
+    const int ring = gemv_tile_dw(xt) * rows_wg * 17 * 16 + gemv_tile_dx(xt) * 16 * xt * kTileRowPitch;
+    const int sums = 8 * xt * gemv_dma_tiles(ni) * 64 * 16;
+    return ring > sums ? ring : sums;
+}
+
+template <int XT, int NI>
+__global__ void __launch_bounds__(512, 1) gemv_q8_dma_tile_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x,
+                                                                   float *__restrict__ y, int m, int k, int rows,
+                                                                   int rows_wg)
+{
+    constexpr int kNT = gemv_dma_tiles(NI);
+    constexpr int kXRows = 16 * XT;
+    constexpr int kDX = gemv_tile_dx(XT), kDW = gemv_tile_dw(XT);
+    static_assert(kDW > kDX, "a chunk's weights are asked for before its activations");
+    constexpr int kNX = 2 * XT;              // activation requests of a wave per chunk (one per row, 16 XT rows)
+    constexpr int kWMost = (NI + 7) / 8;     // weight requests of a wave per chunk, or one less
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int lane = threadIdx.x & 63;
+    const int lm = lane & 15, lg = lane >> 4;
+    const int nb = k >> 5;
+    const int nchunk = nb >> 3;
+    const uint32_t row_bytes = (uint32_t)nb * kQ8Block;
+    const int m0 = blockIdx.x * rows_wg;
+    const int r0 = blockIdx.y * kXRows;
+    const int nrows = rows - r0 < kXRows ? rows - r0 : kXRows;
+    const int pieces = rows_wg * 17;
+    if ((pieces + 63) / 64 != NI)
+        return; // (the launcher's contract: a chunk of weights is NI requests)
+    const int wbytes = pieces * 16;
+    constexpr int kXBytes = kXRows * kTileRowPitch;
+    uint8_t *wring = lds, *xring = lds + kDW * wbytes;
+    const uint32_t wring_at = proj_lds_address(wring), xring_at = proj_lds_address(xring);
+
+    // weights of chunk c: request q = wave + 8 j < NI brings 64 pieces (piece p: row p / 17 of the workgroup, 16
+    // bytes p % 17 of its 272; rows past the end of the matrix repeat the last)
+    uint32_t woff[kWMost];
+#pragma unroll
+    for (int j = 0; j < kWMost; j++) {
+        const int p = (wave + 8 * j) * 64 + lane;
+        const int pr = p / 17, pq = p - pr * 17;
+        const int row = m0 + pr < m ? m0 + pr : m - 1;
+        woff[j] = (uint32_t)row * row_bytes + (uint32_t)pq * 16u;
+    }
+    auto issue_w = [&](int c) {
+        const uint32_t at = wring_at + (uint32_t)((c % kDW) * wbytes);
+#pragma unroll
+        for (int j = 0; j < kWMost; j++) {
+            const int q = wave + 8 * j;
+            if (q < NI && q * 64 + lane < pieces)
+                proj_dma16<true>(at + q * 1024, w, woff[j] + (uint32_t)c * kDmaChunkBytes);
+        }
+    };
+    // activations of chunk c: rows wave + 8 j of the pass (rows past the live ones repeat the last), 256 floats each
+    const uint8_t *xb = reinterpret_cast<const uint8_t *>(x + (size_t)r0 * k);
+    uint32_t xoff[kNX];
+#pragma unroll
+    for (int j = 0; j < kNX; j++) {
+        const int r = wave + 8 * j;
+        xoff[j] = (uint32_t)(r < nrows ? r : nrows - 1) * (uint32_t)k * 4u + lane * 16u;
+    }
+    auto issue_x = [&](int c) {
+        const uint32_t at = xring_at + (uint32_t)((c % kDX) * kXBytes);
+#pragma unroll
+        for (int j = 0; j < kNX; j++)
+            proj_dma16<false>(at + (wave + 8 * j) * kTileRowPitch, xb, xoff[j] + (uint32_t)c * 1024u);
+    };
+#pragma unroll
+    for (int c = 0; c < kDW; c++)
+        if (c < nchunk)
+            issue_w(c);
+#pragma unroll
+    for (int c = 0; c < kDX; c++)
+        if (c < nchunk)
+            issue_x(c);
+
+    float4v acc[XT][kNT];
+#pragma unroll
+    for (int xt = 0; xt < XT; xt++)
+#pragma unroll
+        for (int t = 0; t < kNT; t++)
+            acc[xt][t] = (float4v){0, 0, 0, 0};
+    int wrow[kNT]; // (rows of the second tile past rows_wg repeat the last: never stored)
+#pragma unroll
+    for (int t = 0; t < kNT; t++)
+        wrow[t] = (t * 16 + lm < rows_wg ? t * 16 + lm : rows_wg - 1) * kDmaChunkBytes;
+    const int b = wave; // this wave's block of every chunk
+
+    for (int c = 0; c < nchunk; c++) {
+        // this wave's requests for chunk c have arrived: behind its activation requests of chunk c there are, among
+        // others, those of the chunks up to c + kDX - 1 that exist (counting only those errs on the side of waiting)
+        {
+            const int behind = nchunk - 1 - c < kDX - 1 ? nchunk - 1 - c : kDX - 1;
+            if (behind >= 3 && kDX > 3)
+                wait_vm<(kDX > 3 ? 3 : 0) * kNX>();
+            else if (behind >= 2 && kDX > 2)
+                wait_vm<(kDX > 2 ? 2 : 0) * kNX>();
+            else if (behind >= 1)
+                wait_vm<kNX>();
+            else
+                wait_vm<0>();
+        }
+        __syncthreads(); // ... and every wave's
+        const uint8_t *wbuf = wring + (c % kDW) * wbytes;
+        const uint8_t *xa = xring + (c % kDX) * kXBytes + b * 128 + lg * 32;
+        half8 wv[kNT];
+        float d[kNT];
+#pragma unroll
+        for (int t = 0; t < kNT; t++) {
+            const uint8_t *blk = wbuf + wrow[t] + b * kQ8Block;
+            uint32_t q0, q1;
+            if ((b & 1) == 0) { // (uniform) even blocks sit 2 bytes past a dword boundary
+                const uint3a4 e = *reinterpret_cast<const uint3a4 *>(blk + lg * 8);
+                q0 = __builtin_amdgcn_alignbit(e[1], e[0], 16);
+                q1 = __builtin_amdgcn_alignbit(e[2], e[1], 16);
+            } else {
+                const uint2a4 o = *reinterpret_cast<const uint2a4 *>(blk + 2 + lg * 8);
+                q0 = o[0];
+                q1 = o[1];
+            }
+            d[t] = (float)*reinterpret_cast<const _Float16 *>(blk);
+            wv[t] = int8x8_to_f16(q0, q1);
+        }
+#pragma unroll
+        for (int xt = 0; xt < XT; xt++) {
+            const uint8_t *src = xa + (xt * 16 + lm) * kTileRowPitch;
+            const float4v a4 = *reinterpret_cast<const float4v *>(src);
+            const float4v b4 = *reinterpret_cast<const float4v *>(src + 16);
+            half8 hi, lo;
+            split_hi_lo(a4, b4, hi, lo);
+#pragma unroll
+            for (int t = 0; t < kNT; t++) {
+                float4v p = {0, 0, 0, 0};
+                p = __builtin_amdgcn_mfma_f32_16x16x32_f16(hi, wv[t], p, 0, 0, 0);
+                p = __builtin_amdgcn_mfma_f32_16x16x32_f16(lo, wv[t], p, 0, 0, 0);
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    acc[xt][t][j] = fmaf(d[t], p[j], acc[xt][t][j]);
+            }
+        }
+        __syncthreads(); // every wave is done with the chunk's entries: later chunks may land in them
+        if (c + kDX < nchunk)
+            issue_x(c + kDX);
+        if (c + kDW < nchunk)
+            issue_w(c + kDW);
+    }
+
+    // ---- the waves' sums meet in wave order (the rings are free: the loop ended on a barrier) --------------------
+    float4v *red = reinterpret_cast<float4v *>(lds);
+#pragma unroll
+    for (int xt = 0; xt < XT; xt++)
+#pragma unroll
+        for (int t = 0; t < kNT; t++)
+            red[((wave * XT + xt) * kNT + t) * 64 + lane] = acc[xt][t];
+    __syncthreads();
+    for (int e = threadIdx.x; e < XT * kNT * 64; e += 512) {
+        const int l = e & 63, xt_t = e >> 6;
+        const int xt = xt_t / kNT, t = xt_t - xt * kNT;
+        float4v s = red[e];
+#pragma unroll
+        for (int u = 1; u < 8; u++)
+            s += red[u * (XT * kNT * 64) + e];
+        const int wr = t * 16 + (l & 15);
+        if (wr < rows_wg && m0 + wr < m) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int r = xt * 16 + (l >> 4) * 4 + j;
+                if (r < nrows)
+                    y[(size_t)(r0 + r) * m + m0 + wr] = s[j];
+            }
+        }
+    }
+}
+
 // ---- gemv_q8_tile_kernel: 3 to 128 activation rows (batched decode, verify groups) --------------
 //
 // The same streaming of W as above, with the activations as full 16-row A tiles: A row = activation
@@ -959,9 +1158,58 @@ static int try_gemv_dma(hipStream_t st, const uint8_t *w, const float *x, float 
     }
 }
 
+template <int XT, int NI>
+static int launch_gemv_dma_tile(hipStream_t st, const uint8_t *w, const float *x, float *y, int m, int k, int rows,
+                                int rows_wg)
+{
+    const dim3 grid((unsigned)((m + rows_wg - 1) / rows_wg), (unsigned)((rows + 16 * XT - 1) / (16 * XT)), 1);
+    HIPML_LAUNCH((gemv_q8_dma_tile_kernel<XT, NI>), grid, dim3(512, 1, 1), (size_t)gemv_dma_tile_lds(XT, NI, rows_wg), st, w, x,
+                 y, m, k, rows, rows_wg);
+    return launched("gemv_q8_0_rows");
+}
+
+template <int NI>
+static int launch_gemv_dma_tiles(hipStream_t st, const uint8_t *w, const float *x, float *y, int m, int k, int rows,
+                                 int rows_wg)
+{
+    // the activation tiles of a pass: as many as the rows need, up to four (more rows: passes of 64)
+    const int xt = rows > 48 ? 4 : (rows + 15) / 16;
+    switch (xt) {
+    case 1: return launch_gemv_dma_tile<1, NI>(st, w, x, y, m, k, rows, rows_wg);
+    case 2: return launch_gemv_dma_tile<2, NI>(st, w, x, y, m, k, rows, rows_wg);
+    case 3: return launch_gemv_dma_tile<3, NI>(st, w, x, y, m, k, rows, rows_wg);
+    default: return launch_gemv_dma_tile<4, NI>(st, w, x, y, m, k, rows, rows_wg);
+    }
+}
+
+// 9 rows and more over the raw-row tile kernel, under the conditions of try_gemv_dma.  Returns -1 where the shape
+// does not qualify.
+static int try_gemv_dma_tile(hipStream_t st, const uint8_t *w, const float *x, float *y, int m, int k, int rows)
+{
+    if (k % 256 != 0 || (reinterpret_cast<uintptr_t>(w) & 15) != 0 || (reinterpret_cast<uintptr_t>(x) & 15) != 0 ||
+        (size_t)m * (k >> 5) * kQ8Block >= ((size_t)1 << 32) || (size_t)rows * k * sizeof(float) >= ((size_t)1 << 32))
+        return -1;
+    static const int kRowsWg[4] = {16, 20, 24, 32};
+    int v = 3;
+    for (int i = 0; i < 4; i++)
+        if ((m + kRowsWg[i] - 1) / kRowsWg[i] <= 256) {
+            v = i;
+            break;
+        }
+    switch (v) {
+    case 0: return launch_gemv_dma_tiles<5>(st, w, x, y, m, k, rows, 16);
+    case 1: return launch_gemv_dma_tiles<6>(st, w, x, y, m, k, rows, 20);
+    case 2: return launch_gemv_dma_tiles<7>(st, w, x, y, m, k, rows, 24);
+    default: return launch_gemv_dma_tiles<9>(st, w, x, y, m, k, rows, 32);
+    }
+}
+
 int launch_gemv_q8_rows(hipStream_t st, const uint8_t *w, const float *x, float *y, int m, int k, int rows)
 {
-    const int dma = try_gemv_dma(st, w, x, y, m, k, rows);
+    // (10 to 64 rows: the raw-row tile kernel; 9 rows, and two passes of 64 for 128, measured slower than the tile
+    // kernel below: 17.2 against 16.0 and 86 against 81 us at 5120 x 6144)
+    const int dma = rows <= 8 ? try_gemv_dma(st, w, x, y, m, k, rows)
+                              : (rows >= 10 && rows <= 64 ? try_gemv_dma_tile(st, w, x, y, m, k, rows) : -1);
     if (dma >= 0)
         return dma;
     // three rows or more: full A tiles of 16 or 32 rows (measured at 5120 x 6144, 4 rows: 14.6 us
@@ -1324,6 +1572,13 @@ int proj_init()
     raise(reinterpret_cast<const void *>(&gemv_q8_dma_kernel<8, ni, 4>));
     HIPML_RAISE_DMA(5) HIPML_RAISE_DMA(6) HIPML_RAISE_DMA(7) HIPML_RAISE_DMA(9)
 #undef HIPML_RAISE_DMA
+#define HIPML_RAISE_TILE(ni) \
+    raise(reinterpret_cast<const void *>(&gemv_q8_dma_tile_kernel<1, ni>)); \
+    raise(reinterpret_cast<const void *>(&gemv_q8_dma_tile_kernel<2, ni>)); \
+    raise(reinterpret_cast<const void *>(&gemv_q8_dma_tile_kernel<3, ni>)); \
+    raise(reinterpret_cast<const void *>(&gemv_q8_dma_tile_kernel<4, ni>));
+    HIPML_RAISE_TILE(5) HIPML_RAISE_TILE(6) HIPML_RAISE_TILE(7) HIPML_RAISE_TILE(9)
+#undef HIPML_RAISE_TILE
     if (e != hipSuccess)
         return fail((int)e, "hipFuncSetAttribute(projection LDS) failed: %d (%s)", (int)e, hipGetErrorString(e));
     return 0;

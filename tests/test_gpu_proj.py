@@ -64,7 +64,7 @@ def test_integer_case_is_exact():
     assert np.array_equal(run_gemv(w.ravel(), x, m, k, rows), want)
 
 
-@pytest.mark.parametrize("rows", [1, 2, 3, 4, 5, 8, 9, 16, 17, 24])
+@pytest.mark.parametrize("rows", [1, 2, 3, 4, 5, 8, 9, 10, 16, 17, 24, 33, 49, 64, 70])
 def test_output_projection_shape(rows):
     # W_o of the model: 6144 -> 5120; activations of the size the gated attention output has
     r = orc.Rng(0x0E00 + rows)
@@ -78,13 +78,16 @@ def test_output_projection_shape(rows):
     # a row does not depend on how many rows travel with it (the reference's batched GEMVs are bit-identical
     # per row to the single-sequence one, so that verify columns match a plain decode:
     # crates/hipml-kernels/src/attn_gpu.rs:930-932): up to 8 rows take one kernel whose per-row arithmetic
-    # does not depend on the row count, more take the tile kernel
+    # does not depend on the row count, more take the tile kernels
     if 2 <= rows <= 8:
         for r in {0, rows - 1}:
             assert np.array_equal(run_gemv(w, x[r], m, k, 1)[0], got[r])
     if rows == 8:
         assert np.array_equal(run_gemv(w, x[2:5], m, k, 3)[1], got[3])
-    if rows == 24:
+    # 10 to 64 rows share one kernel, 9 rows and 65 to 128 another
+    if rows in (24, 64):
+        assert np.array_equal(run_gemv(w, x[3:13], m, k, 10)[2], got[5])
+    if rows == 70:
         assert np.array_equal(run_gemv(w, x[3:12], m, k, 9)[2], got[5])
 
 
