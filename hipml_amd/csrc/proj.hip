@@ -701,7 +701,10 @@ __global__ void __launch_bounds__(64 * WAVES, 1) gemv_q8_dma_kernel(const uint8_
 constexpr int kTileRowPitch = 1040;
 // (chunks of activations / of weights in flight, measured at 5120 x 6144 over 16 / 24 / 32 / 64 rows: 2 / 3: 17.5 / 23.4 /
 // 23.5 / 39.8 us; 2 / 4: 17.9 / 29.0 / 29.1 / 41.4; 3 / 6: 18.3 / 25.5 / 25.6 / -; the tile kernel below: 19.6 / 25.8 / 29.7 /
-// 54.5)
+// 54.5.  The figures for 24 and 32 rows move between 23.4 and 29.6 us from run to run of the same build, those for 16 and 64
+// do not.  Two chunks a turn of the loop, half the barriers: 20.5 / 26.7 / 26.9 against 17.5 / 29.6 / 29.7 in one run; every
+// workgroup starting at another chunk, so that they do not all ask for the same activation bytes at once: 20.8 / 24.3 / 24.5 /
+// 39.2 against 17.4 / 23.4 / 23.5 / 39.7 in one run.)
 constexpr int gemv_tile_dx(int) { return 2; }
 constexpr int gemv_tile_dw(int) { return 3; }
 inline int gemv_dma_tile_lds(int xt, int ni, int rows_wg)
@@ -1196,6 +1199,10 @@ static int try_gemv_dma_tile(hipStream_t st, const uint8_t *w, const float *x, f
             v = i;
             break;
         }
+    static const int kNi[4] = {5, 6, 7, 9};
+    const int xt = rows > 48 ? 4 : (rows + 15) / 16;
+    if (gemv_dma_tile_lds(xt, kNi[v], kRowsWg[v]) > (160 << 10))
+        return -1;
     switch (v) {
     case 0: return launch_gemv_dma_tiles<5>(st, w, x, y, m, k, rows, 16);
     case 1: return launch_gemv_dma_tiles<6>(st, w, x, y, m, k, rows, 20);
