@@ -156,6 +156,12 @@ def counters(workload: str, kernel: str):
         return {}
     for name, v in t.items():
         if kernel in name:
+            if v.get("us", 0.0) < 500.0:
+                # (GRBM_GUI_ACTIVE also counts the cycles around a dispatch: over a launch of tens of microseconds
+                # the quotient is no clock, 2.8 "GHz" for the 25-us kernel)
+                return {"mfma_busy": v.get("mfma_busy"),
+                        "mfma_busy_source": "profiles/mfma_counters.json (SQ_VALU_MFMA_BUSY_CYCLES; a lower bound for a "
+                                            "launch this short)"}
             return {"clock_ghz": v.get("clock_ghz"), "mfma_busy": v.get("mfma_busy"),
                     "clock_source": "profiles/mfma_counters.json (GRBM_GUI_ACTIVE / 8 / kernel duration)"}
     return {}
