@@ -132,6 +132,47 @@ def test_q4_mtp_columns_equal_single_row_decodes(pos0, cols, stride, splits):
         assert np.array_equal(host(single).view(np.uint32), host(out)[c].view(np.uint32))
 
 
+def test_q4_batched_decode_with_mtp_slots():
+    # slots of different depths in one launch (the worker window of the batched decode), two of them verify groups
+    # of 3 and 4 rows, the rows of a slot garbage past its live length; every row against the oracle and bit for
+    # bit against the plain decode of its row with the same split count
+    r = orc.Rng(0x0404_0040)
+    depths = [700, 33, 5000, 1, 2049, 12000, 255, 8191]
+    cols = [3, 1, 1, 1, 4, 1, 1, 1]
+    stride = 12160
+    slots = len(depths)
+    kc = np.zeros((slots, N_KV, stride, ROW4), dtype=np.uint8)
+    vc = np.zeros((slots, N_KV, stride, ROW4), dtype=np.uint8)
+    qs, pos = [], []
+    for s, (d, c) in enumerate(zip(depths, cols)):
+        live = d + c
+        kc[s], vc[s] = q4_cache(r.normal_array((N_KV, live, HD)), r.normal_array((N_KV, live, HD)), stride)
+        for j in range(c):
+            qs.append(r.normal_array((N_HEADS, HD)))
+            pos.append((d + j, d + j + 1))
+    q = np.stack(qs)
+    rows = len(pos)
+    splits = attn.batch_splits(stride, N_KV, slots)
+    acc = torch.full((rows, N_HEADS, splits, HD), float("nan"), device="cuda")
+    ml = torch.full((rows, N_HEADS, splits, 2), float("nan"), device="cuda")
+    out = torch.full((rows, N_HEADS, HD), float("nan"), dtype=torch.float32, device="cuda")
+    kd, vd = dev(kc), dev(vc)
+    attn.attn_decode_batch_cols(Q4, torch.tensor(pos, dtype=torch.int32, device="cuda"), dev(q), kd, vd, acc, ml, out,
+                                N_HEADS, N_KV, HD, stride, SCALE, splits, N_KV * stride * ROW4,
+                                N_HEADS * splits * HD, N_HEADS * splits * 2, N_HEADS * HD, cols)
+    torch.cuda.synchronize()
+    got = host(out)
+    assert np.isfinite(got).all()
+    row = 0
+    for s, c in enumerate(cols):
+        for j in range(c):
+            want = orc.attn_decode_kv(q[row], kc[s], vc[s], N_HEADS, N_KV, HD, pos[row][1], SCALE, dtype=Q4,
+                                      stride=stride)
+            ok, ma, _ = orc.compare(want, got[row].ravel(), *KERNEL_CLASS)
+            assert ok, f"slot {s} row {j} seq {pos[row][1]}: max_abs {ma}"
+            row += 1
+
+
 @pytest.mark.parametrize("tok,pos0,pad,splits", [(37, 29, 5, 1), (37, 29, 5, 4), (200, 0, 0, 3),
                                                  (96, 3000, 40, 2)])
 def test_q4_chunk_prefill_matches_oracle(tok, pos0, pad, splits):
