@@ -147,6 +147,26 @@ def test_raw_row_kernel_over_ragged_shapes(m, k):
             assert np.array_equal(got[i], alone[i]), f"rows={rows} row {i}"
 
 
+@pytest.mark.parametrize("rows", [1, 4, 12])
+def test_weights_at_a_4_byte_aligned_address(rows):
+    # the raw-row kernels want W at a 16-byte boundary; a matrix that only meets the interface's 4-byte alignment
+    # takes the kernels that load it in dwords, with the same answer class
+    r = orc.Rng(0x0A11 + rows)
+    m, k = 96, 1024
+    w = orc.random_q8_0_bytes(r, m * k // 32)
+    x = r.normal_array((rows, k), 0.5)
+    want = orc.gemm_q8_0(w, x, rows, m, k)
+    buf = torch.zeros(w.size + 16, dtype=torch.uint8, device="cuda")
+    buf[4:4 + w.size] = torch.from_numpy(w).cuda()
+    wd = buf[4:4 + w.size]
+    assert wd.data_ptr() % 16 == 4
+    y = torch.full((rows, m), float("nan"), dtype=torch.float32, device="cuda")
+    attn.gemv_q8_0_rows(wd, dev(x), y, m, k, rows)
+    torch.cuda.synchronize()
+    ok, _, _ = report(f"W at +4 bytes, rows={rows}", want, host(y), *DEFAULT)
+    assert ok
+
+
 def test_argument_errors():
     w = torch.zeros(34 * 4, dtype=torch.uint8, device="cuda")
     x = torch.zeros(64, device="cuda")
