@@ -126,6 +126,9 @@ def timed(torch, fn, steps, warm=3, wall=False, min_ms=MIN_TIMED_MS):
     return total / n, total, n
 
 
+GRAPH_CAPTURE_FAILED = []  # messages of captures that failed (the figures concerned were then timed eagerly)
+
+
 def timed_graph(torch, fn, calls, min_ms=MIN_TIMED_MS):
     """Mean duration of fn(i) in ms with fn(0) .. fn(calls - 1) captured once in a HIP graph and the graph
     replayed until `min_ms` of work have been timed (HIP events around the replays): what the launches cost when
@@ -138,10 +141,15 @@ def timed_graph(torch, fn, calls, min_ms=MIN_TIMED_MS):
             fn(i)
     torch.cuda.current_stream().wait_stream(side)
     torch.cuda.synchronize()
-    graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph):
-        for i in range(calls):
-            fn(i)
+    try:
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for i in range(calls):
+                fn(i)
+    except Exception as e:  # (no box has refused a capture so far; if one does, say so and time the calls one by one)
+        GRAPH_CAPTURE_FAILED.append(repr(e))
+        torch.cuda.synchronize()
+        return timed(torch, fn, calls, min_ms=min_ms)
     ms, total, n = timed(torch, lambda i: graph.replay(), 2, 2, min_ms=min_ms)
     return ms / calls, total, n * calls
 
@@ -1030,6 +1038,8 @@ def main() -> int:
         if not args.main_only:
             line["cpu_baseline"]["decode_us_per_layer"] = {
                 "8192": cpu_decode(orc, 8192), "32768": cpu_decode(orc, 32768)}
+    if GRAPH_CAPTURE_FAILED:
+        line["graph_capture_failed"] = GRAPH_CAPTURE_FAILED
     print(json.dumps(line))
     return 0
 
