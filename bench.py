@@ -812,8 +812,10 @@ def bench_gemv(torch, attn, rows, steps, layers, m=5120, k=6144):
             "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": gbs / HBM_PEAK_GBS,
                          "traffic": measured_traffic({1: "gemv1", 24: "gemv24"}.get(rows, ""),
-                                                     ["gemv_q8_dma_kernel", "gemv_q8_rows_kernel", "gemv_q8_tile_kernel"]),
-                         "kernel": "gemv_q8_dma_kernel" if rows <= 8 else "gemv_q8_tile_kernel",
+                                                     ["gemv_q8_dma_kernel", "gemv_q8_dma_tile_kernel", "gemv_q8_rows_kernel",
+                                                      "gemv_q8_tile_kernel"]),
+                         "kernel": ("gemv_q8_dma_kernel" if rows <= 8 else
+                                    "gemv_q8_dma_tile_kernel" if 10 <= rows <= 64 else "gemv_q8_tile_kernel"),
                          "bytes_per_launch": nbytes, "launch_us": us}}
 
 

@@ -704,7 +704,8 @@ constexpr int kTileRowPitch = 1040;
 // 54.5.  The figures for 24 and 32 rows move between 23.4 and 29.6 us from run to run of the same build, those for 16 and 64
 // do not.  Two chunks a turn of the loop, half the barriers: 20.5 / 26.7 / 26.9 against 17.5 / 29.6 / 29.7 in one run; every
 // workgroup starting at another chunk, so that they do not all ask for the same activation bytes at once: 20.8 / 24.3 / 24.5 /
-// 39.2 against 17.4 / 23.4 / 23.5 / 39.7 in one run.)
+// 39.2 against 17.4 / 23.4 / 23.5 / 39.7 in one run.  Not fetching the 8 rows of a last tile that has no more than 8 live
+// ones (HALF): 17 and 24 rows 21.9 us where 32 rows take 23.5, 33 and 40 rows 34.7 / 34.8 where 48 take 35.1.)
 constexpr int gemv_tile_dx(int) { return 2; }
 constexpr int gemv_tile_dw(int) { return 3; }
 inline int gemv_dma_tile_lds(int xt, int ni, int rows_wg)
@@ -714,7 +715,7 @@ inline int gemv_dma_tile_lds(int xt, int ni, int rows_wg)
     return ring > sums ? ring : sums;
 }
 
-template <int XT, int NI>
+template <int XT, int NI, bool HALF>
 __global__ void __launch_bounds__(512, 1) gemv_q8_dma_tile_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x,
                                                                    float *__restrict__ y, int m, int k, int rows,
                                                                    int rows_wg)
@@ -723,7 +724,9 @@ __global__ void __launch_bounds__(512, 1) gemv_q8_dma_tile_kernel(const uint8_t 
     constexpr int kXRows = 16 * XT;
     constexpr int kDX = gemv_tile_dx(XT), kDW = gemv_tile_dw(XT);
     static_assert(kDW > kDX, "a chunk's weights are asked for before its activations");
-    constexpr int kNX = 2 * XT;              // activation requests of a wave per chunk (one per row, 16 XT rows)
+    // activation requests of a wave per chunk: one per row, 16 XT rows, or 8 fewer (HALF: the last tile has at most
+    // 8 live rows; the other 8 are never fetched, hold whatever the ring held, and their sums are never stored)
+    constexpr int kNX = 2 * XT - (HALF ? 1 : 0);
     constexpr int kWMost = (NI + 7) / 8;     // weight requests of a wave per chunk, or one less
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
@@ -1166,8 +1169,11 @@ static int launch_gemv_dma_tile(hipStream_t st, const uint8_t *w, const float *x
                                 int rows_wg)
 {
     const dim3 grid((unsigned)((m + rows_wg - 1) / rows_wg), (unsigned)((rows + 16 * XT - 1) / (16 * XT)), 1);
-    HIPML_LAUNCH((gemv_q8_dma_tile_kernel<XT, NI>), grid, dim3(512, 1, 1), (size_t)gemv_dma_tile_lds(XT, NI, rows_wg), st, w, x,
-                 y, m, k, rows, rows_wg);
+    const size_t lds = (size_t)gemv_dma_tile_lds(XT, NI, rows_wg);
+    if (grid.y == 1 && rows <= 16 * XT - 8)
+        HIPML_LAUNCH((gemv_q8_dma_tile_kernel<XT, NI, true>), grid, dim3(512, 1, 1), lds, st, w, x, y, m, k, rows, rows_wg);
+    else
+        HIPML_LAUNCH((gemv_q8_dma_tile_kernel<XT, NI, false>), grid, dim3(512, 1, 1), lds, st, w, x, y, m, k, rows, rows_wg);
     return launched("gemv_q8_0_rows");
 }
 
@@ -1580,10 +1586,14 @@ int proj_init()
     HIPML_RAISE_DMA(5) HIPML_RAISE_DMA(6) HIPML_RAISE_DMA(7) HIPML_RAISE_DMA(9)
 #undef HIPML_RAISE_DMA
 #define HIPML_RAISE_TILE(ni) \
-    raise(reinterpret_cast<const void *>(&gemv_q8_dma_tile_kernel<1, ni>)); \
-    raise(reinterpret_cast<const void *>(&gemv_q8_dma_tile_kernel<2, ni>)); \
-    raise(reinterpret_cast<const void *>(&gemv_q8_dma_tile_kernel<3, ni>)); \
-    raise(reinterpret_cast<const void *>(&gemv_q8_dma_tile_kernel<4, ni>));
+    raise(reinterpret_cast<const void *>(&gemv_q8_dma_tile_kernel<1, ni, false>)); \
+    raise(reinterpret_cast<const void *>(&gemv_q8_dma_tile_kernel<2, ni, false>)); \
+    raise(reinterpret_cast<const void *>(&gemv_q8_dma_tile_kernel<3, ni, false>)); \
+    raise(reinterpret_cast<const void *>(&gemv_q8_dma_tile_kernel<4, ni, false>)); \
+    raise(reinterpret_cast<const void *>(&gemv_q8_dma_tile_kernel<1, ni, true>)); \
+    raise(reinterpret_cast<const void *>(&gemv_q8_dma_tile_kernel<2, ni, true>)); \
+    raise(reinterpret_cast<const void *>(&gemv_q8_dma_tile_kernel<3, ni, true>)); \
+    raise(reinterpret_cast<const void *>(&gemv_q8_dma_tile_kernel<4, ni, true>));
     HIPML_RAISE_TILE(5) HIPML_RAISE_TILE(6) HIPML_RAISE_TILE(7) HIPML_RAISE_TILE(9)
 #undef HIPML_RAISE_TILE
     if (e != hipSuccess)
