@@ -61,8 +61,13 @@ __device__ __forceinline__ void split_hi_lo(const float4v &a, const float4v &b, 
         const float x0 = j < 2 ? a[2 * j] : b[2 * j - 4];
         const float x1 = j < 2 ? a[2 * j + 1] : b[2 * j - 3];
         const half2v h = __builtin_bit_cast(half2v, __builtin_amdgcn_cvt_pkrtz(x0, x1));
-        const half2v l =
-            __builtin_bit_cast(half2v, __builtin_amdgcn_cvt_pkrtz(x0 - (float)h[0], x1 - (float)h[1]));
+        // x - h (exact: h holds the leading bits of x) in one mixed-precision instruction per value, which reads
+        // the f16 half in place; the compiler turns the same expression into a conversion and a subtraction
+        const uint32_t hb = __builtin_bit_cast(uint32_t, h);
+        float r0, r1;
+        asm("v_fma_mix_f32 %0, -%1, 1.0, %2 op_sel_hi:[1,0,0]" : "=v"(r0) : "v"(hb), "v"(x0));
+        asm("v_fma_mix_f32 %0, -%1, 1.0, %2 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(r1) : "v"(hb), "v"(x1));
+        const half2v l = __builtin_bit_cast(half2v, __builtin_amdgcn_cvt_pkrtz(r0, r1));
         hi[2 * j] = h[0];
         hi[2 * j + 1] = h[1];
         lo[2 * j] = l[0];
@@ -756,6 +761,10 @@ __global__ void __launch_bounds__(512, 1) gemv_q8_dma_tile_kernel(const uint8_t 
         const int row = m0 + pr < m ? m0 + pr : m - 1;
         woff[j] = (uint32_t)row * row_bytes + (uint32_t)pq * 16u;
     }
+    int wreq = 0; // weight requests of this wave per chunk
+#pragma unroll
+    for (int j = 0; j < kWMost; j++)
+        wreq += wave + 8 * j < NI ? 1 : 0;
     auto issue_w = [&](int c) {
         const uint32_t at = wring_at + (uint32_t)((c % kDW) * wbytes);
 #pragma unroll
@@ -801,18 +810,28 @@ __global__ void __launch_bounds__(512, 1) gemv_q8_dma_tile_kernel(const uint8_t 
     const int b = wave; // this wave's block of every chunk
 
     for (int c = 0; c < nchunk; c++) {
-        // this wave's requests for chunk c have arrived: behind its activation requests of chunk c there are, among
-        // others, those of the chunks up to c + kDX - 1 that exist (counting only those errs on the side of waiting)
+        // This wave's requests for chunk c have arrived once only those made after them are outstanding.  In the
+        // steady state these are, in order, the weights of chunk c + 1, then per chunk finished since (kDX of them)
+        // the activations and the weights asked for behind it: kDX - 1 sets of activations and kDX of weights in
+        // all.  Counting the activation sets alone waits for requests made a chunk ago as well; measured at 16 / 24 /
+        // 48 / 64 rows: 17.5 / 21.9 / 35.1 / 39.7 us so, 17.5 / 23.2 / 31.2 / 35.7 with the full count, hence the full
+        // count from three activation tiles on.  At the ends, where some of those chunks do not exist, only the
+        // activation sets that do are counted, which errs on the side of waiting.
         {
+            static_assert(kDX == 2 && kDW == 3 && kWMost <= 2, "the counts below");
             const int behind = nchunk - 1 - c < kDX - 1 ? nchunk - 1 - c : kDX - 1;
-            if (behind >= 3 && kDX > 3)
-                wait_vm<(kDX > 3 ? 3 : 0) * kNX>();
-            else if (behind >= 2 && kDX > 2)
-                wait_vm<(kDX > 2 ? 2 : 0) * kNX>();
-            else if (behind >= 1)
+            if (XT >= 3 && c >= kDX && c + kDW - 1 < nchunk) {
+                if (wreq == 0)
+                    wait_vm<kNX>();
+                else if (wreq == 1)
+                    wait_vm<kNX + kDX>();
+                else
+                    wait_vm<kNX + 2 * kDX>();
+            } else if (behind >= 1) {
                 wait_vm<kNX>();
-            else
+            } else {
                 wait_vm<0>();
+            }
         }
         __syncthreads(); // ... and every wave's
         const uint8_t *wbuf = wring + (c % kDW) * wbytes;
