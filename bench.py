@@ -815,7 +815,7 @@ def bench_gemv(torch, attn, rows, steps, layers, m=5120, k=6144):
                                                      ["gemv_q8_dma_kernel", "gemv_q8_dma_tile_kernel", "gemv_q8_rows_kernel",
                                                       "gemv_q8_tile_kernel"]),
                          "kernel": ("gemv_q8_dma_kernel" if rows <= 8 else
-                                    "gemv_q8_dma_tile_kernel" if 10 <= rows <= 64 else "gemv_q8_tile_kernel"),
+                                    "gemv_q8_dma_tile_kernel" if rows >= 10 else "gemv_q8_tile_kernel"),
                          "bytes_per_launch": nbytes, "launch_us": us}}
 
 

@@ -686,7 +686,7 @@ __global__ void __launch_bounds__(64 * WAVES, 1) gemv_q8_dma_kernel(const uint8_
     }
 }
 
-// ---- gemv_q8_dma_tile_kernel: 9 to 64 activation rows over the same stream of raw weight rows ------------------
+// ---- gemv_q8_dma_tile_kernel: 10 to 128 activation rows over the same stream of raw weight rows, 64 a pass ------
 //
 // More rows than the kernel above holds operands for.  The workgroups are the same (rows_wg consecutive weight
 // rows, one workgroup per CU, eight waves), but the waves walk the chunks together: for a chunk of 256 values the
@@ -1183,6 +1183,12 @@ static int try_gemv_dma(hipStream_t st, const uint8_t *w, const float *x, float 
     }
 }
 
+static int gemv_tile_xt(int rows)
+{
+    const int pass = rows > 64 ? (rows + 1) / 2 : rows;
+    return (pass + 15) / 16;
+}
+
 template <int XT, int NI>
 static int launch_gemv_dma_tile(hipStream_t st, const uint8_t *w, const float *x, float *y, int m, int k, int rows,
                                 int rows_wg)
@@ -1200,8 +1206,9 @@ template <int NI>
 static int launch_gemv_dma_tiles(hipStream_t st, const uint8_t *w, const float *x, float *y, int m, int k, int rows,
                                  int rows_wg)
 {
-    // the activation tiles of a pass: as many as the rows need, up to four (more rows: passes of 64)
-    const int xt = rows > 48 ? 4 : (rows + 15) / 16;
+    // the activation tiles of a pass: as many as the rows need, up to four; more than 64 rows: two passes (the
+    // grid's second dimension) that share the rows evenly
+    const int xt = gemv_tile_xt(rows);
     switch (xt) {
     case 1: return launch_gemv_dma_tile<1, NI>(st, w, x, y, m, k, rows, rows_wg);
     case 2: return launch_gemv_dma_tile<2, NI>(st, w, x, y, m, k, rows, rows_wg);
@@ -1225,7 +1232,7 @@ static int try_gemv_dma_tile(hipStream_t st, const uint8_t *w, const float *x, f
             break;
         }
     static const int kNi[4] = {5, 6, 7, 9};
-    const int xt = rows > 48 ? 4 : (rows + 15) / 16;
+    const int xt = gemv_tile_xt(rows);
     if (gemv_dma_tile_lds(xt, kNi[v], kRowsWg[v]) > (160 << 10))
         return -1;
     switch (v) {
@@ -1238,10 +1245,10 @@ static int try_gemv_dma_tile(hipStream_t st, const uint8_t *w, const float *x, f
 
 int launch_gemv_q8_rows(hipStream_t st, const uint8_t *w, const float *x, float *y, int m, int k, int rows)
 {
-    // (10 to 64 rows: the raw-row tile kernel; 9 rows, and two passes of 64 for 128, measured slower than the tile
-    // kernel below: 17.2 against 16.0 and 86 against 81 us at 5120 x 6144)
+    // (10 rows and more: the raw-row tile kernel, in two passes beyond 64; 9 rows measured slower there than in the
+    // tile kernel below: 17.2 against 16.0 us at 5120 x 6144)
     const int dma = rows <= 8 ? try_gemv_dma(st, w, x, y, m, k, rows)
-                              : (rows >= 10 && rows <= 64 ? try_gemv_dma_tile(st, w, x, y, m, k, rows) : -1);
+                              : (rows >= 10 && rows <= 128 ? try_gemv_dma_tile(st, w, x, y, m, k, rows) : -1);
     if (dma >= 0)
         return dma;
     // three rows or more: full A tiles of 16 or 32 rows (measured at 5120 x 6144, 4 rows: 14.6 us

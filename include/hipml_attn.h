@@ -508,9 +508,9 @@ int hipml_kv_rows_copy(hipml_stream_t stream, int dtype, const void *k_src, cons
  * every row has the precision class of the reference's f32 GEMV kernels.  Up to 8 rows W streams from
  * memory once and a row's result has the same bits whatever `rows` is and whichever rows travel with it:
  * the rows of a verify group match their plain decodes, as the reference's batched GEMVs do
- * (crates/hipml-kernels/src/attn_gpu.rs:930-932).  From 10 to 64 rows W also streams once and a row's bits
- * are the same for every such `rows`; 9 rows and 65 to 128 rows stream W once per 16 or 32 rows, again with the
- * same bits within that class.  The three classes differ from each other in the last bits.
+ * (crates/hipml-kernels/src/attn_gpu.rs:930-932).  From 10 to 128 rows W streams once per pass of up to 64 rows
+ * (two passes beyond 64) and a row's bits are the same for every such `rows`; 9 rows take a kernel of their own.
+ * The three classes differ from each other in the last bits.
  * (W at a 16-byte aligned address and k a multiple of 256 take the fastest road.)
  * Replaces AttnLayer::gemv / gemv_rows / gemv_batched over a Q8_0 ResidentMat (the output
  * projection of apply_output / output_rows, and W_q, W_k, W_v in prepare_rows),

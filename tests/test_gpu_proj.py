@@ -64,7 +64,7 @@ def test_integer_case_is_exact():
     assert np.array_equal(run_gemv(w.ravel(), x, m, k, rows), want)
 
 
-@pytest.mark.parametrize("rows", [1, 2, 3, 4, 5, 8, 9, 10, 16, 17, 24, 33, 49, 64, 70])
+@pytest.mark.parametrize("rows", [1, 2, 3, 4, 5, 8, 9, 10, 16, 17, 24, 33, 49, 64, 70, 128])
 def test_output_projection_shape(rows):
     # W_o of the model: 6144 -> 5120; activations of the size the gated attention output has
     r = orc.Rng(0x0E00 + rows)
@@ -84,11 +84,10 @@ def test_output_projection_shape(rows):
             assert np.array_equal(run_gemv(w, x[r], m, k, 1)[0], got[r])
     if rows == 8:
         assert np.array_equal(run_gemv(w, x[2:5], m, k, 3)[1], got[3])
-    # 10 to 64 rows share one kernel, 9 rows and 65 to 128 another
-    if rows in (24, 64):
+    # 10 to 128 rows share one kernel (two passes of it beyond 64), 9 rows take another
+    if rows in (24, 64, 70, 128):
         assert np.array_equal(run_gemv(w, x[3:13], m, k, 10)[2], got[5])
-    if rows == 70:
-        assert np.array_equal(run_gemv(w, x[3:12], m, k, 9)[2], got[5])
+        assert np.array_equal(run_gemv(w, x[rows - 10:], m, k, 10)[9], got[rows - 1])
 
 
 def test_ragged_shapes_and_scales():
