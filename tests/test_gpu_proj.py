@@ -146,6 +146,35 @@ def test_raw_row_kernel_over_ragged_shapes(m, k):
             assert np.array_equal(got[i], alone[i]), f"rows={rows} row {i}"
 
 
+@pytest.mark.parametrize("m,k", [(100, 2304), (5121, 1024), (300, 8192)])
+def test_raw_row_tile_kernel_over_row_counts(m, k):
+    # 10 to 128 rows over the tile kernel that moves the weight rows into LDS as they lie: one to four activation
+    # tiles, a last tile with at most 8 live rows (whose other rows are not fetched), two passes beyond 64 rows with
+    # a short second pass; real scales.  Every row count against the oracle, and a row's bits the same whatever
+    # travels with it and whichever pass and tile it falls in.
+    r = orc.Rng(0x711E + m + k)
+    w = orc.random_q8_0_bytes(r, m * k // 32).reshape(-1, 34)
+    scales = (r.uniform_array(w.shape[0]) * 0.05 + 0.001).astype(np.float16)
+    w[:, :2] = scales.view(np.uint8).reshape(-1, 2)
+    w = w.ravel()
+    x = r.normal_array((128, k), 0.25)  # (outputs of magnitude ~40: two fp32 summation orders stay inside the gate)
+    want = orc.gemm_q8_0(w, x, 128, m, k, n_threads=8)
+    blocks = w.reshape(m, k // 32, 34)
+    dense = (blocks[:, :, :2].copy().view(np.float16).astype(np.float64)
+             * blocks[:, :, 2:].view(np.int8).astype(np.float64)).reshape(m, k)
+    exact = x.astype(np.float64) @ dense.T
+    full = run_gemv(w, x, m, k, 128)
+    for rows in (10, 16, 17, 24, 32, 33, 40, 48, 49, 64, 65, 80, 96, 97, 127):
+        got = run_gemv(w, x[:rows], m, k, rows)
+        ok, _, _ = report(f"raw-row tiles {m}x{k} rows={rows}", want[:rows], got, 2e-3, 3e-2)
+        assert ok
+        bound = max(2 * np.max(np.abs(want[:rows] - exact[:rows])), 2e-6 * np.max(np.abs(exact[:rows])) + 1e-5)
+        assert np.max(np.abs(got - exact[:rows])) <= bound
+        assert np.array_equal(got, full[:rows]), f"rows={rows}"
+    # rows taken from the middle: other tiles, other passes
+    assert np.array_equal(run_gemv(w, x[60:75], m, k, 15), full[60:75])
+
+
 @pytest.mark.parametrize("rows", [1, 4, 12])
 def test_weights_at_a_4_byte_aligned_address(rows):
     # the raw-row kernels want W at a 16-byte boundary; a matrix that only meets the interface's 4-byte alignment
