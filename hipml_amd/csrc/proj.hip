@@ -710,7 +710,8 @@ constexpr int kTileRowPitch = 1040;
 // do not.  Two chunks a turn of the loop, half the barriers: 20.5 / 26.7 / 26.9 against 17.5 / 29.6 / 29.7 in one run; every
 // workgroup starting at another chunk, so that they do not all ask for the same activation bytes at once: 20.8 / 24.3 / 24.5 /
 // 39.2 against 17.4 / 23.4 / 23.5 / 39.7 in one run.  Not fetching the 8 rows of a last tile that has no more than 8 live
-// ones (HALF): 17 and 24 rows 21.9 us where 32 rows take 23.5, 33 and 40 rows 34.7 / 34.8 where 48 take 35.1.)
+// ones (HALF): 17 and 24 rows 21.9 us where 32 rows take 23.5, 33 and 40 rows 34.7 / 34.8 where 48 take 35.1.  Sixteen waves,
+// two per block of a chunk with one weight tile each: 18.4 / 24.9 / 45.9 us at 16 / 24 / 64 rows against 17.0 / 22.7 / 34.0.)
 constexpr int gemv_tile_dx(int) { return 2; }
 constexpr int gemv_tile_dw(int) { return 3; }
 inline int gemv_dma_tile_lds(int xt, int ni, int rows_wg)
